@@ -1,0 +1,123 @@
+/* libtmb_hip — C ABI of the MI355X (gfx950) kernels behind torch_mojo_backend's hot ATen ops.
+ *
+ * Conventions (shared by every entry point):
+ *   - plain pointers are DEVICE pointers supplied by the caller; the caller owns every buffer,
+ *     outputs included (the reference's "classic" raw-pointer ABI, e.g.
+ *     torch_mojo_backend/eager_kernels/aten_fast.py:2763-2776 and :4588-4600);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the legacy default stream); launches
+ *     are asynchronous and never synchronise, like the reference's enqueue-and-return kernels
+ *     (torch_mojo_backend/eager_kernels/__init__.py:9-12);
+ *   - dtypes cross as `tmb_dtype` ints;
+ *   - the return value is 0 on success, a negative `tmb_status` for argument errors detected
+ *     on the host before anything is enqueued, or a positive hipError_t from the launch.
+ *   - no entry point allocates or frees device memory; kernels that need scratch take a
+ *     caller-provided workspace whose size `tmb_*_workspace_bytes` reports.
+ */
+#ifndef TMB_HIP_H_
+#define TMB_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tmb_dtype {
+  TMB_F32 = 0,
+  TMB_F16 = 1,
+  TMB_BF16 = 2,
+  TMB_I64 = 3,
+  TMB_I32 = 4
+} tmb_dtype;
+
+typedef enum tmb_status {
+  TMB_OK = 0,
+  TMB_ERR_INVALID_ARGUMENT = -1, /* null pointer, negative size, unknown enum */
+  TMB_ERR_UNSUPPORTED = -2,      /* well-formed request this build has no kernel for */
+  TMB_ERR_WORKSPACE = -3         /* workspace missing or too small */
+} tmb_status;
+
+typedef enum tmb_reduce_op { TMB_SUM = 0, TMB_MEAN = 1, TMB_AMAX = 2 } tmb_reduce_op;
+
+typedef enum tmb_epilogue {
+  TMB_EPI_NONE = 0,
+  TMB_EPI_GELU_TANH = 1, /* 0.5*x*(1+tanh(sqrt(2/pi)*(x+0.044715*x^3))) applied after bias */
+  TMB_EPI_GELU_ERF = 2   /* 0.5*x*(1+erf(x/sqrt(2))) applied after bias */
+} tmb_epilogue;
+
+/* Library/ABI version (major*1000 + minor). */
+int tmb_version(void);
+
+/* Human-readable text for a return code of any entry point (static storage). */
+const char* tmb_status_string(int code);
+
+/* Row softmax / log-softmax over the last (contiguous) dimension of a [rows, cols] matrix.
+ * fp32 arithmetic, one cast on store: m = max_j x; s = sum_j exp(x - m);
+ * softmax = exp(x - m)/s, log_softmax = x - m - log(s).
+ * `in_dtype` in {F32,F16,BF16}; `out_dtype` equals `in_dtype` or F32 (half_to_float).
+ * Replaces nn_ops.mojo:413-493 (`_softmax_rows`, scale=1, causal=0) behind SoftmaxSpec
+ * (nn_ops.mojo:2818-2864) and reduction_ops.mojo:778-933 (`_log_softmax_rows`). */
+int tmb_softmax_rows(void* out, const void* in, int64_t rows, int64_t cols, int in_dtype,
+                     int out_dtype, int log_mode, void* stream);
+
+/* Layer norm over the last dimension of [rows, cols]: two-pass fp32 statistics
+ * (mean = sum(x)/cols, var = sum((x-mean)^2)/cols biased, rstd = 1/sqrt(var+eps)),
+ * out = (x-mean)*rstd*gamma + beta cast once. `gamma`/`beta` may be NULL (no affine);
+ * `mean`/`rstd` ([rows] fp32) may be NULL when the caller proved them dead.
+ * Replaces normalization_forward_ops.mojo `LayerNormForwardF32`
+ * (called at aten_fast.py:2763-2776) and nn_ops.mojo:208-346 `LayerNorm` (aten_fast.py:2783-2793). */
+int tmb_layer_norm_rows(void* out, float* mean, float* rstd, const void* x, const void* gamma,
+                        const void* beta, int64_t rows, int64_t cols, double eps, int dtype,
+                        void* stream);
+
+/* Bytes of device workspace `tmb_reduce_rows` / `tmb_argmax_rows` need for a shape (may be 0). */
+size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+
+/* Row reduction of [rows, cols] (cols contiguous) to [rows]; a full reduction is rows == 1.
+ * Floats accumulate in fp32 and are cast once (F32/F16/BF16); I64 sums and I64/I32 maxima use
+ * their own type. The combine order is a fixed tree that depends only on (rows, cols), so
+ * results are bit-reproducible. MEAN is the fp32 sum divided by cols.
+ * AMAX propagates NaN. Replaces reduction_ops.mojo:161-263 (`_reduce_rows`), nn_ops.mojo:981-1027
+ * (`_mean_rows`) behind SumSpec/MeanSpec/AmaxSpec (reduction_ops.mojo:1094-1184). */
+int tmb_reduce_rows(void* out, const void* in, int64_t rows, int64_t cols, int op, int dtype,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* First-occurrence argmax of every row of [rows, cols] to int64 [rows]; NaN counts as the
+ * maximum (first NaN wins), otherwise greater value wins and equal values keep the lower index
+ * at every stage of the tree. `dtype` in {F32,F16,BF16,I64,I32}.
+ * Replaces nn_ops.mojo:1424-1522 (`_argmax_rows`) behind ArgmaxSpec (nn_ops.mojo:2599-2653). */
+int tmb_argmax_rows(int64_t* out, const void* in, int64_t rows, int64_t cols, int dtype,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Batched GEMM  C[b] = epilogue(op(A[b]) . op(B[b]) + bias)  with fp32 accumulation; bias
+ * (length n, same dtype, may be NULL) is added in fp32 before the single down-cast
+ * (matmul_ops.mojo:2651-2657). Logical shapes: op(A) is [m,k], op(B) is [k,n], C is [m,n]
+ * row-major with leading dimension ldc. `trans_a`/`trans_b` = 0: the operand is stored
+ * row-major as its logical shape ([m,k] with lda / [k,n] with ldb); = 1: stored as the
+ * transpose ([k,m] with lda / [n,k] with ldb — the layout of a torch `weight.t()` view).
+ * stride_* are element strides between batch entries (stride 0 broadcasts an operand).
+ * `dtype` in {F32,F16,BF16} for A, B, bias and C alike.
+ * Replaces the raw-pointer GEMM bridges `Bf16GemmBF16` (aten_fast.py:4588-4600),
+ * `Bf16BmmBF16` (aten_fast.py:4707-4721) and MatmulSpec/MatmulBiasSpec/BmmSpec
+ * (matmul_ops.mojo:3451-3636). */
+int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t batch, int64_t m,
+             int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+             int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
+             int epilogue, void* stream);
+
+/* Elementwise GELU over `numel` contiguous elements, fp32 inside, one cast.
+ * `approximate_tanh` != 0 selects the tanh form. Replaces activation_forward_kernels.mojo:22-56
+ * (used when the GELU cannot be fused into the producing GEMM's epilogue). */
+int tmb_gelu(void* out, const void* in, int64_t numel, int dtype, int approximate_tanh,
+             void* stream);
+
+/* Plain device copy kernel (16-byte vectors, grid-stride) — the bandwidth yardstick the
+ * benchmark and the counter calibration use. No reference counterpart. */
+int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TMB_HIP_H_ */

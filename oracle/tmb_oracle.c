@@ -1,0 +1,268 @@
+/* CPU oracle for the hot ATen ops — TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load this library;
+ * it is the checker the HIP kernels are compared with, never a fallback for them.
+ *
+ * Each function restates, in plain C, the arithmetic of one CPU kernel body of the reference
+ * (paths relative to torch_mojo_backend/eager_kernels/):
+ *   orc_gemm        matmul_ops.mojo:2671-2720  (_cpu_gemm_naive: sequential-k fp32 accumulate,
+ *                                               bias added in fp32, one cast) and :2651-2657
+ *   orc_softmax     nn_ops.mojo:428-455        (max, sum of exp(x-m), exp(x-m)/denom; fp32)
+ *                   reduction_ops.mojo:874-895 (log-softmax: x - m - log(denom))
+ *   orc_layer_norm  nn_ops.mojo:299-326        (two-pass mean / centered variance, fp32) with the
+ *                                               NaN-mean rule of normalization_forward_kernels.mojo:60-70
+ *   orc_reduce      reduction_ops.mojo:161-194 (fp32 accumulator for floats, own type for ints,
+ *                                               one cast) and nn_ops.mojo:981-1027 (mean)
+ *   orc_argmax      nn_ops.mojo:1488-1505      (sequential strict-greater scan from index 0).
+ *                   Deviation, on purpose: a NaN counts as the maximum (first NaN wins), which
+ *                   is what ATen does and what the reference's tests compare with; the
+ *                   reference's scan only keeps a NaN that sits at index 0.
+ *   orc_gelu        activation_forward_kernels.mojo:22-56 (fp32 inside, one cast)
+ *
+ * Pinning: tests/test_oracle_pins.py checks every function against float64 closed forms,
+ * brute-force Python loops on tiny inputs, mathematical invariants and PyTorch CPU eager (the
+ * comparison the reference's own tests make, torch_mojo_backend/testing.py:186-229), and against
+ * the fixtures under tests/golden/. The low-order bits of Modular MAX's CPU kernels (a
+ * third-party dependency that is not part of the reference tree) are not observable here, so
+ * bit-level parity with MAX is "parity unpinned"; parity is pinned at assert_close tolerances.
+ *
+ * dtype codes match include/tmb_hip.h: 0 f32, 1 f16, 2 bf16, 3 i64, 4 i32.
+ * Rows are processed in parallel with OpenMP when compiled with -fopenmp.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2, ORC_I64 = 3, ORC_I32 = 4 };
+enum { ORC_SUM = 0, ORC_MEAN = 1, ORC_AMAX = 2 };
+enum { ORC_EPI_NONE = 0, ORC_EPI_GELU_TANH = 1, ORC_EPI_GELU_ERF = 2 };
+
+static float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+static float bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+static uint16_t f32_to_bf16(float f) {
+  uint32_t u = f32_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+  u += 0x7fffu + ((u >> 16) & 1u); /* round to nearest even */
+  return (uint16_t)(u >> 16);
+}
+static float f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu, man = h & 0x3ffu;
+  if (exp == 0) {
+    if (man == 0) return bits_f32(sign);
+    float v = (float)man * 5.9604644775390625e-08f; /* 2^-24 */
+    return sign ? -v : v;
+  }
+  if (exp == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+  return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+static uint16_t f32_to_f16(float f) {
+  uint32_t u = f32_bits(f);
+  uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);            /* NaN */
+  if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);           /* >= 65536 -> inf (65520 rounds below) */
+  if (a < 0x33000000u) return sign;                                   /* < 2^-25 -> 0 */
+  int e = (int)(a >> 23) - 127;
+  uint32_t man = (a & 0x7fffffu) | 0x800000u;
+  int shift;
+  uint32_t base;
+  if (e < -14) { shift = 13 + (-14 - e); base = 0; }                  /* subnormal half */
+  else { shift = 13; base = (uint32_t)(e + 15) << 10; man &= 0x7fffffu; }
+  uint32_t q = man >> shift, rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1u))) q++;
+  uint32_t r = base + q; /* carry into the exponent is the right answer, incl. -> inf */
+  return (uint16_t)(sign | r);
+}
+
+static float load_f(const void* p, int64_t i, int dtype) {
+  switch (dtype) {
+    case ORC_F32: return ((const float*)p)[i];
+    case ORC_F16: return f16_to_f32(((const uint16_t*)p)[i]);
+    default: return bf16_to_f32(((const uint16_t*)p)[i]);
+  }
+}
+static void store_f(void* p, int64_t i, int dtype, float v) {
+  switch (dtype) {
+    case ORC_F32: ((float*)p)[i] = v; break;
+    case ORC_F16: ((uint16_t*)p)[i] = f32_to_f16(v); break;
+    default: ((uint16_t*)p)[i] = f32_to_bf16(v); break;
+  }
+}
+static float round_to(float v, int dtype) {
+  if (dtype == ORC_F16) return f16_to_f32(f32_to_f16(v));
+  if (dtype == ORC_BF16) return bf16_to_f32(f32_to_bf16(v));
+  return v;
+}
+
+static float gelu_tanh(float x) {
+  const float k = 0.7978845608028654f;
+  return 0.5f * x * (1.0f + tanhf(k * (x + 0.044715f * x * x * x)));
+}
+static float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+
+/* C[b] = epi(op(A[b]) op(B[b]) + bias). The GELU epilogue acts on the value already rounded to
+ * the storage dtype, i.e. exactly what an unfused addmm followed by gelu produces. */
+int orc_gemm(void* c, const void* a, const void* b, const void* bias, int64_t batch, int64_t m,
+             int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+             int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
+             int epilogue) {
+  if (dtype != ORC_F32 && dtype != ORC_F16 && dtype != ORC_BF16) return -2;
+  const int64_t sa_m = trans_a ? 1 : lda, sa_k = trans_a ? lda : 1;
+  const int64_t sb_k = trans_b ? 1 : ldb, sb_n = trans_b ? ldb : 1;
+  const int64_t total_rows = batch * m;
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < total_rows; ++row) {
+    const int64_t bz = row / m, i = row % m;
+    for (int64_t j = 0; j < n; ++j) {
+      float acc = 0.0f;
+      for (int64_t kk = 0; kk < k; ++kk) {
+        acc += load_f(a, bz * stride_a + i * sa_m + kk * sa_k, dtype) *
+               load_f(b, bz * stride_b + kk * sb_k + j * sb_n, dtype);
+      }
+      if (bias) acc += load_f(bias, j, dtype);
+      if (epilogue != ORC_EPI_NONE) {
+        acc = round_to(acc, dtype);
+        acc = epilogue == ORC_EPI_GELU_TANH ? gelu_tanh(acc) : gelu_erf(acc);
+      }
+      store_f(c, bz * stride_c + i * ldc + j, dtype, acc);
+    }
+  }
+  return 0;
+}
+
+int orc_softmax(void* out, const void* in, int64_t rows, int64_t cols, int in_dtype,
+                int out_dtype, int log_mode) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * cols;
+    float m = -INFINITY;
+    for (int64_t j = 0; j < cols; ++j) {
+      float x = load_f(in, base + j, in_dtype);
+      if (x > m) m = x;
+      if (x != x) m = x; /* a NaN anywhere poisons the row, as it does through exp/sum */
+    }
+    float denom = 0.0f;
+    for (int64_t j = 0; j < cols; ++j) denom += expf(load_f(in, base + j, in_dtype) - m);
+    if (log_mode) {
+      const float lg = logf(denom);
+      for (int64_t j = 0; j < cols; ++j)
+        store_f(out, base + j, out_dtype, load_f(in, base + j, in_dtype) - m - lg);
+    } else {
+      for (int64_t j = 0; j < cols; ++j)
+        store_f(out, base + j, out_dtype, expf(load_f(in, base + j, in_dtype) - m) / denom);
+    }
+  }
+  return 0;
+}
+
+int orc_layer_norm(void* out, float* mean_out, float* rstd_out, const void* x, const void* gamma,
+                   const void* beta, int64_t rows, int64_t cols, double eps, int dtype) {
+  const float e = (float)eps;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * cols;
+    float total = 0.0f;
+    for (int64_t j = 0; j < cols; ++j) total += load_f(x, base + j, dtype);
+    float mean = total / (float)cols;
+    float var_sum = 0.0f;
+    for (int64_t j = 0; j < cols; ++j) {
+      const float d = load_f(x, base + j, dtype) - mean;
+      var_sum += d * d;
+    }
+    const float var = var_sum / (float)cols;
+    const float rstd = 1.0f / sqrtf(var + e);
+    for (int64_t j = 0; j < cols; ++j) {
+      float y = (load_f(x, base + j, dtype) - mean) * rstd;
+      if (gamma) y *= load_f(gamma, j, dtype);
+      if (beta) y += load_f(beta, j, dtype);
+      store_f(out, base + j, dtype, y);
+    }
+    if (var != var) mean = var;
+    if (mean_out) mean_out[r] = mean;
+    if (rstd_out) rstd_out[r] = rstd;
+  }
+  return 0;
+}
+
+int orc_reduce(void* out, const void* in, int64_t rows, int64_t cols, int op, int dtype) {
+  if (dtype == ORC_I64 || dtype == ORC_I32) {
+    if (op == ORC_MEAN) return -2;
+    if (dtype == ORC_I32 && op == ORC_SUM) return -2;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+      if (dtype == ORC_I64) {
+        const int64_t* p = (const int64_t*)in + r * cols;
+        int64_t acc = op == ORC_SUM ? 0 : INT64_MIN;
+        for (int64_t j = 0; j < cols; ++j) acc = op == ORC_SUM ? acc + p[j] : (p[j] > acc ? p[j] : acc);
+        ((int64_t*)out)[r] = acc;
+      } else {
+        const int32_t* p = (const int32_t*)in + r * cols;
+        int32_t acc = INT32_MIN;
+        for (int64_t j = 0; j < cols; ++j) acc = p[j] > acc ? p[j] : acc;
+        ((int32_t*)out)[r] = acc;
+      }
+    }
+    return 0;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * cols;
+    float acc = op == ORC_AMAX ? -INFINITY : 0.0f;
+    int saw_nan = 0;
+    for (int64_t j = 0; j < cols; ++j) {
+      const float x = load_f(in, base + j, dtype);
+      if (op == ORC_AMAX) { if (x > acc) acc = x; if (x != x) saw_nan = 1; }
+      else acc += x;
+    }
+    if (op == ORC_AMAX && saw_nan) acc = NAN;
+    if (op == ORC_MEAN) acc = acc / (float)cols;
+    store_f(out, r, dtype, acc);
+  }
+  return 0;
+}
+
+int orc_argmax(int64_t* out, const void* in, int64_t rows, int64_t cols, int dtype) {
+  if (cols <= 0) return -1;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    int64_t best_idx = 0;
+    if (dtype == ORC_I64) {
+      const int64_t* p = (const int64_t*)in + r * cols;
+      int64_t best = p[0];
+      for (int64_t j = 1; j < cols; ++j) if (p[j] > best) { best = p[j]; best_idx = j; }
+    } else if (dtype == ORC_I32) {
+      const int32_t* p = (const int32_t*)in + r * cols;
+      int32_t best = p[0];
+      for (int64_t j = 1; j < cols; ++j) if (p[j] > best) { best = p[j]; best_idx = j; }
+    } else {
+      const int64_t base = r * cols;
+      float best = load_f(in, base, dtype);
+      for (int64_t j = 1; j < cols; ++j) {
+        const float v = load_f(in, base + j, dtype);
+        if (v > best || (v != v && best == best)) { best = v; best_idx = j; }
+      }
+    }
+    out[r] = best_idx;
+  }
+  return 0;
+}
+
+int orc_gelu(void* out, const void* in, int64_t numel, int dtype, int approximate_tanh) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < numel; ++i) {
+    const float x = load_f(in, i, dtype);
+    store_f(out, i, dtype, approximate_tanh ? gelu_tanh(x) : gelu_erf(x));
+  }
+  return 0;
+}
+
+/* Round-trip helpers so the tests can pin the 16-bit conversions themselves. */
+void orc_convert_to_f32(float* out, const void* in, int64_t n, int dtype) {
+  for (int64_t i = 0; i < n; ++i) out[i] = load_f(in, i, dtype);
+}
+void orc_convert_from_f32(void* out, const float* in, int64_t n, int dtype) {
+  for (int64_t i = 0; i < n; ++i) store_f(out, i, dtype, in[i]);
+}

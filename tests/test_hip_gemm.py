@@ -1,0 +1,205 @@
+"""GPU parity of the GEMM family (mm / addmm / bmm / linear, bias + GELU epilogue)."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import closed_form as cf
+from helpers import as64, assert_close64, rel_frobenius, seeded
+
+pytestmark = pytest.mark.gpu
+
+HALF = [torch.bfloat16, torch.float16]
+
+
+def _ops():
+    from torch_mojo_backend.eager_kernels import hip_ops
+    return hip_ops
+
+
+def _ek():
+    from torch_mojo_backend import eager_kernels
+    return eager_kernels
+
+
+def _dev(t):
+    return t.to("cuda")
+
+
+def _abc(m, n, k, dtype, seed=0):
+    return (seeded((m, k), seed=seed, dtype=dtype), seeded((k, n), seed=seed + 1, dtype=dtype),
+            seeded((n,), seed=seed + 2, dtype=dtype))
+
+
+# Tiny cases: the C oracle (sequential fp32, the reference's _cpu_gemm_naive) is the yardstick.
+TINY = [(1, 1, 8), (3, 5, 16), (33, 65, 72), (64, 64, 64), (129, 131, 200), (257, 96, 1000)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32] + HALF)
+@pytest.mark.parametrize("mnk", TINY)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_addmm_small_vs_c_oracle(mnk, dtype, trans_b):
+    m, n, k = mnk
+    a, b, bias = _abc(m, n, k, dtype)
+    if trans_b:  # B given as the .t() view of an [n, k] weight
+        b = b.t().contiguous().t()
+    got = _ops().gemm(_dev(a), _dev(b), _dev(bias))
+    assert got.dtype == dtype and tuple(got.shape) == (m, n)
+    want = cf.gemm(as64(a), as64(b), as64(bias))
+    # fp32 accumulation of k products of magnitude ~1: error <= k*2^-24*sum|a||b| a priori
+    bound = k * 2.0 ** -24 * (np.abs(as64(a)) @ np.abs(as64(b)) + np.abs(as64(bias)))
+    assert_close64(got, want, extra_abs=bound, what=f"addmm {mnk} {dtype}")
+    ref = oracle.gemm(a, b, bias)
+    assert_close64(got, as64(ref), extra_abs=2 * bound, rounded_want=True, what="vs C oracle")
+
+
+# BASELINE config 1 shapes that the CPU can check in seconds + the reference's awkward shapes
+# (N=50257 / 3001 unaligned, K=1000, M=257).
+MID = [(128, 768, 768), (1024, 3072, 768), (1024, 768, 3072), (512, 2304, 768), (257, 3001, 1000),
+       (512, 50257, 768), (300, 260, 264)]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", MID)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_addmm_half_frobenius(mnk, dtype, trans_b):
+    m, n, k = mnk
+    a, b, bias = _abc(m, n, k, dtype, seed=3)
+    if trans_b:
+        b = b.t().contiguous().t()
+    got = _ops().gemm(_dev(a), _dev(b), _dev(bias))
+    want = (a.float() @ b.float() + bias.float()).double().numpy()
+    assert rel_frobenius(got, want) <= 1e-2
+    # elementwise: one storage ulp of the exact value plus fp32 accumulation slack
+    assert_close64(got, want, rtol=2e-5, atol=1e-3, what=f"addmm {mnk} {dtype}")
+
+
+@pytest.mark.parametrize("mnk", [(128, 768, 768), (1024, 3072, 768), (130, 50257, 768)])
+def test_mm_fp32(mnk):
+    m, n, k = mnk
+    a, b, _ = _abc(m, n, k, torch.float32, seed=5)
+    got = _ops().gemm(_dev(a), _dev(b.t().contiguous().t()))
+    want = a.double().numpy() @ b.double().numpy()
+    bound = k * 2.0 ** -24 * (np.abs(as64(a)) @ np.abs(as64(b)))
+    assert_close64(got, want, extra_abs=bound, what=f"mm fp32 {mnk}")
+
+
+@pytest.mark.parametrize("mnk", [(4096, 4096, 4096), (8192, 8192, 8192)])
+def test_addmm_bf16_large_sampled_rows(mnk):
+    """Benchmark sizes: float64 check on 64 sampled rows + linearity over the whole product."""
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = torch.randn(m, k, generator=g, device="cuda").bfloat16()
+    b = torch.randn(k, n, generator=g, device="cuda").bfloat16()
+    bias = torch.randn(n, generator=g, device="cuda").bfloat16()
+    got = _ops().gemm(a, b, bias)
+    rows = torch.randperm(m, generator=torch.Generator().manual_seed(1))[:64]
+    a_s = a[rows.to("cuda")].cpu().double()
+    want = (a_s @ b.cpu().double() + bias.cpu().double()).numpy()
+    assert rel_frobenius(got[rows.to("cuda")], want) <= 1e-2
+    assert_close64(got[rows.to("cuda")], want, rtol=2e-5, atol=2e-3, what=f"rows of {mnk}")
+    # (2A)B + bias - bias == 2(AB) exactly in every rounding step => compare against no-bias runs
+    c1 = _ops().gemm(a, b)
+    c2 = _ops().gemm(a * 2, b)
+    assert torch.equal(c2, c1 * 2)
+    # determinism
+    assert torch.equal(got, _ops().gemm(a, b, bias))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32] + HALF)
+def test_bmm(dtype):
+    a = seeded((12, 128, 64), seed=1, dtype=dtype)
+    b = seeded((12, 128, 64), seed=2, dtype=dtype)
+    v = seeded((12, 128, 64), seed=3, dtype=dtype)
+    scores = _ops().gemm(_dev(a), _dev(b).transpose(1, 2))        # q @ k^T   (K-major B)
+    want = torch.bmm(a.double(), b.double().transpose(1, 2)).numpy()
+    assert_close64(scores, want, rtol=2e-5, atol=1e-4, what="q@k^T")
+    ctx = _ops().gemm(_dev(seeded((12, 128, 128), seed=4, dtype=dtype)), _dev(v))  # att @ v (N-major B)
+    want2 = torch.bmm(seeded((12, 128, 128), seed=4, dtype=dtype).double(), v.double()).numpy()
+    assert_close64(ctx, want2, rtol=2e-5, atol=1e-4, what="att@v")
+    ref = oracle.gemm(a, b.transpose(1, 2))
+    assert_close64(scores, as64(ref), rtol=2e-5, atol=1e-4, rounded_want=True, what="vs C oracle")
+
+
+def test_bmm_benchmark_shape_bf16():
+    a = seeded((48, 1024, 64), seed=1, dtype=torch.bfloat16)
+    b = seeded((48, 64, 1024), seed=2, dtype=torch.bfloat16)
+    got = _ops().gemm(_dev(a), _dev(b))
+    want = torch.bmm(a.float(), b.float()).double().numpy()
+    assert rel_frobenius(got, want) <= 1e-2
+    assert_close64(got, want, rtol=2e-5, atol=1e-4, what="bmm [48,1024,64]x[48,64,1024]")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32] + HALF)
+@pytest.mark.parametrize("approximate", ["tanh", "none"])
+def test_gelu_epilogue_equals_unfused(dtype, approximate):
+    """The fused epilogue must be bit-identical to addmm followed by the standalone GELU."""
+    m, n, k = 200, 3072, 768
+    a, b, bias = _abc(m, n, k, dtype, seed=9)
+    b = (b * 0.05).to(dtype)
+    ek = _ek()
+    epi = ek.EPI_GELU_TANH if approximate == "tanh" else ek.EPI_GELU_ERF
+    fused = _ops().gemm(_dev(a), _dev(b), _dev(bias), epilogue=epi)
+    unfused = _ops().gelu(_ops().gemm(_dev(a), _dev(b), _dev(bias)), approximate)
+    assert torch.equal(fused, unfused)
+    pre = (a.double() @ b.double() + bias.double()).numpy()
+    want = cf.gelu_tanh(pre) if approximate == "tanh" else cf.gelu_erf(pre)
+    assert_close64(fused, want, rtol=2e-2 if dtype != torch.float32 else 1e-4, atol=2e-3,
+                   what="gelu epilogue vs closed form")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32] + HALF)
+@pytest.mark.parametrize("approximate", ["tanh", "none"])
+def test_gelu_standalone(dtype, approximate):
+    x = seeded((1000, 129), seed=2, scale=3.0, dtype=dtype)
+    got = _ops().gelu(_dev(x), approximate)
+    want = cf.gelu_tanh(as64(x)) if approximate == "tanh" else cf.gelu_erf(as64(x))
+    assert_close64(got, want, rtol=1e-5, atol=2e-6, what="gelu")
+    assert_close64(got, as64(oracle.gelu(x, approximate)), rtol=1e-5, atol=2e-6, rounded_want=True, what="vs C oracle")
+
+
+def test_bias_is_added_before_the_cast():
+    """acc + bias is rounded once. acc = 1 + 2^-8 is a bf16 tie that rounds to 1.0 on its own;
+    with bias 2^-10 the fp32 sum lies above the tie and must round UP to 1 + 2^-7, whereas
+    round(acc) + bias would give 1.0."""
+    k = 8
+    a = torch.zeros(1, k, dtype=torch.bfloat16)
+    b = torch.zeros(k, 1, dtype=torch.bfloat16)
+    a[0, 0], b[0, 0] = 1.0, 1.0
+    a[0, 1], b[1, 0] = 2.0 ** -8, 1.0
+    bias = torch.tensor([2.0 ** -10], dtype=torch.bfloat16)
+    want = torch.tensor([[1.0 + 2.0 ** -7]]).bfloat16()
+    assert torch.equal(oracle.gemm(a, b, bias), want)
+    assert torch.equal(_ops().gemm(_dev(a), _dev(b), _dev(bias)).cpu(), want)
+    # same thing through the MFMA path (needs k % 8 == 0, which k = 8 satisfies) and the SIMT
+    # path (fp32 storage keeps every bit, so only check it runs and is exact)
+    got32 = _ops().gemm(_dev(a.float()), _dev(b.float()), _dev(bias.float())).cpu()
+    assert got32.item() == 1.0 + 2.0 ** -8 + 2.0 ** -10
+
+
+def test_degenerate_shapes():
+    ops = _ops()
+    a = _dev(seeded((0, 16), dtype=torch.float32))
+    b = _dev(seeded((16, 8), dtype=torch.float32))
+    assert ops.gemm(a, b).shape == (0, 8)
+    a2 = _dev(seeded((4, 0), dtype=torch.float32))
+    b2 = _dev(seeded((0, 8), dtype=torch.float32))
+    bias = _dev(seeded((8,), dtype=torch.float32))
+    assert torch.equal(ops.gemm(a2, b2), torch.zeros(4, 8, device="cuda"))
+    assert torch.equal(ops.gemm(a2, b2, bias), bias.expand(4, 8))
+    one = ops.gemm(_dev(seeded((1, 768), seed=1)), _dev(seeded((768, 1), seed=2)))
+    assert one.shape == (1, 1)
+
+
+def test_gemm_rejects_cpu_tensors():
+    with pytest.raises(TypeError, match="no CPU path"):
+        _ops().gemm(torch.randn(2, 2), torch.randn(2, 2))
+
+
+def test_queued_launches_are_bit_identical():
+    a, b, bias = _abc(512, 768, 768, torch.bfloat16, seed=4)
+    ad, bd, cd = _dev(a), _dev(b), _dev(bias)
+    outs = [_ops().gemm(ad, bd, cd) for _ in range(3)]
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])

@@ -1,0 +1,174 @@
+"""GPU parity of sum / mean / amax / argmax against the CPU oracle and float64 closed forms."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import closed_form as cf
+from helpers import as64, assert_close64, seeded
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _ops():
+    from torch_mojo_backend.eager_kernels import hip_ops
+    return hip_ops
+
+
+def _ek():
+    from torch_mojo_backend import eager_kernels
+    return eager_kernels
+
+
+def _dev(t):
+    return t.to("cuda")
+
+
+# (rows, cols): wave-per-row, block-per-row, split rows, unaligned widths, a single long row.
+REDUCE_SHAPES = [(1, 1), (5, 3), (64, 64), (33, 257), (1000, 768), (2048, 4096), (300, 4097),
+                 (7, 50257), (3, 100003), (1, 1 << 20), (1, (1 << 22) + 5), (2, 300000)]
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", REDUCE_SHAPES)
+def test_sum_mean_amax_rows(shape, dtype):
+    x = seeded(shape, seed=shape[1] % 997, dtype=dtype)
+    xd = _dev(x)
+    x64 = as64(x)
+    bound = cf.sum_error_bound(x64, axis=-1)
+    n = shape[1]
+    s = _ops().reduce(xd, [1], False, _ek().SUM)
+    assert s.dtype == dtype and tuple(s.shape) == (shape[0],)
+    assert_close64(s, x64.sum(-1), extra_abs=bound, what=f"sum {shape}")
+    m = _ops().reduce(xd, [1], False, _ek().MEAN)
+    assert_close64(m, x64.mean(-1), extra_abs=bound / n, what=f"mean {shape}")
+    a = _ops().reduce(xd, [1], False, _ek().AMAX)
+    assert np.array_equal(as64(a), x64.max(-1)), "amax must be exact"
+    # C restatement of the reference kernel (sequential fp32): same bound applies to it
+    ref = oracle.reduce_rows(x, oracle.SUM)
+    assert_close64(s, as64(ref), extra_abs=2 * bound, rounded_want=True, what="sum vs C oracle")
+
+
+@pytest.mark.parametrize("dims,keepdim", [([0], False), ([1], True), ([0, 2], False), ([2], True),
+                                          ([0, 1, 2], False), ([0, 1, 2], True), ([1, 2], False)])
+def test_reduce_dims_and_keepdim(dims, keepdim):
+    x = seeded((6, 10, 12), seed=4)
+    for op, ref in ((_ek().SUM, torch.sum), (_ek().MEAN, torch.mean), (_ek().AMAX, torch.amax)):
+        got = _ops().reduce(_dev(x), dims, keepdim, op)
+        want = ref(x, dim=dims, keepdim=keepdim)
+        assert got.shape == want.shape
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+
+
+def test_full_reduction_benchmark_size_properties():
+    """[65536, 4096] fp32 (the benchmark tensor): linearity and a sum of row sums."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(65536, 4096, generator=g, device="cuda")
+    ops, ek = _ops(), _ek()
+    total = ops.reduce(x, [0, 1], False, ek.SUM)
+    rows = ops.reduce(x, [1], False, ek.SUM)
+    total_of_rows = ops.reduce(rows, [0], False, ek.SUM)
+    exact = x.double().sum().item()
+    l1 = x.double().abs().sum().item()
+    assert abs(total.item() - exact) <= 1e-6 * l1 * 1e-1 + 1e-5 * abs(exact)
+    assert abs(total_of_rows.item() - exact) <= 1e-6 * l1 * 1e-1 + 1e-5 * abs(exact)
+    # bit-reproducible: same launch twice, identical bits
+    again = ops.reduce(x, [0, 1], False, ek.SUM)
+    assert total.view(torch.int32).item() == again.view(torch.int32).item()
+    # mean = sum / numel, amax exact
+    mean = ops.reduce(x, [0, 1], False, ek.MEAN)
+    assert abs(mean.item() - exact / x.numel()) <= 1e-6
+    assert ops.reduce(x, [0, 1], False, ek.AMAX).item() == x.max().item()
+    # linearity: sum(2x) == 2 sum(x) exactly (scaling by 2 is exact in fp32)
+    assert ops.reduce(x * 2, [0, 1], False, ek.SUM).item() == 2 * total.item()
+
+
+def test_amax_propagates_nan_and_handles_inf():
+    x = seeded((4, 5000), seed=3)
+    x[1, 4321] = float("nan")
+    x[2, 17] = float("inf")
+    x[3, :] = float("-inf")
+    got = _ops().reduce(_dev(x), [1], False, _ek().AMAX).cpu()
+    want = torch.amax(x, dim=1)
+    assert torch.isnan(got[1]) and got[2] == float("inf") and got[3] == float("-inf")
+    assert got[0] == want[0]
+
+
+def test_integer_reductions_are_exact():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randint(-2 ** 40, 2 ** 40, (37, 5001), generator=g, dtype=torch.int64)
+    assert torch.equal(_ops().reduce(_dev(x), [1], False, _ek().SUM).cpu(), x.sum(1))
+    assert torch.equal(_ops().reduce(_dev(x), [1], False, _ek().AMAX).cpu(), x.amax(1))
+    assert torch.equal(_ops().reduce(_dev(x), [0, 1], False, _ek().SUM).cpu(), x.sum())
+    xi = torch.randint(-2 ** 31, 2 ** 31 - 1, (3, 70001), generator=g, dtype=torch.int32)
+    assert torch.equal(_ops().reduce(_dev(xi), [1], False, _ek().AMAX).cpu(), xi.amax(1))
+    assert torch.equal(_ops().argmax(_dev(xi), 1, False).cpu(), xi.argmax(1))
+    assert torch.equal(_ops().argmax(_dev(x), 1, False).cpu(), x.argmax(1))
+
+
+def _logits_with_ties(rows=512, cols=50257, seed=0):
+    """Benchmark logits: 1% of rows carry an injected tie above the row maximum."""
+    x = seeded((rows, cols), seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    n_tied = max(1, -(-rows // 100))
+    tied_rows = torch.randperm(rows, generator=g)[: n_tied + 2].tolist()
+    expected = {}
+    for r in tied_rows[:n_tied]:
+        j = sorted(torch.randint(0, cols, (2,), generator=g).tolist())
+        if j[0] == j[1]:
+            j[1] = (j[0] + 1) % cols
+            j.sort()
+        x[r, j[0]] = x[r, j[1]] = x[r].max() + 1
+        expected[r] = j[0]
+    r3, rl = tied_rows[n_tied], tied_rows[n_tied + 1]
+    top = x[r3].max() + 1
+    x[r3, 0] = x[r3, cols // 2] = x[r3, cols - 1] = top   # three-way tie including column 0
+    expected[r3] = 0
+    top = x[rl].max() + 1
+    x[rl, cols - 2] = x[rl, cols - 1] = top               # tie at the very end of the row
+    expected[rl] = cols - 2
+    return x, expected
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_argmax_vocab_with_ties_is_bit_exact(dtype):
+    x, expected = _logits_with_ties()
+    x = x.to(dtype)
+    got = _ops().argmax(_dev(x), -1, False)
+    assert got.dtype == torch.int64
+    got = got.cpu()
+    assert torch.equal(got, oracle.argmax_rows(x))
+    assert torch.equal(got, torch.argmax(x, dim=-1))
+    if dtype == torch.float32:
+        for r, j in expected.items():
+            assert got[r].item() == j
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 64), (257, 1000), (5, 65537), (2, 1 << 21),
+                                   (1, (1 << 23) + 3)])
+def test_argmax_shapes(shape):
+    x = seeded(shape, seed=shape[1] % 991)
+    x[:, shape[1] // 2] = x.max() + 1  # a planted maximum, as the reference's vocab test does
+    if shape[1] > 2:
+        x[0, shape[1] - 1] = x.max()   # and a tie with a later column in row 0
+    got = _ops().argmax(_dev(x), 1, False).cpu()
+    assert torch.equal(got, torch.argmax(x, dim=1))
+    assert torch.equal(got, oracle.argmax_rows(x))
+
+
+def test_argmax_dim_none_keepdim_and_nan():
+    x = seeded((7, 9, 11), seed=8)
+    ops = _ops()
+    assert torch.equal(ops.argmax(_dev(x), None, False).cpu(), torch.argmax(x))
+    assert ops.argmax(_dev(x), None, True).shape == (1, 1, 1)
+    for d in (0, 1, 2, -1):
+        for keep in (False, True):
+            assert torch.equal(ops.argmax(_dev(x), d, keep).cpu(), torch.argmax(x, dim=d, keepdim=keep))
+    x[2, 3, 5] = float("nan")
+    x[2, 3, 7] = float("nan")
+    assert torch.equal(ops.argmax(_dev(x), 2, False).cpu(), torch.argmax(x, dim=2))
+    all_equal = torch.zeros(3, 70000)
+    assert torch.equal(ops.argmax(_dev(all_equal), 1, False).cpu(), torch.zeros(3, dtype=torch.int64))

@@ -1,0 +1,157 @@
+"""GPU parity of softmax / log_softmax / native_layer_norm: HIP kernels (through the C ABI)
+against the CPU oracle and the float64 closed forms, on seeded inputs."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import closed_form as cf
+from helpers import as64, assert_close64, seeded
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _dev(t):
+    return t.to("cuda")
+
+
+def _ops():
+    from torch_mojo_backend.eager_kernels import hip_ops
+    return hip_ops
+
+
+# cols chosen to hit every register-resident configuration, the 16-wave one, the generic
+# fallback (unaligned widths, beyond-register widths) and the GPT-2 / benchmark shapes.
+SOFTMAX_SHAPES = [(7, 1), (5, 8), (33, 257), (64, 64), (19, 128), (300, 768), (130, 1024),
+                  (67, 2048), (35, 4096), (9, 8192), (5, 16384), (3, 32768), (2, 40000),
+                  (4, 50257), (3, 70000)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_matches_oracle(shape, dtype, log):
+    x = seeded(shape, seed=shape[1], scale=4.0, dtype=dtype)
+    got = _ops().softmax(_dev(x), -1, log=log)
+    assert got.dtype == dtype and tuple(got.shape) == shape
+    want = (cf.log_softmax if log else cf.softmax)(as64(x))
+    assert_close64(got, want, what=f"softmax{shape} log={log}")
+    # and against the C restatement of the reference CPU kernel
+    ref = oracle.softmax_rows(x, log=log)
+    assert_close64(got, as64(ref), rtol=2e-5, atol=2e-6, rounded_want=True, what="vs C oracle")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_softmax_half_to_float(dtype):
+    x = seeded((37, 1024), seed=3, scale=4.0, dtype=dtype)
+    got = _ops().softmax(_dev(x), -1, half_to_float=True)
+    assert got.dtype == torch.float32
+    assert_close64(got, cf.softmax(as64(x)), what="half_to_float")
+
+
+@pytest.mark.parametrize("dim", [0, 1, 2, -1, -2])
+def test_softmax_any_dim(dim):
+    x = seeded((6, 10, 12), seed=11, scale=2.0)
+    got = _ops().softmax(_dev(x), dim)
+    assert_close64(got, cf.softmax(as64(x), axis=dim), what=f"dim={dim}")
+    assert got.shape == x.shape
+
+
+def test_softmax_invariants_full_size():
+    """Benchmark-size rows: sums to one and shift invariance (size-independent properties)."""
+    x = seeded((4096, 4096), seed=5, scale=4.0)
+    xd = _dev(x)
+    p = _ops().softmax(xd, -1)
+    sums = p.double().sum(-1).cpu().numpy()
+    assert np.abs(sums - 1.0).max() < 1e-5
+    assert (p >= 0).all()
+    shifted = _ops().softmax(xd + 3.0, -1)
+    assert torch.allclose(p, shifted, rtol=2e-5, atol=1e-7)
+    # argmax of probabilities is the argmax of the logits
+    assert torch.equal(p.argmax(-1).cpu(), x.argmax(-1))
+
+
+def test_softmax_extremes():
+    x = torch.tensor([[1e4, -1e4, 0.0, 1e4], [-1e30, -1e30, -1e30, -1e30],
+                      [float("-inf"), 0.0, 1.0, 2.0], [88.0, 89.0, -88.0, 0.0]])
+    got = _ops().softmax(_dev(x), -1)
+    assert_close64(got, cf.softmax(as64(x)), what="extremes")
+    nan_row = torch.tensor([[1.0, float("nan"), 2.0, 3.0]])
+    assert torch.isnan(_ops().softmax(_dev(nan_row), -1)).all()
+
+
+def test_softmax_rank0_and_offset_storage():
+    ops = _ops()
+    assert ops.softmax(_dev(torch.tensor(3.0)), -1).item() == 1.0
+    assert ops.softmax(_dev(torch.tensor(3.0)), -1, log=True).item() == 0.0
+    base = seeded((5 * 64 + 1,), seed=2)
+    view = _dev(base)[1:].view(5, 64)  # 4-byte aligned only: must take the generic kernel
+    assert_close64(ops.softmax(view, -1), cf.softmax(as64(base[1:].view(5, 64))), what="offset")
+
+
+LN_SHAPES = [(3, 7), (6, 768), (5, 769), (3, 65), (16, 1024), (33, 2048), (9, 4096), (4, 8192),
+             (3, 16384), (2, 40000), (257, 768)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", LN_SHAPES)
+def test_layer_norm_matches_oracle(shape, dtype):
+    rows, cols = shape
+    x = seeded(shape, seed=cols, dtype=dtype)
+    g = seeded((cols,), seed=1, scale=0.1, shift=1.0, dtype=dtype)
+    b = seeded((cols,), seed=2, scale=0.1, dtype=dtype)
+    out, mean, rstd = _ops().layer_norm(_dev(x), [cols], _dev(g), _dev(b), 1e-5)
+    assert out.dtype == dtype and mean.dtype == torch.float32 and rstd.dtype == torch.float32
+    assert tuple(mean.shape) == (rows, 1) and tuple(rstd.shape) == (rows, 1)
+    w_out, w_mean, w_rstd = cf.layer_norm(as64(x), as64(g), as64(b), 1e-5)
+    # out = (x-mean)*rstd*g+b: error scales with |x-mean|*rstd*|g|, so allow rtol on that scale
+    scale = np.abs(as64(x) - w_mean) * w_rstd * np.abs(as64(g)) + np.abs(as64(b))
+    assert_close64(out, w_out, extra_abs=1e-5 * scale, what=f"ln out {shape}")
+    assert_close64(mean, w_mean, atol=1e-6, what="ln mean")
+    assert_close64(rstd, w_rstd, rtol=1e-5, what="ln rstd")
+    r_out, r_mean, r_rstd = oracle.layer_norm_rows(x, g, b, 1e-5)
+    assert_close64(mean.reshape(-1), as64(r_mean), atol=2e-6, rounded_want=True, what="mean vs C oracle")
+    assert_close64(rstd.reshape(-1), as64(r_rstd), rtol=2e-5, rounded_want=True, what="rstd vs C oracle")
+
+
+@pytest.mark.parametrize("has_weight,has_bias", [(False, False), (True, False), (False, True)])
+@pytest.mark.parametrize("shape,normalized,eps", [((3, 7), (7,), 1e-5), ((2, 3, 4), (3, 4), 0.5)])
+def test_layer_norm_optional_affine(shape, normalized, eps, has_weight, has_bias):
+    x = seeded(shape, seed=20260720 % 1000)
+    w = seeded(normalized, seed=4) if has_weight else None
+    b = seeded(normalized, seed=5) if has_bias else None
+    out, mean, rstd = _ops().layer_norm(_dev(x), list(normalized), None if w is None else _dev(w),
+                                        None if b is None else _dev(b), eps)
+    want = torch.native_layer_norm(x, normalized, w, b, eps)
+    for got, ref, tol in zip((out, mean, rstd), want, (1e-5, 1e-5, 1e-4)):
+        torch.testing.assert_close(got.cpu(), ref, atol=tol, rtol=tol)
+    k = len(normalized)
+    assert tuple(mean.shape) == tuple(shape[:-k]) + (1,) * k
+
+
+@pytest.mark.parametrize("cols", [768, 769])
+@pytest.mark.parametrize("value", [float("nan"), float("inf"), float("-inf")])
+def test_layer_norm_nonfinite_rows(cols, value):
+    x = torch.full((2, cols), value)
+    out, mean, rstd = _ops().layer_norm(_dev(x), [cols], None, None, 1e-5)
+    assert torch.isnan(out).all() and torch.isnan(mean).all() and torch.isnan(rstd).all()
+
+
+def test_layer_norm_without_stats_and_invariants():
+    x = seeded((8192, 768), seed=9, scale=3.0, shift=0.5)
+    out, mean, rstd = _ops().layer_norm(_dev(x), [768], None, None, 1e-5, need_stats=False)
+    assert mean is None and rstd is None
+    o = out.double()
+    assert o.mean(-1).abs().max().item() < 1e-5          # gamma=1, beta=0 => zero mean
+    assert (o.var(-1, unbiased=False) - 1).abs().max().item() < 1e-3  # ... and unit variance
+
+
+def test_row_kernels_are_deterministic():
+    """Queue three launches before syncing; outputs must be bit-identical."""
+    x = _dev(seeded((2048, 1024), seed=1, scale=4.0))
+    outs = [_ops().softmax(x, -1) for _ in range(3)]
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])

@@ -1,0 +1,539 @@
+// Row reductions (sum / mean / amax) and first-occurrence argmax for gfx950.
+//
+// Work decomposition depends only on (rows, cols): every row is cut into `splits` contiguous
+// chunks; one workgroup streams one chunk with 16-byte loads (scalar head/tail for unaligned
+// rows, e.g. 50257-wide vocab rows), reduces it in a fixed order (per-lane strided accumulate
+// -> DPP wave tree -> LDS combine in wave order) and either writes the final value
+// (splits == 1) or a partial into the caller's workspace, which a second launch combines in
+// chunk order. No atomics anywhere, so floating-point results are bit-reproducible.
+//
+// Arithmetic contract (torch_mojo_backend/eager_kernels/reduction_ops.mojo:161-194,
+// nn_ops.mojo:981-1027, nn_ops.mojo:1424-1478): floats accumulate in fp32 and are cast once;
+// integers reduce in their own type; argmax keeps the lower index among equal values at
+// every combine step.
+#include "tmb_common.h"
+
+namespace tmb {
+
+constexpr int kRedBlock = 256;
+constexpr int kRedWaves = kRedBlock / kWave;
+
+struct SplitPlan {
+  int splits;
+  int64_t chunk;  // elements per chunk (multiple of 64 unless splits == 1)
+};
+
+// Must stay a pure function of (rows, cols): the Python side sizes the workspace from it and
+// reproducibility relies on it.
+static SplitPlan plan_splits(int64_t rows, int64_t cols) {
+  constexpr int64_t kTargetBlocks = 2048;   // 8 workgroups per CU on 256 CUs
+  constexpr int64_t kMinChunk = 16384;      // elements; below this a split is not worth a launch
+  constexpr int64_t kMaxChunk = int64_t{1} << 30;
+  int64_t splits = 1;
+  if (rows < kTargetBlocks / 2) {
+    splits = (kTargetBlocks + rows - 1) / rows;
+    const int64_t by_size = cols / kMinChunk;
+    if (splits > by_size) splits = by_size;
+    if (splits < 1) splits = 1;
+  }
+  const int64_t need = (cols + kMaxChunk - 1) / kMaxChunk;
+  if (splits < need) splits = need;
+  if (splits > 4096) splits = 4096;
+  int64_t chunk = (cols + splits - 1) / splits;
+  if (splits > 1) {
+    chunk = (chunk + 63) / 64 * 64;
+    splits = (cols + chunk - 1) / chunk;
+  }
+  return SplitPlan{static_cast<int>(splits), chunk};
+}
+
+// ---------------------------------------------------------------------------
+// Value reductions
+// ---------------------------------------------------------------------------
+template <typename Acc>
+struct AccSum {
+  using acc_t = Acc;
+  static __device__ __forceinline__ Acc identity() { return Acc(0); }
+  static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return a + b; }
+};
+// Float max carried as (value, saw_nan) so the streaming loop is one v_max + one compare.
+struct FMax {
+  float v;
+  bool nan;
+};
+struct AccFMax {
+  using acc_t = FMax;
+  static __device__ __forceinline__ FMax identity() { return FMax{-__builtin_inff(), false}; }
+  static __device__ __forceinline__ FMax combine(FMax a, FMax b) {
+    return FMax{fmaxf(a.v, b.v), a.nan || b.nan};
+  }
+};
+template <typename I>
+struct AccIMax {
+  using acc_t = I;
+  static __device__ __forceinline__ I identity() {
+    if constexpr (sizeof(I) == 8) {
+      return static_cast<I>(INT64_MIN);
+    } else {
+      return static_cast<I>(INT32_MIN);
+    }
+  }
+  static __device__ __forceinline__ I combine(I a, I b) { return a > b ? a : b; }
+};
+
+template <typename T>
+__device__ __forceinline__ void accumulate(float& acc, T x) { acc += to_f32(x); }
+__device__ __forceinline__ void accumulate(int64_t& acc, int64_t x) { acc += x; }
+template <typename T>
+__device__ __forceinline__ void accumulate(FMax& acc, T x) {
+  const float f = to_f32(x);
+  acc.v = fmaxf(acc.v, f);
+  acc.nan = acc.nan || (f != f);
+}
+__device__ __forceinline__ void accumulate_imax(int64_t& acc, int64_t x) { acc = x > acc ? x : acc; }
+__device__ __forceinline__ void accumulate_imax(int32_t& acc, int32_t x) { acc = x > acc ? x : acc; }
+
+template <typename Policy, typename T, bool IMAX>
+__device__ __forceinline__ void acc_one(typename Policy::acc_t& acc, T x) {
+  if constexpr (IMAX) {
+    accumulate_imax(acc, x);
+  } else {
+    accumulate(acc, x);
+  }
+}
+
+// Generic (non-fp32-sum) wave butterfly; used for exact/associative combines.
+template <typename V>
+__device__ __forceinline__ V shfl_xor_any(V v, int mask) {
+  static_assert(sizeof(V) % 4 == 0, "4-byte multiples only");
+  union {
+    V v;
+    int w[sizeof(V) / 4];
+  } a, b;
+  a.v = v;
+#pragma unroll
+  for (int i = 0; i < static_cast<int>(sizeof(V) / 4); ++i) b.w[i] = __shfl_xor(a.w[i], mask, kWave);
+  return b.v;
+}
+
+struct FMaxPacked {
+  float v;
+  int nan;
+};
+
+template <typename Policy>
+__device__ __forceinline__ typename Policy::acc_t wave_combine(typename Policy::acc_t a) {
+  using A = typename Policy::acc_t;
+  if constexpr (__is_same(A, float)) {
+    return wave_sum(a);
+  } else if constexpr (__is_same(A, FMax)) {
+    const float v = wave_max(a.v);
+    const bool any_nan = __builtin_amdgcn_ballot_w64(a.nan) != 0;
+    return FMax{v, any_nan};
+  } else {
+#pragma unroll
+    for (int mask = 1; mask < kWave; mask <<= 1) a = Policy::combine(a, shfl_xor_any(a, mask));
+    return a;
+  }
+}
+
+// Streams [p, p+n) with `NT` cooperating threads (this thread is `tid`) in a fixed order.
+template <typename Policy, typename T, bool IMAX, int NT>
+__device__ __forceinline__ typename Policy::acc_t stream_range(const T* __restrict__ p, int64_t n,
+                                                               int tid) {
+  using A = typename Policy::acc_t;
+  constexpr int EPV = Vec16<T>::N;
+  A acc0 = Policy::identity(), acc1 = Policy::identity();
+  A acc2 = Policy::identity(), acc3 = Policy::identity();
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+  int64_t head = static_cast<int64_t>(((16u - (addr & 15u)) & 15u) / sizeof(T));
+  if (head > n) head = n;
+  if (tid < head) acc_one<Policy, T, IMAX>(acc0, p[tid]);
+  const T* body = p + head;
+  const int64_t nvec = (n - head) / EPV;
+  int64_t i = tid;
+  for (; i + 3 * NT < nvec; i += 4 * NT) {
+    const Vec16<T> v0 = load_vec16(body + i * EPV);
+    const Vec16<T> v1 = load_vec16(body + (i + NT) * EPV);
+    const Vec16<T> v2 = load_vec16(body + (i + 2 * NT) * EPV);
+    const Vec16<T> v3 = load_vec16(body + (i + 3 * NT) * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      acc_one<Policy, T, IMAX>(acc0, v0.v[e]);
+      acc_one<Policy, T, IMAX>(acc1, v1.v[e]);
+      acc_one<Policy, T, IMAX>(acc2, v2.v[e]);
+      acc_one<Policy, T, IMAX>(acc3, v3.v[e]);
+    }
+  }
+  for (; i < nvec; i += NT) {
+    const Vec16<T> v0 = load_vec16(body + i * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) acc_one<Policy, T, IMAX>(acc0, v0.v[e]);
+  }
+  const int64_t tail = head + nvec * EPV;
+  if (tail + tid < n) acc_one<Policy, T, IMAX>(acc1, p[tail + tid]);
+  return Policy::combine(Policy::combine(acc0, acc1), Policy::combine(acc2, acc3));
+}
+
+template <typename A>
+struct AccStore {  // what a partial looks like in the workspace (8 bytes per partial)
+  static __device__ __forceinline__ void put(void* ws, int64_t i, A a) {
+    static_cast<A*>(ws)[i] = a;
+  }
+  static __device__ __forceinline__ A get(const void* ws, int64_t i) {
+    return static_cast<const A*>(ws)[i];
+  }
+};
+template <>
+struct AccStore<FMax> {
+  static __device__ __forceinline__ void put(void* ws, int64_t i, FMax a) {
+    static_cast<FMaxPacked*>(ws)[i] = FMaxPacked{a.v, a.nan ? 1 : 0};
+  }
+  static __device__ __forceinline__ FMax get(const void* ws, int64_t i) {
+    const FMaxPacked p = static_cast<const FMaxPacked*>(ws)[i];
+    return FMax{p.v, p.nan != 0};
+  }
+};
+
+template <typename TOut, typename A>
+__device__ __forceinline__ TOut finalize(A a, int op, int64_t cols) {
+  if constexpr (__is_same(A, FMax)) {
+    return from_f32<TOut>(a.nan ? __builtin_nanf("") : a.v);
+  } else if constexpr (__is_same(A, float)) {
+    return from_f32<TOut>(op == TMB_MEAN ? a / static_cast<float>(cols) : a);
+  } else {
+    return static_cast<TOut>(a);
+  }
+}
+
+// One workgroup per (row, split) chunk.
+template <typename Policy, typename T, bool IMAX>
+__global__ __launch_bounds__(kRedBlock) void reduce_chunk_kernel(T* __restrict__ out,
+                                                                 void* __restrict__ ws,
+                                                                 const T* __restrict__ in,
+                                                                 int64_t rows, int64_t cols,
+                                                                 int splits, int64_t chunk, int op) {
+  using A = typename Policy::acc_t;
+  __shared__ A slot[kRedWaves];
+  const int64_t item = blockIdx.x;
+  const int64_t row = item / splits;
+  const int split = static_cast<int>(item - row * splits);
+  const int64_t c0 = static_cast<int64_t>(split) * chunk;
+  int64_t n = cols - c0;
+  if (n > chunk) n = chunk;
+  A acc = stream_range<Policy, T, IMAX, kRedBlock>(in + row * cols + c0, n, threadIdx.x);
+  acc = wave_combine<Policy>(acc);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) slot[wave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    A r = slot[0];
+#pragma unroll
+    for (int w = 1; w < kRedWaves; ++w) r = Policy::combine(r, slot[w]);
+    if (splits == 1) {
+      out[row] = finalize<T>(r, op, cols);
+    } else {
+      AccStore<A>::put(ws, item, r);
+    }
+  }
+}
+
+// One wave per row: rows that are short enough that a workgroup per row would idle lanes.
+template <typename Policy, typename T, bool IMAX>
+__global__ __launch_bounds__(kRedBlock) void reduce_wave_kernel(T* __restrict__ out,
+                                                                const T* __restrict__ in,
+                                                                int64_t rows, int64_t cols, int op) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRedWaves + (threadIdx.x >> 6);
+  if (row >= rows) return;  // wave-uniform
+  auto acc = stream_range<Policy, T, IMAX, kWave>(in + row * cols, cols, threadIdx.x & 63);
+  acc = wave_combine<Policy>(acc);
+  if ((threadIdx.x & 63) == 0) out[row] = finalize<T>(acc, op, cols);
+}
+
+// Second stage: combines the `splits` partials of each row in chunk order.
+template <typename Policy, typename T>
+__global__ __launch_bounds__(kWave) void reduce_final_kernel(T* __restrict__ out,
+                                                             const void* __restrict__ ws,
+                                                             int64_t rows, int64_t cols,
+                                                             int splits, int op) {
+  using A = typename Policy::acc_t;
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x;
+  A acc = Policy::identity();
+  for (int i = lane; i < splits; i += kWave)
+    acc = Policy::combine(acc, AccStore<A>::get(ws, row * splits + i));
+  acc = wave_combine<Policy>(acc);
+  if (lane == 0) out[row] = finalize<T>(acc, op, cols);
+}
+
+template <typename Policy, typename T, bool IMAX>
+static int launch_reduce(void* out_, const void* in_, int64_t rows, int64_t cols, int op,
+                         void* ws, size_t ws_bytes, hipStream_t stream) {
+  T* out = static_cast<T*>(out_);
+  const T* in = static_cast<const T*>(in_);
+  const SplitPlan plan = plan_splits(rows, cols);
+  if (plan.splits == 1 && cols * static_cast<int64_t>(sizeof(T)) <= 8192) {
+    const int64_t blocks = (rows + kRedWaves - 1) / kRedWaves;
+    if (blocks >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+    reduce_wave_kernel<Policy, T, IMAX>
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(kRedBlock), 0, stream>>>(out, in, rows, cols, op);
+    return check_launch();
+  }
+  const int64_t items = rows * plan.splits;
+  if (items >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  if (plan.splits > 1) {
+    if (ws == nullptr || ws_bytes < static_cast<size_t>(items) * 16) return TMB_ERR_WORKSPACE;
+  }
+  reduce_chunk_kernel<Policy, T, IMAX><<<dim3(static_cast<unsigned>(items)), dim3(kRedBlock), 0, stream>>>(
+      out, ws, in, rows, cols, plan.splits, plan.chunk, op);
+  int rc = check_launch();
+  if (rc != 0 || plan.splits == 1) return rc;
+  reduce_final_kernel<Policy, T><<<dim3(static_cast<unsigned>(rows)), dim3(kWave), 0, stream>>>(
+      out, ws, rows, cols, plan.splits, op);
+  return check_launch();
+}
+
+// ---------------------------------------------------------------------------
+// Argmax
+// ---------------------------------------------------------------------------
+template <typename V>
+struct Best {
+  V val;
+  int64_t idx;
+};
+
+template <typename V>
+__device__ __forceinline__ bool is_nan(V v) {
+  if constexpr (__is_same(V, float)) {
+    return v != v;
+  } else {
+    return false;
+  }
+}
+
+// true when b must replace a: NaN beats numbers, greater beats smaller, ties keep the lower index.
+template <typename V>
+__device__ __forceinline__ bool replaces(const Best<V>& a, const Best<V>& b) {
+  if (a.idx < 0) return b.idx >= 0;
+  if (b.idx < 0) return false;
+  const bool an = is_nan(a.val), bn = is_nan(b.val);
+  if (an || bn) {
+    if (an && bn) return b.idx < a.idx;
+    return bn;
+  }
+  if (b.val > a.val) return true;
+  if (b.val == a.val) return b.idx < a.idx;
+  return false;
+}
+
+template <typename V>
+__device__ __forceinline__ Best<V> best_combine(Best<V> a, Best<V> b) {
+  return replaces(a, b) ? b : a;
+}
+
+template <typename T>
+struct ArgTraits {
+  using val_t = float;
+  static __device__ __forceinline__ float conv(T x) { return to_f32(x); }
+};
+template <>
+struct ArgTraits<int64_t> {
+  using val_t = int64_t;
+  static __device__ __forceinline__ int64_t conv(int64_t x) { return x; }
+};
+template <>
+struct ArgTraits<int32_t> {
+  using val_t = int32_t;
+  static __device__ __forceinline__ int32_t conv(int32_t x) { return x; }
+};
+
+// Per-thread scan in ascending index order: strict "greater" keeps the first occurrence;
+// the first NaN sticks.
+template <typename V>
+__device__ __forceinline__ void scan_one(V& best, int& best_off, V x, int off) {
+  bool take;
+  if constexpr (__is_same(V, float)) {
+    take = (best_off < 0) || (x > best) || ((x != x) && (best == best));
+  } else {
+    take = (best_off < 0) || (x > best);
+  }
+  best = take ? x : best;
+  best_off = take ? off : best_off;
+}
+
+template <typename T, int NT>
+__device__ __forceinline__ Best<typename ArgTraits<T>::val_t> argmax_range(const T* __restrict__ p,
+                                                                           int64_t n, int tid,
+                                                                           int64_t base) {
+  using V = typename ArgTraits<T>::val_t;
+  constexpr int EPV = Vec16<T>::N;
+  V best = V(0);
+  int off = -1;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+  int head = static_cast<int>(((16u - (addr & 15u)) & 15u) / sizeof(T));
+  if (head > n) head = static_cast<int>(n);
+  if (tid < head) scan_one(best, off, ArgTraits<T>::conv(p[tid]), tid);
+  const T* body = p + head;
+  const int nvec = static_cast<int>((n - head) / EPV);
+  int i = tid;
+  for (; i + NT < nvec; i += 2 * NT) {
+    const Vec16<T> v0 = load_vec16(body + static_cast<int64_t>(i) * EPV);
+    const Vec16<T> v1 = load_vec16(body + static_cast<int64_t>(i + NT) * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) scan_one(best, off, ArgTraits<T>::conv(v0.v[e]), head + i * EPV + e);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e)
+      scan_one(best, off, ArgTraits<T>::conv(v1.v[e]), head + (i + NT) * EPV + e);
+  }
+  for (; i < nvec; i += NT) {
+    const Vec16<T> v0 = load_vec16(body + static_cast<int64_t>(i) * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) scan_one(best, off, ArgTraits<T>::conv(v0.v[e]), head + i * EPV + e);
+  }
+  const int tail = head + nvec * EPV;
+  if (tail + tid < n) scan_one(best, off, ArgTraits<T>::conv(p[tail + tid]), tail + tid);
+  return Best<V>{best, off < 0 ? int64_t{-1} : base + off};
+}
+
+template <typename V>
+__device__ __forceinline__ Best<V> wave_best(Best<V> b) {
+#pragma unroll
+  for (int mask = 1; mask < kWave; mask <<= 1) {
+    Best<V> o;
+    o.val = shfl_xor_any(b.val, mask);
+    o.idx = shfl_xor_any(b.idx, mask);
+    b = best_combine(b, o);
+  }
+  return b;
+}
+
+template <typename V>
+struct alignas(16) BestSlot {
+  int64_t idx;
+  V val;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kRedBlock) void argmax_chunk_kernel(int64_t* __restrict__ out,
+                                                                 void* __restrict__ ws,
+                                                                 const T* __restrict__ in,
+                                                                 int64_t rows, int64_t cols,
+                                                                 int splits, int64_t chunk) {
+  using V = typename ArgTraits<T>::val_t;
+  __shared__ BestSlot<V> slot[kRedWaves];
+  const int64_t item = blockIdx.x;
+  const int64_t row = item / splits;
+  const int split = static_cast<int>(item - row * splits);
+  const int64_t c0 = static_cast<int64_t>(split) * chunk;
+  int64_t n = cols - c0;
+  if (n > chunk) n = chunk;
+  Best<V> b = argmax_range<T, kRedBlock>(in + row * cols + c0, n, threadIdx.x, c0);
+  b = wave_best(b);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) slot[wave] = BestSlot<V>{b.idx, b.val};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Best<V> r{slot[0].val, slot[0].idx};
+#pragma unroll
+    for (int w = 1; w < kRedWaves; ++w) r = best_combine(r, Best<V>{slot[w].val, slot[w].idx});
+    if (splits == 1) {
+      out[row] = r.idx;
+    } else {
+      static_cast<BestSlot<V>*>(ws)[item] = BestSlot<V>{r.idx, r.val};
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWave) void argmax_final_kernel(int64_t* __restrict__ out,
+                                                             const void* __restrict__ ws,
+                                                             int64_t rows, int splits) {
+  using V = typename ArgTraits<T>::val_t;
+  const int64_t row = blockIdx.x;
+  Best<V> b{V(0), int64_t{-1}};
+  for (int i = threadIdx.x; i < splits; i += kWave) {
+    const BestSlot<V> s = static_cast<const BestSlot<V>*>(ws)[row * splits + i];
+    b = best_combine(b, Best<V>{s.val, s.idx});
+  }
+  b = wave_best(b);
+  if (threadIdx.x == 0) out[row] = b.idx;
+}
+
+template <typename T>
+static int launch_argmax(int64_t* out, const void* in_, int64_t rows, int64_t cols, void* ws,
+                         size_t ws_bytes, hipStream_t stream) {
+  const T* in = static_cast<const T*>(in_);
+  const SplitPlan plan = plan_splits(rows, cols);
+  const int64_t items = rows * plan.splits;
+  if (items >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  if (plan.splits > 1) {
+    if (ws == nullptr || ws_bytes < static_cast<size_t>(items) * 16) return TMB_ERR_WORKSPACE;
+  }
+  argmax_chunk_kernel<T><<<dim3(static_cast<unsigned>(items)), dim3(kRedBlock), 0, stream>>>(
+      out, ws, in, rows, cols, plan.splits, plan.chunk);
+  int rc = check_launch();
+  if (rc != 0 || plan.splits == 1) return rc;
+  argmax_final_kernel<T><<<dim3(static_cast<unsigned>(rows)), dim3(kWave), 0, stream>>>(
+      out, ws, rows, plan.splits);
+  return check_launch();
+}
+
+}  // namespace tmb
+
+extern "C" size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
+  (void)dtype;
+  if (rows <= 0 || cols <= 0) return 0;
+  const tmb::SplitPlan plan = tmb::plan_splits(rows, cols);
+  if (plan.splits == 1) return 0;
+  return static_cast<size_t>(rows) * static_cast<size_t>(plan.splits) * 16;
+}
+
+extern "C" int tmb_reduce_rows(void* out, const void* in, int64_t rows, int64_t cols, int op,
+                               int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace tmb;
+  if (rows < 0 || cols < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (op != TMB_SUM && op != TMB_MEAN && op != TMB_AMAX) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0) return TMB_OK;
+  if (cols == 0) return TMB_ERR_INVALID_ARGUMENT;  // empty rows have no max/mean; caller decides
+  if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool is_max = op == TMB_AMAX;
+  switch (dtype) {
+    case TMB_F32:
+      return is_max ? launch_reduce<AccFMax, float, false>(out, in, rows, cols, op, workspace, workspace_bytes, s)
+                    : launch_reduce<AccSum<float>, float, false>(out, in, rows, cols, op, workspace, workspace_bytes, s);
+    case TMB_F16:
+      return is_max ? launch_reduce<AccFMax, f16_t, false>(out, in, rows, cols, op, workspace, workspace_bytes, s)
+                    : launch_reduce<AccSum<float>, f16_t, false>(out, in, rows, cols, op, workspace, workspace_bytes, s);
+    case TMB_BF16:
+      return is_max ? launch_reduce<AccFMax, bf16_t, false>(out, in, rows, cols, op, workspace, workspace_bytes, s)
+                    : launch_reduce<AccSum<float>, bf16_t, false>(out, in, rows, cols, op, workspace, workspace_bytes, s);
+    case TMB_I64:
+      if (op == TMB_MEAN) return TMB_ERR_UNSUPPORTED;
+      return is_max ? launch_reduce<AccIMax<int64_t>, int64_t, true>(out, in, rows, cols, op, workspace, workspace_bytes, s)
+                    : launch_reduce<AccSum<int64_t>, int64_t, false>(out, in, rows, cols, op, workspace, workspace_bytes, s);
+    case TMB_I32:
+      if (!is_max) return TMB_ERR_UNSUPPORTED;
+      return launch_reduce<AccIMax<int32_t>, int32_t, true>(out, in, rows, cols, op, workspace, workspace_bytes, s);
+    default:
+      return TMB_ERR_UNSUPPORTED;
+  }
+}
+
+extern "C" int tmb_argmax_rows(int64_t* out, const void* in, int64_t rows, int64_t cols,
+                               int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace tmb;
+  if (rows < 0 || cols < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0) return TMB_OK;
+  if (cols == 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case TMB_F32: return launch_argmax<float>(out, in, rows, cols, workspace, workspace_bytes, s);
+    case TMB_F16: return launch_argmax<f16_t>(out, in, rows, cols, workspace, workspace_bytes, s);
+    case TMB_BF16: return launch_argmax<bf16_t>(out, in, rows, cols, workspace, workspace_bytes, s);
+    case TMB_I64: return launch_argmax<int64_t>(out, in, rows, cols, workspace, workspace_bytes, s);
+    case TMB_I32: return launch_argmax<int32_t>(out, in, rows, cols, workspace, workspace_bytes, s);
+    default: return TMB_ERR_UNSUPPORTED;
+  }
+}

@@ -1,0 +1,155 @@
+// Shared device helpers for the gfx950 (MI355X, wave64) kernels of libtmb_hip.
+//
+// Everything here is written for CDNA4 only: 64-lane wavefronts, DPP row
+// operations for intra-wave reductions, 16-byte vector memory accesses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tmb_hip.h"
+
+namespace tmb {
+
+using bf16_t = __bf16;
+using f16_t = _Float16;
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------
+// Scalar conversions. All arithmetic is done in fp32; storage types are cast
+// exactly once on the way out (round-to-nearest-even, the hardware default).
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float to_f32(T v) {
+  return static_cast<float>(v);
+}
+template <typename T>
+__device__ __forceinline__ T from_f32(float v) {
+  return static_cast<T>(v);
+}
+
+// 16-byte vector of storage elements.
+template <typename T>
+struct alignas(16) Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ Vec16<T> load_vec16(const T* p) {
+  return *reinterpret_cast<const Vec16<T>*>(p);
+}
+template <typename T>
+__device__ __forceinline__ void store_vec16(T* p, const Vec16<T>& v) {
+  *reinterpret_cast<Vec16<T>*>(p) = v;
+}
+
+// Stores N = 16/sizeof(TIn) fp32 values as TOut elements. When TOut is wider
+// than TIn (half_to_float softmax) this issues several 16-byte stores.
+template <typename TOut, int N>
+__device__ __forceinline__ void store_converted(TOut* p, const float (&x)[N]) {
+  constexpr int OUT_PER_VEC = 16 / sizeof(TOut);
+  static_assert(N % OUT_PER_VEC == 0, "vector width mismatch");
+#pragma unroll
+  for (int c = 0; c < N / OUT_PER_VEC; ++c) {
+    Vec16<TOut> o;
+#pragma unroll
+    for (int e = 0; e < OUT_PER_VEC; ++e) o.v[e] = from_f32<TOut>(x[c * OUT_PER_VEC + e]);
+    store_vec16(p + c * OUT_PER_VEC, o);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// exp with fp32-accurate argument reduction on top of v_exp_f32 (2^x).
+// x*log2(e) is formed as hi+lo so the result keeps ~1-2 ulp even for |x|~80.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float exp_f32(float x) {
+  constexpr float kLog2eHi = 1.44269502162933349609375f;   // float(log2 e)
+  constexpr float kLog2eLo = 1.92596299112661746e-08f;     // log2 e - hi
+  constexpr float kLn2 = 0.693147180559945309417f;
+  float hi = x * kLog2eHi;
+  float lo = __builtin_fmaf(x, kLog2eHi, -hi) + x * kLog2eLo;
+  float e = __builtin_amdgcn_exp2f(hi);
+  // 2^(hi+lo) = 2^hi * (1 + lo*ln2 + ...), |lo| < 1e-5 so first order is exact to fp32.
+  float r = __builtin_fmaf(e, lo * kLn2, e);
+  // exp(-inf) must be exactly 0 (0 * nan hazards: lo is nan when x is -inf).
+  return (x == -__builtin_inff()) ? 0.0f : r;
+}
+
+// ---------------------------------------------------------------------------
+// Wave64 reductions built on DPP row operations. After the four DPP steps all
+// 16 lanes of a DPP row hold that row's reduction; the four rows are combined
+// through v_readlane in a fixed order, so the result is wave-uniform and
+// bit-reproducible from launch to launch.
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+
+constexpr int kDppQuadXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;  // lane i <- lane 7-i within 8
+constexpr int kDppRowMirror = 0x140;      // lane i <- lane 15-i within 16
+
+__device__ __forceinline__ float readlane_f32(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+struct SumOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+// max that propagates NaN like torch.amax / torch.max do.
+struct MaxNanOp {
+  __device__ __forceinline__ float operator()(float a, float b) const {
+    return (a != a) ? a : ((b != b) ? b : (a > b ? a : b));
+  }
+};
+// plain max for softmax (rows containing NaN produce NaN through the exp/sum anyway).
+struct MaxOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+
+template <typename Op>
+__device__ __forceinline__ float wave_reduce(float v, Op op) {
+  v = op(v, dpp_f32<kDppQuadXor1>(v));
+  v = op(v, dpp_f32<kDppQuadXor2>(v));
+  v = op(v, dpp_f32<kDppRowHalfMirror>(v));
+  v = op(v, dpp_f32<kDppRowMirror>(v));
+  float r0 = readlane_f32(v, 0), r1 = readlane_f32(v, 16);
+  float r2 = readlane_f32(v, 32), r3 = readlane_f32(v, 48);
+  return op(op(r0, r1), op(r2, r3));
+}
+
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, SumOp{}); }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, MaxOp{}); }
+
+// Reduction across the waves that cooperate on one row. `slot` is an LDS array
+// of at least (waves in block) floats; `group` is the index of the first wave
+// of the row's group, `n` the number of waves per row. Fixed combine order.
+template <typename Op>
+__device__ __forceinline__ float group_reduce(float wave_val, float* slot, int wave, int group0,
+                                              int n, Op op) {
+  if (n == 1) return wave_val;
+  __syncthreads();  // protect slot reuse between successive reductions
+  if ((threadIdx.x & (kWave - 1)) == 0) slot[wave] = wave_val;
+  __syncthreads();
+  float r = slot[group0];
+  for (int i = 1; i < n; ++i) r = op(r, slot[group0 + i]);
+  return r;
+}
+
+inline int check_launch() {
+  hipError_t e = hipGetLastError();
+  return static_cast<int>(e);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace tmb

@@ -1,0 +1,310 @@
+"""The aten -> kernel registry of the ``mojo_backend`` graph surface.
+
+Mirrors the contract of the reference's ``torch_mojo_backend/aten_functions.py``:
+
+* ``MAPPING_TORCH_ATEN_TO_MOJO`` (reference :116) is a plain mutable dict keyed by
+  ``OpOverload`` / ``OpOverloadPacket`` / python builtins; users may add, override or delete
+  entries at run time;
+* ``map_to(op)`` (reference :157-198) registers a function, counts its calls under
+  ``TORCH_MOJO_BACKEND_TESTING=1`` and removes the op (every overload of a packet) from
+  ``DECOMPOSITION_TABLE`` (reference :113) so AOTAutograd hands the op over undecomposed;
+* mapping functions take the ATen schema's arguments. Here the tensors are real
+  ``torch.Tensor``s on a HIP device instead of MAX graph values, and a mapping function
+  *executes* its op.
+
+The hot ops (mm / addmm / bmm / linear, _softmax / softmax / _log_softmax, native_layer_norm,
+sum / mean / amax / argmax, gelu) run on the hand-written gfx950 kernels of ``libtmb_hip.so``.
+Every other op the reference maps is registered as the PyTorch-ROCm op itself, so whole
+models run with ``fullgraph=True``; those are not part of this package's kernel layer.
+"""
+
+from __future__ import annotations
+
+import contextvars
+import functools
+import operator
+import os
+from typing import List, Optional
+
+import torch
+from torch._decomp import core_aten_decompositions
+from torch._ops import OpOverload, OpOverloadPacket
+
+import torch_mojo_backend.is_running_tests
+from torch_mojo_backend import eager_kernels as _ek
+from torch_mojo_backend.eager_kernels import hip_ops
+from torch_mojo_backend.flags import verbose_enabled
+
+aten = torch.ops.aten
+
+# The fx node currently executed, set by the graph executor; lets multi-output mappings see
+# which outputs are consumed (reference :98-109).
+CURRENT_FX_NODE: contextvars.ContextVar = contextvars.ContextVar("CURRENT_FX_NODE", default=None)
+
+
+def _only_first_output_used() -> bool:
+    node = CURRENT_FX_NODE.get()
+    if node is None:
+        return False
+    return all(user.target is operator.getitem and user.args[1] == 0 for user in node.users)
+
+
+DECOMPOSITION_TABLE = core_aten_decompositions()
+original_decomposition_table_size = len(DECOMPOSITION_TABLE)
+MAPPING_TORCH_ATEN_TO_MOJO: dict = {}
+
+IDENTICAL_FUNCTIONS = [
+    operator.add, operator.sub, operator.mul, operator.truediv, operator.floordiv, operator.pow,
+    operator.mod, operator.matmul, operator.neg, operator.gt, operator.ge, operator.lt,
+    operator.le, operator.eq, operator.ne, operator.and_, operator.or_, operator.xor,
+    operator.iadd, operator.isub, operator.imul, operator.ifloordiv, operator.ipow,
+    operator.imod, operator.getitem, str, max, min,
+]
+for _func in IDENTICAL_FUNCTIONS:
+    MAPPING_TORCH_ATEN_TO_MOJO[_func] = _func
+
+number_of_decompositions_removed = 0
+
+
+def map_to(func):
+    """Register the decorated function as the implementation of ``func``."""
+
+    def decorator(func_to_map):
+        global number_of_decompositions_removed
+        if os.environ.get("TORCH_MOJO_BACKEND_BEARTYPE", "0") == "1":
+            try:
+                from beartype import beartype
+            except ImportError:  # optional dependency
+                beartype = None
+            if beartype is not None:
+                func_to_map = beartype(func_to_map)
+
+        registered = func_to_map
+        if torch_mojo_backend.is_running_tests.IS_RUNNING_TESTS:
+
+            @functools.wraps(func_to_map)
+            def counted(*args, **kwargs):
+                counted.call_count += 1
+                return func_to_map(*args, **kwargs)
+
+            counted.call_count = 0
+            registered = counted
+
+        if isinstance(func, OpOverload):
+            DECOMPOSITION_TABLE.pop(func, None)
+        elif isinstance(func, OpOverloadPacket):
+            for overload_name in func.overloads():
+                if DECOMPOSITION_TABLE.pop(getattr(func, overload_name), None) is not None:
+                    number_of_decompositions_removed += 1
+        else:
+            raise TypeError(f"Expected OpOverload or OpOverloadPacket, got {type(func)}")
+        MAPPING_TORCH_ATEN_TO_MOJO[func] = registered
+        return registered
+
+    return decorator
+
+
+# ---------------------------------------------------------------------------
+# Hot ops on the HIP kernels
+# ---------------------------------------------------------------------------
+def _normalize_dims(dim, rank: int) -> List[int]:
+    """None / [] -> all dims; ints wrapped; sorted (reference :1002-1020, :3311-3346)."""
+    if dim is None:
+        return list(range(rank))
+    if isinstance(dim, int):
+        dim = [dim]
+    dims = [d % rank if rank else 0 for d in dim]
+    if not dims:
+        return list(range(rank))
+    if len(set(dims)) != len(dims):
+        raise ValueError(f"dim {tuple(dim)} has duplicates")
+    return sorted(dims)
+
+
+@map_to(aten.mm)
+def aten_mm(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """reference :2632-2634."""
+    return hip_ops.gemm(x, y)
+
+
+@map_to(aten.bmm)
+def aten_bmm(input: torch.Tensor, mat2: torch.Tensor) -> torch.Tensor:
+    """reference :1415-1428."""
+    return hip_ops.gemm(input, mat2)
+
+
+@map_to(aten.addmm)
+def aten_addmm(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor, *, beta=1.0,
+               alpha=1.0) -> torch.Tensor:
+    """``beta*input + alpha*(mat1 @ mat2)`` (reference :971-992). A ``[n]`` bias with
+    beta == alpha == 1 is fused into the GEMM epilogue (added in fp32 before the one cast,
+    matmul_ops.mojo:2651-2657); any other case scales and adds afterwards."""
+    n = mat2.shape[-1]
+    if beta == 1 and alpha == 1 and input.dim() == 1 and input.shape[0] == n \
+            and input.dtype == mat1.dtype:
+        return hip_ops.gemm(mat1, mat2, input)
+    result = hip_ops.gemm(mat1, mat2)
+    if alpha != 1:
+        result = result * alpha
+    scaled = input * beta if beta != 1 else input
+    return scaled + result
+
+
+def addmm_gelu(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor,
+               approximate: str = "none") -> torch.Tensor:
+    """``gelu(addmm(bias, mat1, mat2))`` in one kernel. Produced by the executor's
+    addmm -> view -> gelu fusion; the epilogue rounds to the storage dtype before the GELU, so
+    the result is bit-identical to the unfused pair."""
+    epi = _ek.EPI_GELU_TANH if approximate == "tanh" else _ek.EPI_GELU_ERF
+    return hip_ops.gemm(mat1, mat2, input, epilogue=epi)
+
+
+@map_to(aten.linear)
+def aten_linear(input: torch.Tensor, weight: torch.Tensor,
+                bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``input @ weight.T + bias`` (reference :2313-2320); the weight is read K-major in place."""
+    lead = input.shape[:-1]
+    x2 = input.reshape(-1, input.shape[-1]) if input.dim() != 2 else input
+    out = hip_ops.gemm(x2, weight.t(), bias)
+    return out if input.dim() == 2 else out.reshape(*lead, weight.shape[0])
+
+
+@map_to(aten._softmax)
+def aten__softmax(self: torch.Tensor, dim: int, half_to_float: bool) -> torch.Tensor:
+    """reference :681-687."""
+    return hip_ops.softmax(self, dim, half_to_float=half_to_float)
+
+
+@map_to(aten.softmax)
+def aten_softmax(input: torch.Tensor, dim: int = -1, dtype=None) -> torch.Tensor:
+    """reference :690-714: an explicit dtype casts the input first."""
+    if dtype is not None and dtype != input.dtype:
+        if dtype == torch.float32 and input.dtype in (torch.float16, torch.bfloat16):
+            return hip_ops.softmax(input, dim, half_to_float=True)
+        input = input.to(dtype)
+    return hip_ops.softmax(input, dim)
+
+
+@map_to(aten._log_softmax)
+def aten__log_softmax(input: torch.Tensor, dim: int, half_to_float: bool) -> torch.Tensor:
+    """reference :718-785: half_to_float is float16-only."""
+    if half_to_float and input.dtype != torch.float16:
+        raise ValueError(
+            f"half_to_float conversion is supported for Half (float16) type only, got {input.dtype}")
+    return hip_ops.softmax(input, dim, half_to_float=half_to_float, log=True)
+
+
+@map_to(aten.native_layer_norm)
+def aten_native_layer_norm(input: torch.Tensor, normalized_shape, weight: Optional[torch.Tensor],
+                           bias: Optional[torch.Tensor], eps: float):
+    """(out, mean, rstd) with keepdim float32 statistics (reference :2829-2868). When only
+    output 0 is consumed the statistics are neither allocated nor written (reference
+    :2837-2849)."""
+    normalized_shape = [int(s) for s in normalized_shape]
+    if _only_first_output_used():
+        out, _, _ = hip_ops.layer_norm(input, normalized_shape, weight, bias, eps, need_stats=False)
+        return out, None, None
+    return hip_ops.layer_norm(input, normalized_shape, weight, bias, eps)
+
+
+_INT_PROMOTE = (torch.bool, torch.uint8, torch.int8, torch.int16, torch.int32)
+
+
+@map_to(aten.sum)
+def aten_sum(input: torch.Tensor, dim=None, keepdim: bool = False, *, dtype=None) -> torch.Tensor:
+    """reference :3311-3346: small integer / bool inputs are summed as int64."""
+    if dtype is not None:
+        input = input.to(dtype)
+    elif input.dtype in _INT_PROMOTE:
+        input = input.to(torch.int64)
+    dims = _normalize_dims(dim, input.dim())
+    if input.numel() == 0:
+        shape = [1 if d in dims else s for d, s in enumerate(input.shape)] if keepdim else \
+            [s for d, s in enumerate(input.shape) if d not in dims]
+        return torch.zeros(shape, dtype=input.dtype, device=input.device)
+    return hip_ops.reduce(input, dims, keepdim, _ek.SUM)
+
+
+@map_to(aten.mean)
+def aten_mean(input: torch.Tensor, dim=None, keepdim: bool = False, *, dtype=None) -> torch.Tensor:
+    """reference :2556-2590."""
+    if dtype is not None:
+        input = input.to(dtype)
+    return hip_ops.reduce(input, _normalize_dims(dim, input.dim()), keepdim, _ek.MEAN)
+
+
+@map_to(aten.amax)
+def aten_amax(input: torch.Tensor, dim=[], keepdim: bool = False) -> torch.Tensor:
+    """reference :1002-1020."""
+    return hip_ops.reduce(input, _normalize_dims(dim, input.dim()), keepdim, _ek.AMAX)
+
+
+@map_to(aten.argmax)
+def aten_argmax(input: torch.Tensor, dim: Optional[int] = None, keepdim: bool = False) -> torch.Tensor:
+    """reference :1141-1196."""
+    return hip_ops.argmax(input, dim, keepdim)
+
+
+@map_to(aten.gelu)
+def aten_gelu(input: torch.Tensor, approximate: str = "none") -> torch.Tensor:
+    """reference :2063-2067."""
+    return hip_ops.gelu(input, approximate)
+
+
+HOT_OPS = (aten.mm, aten.bmm, aten.addmm, aten.linear, aten._softmax, aten.softmax,
+           aten._log_softmax, aten.native_layer_norm, aten.sum, aten.mean, aten.amax,
+           aten.argmax, aten.gelu)
+
+# ---------------------------------------------------------------------------
+# Every other op the reference maps: the PyTorch-ROCm op itself.
+# ---------------------------------------------------------------------------
+_PASSTHROUGH = """
+floordiv _local_scalar_dense all _adaptive_avg_pool2d _adaptive_avg_pool2d_backward
+_native_batch_norm_legit_no_training _scaled_dot_product_attention_math
+_scaled_dot_product_efficient_attention _scaled_dot_product_flash_attention
+_log_softmax_backward_data.default _to_copy abs acos add addcdiv addcmul alias amin any arange
+argmin asinh atanh avg_pool2d bitwise_and.Scalar bitwise_and.Tensor bitwise_not bitwise_or.Scalar
+bitwise_or.Tensor bitwise_xor.Scalar bitwise_xor.Tensor cat ceil clamp clone constant_pad_nd
+convolution copy cos cosh cumsum detach div embedding empty.memory_format empty_strided empty_like
+empty_permuted eq erf exp expand fill fill_ floor full full_like ge gelu_backward gt index isin
+isnan le linear_backward.default lift_fresh_copy log log1p logical_and logical_not logical_xor lt
+max max_pool2d_with_indices maximum mean.out min minimum mul native_batch_norm native_group_norm
+normal_ ne neg nonzero ones_like permute pow reciprocal relu remainder repeat relu_ rsqrt
+scalar_tensor scaled_dot_product_attention scatter.src scatter.value select select_scatter sigmoid
+sign silu sin tan tanh sinh slice split_with_sizes sqrt squeeze sub unsqueeze upsample_bilinear2d
+var view _unsafe_view where stack tril triu split unbind t.default _foreach_add.Scalar
+_foreach_add.ScalarList _foreach_add.Tensor _foreach_add.List _foreach_sub.Scalar
+_foreach_sub.ScalarList _foreach_sub.List _foreach_mul.Scalar _foreach_mul.ScalarList
+_foreach_mul.Tensor _foreach_mul.List _foreach_neg _foreach_pow.Scalar _foreach_pow.ScalarList
+_foreach_pow.List _foreach_pow.ScalarAndTensor _foreach_div.Scalar _foreach_div.ScalarList
+_foreach_div.Tensor _foreach_div.List _foreach_reciprocal _foreach_sqrt _foreach_addcdiv.Scalar
+_foreach_addcdiv.ScalarList _foreach_addcmul.Scalar _foreach_addcmul.ScalarList masked_fill
+transpose sym_size sym_numel sym_stride sym_storage_offset
+""".split()
+
+
+def _resolve(name: str):
+    obj = aten
+    for part in name.split("."):
+        obj = getattr(obj, part, None)
+        if obj is None:
+            return None
+    return obj
+
+
+def _passthrough(op):
+    def run(*args, **kwargs):
+        return op(*args, **kwargs)
+
+    run.__name__ = "aten_" + str(getattr(op, "__name__", op)).replace(".", "_")
+    run.__qualname__ = run.__name__
+    return run
+
+
+for _name in _PASSTHROUGH:
+    _op = _resolve(_name)
+    if _op is not None and _op not in MAPPING_TORCH_ATEN_TO_MOJO:
+        map_to(_op)(_passthrough(_op))
+
+if verbose_enabled():
+    print(f"Removed {number_of_decompositions_removed}/{original_decomposition_table_size} decompositions.")

@@ -1,0 +1,64 @@
+"""Loader of ``libtmb_hip.so``, the C-ABI library of hand-written gfx950 kernels.
+
+Takes the place of the reference's lazy Mojo-extension loader
+(torch_mojo_backend/eager_kernels/__init__.py:36-126): there the kernels are JIT-compiled
+CPython extensions, here they are one prebuilt shared library bound with ctypes. Kernels are
+enqueued on the caller's stream and never synchronise (reference: same file, lines 9-12).
+
+There is no CPU or PyTorch fallback: if the library is missing, loading raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+_CSRC = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", "csrc"))
+LIBRARY_PATH = os.path.join(_CSRC, "libtmb_hip.so")
+
+F32, F16, BF16, I64, I32 = 0, 1, 2, 3, 4
+SUM, MEAN, AMAX = 0, 1, 2
+EPI_NONE, EPI_GELU_TANH, EPI_GELU_ERF = 0, 1, 2
+
+# Every symbol include/tmb_hip.h declares, with its ctypes signature.
+_i64, _vp, _ci, _sz, _dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_double
+SIGNATURES = {
+    "tmb_version": (_ci, []),
+    "tmb_status_string": (ctypes.c_char_p, [_ci]),
+    "tmb_softmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _ci, _vp]),
+    "tmb_layer_norm_rows": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _dbl, _ci, _vp]),
+    "tmb_reduce_workspace_bytes": (_sz, [_i64, _i64, _ci]),
+    "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
+    "tmb_argmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _vp, _sz, _vp]),
+    "tmb_gemm": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp]),
+    "tmb_gelu": (_ci, [_vp, _vp, _i64, _ci, _ci, _vp]),
+    "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+class HipLibraryMissing(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises ``HipLibraryMissing`` (never falls back) when absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIBRARY_PATH):
+            raise HipLibraryMissing(
+                f"{LIBRARY_PATH} is not built. Build it with `sh {os.path.join(_CSRC, 'build.sh')}` "
+                "(hipcc, gfx950). torch_mojo_backend has no CPU or PyTorch fallback for its hot ops."
+            )
+        handle = ctypes.CDLL(LIBRARY_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def status_string(code: int) -> str:
+    return lib().tmb_status_string(int(code)).decode()

@@ -1,0 +1,281 @@
+"""Tensor-level launchers over the C ABI of ``libtmb_hip.so``.
+
+Both surfaces of the backend — the graph registry (``aten_functions``) and the eager
+``fast_aten_*`` functions (``aten_fast``) — end up here. Each launcher validates on the host,
+allocates its outputs with PyTorch-ROCm's stream-ordered caching allocator (the ownership role
+the reference gives to ``TensorHolder``, op_utils/__init__.mojo:250-263), and enqueues the
+kernel on the current HIP stream without synchronising.
+
+Inputs must live on a HIP device. CPU tensors are rejected: there is no CPU route.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from torch_mojo_backend import eager_kernels as _ek
+
+_CODES = {
+    torch.float32: _ek.F32,
+    torch.float16: _ek.F16,
+    torch.bfloat16: _ek.BF16,
+    torch.int64: _ek.I64,
+    torch.int32: _ek.I32,
+}
+FLOAT_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+
+_OOM_CODE = 2  # hipErrorOutOfMemory
+
+
+class HipKernelError(RuntimeError):
+    def __init__(self, op: str, code: int):
+        self.code = code
+        super().__init__(f"{op} failed: {_ek.status_string(code)} (status {code})")
+
+
+def _check(op: str, code: int) -> None:
+    if code == 0:
+        return
+    if code == _OOM_CODE:
+        raise torch.OutOfMemoryError(f"{op}: HIP out of memory")
+    raise HipKernelError(op, code)
+
+
+def require_hip(*tensors: Optional[torch.Tensor]) -> torch.device:
+    """All tensors on one HIP device, else TypeError (validated before any allocation)."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise TypeError(
+                f"torch_mojo_backend HIP kernels need tensors on a HIP device, got {t.device}; "
+                "there is no CPU path"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise TypeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def code_of(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise TypeError(f"dtype {dtype} has no HIP kernel") from None
+
+
+# ---------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------
+def _matrix_layout(t: torch.Tensor) -> Optional[Tuple[int, int]]:
+    """(transposed, leading_dimension) of the last two dims if they are dense row-major or
+    dense column-major, else None (same classification as aten_fast.py:4457-4492)."""
+    rows, cols = t.shape[-2], t.shape[-1]
+    sr, sc = t.stride(-2), t.stride(-1)
+    if (sc == 1 or cols == 1) and (sr >= cols or rows == 1):
+        return 0, max(sr if rows > 1 else cols, cols, 1)
+    if (sr == 1 or rows == 1) and (sc >= rows or cols == 1):
+        return 1, max(sc if cols > 1 else rows, rows, 1)
+    return None
+
+
+def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
+         epilogue: int = _ek.EPI_NONE) -> torch.Tensor:
+    """``epilogue(a @ b + bias)`` for 2-D operands, or 3-D operands with equal batch sizes.
+
+    Transposed views (``weight.t()``, ``k.transpose(-2, -1)``) are consumed in place through
+    the kernel's transpose flags; other non-dense layouts are materialised once.
+    """
+    require_hip(a, b, bias)
+    if a.dtype != b.dtype or a.dtype not in FLOAT_DTYPES:
+        raise TypeError(f"gemm: unsupported dtypes {a.dtype} x {b.dtype}")
+    batched = a.dim() == 3
+    if a.dim() != b.dim() or a.dim() not in (2, 3):
+        raise ValueError(f"gemm: expected two 2-D or two 3-D operands, got {a.dim()}-D x {b.dim()}-D")
+    if a.shape[-1] != b.shape[-2] or (batched and a.shape[0] != b.shape[0]):
+        raise ValueError(f"gemm: shapes {tuple(a.shape)} and {tuple(b.shape)} do not multiply")
+    m, k, n = a.shape[-2], a.shape[-1], b.shape[-1]
+    batch = a.shape[0] if batched else 1
+    if bias is not None:
+        if bias.dtype != a.dtype or tuple(bias.shape) != (n,):
+            raise ValueError(f"gemm: bias must be [{n}] {a.dtype}, got {tuple(bias.shape)} {bias.dtype}")
+        if not bias.is_contiguous():
+            bias = bias.contiguous()
+
+    la = _matrix_layout(a)
+    if la is None or (batched and batch > 1 and a.stride(0) < 0):
+        a = a.contiguous()
+        la = (0, max(k, 1))
+    lb = _matrix_layout(b)
+    if lb is None or (batched and batch > 1 and b.stride(0) < 0):
+        b = b.contiguous()
+        lb = (0, max(n, 1))
+    out = torch.empty((batch, m, n) if batched else (m, n), dtype=a.dtype, device=a.device)
+    if out.numel() == 0:
+        return out
+    lib = _ek.lib()
+    rc = lib.tmb_gemm(
+        out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
+        batch, m, n, k, la[1], lb[1], n,
+        a.stride(0) if batched else 0, b.stride(0) if batched else 0, m * n,
+        la[0], lb[0], code_of(a.dtype), epilogue, _stream())
+    _check("tmb_gemm", rc)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Row kernels
+# ---------------------------------------------------------------------------
+def _as_rows(x: torch.Tensor, dim: int) -> Tuple[torch.Tensor, bool]:
+    """x with `dim` moved last and made contiguous; flag tells whether a move happened."""
+    if dim == x.dim() - 1:
+        return (x if x.is_contiguous() else x.contiguous()), False
+    return x.movedim(dim, -1).contiguous(), True
+
+
+def softmax(x: torch.Tensor, dim: int, half_to_float: bool = False, log: bool = False) -> torch.Tensor:
+    require_hip(x)
+    if x.dtype not in FLOAT_DTYPES:
+        raise TypeError(f"softmax: unsupported dtype {x.dtype}")
+    out_dtype = torch.float32 if half_to_float else x.dtype
+    if x.dim() == 0:
+        return torch.full((), 0.0 if log else 1.0, dtype=out_dtype, device=x.device)
+    dim %= x.dim()
+    rows_t, moved = _as_rows(x, dim)
+    cols = rows_t.shape[-1]
+    out = torch.empty(rows_t.shape, dtype=out_dtype, device=x.device)
+    if out.numel():
+        rc = _ek.lib().tmb_softmax_rows(out.data_ptr(), rows_t.data_ptr(), rows_t.numel() // cols,
+                                        cols, code_of(x.dtype), code_of(out_dtype), int(log),
+                                        _stream())
+        _check("tmb_softmax_rows", rc)
+    return out.movedim(-1, dim) if moved else out
+
+
+def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optional[torch.Tensor],
+               bias: Optional[torch.Tensor], eps: float, need_stats: bool = True):
+    """(out, mean, rstd); mean/rstd are float32 with shape ``x.shape[:-k] + (1,)*k`` or None
+    when ``need_stats`` is False."""
+    require_hip(x, weight, bias)
+    k = len(normalized_shape)
+    if x.dtype not in FLOAT_DTYPES or k < 1 or x.dim() < k or \
+            tuple(x.shape[x.dim() - k:]) != tuple(normalized_shape):
+        raise ValueError(f"layer_norm: input {tuple(x.shape)} {x.dtype} vs normalized_shape "
+                         f"{tuple(normalized_shape)}")
+    for name, p in (("weight", weight), ("bias", bias)):
+        if p is not None and (p.dtype != x.dtype or tuple(p.shape) != tuple(normalized_shape)):
+            raise ValueError(f"layer_norm: {name} must be {tuple(normalized_shape)} {x.dtype}")
+    cols = math.prod(normalized_shape)
+    xc = x if x.is_contiguous() else x.contiguous()
+    rows = xc.numel() // cols if cols else 0
+    out = torch.empty_like(xc)
+    stat_shape = tuple(x.shape[: x.dim() - k]) + (1,) * k
+    mean = rstd = None
+    if need_stats:
+        mean = torch.empty(stat_shape, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(stat_shape, dtype=torch.float32, device=x.device)
+    if xc.numel():
+        w = None if weight is None else (weight if weight.is_contiguous() else weight.contiguous())
+        b = None if bias is None else (bias if bias.is_contiguous() else bias.contiguous())
+        rc = _ek.lib().tmb_layer_norm_rows(
+            out.data_ptr(), None if mean is None else mean.data_ptr(),
+            None if rstd is None else rstd.data_ptr(), xc.data_ptr(),
+            None if w is None else w.data_ptr(), None if b is None else b.data_ptr(),
+            rows, cols, float(eps), code_of(x.dtype), _stream())
+        _check("tmb_layer_norm_rows", rc)
+    return out, mean, rstd
+
+
+def _reduce_geometry(x: torch.Tensor, dims: Sequence[int]):
+    """Kept dims (ascending) then reduce dims, made contiguous: the [rows, cols] view of
+    op_utils/__init__.mojo:651-720. Returns (rows_tensor, rows, cols, kept_shape)."""
+    rank = x.dim()
+    dims = list(dims)
+    kept = [d for d in range(rank) if d not in dims]
+    trailing = dims == list(range(rank - len(dims), rank))
+    if trailing and x.is_contiguous():
+        moved = x
+    else:
+        moved = x.permute(kept + dims).contiguous()
+    cols = math.prod(x.shape[d] for d in dims)
+    rows = math.prod(x.shape[d] for d in kept)
+    return moved, rows, cols, [x.shape[d] for d in kept]
+
+
+def _workspace(rows: int, cols: int, code: int, device) -> Tuple[Optional[torch.Tensor], int]:
+    nbytes = _ek.lib().tmb_reduce_workspace_bytes(rows, cols, code)
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+
+def reduce(x: torch.Tensor, dims: Sequence[int], keepdim: bool, op: int) -> torch.Tensor:
+    """sum / mean / amax over `dims` (already normalised, sorted, unique, non-empty unless
+    x is 0-d). Output dtype = input dtype."""
+    require_hip(x)
+    code = code_of(x.dtype)
+    rank = x.dim()
+    moved, rows, cols, kept_shape = _reduce_geometry(x, dims)
+    if cols == 0 or rows == 0:
+        raise ValueError("reduce: empty reduction has no kernel; the caller decides its value")
+    out = torch.empty(kept_shape, dtype=x.dtype, device=x.device)
+    ws, ws_bytes = _workspace(rows, cols, code, x.device)
+    rc = _ek.lib().tmb_reduce_rows(out.data_ptr(), moved.data_ptr(), rows, cols, op, code,
+                                   None if ws is None else ws.data_ptr(), ws_bytes, _stream())
+    _check("tmb_reduce_rows", rc)
+    if keepdim:
+        out = out.reshape([1 if d in dims else x.shape[d] for d in range(rank)])
+    return out
+
+
+def argmax(x: torch.Tensor, dim: Optional[int], keepdim: bool) -> torch.Tensor:
+    require_hip(x)
+    code = code_of(x.dtype)
+    if x.numel() == 0:
+        raise ValueError("argmax of an empty tensor")
+    rank = x.dim()
+    if dim is None:
+        dims = list(range(rank))
+    else:
+        dims = [dim % rank] if rank else []
+    moved, rows, cols, kept_shape = _reduce_geometry(x, dims)
+    out = torch.empty(kept_shape, dtype=torch.int64, device=x.device)
+    ws, ws_bytes = _workspace(rows, cols, code, x.device)
+    rc = _ek.lib().tmb_argmax_rows(out.data_ptr(), moved.data_ptr(), rows, cols, code,
+                                   None if ws is None else ws.data_ptr(), ws_bytes, _stream())
+    _check("tmb_argmax_rows", rc)
+    if keepdim:
+        out = out.reshape([1 if d in dims else x.shape[d] for d in range(rank)])
+    return out
+
+
+def gelu(x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
+    require_hip(x)
+    if x.dtype not in FLOAT_DTYPES:
+        raise TypeError(f"gelu: unsupported dtype {x.dtype}")
+    if approximate not in ("none", "tanh"):
+        raise ValueError(f"gelu: approximate must be 'none' or 'tanh', got {approximate!r}")
+    xc = x if x.is_contiguous() else x.contiguous()
+    out = torch.empty_like(xc)
+    if xc.numel():
+        rc = _ek.lib().tmb_gelu(out.data_ptr(), xc.data_ptr(), xc.numel(), code_of(x.dtype),
+                                int(approximate == "tanh"), _stream())
+        _check("tmb_gelu", rc)
+    return out
+
+
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """Plain device copy through the library's yardstick kernel (benchmarks only)."""
+    require_hip(dst, src)
+    nbytes = src.numel() * src.element_size()
+    assert dst.numel() * dst.element_size() == nbytes and dst.is_contiguous() and src.is_contiguous()
+    _check("tmb_copy_bytes", _ek.lib().tmb_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _stream()))

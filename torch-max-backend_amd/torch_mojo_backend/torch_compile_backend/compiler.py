@@ -1,0 +1,363 @@
+"""``mojo_backend``: the ``torch.compile`` backend surface.
+
+Same public contract as the reference's ``torch_compile_backend/compiler.py``:
+
+* ``mojo_backend`` is a class instantiated per graph by dynamo — ``__init__(gm, example_inputs)``
+  wraps ``aot_autograd(fw_compiler=boxed_func, decompositions=DECOMPOSITION_TABLE)`` and
+  ``__call__(*args)`` returns a list (reference :573-583);
+* every FX ``call_function`` node is resolved through ``MAPPING_TORCH_ATEN_TO_MOJO``: the
+  exact ``node.target`` first, then its ``overloadpacket`` (reference :278-285); an unmapped op
+  raises ``MojoCompilerError`` naming the op, the node index and the user stack trace
+  (reference :287-292); an exception inside a mapping function is re-raised as
+  ``MojoCompilerError`` carrying the original message (reference :300-306);
+* ``None`` outputs are preserved and SymInt outputs come back as Python ints
+  (reference :329-369, :483-494).
+
+What differs is the engine underneath. The reference lowers the FX graph to a MAX graph and
+lets MAX compile and run it; here ``BaseMaxCompiler`` turns the FX graph into a flat program of
+(mapping function, argument slots) steps once, and ``__call__`` runs those steps in order on the
+current HIP stream: hot ops enqueue hand-written gfx950 kernels, everything stays asynchronous,
+intermediates are released at their last use. Two graph-level rewrites happen at build time:
+``addmm -> [view] -> gelu`` chains become one GEMM with a GELU epilogue, and
+``native_layer_norm`` nodes whose statistics are dead skip them (reference
+aten_functions.py:2837-2849).
+"""
+
+from __future__ import annotations
+
+import datetime as dt
+import operator
+import os
+import time
+import traceback
+from typing import Any, Callable, List, Optional
+
+import torch
+from functorch.compile import make_boxed_func
+from torch._dynamo.backends.common import aot_autograd
+
+from torch_mojo_backend import aten_functions
+from torch_mojo_backend.aten_functions import (
+    CURRENT_FX_NODE,
+    DECOMPOSITION_TABLE,
+    MAPPING_TORCH_ATEN_TO_MOJO,
+)
+from torch_mojo_backend.flags import debug_graph, profiling_enabled, verbose_enabled
+from torch_mojo_backend.torch_compile_backend.utils import get_accelerators, get_error_message
+
+__all__ = ["mojo_backend", "MojoCompilerError", "MAPPING_TORCH_ATEN_TO_MOJO", "get_accelerators",
+           "BaseMaxCompiler", "boxed_func", "dummy_backend"]
+
+aten = torch.ops.aten
+
+
+class MojoCompilerError(Exception):
+    pass
+
+
+def gather_stats_on_graph(gm: torch.fx.GraphModule) -> None:
+    """Prints a histogram of the graph's call targets (reference :67-79)."""
+    counts: dict = {}
+    for node in gm.graph.nodes:
+        if node.op in ("call_function", "call_method"):
+            counts[str(node.target)] = counts.get(str(node.target), 0) + 1
+    print("Function call statistics:")
+    for name, count in sorted(counts.items(), key=lambda kv: -kv[1]):
+        print(f"  {name}: {count}")
+
+
+def _fusion_enabled() -> bool:
+    return os.environ.get("TORCH_MOJO_BACKEND_NO_FUSION", "0").lower() not in ("1", "true", "yes")
+
+
+def _identity(x, *args, **kwargs):
+    return x
+
+
+class _Slot:
+    """Reference to the value an earlier node produced."""
+
+    __slots__ = ("index",)
+
+    def __init__(self, index: int):
+        self.index = index
+
+
+def _has_slot(value) -> bool:
+    if isinstance(value, _Slot):
+        return True
+    if isinstance(value, (list, tuple)):
+        return any(_has_slot(v) for v in value)
+    if isinstance(value, dict):
+        return any(_has_slot(v) for v in value.values())
+    return False
+
+
+def _materialize(value, env):
+    if isinstance(value, _Slot):
+        return env[value.index]
+    if isinstance(value, list):
+        return [_materialize(v, env) for v in value]
+    if isinstance(value, tuple):
+        return tuple(_materialize(v, env) for v in value)
+    if isinstance(value, dict):
+        return {k: _materialize(v, env) for k, v in value.items()}
+    if isinstance(value, slice):
+        return slice(_materialize(value.start, env), _materialize(value.stop, env),
+                     _materialize(value.step, env))
+    return value
+
+
+class _Step:
+    __slots__ = ("fn", "args", "kwargs", "dynamic_args", "dynamic_kwargs", "out", "node",
+                 "node_idx", "release", "key")
+
+
+class _GraphFactory:
+    """Turns an FX graph into a step program (counterpart of the reference's ``_GraphFactory``,
+    :154-403, which emits MAX graph ops instead)."""
+
+    def __init__(self):
+        self.slots: dict = {}
+        self.steps: List[_Step] = []
+        self.input_slots: List[int] = []
+        self.constants: List[tuple] = []
+        self.output_template: Any = None
+
+    def _slot_of(self, node: torch.fx.Node) -> int:
+        return self.slots[node.name]
+
+    def _convert(self, value):
+        if isinstance(value, torch.fx.Node):
+            return _Slot(self._slot_of(value))
+        if isinstance(value, list):
+            return [self._convert(v) for v in value]
+        if isinstance(value, tuple):
+            return tuple(self._convert(v) for v in value)
+        if isinstance(value, dict):
+            return {k: self._convert(v) for k, v in value.items()}
+        if isinstance(value, slice):
+            return slice(self._convert(value.start), self._convert(value.stop),
+                         self._convert(value.step))
+        return value
+
+    def resolve(self, node_idx: int, node: torch.fx.Node) -> tuple:
+        key = node.target
+        if key not in MAPPING_TORCH_ATEN_TO_MOJO and \
+                getattr(key, "overloadpacket", None) in MAPPING_TORCH_ATEN_TO_MOJO:
+            key = key.overloadpacket
+        if key not in MAPPING_TORCH_ATEN_TO_MOJO:
+            raise MojoCompilerError(
+                "The aten function is not supported by the Mojo backend yet. "
+                + get_error_message(node, node_idx, node.args, node.kwargs)
+                + "You can try to write it yourself and insert it in the "
+                  "MAPPING_TORCH_ATEN_TO_MOJO dictionary."
+            )
+        return key, MAPPING_TORCH_ATEN_TO_MOJO[key]
+
+    @staticmethod
+    def _fuse_bias_gelu(graph: torch.fx.Graph) -> dict:
+        """addmm (single user) -> optional view/_unsafe_view (single user) -> gelu.
+        Returns {addmm_node: approximate, gelu_node: None} for the nodes to rewrite."""
+        rewrites: dict = {}
+        if MAPPING_TORCH_ATEN_TO_MOJO.get(aten.addmm) is not _BUILTIN_ADDMM or \
+                MAPPING_TORCH_ATEN_TO_MOJO.get(aten.gelu) is not _BUILTIN_GELU:
+            return rewrites  # a user replaced one of the two ops: leave the graph alone
+        for node in graph.nodes:
+            if node.op != "call_function" or node.target not in (aten.gelu.default, aten.gelu):
+                continue
+            src = node.args[0]
+            via = None
+            if isinstance(src, torch.fx.Node) and src.op == "call_function" and src.target in (
+                    aten.view.default, aten._unsafe_view.default) and len(src.users) == 1:
+                via, src = src, src.args[0]
+            if not (isinstance(src, torch.fx.Node) and src.op == "call_function"
+                    and src.target is aten.addmm.default and len(src.users) == 1):
+                continue
+            if src.kwargs.get("beta", 1) != 1 or src.kwargs.get("alpha", 1) != 1:
+                continue
+            bias_meta = src.args[0].meta.get("val") if isinstance(src.args[0], torch.fx.Node) else None
+            if bias_meta is None or bias_meta.dim() != 1:
+                continue
+            approximate = node.kwargs.get("approximate", node.args[1] if len(node.args) > 1 else "none")
+            rewrites[src] = approximate
+            rewrites[node] = None
+        return rewrites
+
+    def create_graph(self, graph: torch.fx.Graph):
+        rewrites = self._fuse_bias_gelu(graph) if _fusion_enabled() else {}
+        nodes = list(graph.nodes)
+        last_use: dict = {}
+        for idx, node in enumerate(nodes):
+            for used in node.all_input_nodes:
+                last_use[used.name] = idx
+        for idx, node in enumerate(nodes):
+            if node.op == "placeholder":
+                self.slots[node.name] = len(self.slots)
+                self.input_slots.append(self.slots[node.name])
+            elif node.op == "get_attr":
+                self.slots[node.name] = len(self.slots)
+                owner = graph.owning_module
+                value = owner
+                for part in node.target.split("."):
+                    value = getattr(value, part)
+                self.constants.append((self.slots[node.name], value))
+            elif node.op == "call_function":
+                key, fn = self.resolve(idx, node)
+                args, kwargs = node.args, dict(node.kwargs)
+                if node in rewrites:
+                    if rewrites[node] is None:
+                        fn, args, kwargs = _identity, (node.args[0],), {}
+                    else:
+                        fn = _FUSED_ADDMM_GELU
+                        kwargs = {"approximate": rewrites[node]}
+                step = _Step()
+                step.fn = fn
+                step.key = key
+                step.args = self._convert(args)
+                step.kwargs = self._convert(kwargs)
+                step.dynamic_args = _has_slot(step.args)
+                step.dynamic_kwargs = _has_slot(step.kwargs)
+                self.slots[node.name] = len(self.slots)
+                step.out = self.slots[node.name]
+                step.node = node
+                step.node_idx = idx
+                step.release = ()
+                self.steps.append(step)
+            elif node.op == "output":
+                self.output_template = self._convert(node.args[0])
+            else:
+                raise MojoCompilerError(f"Unsupported FX node kind {node.op!r} ({node.name})")
+        # Release each value after the step that uses it last (never graph outputs).
+        output_node = nodes[-1]
+        keep = {n.name for n in output_node.all_input_nodes}
+        step_of_idx = {s.node_idx: s for s in self.steps}
+        for name, idx in last_use.items():
+            if name in keep or idx not in step_of_idx:
+                continue
+            step_of_idx[idx].release = step_of_idx[idx].release + (self.slots[name],)
+        for s in self.steps:  # a value nobody uses is dropped right away
+            if s.node.name not in last_use and s.node.name not in keep:
+                s.release = s.release + (s.out,)
+        return self
+
+
+def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none"):
+    n = mat2.shape[-1]
+    if input.dim() == 1 and input.shape[0] == n and input.dtype == mat1.dtype:
+        return aten_functions.addmm_gelu(input, mat1, mat2, approximate)
+    return _BUILTIN_GELU(_BUILTIN_ADDMM(input, mat1, mat2), approximate=approximate)
+
+
+_BUILTIN_ADDMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.addmm]
+_BUILTIN_GELU = MAPPING_TORCH_ATEN_TO_MOJO[aten.gelu]
+_FUSED_ADDMM_GELU = _fused_addmm_gelu
+
+
+class BaseMaxCompiler:
+    """Executable form of one FX graph (the name is the reference's, :455-532)."""
+
+    def __init__(self, gm: torch.fx.GraphModule, example_inputs: list, mode=None):
+        self.gm = gm
+        start = time.time_ns() if profiling_enabled() else 0
+        if verbose_enabled():
+            print(f"Graph has {len(gm.graph.nodes)} nodes.")
+            gather_stats_on_graph(gm)
+            gm.graph.print_tabular()
+        self.program = _GraphFactory().create_graph(gm.graph)
+        self.num_slots = len(self.program.slots)
+        if profiling_enabled():
+            elapsed = dt.timedelta(microseconds=(time.time_ns() - start) / 1000)
+            print(f"Building the step program in {elapsed}")
+
+    def _fail(self, step: _Step, args, kwargs, exc: Exception):
+        raise MojoCompilerError(
+            get_error_message(step.node, step.node_idx, args, kwargs)
+            + "There was an error when executing the function. See the original error below. \n"
+            f"{exc}\n"
+            f"{traceback.format_exc()}"
+        ) from exc
+
+    def __call__(self, *args) -> list:
+        start = time.time_ns() if profiling_enabled() else 0
+        program = self.program
+        env: List[Any] = [None] * self.num_slots
+        if len(args) != len(program.input_slots):
+            raise MojoCompilerError(
+                f"graph takes {len(program.input_slots)} inputs, got {len(args)}")
+        for slot, value in zip(program.input_slots, args):
+            env[slot] = value
+        for slot, value in program.constants:
+            env[slot] = value
+        check = debug_graph()
+        for step in program.steps:
+            a = _materialize(step.args, env) if step.dynamic_args else step.args
+            kw = _materialize(step.kwargs, env) if step.dynamic_kwargs else step.kwargs
+            token = CURRENT_FX_NODE.set(step.node)
+            try:
+                out = step.fn(*a, **kw)
+            except Exception as exc:  # noqa: BLE001 - re-raised with the node's context
+                self._fail(step, a, kw, exc)
+            finally:
+                CURRENT_FX_NODE.reset(token)
+            if check:
+                _compare_with_torch(step, a, kw, out)
+            env[step.out] = out
+            for slot in step.release:
+                env[slot] = None
+        result = _materialize(program.output_template, env)
+        if profiling_enabled():
+            elapsed = dt.timedelta(microseconds=(time.time_ns() - start) / 1000)
+            print(f"Enqueueing the graph in {elapsed}")
+        if isinstance(result, tuple):
+            result = list(result)
+        elif not isinstance(result, list):
+            result = [result]
+        return [int(r) if isinstance(r, torch.SymInt) else r for r in result]
+
+
+def _compare_with_torch(step: _Step, args, kwargs, out) -> None:
+    """TORCH_MOJO_BACKEND_DEBUG_GRAPH=1: run the node's own aten op with PyTorch-ROCm and report
+    the largest deviation (the reference compares MAX against torch per node, debug.py:27-128)."""
+    target = step.node.target
+    if step.fn is _identity or not callable(target) or step.key not in aten_functions.HOT_OPS:
+        return
+    try:
+        if step.fn is _FUSED_ADDMM_GELU:
+            expected = torch.nn.functional.gelu(target(*args), approximate=kwargs["approximate"])
+        else:
+            expected = target(*args, **kwargs)
+    except Exception as exc:  # noqa: BLE001
+        print(f"[debug_graph] node {step.node_idx} {target}: torch failed: {exc}")
+        return
+    outs = out if isinstance(out, (tuple, list)) else (out,)
+    exps = expected if isinstance(expected, (tuple, list)) else (expected,)
+    for i, (o, e) in enumerate(zip(outs, exps)):
+        if isinstance(o, torch.Tensor) and isinstance(e, torch.Tensor) and o.numel():
+            diff = (o.double() - e.double()).abs().max().item()
+            print(f"[debug_graph] node {step.node_idx} {target} out{i}: max abs diff {diff:.3e}")
+
+
+def boxed_func(*args, **kwargs):
+    return make_boxed_func(BaseMaxCompiler(*args, **kwargs).__call__)
+
+
+class mojo_backend:
+    def __init__(self, gm: torch.fx.GraphModule, example_inputs: list):
+        self.func_to_execute = aot_autograd(
+            fw_compiler=boxed_func, decompositions=DECOMPOSITION_TABLE
+        )(gm, example_inputs)
+
+    def __call__(self, *args) -> list:
+        result = self.func_to_execute(*args)
+        if isinstance(result, tuple):
+            return list(result)
+        return result
+
+
+def dummy_compiler(gm: torch.fx.GraphModule, example_inputs: list):
+    return make_boxed_func(gm.forward)
+
+
+# To tell a backend problem from a model problem: same pipeline, PyTorch's own kernels.
+dummy_backend = aot_autograd(fw_compiler=dummy_compiler)
