@@ -1,0 +1,102 @@
+"""The C-ABI library: it loads without a GPU, exports every symbol include/tmb_hip.h declares,
+and rejects malformed arguments on the host before anything would be enqueued."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tmb_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tmb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from torch_mojo_backend import eager_kernels as ek
+
+    declared = _declared_symbols()
+    assert len(declared) >= 10
+    handle = ctypes.CDLL(ek.LIBRARY_PATH)
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in tmb_hip.h but not exported"
+    assert sorted(ek.SIGNATURES) == declared, "ctypes signature table out of sync with the header"
+
+
+def test_version_and_status_strings():
+    from torch_mojo_backend import eager_kernels as ek
+
+    L = ek.lib()
+    assert L.tmb_version() == 1000
+    assert ek.status_string(0) == "ok"
+    assert "invalid" in ek.status_string(-1)
+    assert "unsupported" in ek.status_string(-2)
+    assert "workspace" in ek.status_string(-3)
+
+
+def test_host_side_argument_validation_needs_no_gpu():
+    from torch_mojo_backend import eager_kernels as ek
+
+    L = ek.lib()
+    # negative sizes / null pointers / unknown enums are refused before any launch
+    assert L.tmb_softmax_rows(None, None, -1, 4, ek.F32, ek.F32, 0, None) == -1
+    assert L.tmb_softmax_rows(None, None, 3, 4, ek.F32, ek.F32, 0, None) == -1
+    assert L.tmb_softmax_rows(None, None, 0, 4, ek.F32, ek.F32, 0, None) == 0   # empty: nothing to do
+    assert L.tmb_layer_norm_rows(None, None, None, None, None, None, 2, 2, 1e-5, ek.F32, None) == -1
+    assert L.tmb_reduce_rows(None, None, 2, 2, 7, ek.F32, None, 0, None) == -1  # unknown op
+    assert L.tmb_reduce_rows(None, None, 2, 0, ek.SUM, ek.F32, None, 0, None) == -1
+    assert L.tmb_argmax_rows(None, None, 2, 0, ek.F32, None, 0, None) == -1
+    assert L.tmb_gemm(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 0, None) == -1
+    assert L.tmb_gemm(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.I64, 0, None) == -2
+    assert L.tmb_gemm(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 9, None) == -1
+    assert L.tmb_gemm(None, None, None, None, 0, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 0, None) == 0
+    assert L.tmb_gelu(None, None, -5, ek.F32, 1, None) == -1
+
+
+def test_workspace_plan_is_a_pure_function_of_the_shape():
+    from torch_mojo_backend import eager_kernels as ek
+
+    L = ek.lib()
+    assert L.tmb_reduce_workspace_bytes(65536, 4096, ek.F32) == 0        # one pass, no scratch
+    full = L.tmb_reduce_workspace_bytes(1, 65536 * 4096, ek.F32)
+    assert full > 0 and full % 16 == 0
+    assert full == L.tmb_reduce_workspace_bytes(1, 65536 * 4096, ek.BF16)
+    assert L.tmb_reduce_workspace_bytes(512, 50257, ek.F32) == 512 * 3 * 16
+    assert L.tmb_reduce_workspace_bytes(0, 10, ek.F32) == 0
+
+
+def test_product_refuses_cpu_tensors_and_never_falls_back():
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    x = torch.randn(4, 8)
+    for call in (lambda: hip_ops.softmax(x, -1), lambda: hip_ops.gemm(x, x.t()),
+                 lambda: hip_ops.layer_norm(x, [8], None, None, 1e-5),
+                 lambda: hip_ops.reduce(x, [1], False, 0), lambda: hip_ops.argmax(x, 1, False),
+                 lambda: hip_ops.gelu(x)):
+        with pytest.raises(TypeError, match="no CPU path"):
+            call()
+
+
+def test_missing_library_raises(monkeypatch, tmp_path):
+    from torch_mojo_backend import eager_kernels as ek
+
+    monkeypatch.setattr(ek, "_lib", None)
+    monkeypatch.setattr(ek, "LIBRARY_PATH", str(tmp_path / "libtmb_hip.so"))
+    with pytest.raises(ek.HipLibraryMissing, match="no CPU or PyTorch fallback"):
+        ek.lib()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "torch-max-backend_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".sh")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
+                assert "libtmb_oracle" not in text, f

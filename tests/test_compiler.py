@@ -1,0 +1,198 @@
+"""Host logic of the graph surface, runnable without a GPU: registry semantics, error text,
+decomposition skipping, the step program (fusion, liveness, output blueprint).
+
+Where a graph has to *execute* on this GPU-less host the hot entries of the registry are
+monkeypatched with PyTorch CPU functions — the reference's own "fake backend" pattern
+(tests/test_tensor_spec_oom.py:14-143) — so the executor is exercised, not the kernels."""
+
+import operator
+
+import pytest
+import torch
+
+import torch_mojo_backend
+from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO, MojoCompilerError, mojo_backend
+from torch_mojo_backend import aten_functions as af
+from torch_mojo_backend.torch_compile_backend import compiler
+
+aten = torch.ops.aten
+
+
+def test_public_names():
+    for name in ("mojo_backend", "MAPPING_TORCH_ATEN_TO_MOJO", "MojoCompilerError",
+                 "get_accelerators", "log_aten_calls"):
+        assert hasattr(torch_mojo_backend, name)
+    assert torch_mojo_backend.get_accelerators()[-1] == torch.device("cpu")
+
+
+def test_registry_has_the_hot_entries_and_identity_functions():
+    for op in (aten.mm, aten.addmm, aten.bmm, aten.linear, aten._softmax, aten.softmax,
+               aten._log_softmax, aten.native_layer_norm, aten.sum, aten.mean, aten.amax,
+               aten.argmax, aten.gelu):
+        assert op in MAPPING_TORCH_ATEN_TO_MOJO
+        assert hasattr(MAPPING_TORCH_ATEN_TO_MOJO[op], "call_count")
+    for fn in (operator.add, operator.getitem, max, min, str):
+        assert MAPPING_TORCH_ATEN_TO_MOJO[fn] is fn
+    assert MAPPING_TORCH_ATEN_TO_MOJO is compiler.MAPPING_TORCH_ATEN_TO_MOJO is af.MAPPING_TORCH_ATEN_TO_MOJO
+
+
+def test_map_to_removes_decompositions_and_rejects_other_keys():
+    assert len(af.DECOMPOSITION_TABLE) < af.original_decomposition_table_size
+    for overload in (aten.addmm.default, aten.native_layer_norm.default, aten._softmax.default,
+                     aten._log_softmax.default, aten.gelu.default, aten.mean.dim):
+        assert overload not in af.DECOMPOSITION_TABLE
+    with pytest.raises(TypeError, match="OpOverload"):
+        af.map_to("aten.tanh")(lambda x: x)
+    # decorator registers, counts and pops a single overload
+    table_had = aten.hardswish.default in af.DECOMPOSITION_TABLE
+    saved = af.DECOMPOSITION_TABLE.get(aten.hardswish.default)
+    try:
+        @af.map_to(aten.hardswish.default)
+        def my_hardswish(x):
+            return torch.nn.functional.hardswish(x)
+
+        assert MAPPING_TORCH_ATEN_TO_MOJO[aten.hardswish.default] is my_hardswish
+        assert aten.hardswish.default not in af.DECOMPOSITION_TABLE
+        my_hardswish(torch.zeros(2))
+        assert my_hardswish.call_count == 1
+    finally:
+        MAPPING_TORCH_ATEN_TO_MOJO.pop(aten.hardswish.default, None)
+        if table_had:
+            af.DECOMPOSITION_TABLE[aten.hardswish.default] = saved
+
+
+def test_unmapped_op_raises_with_the_reference_text(monkeypatch):
+    monkeypatch.delitem(MAPPING_TORCH_ATEN_TO_MOJO, aten.cos)
+
+    def fn(x):
+        return torch.cos(x) + 1
+
+    with pytest.raises(Exception) as info:
+        torch.compile(fn, backend=mojo_backend)(torch.randn(3))
+    text = str(info.value)
+    assert "The aten function is not supported by the Mojo backend yet" in text
+    assert "torch._ops.aten.aten::cos" in text or "cos" in text
+    assert "Failing at node" in text
+    assert "https://github.com/gabrieldemarmiesse/torch-mojo-backend/issues" in text
+    assert "MAPPING_TORCH_ATEN_TO_MOJO" in text
+    assert "return torch.cos(x) + 1" in text   # the user stack trace
+
+
+def test_exception_in_mapping_function_is_wrapped(monkeypatch):
+    def broken(x):
+        raise ValueError("boom from mapping")
+
+    monkeypatch.setitem(MAPPING_TORCH_ATEN_TO_MOJO, aten.cos, broken)
+    with pytest.raises(Exception) as info:
+        torch.compile(lambda x: torch.cos(x), backend=mojo_backend)(torch.randn(3))
+    text = str(info.value)
+    assert "boom from mapping" in text and "There was an error when executing the function" in text
+    cause = info.value
+    while cause is not None and not isinstance(cause, MojoCompilerError):
+        cause = cause.__cause__ or cause.__context__
+    assert isinstance(cause, MojoCompilerError)
+
+
+def test_user_can_override_an_entry(monkeypatch):
+    calls = []
+
+    def my_tanh(x):
+        calls.append(1)
+        return torch.tanh(x) * 0 + 7
+
+    monkeypatch.setitem(MAPPING_TORCH_ATEN_TO_MOJO, aten.tanh, my_tanh)
+    out = torch.compile(lambda x: torch.tanh(x), backend=mojo_backend)(torch.randn(4))
+    assert calls and torch.equal(out, torch.full((4,), 7.0))
+
+
+@pytest.fixture()
+def cpu_hot_ops(monkeypatch):
+    """Stand-ins so graphs can execute on this host; they record what the executor asked for."""
+    log = []
+
+    def rec(name, fn):
+        def run(*a, **k):
+            log.append(name)
+            return fn(*a, **k)
+        run.__name__ = name
+        return run
+
+    fake = {
+        aten.addmm: rec("addmm", lambda i, a, b, **k: torch.addmm(i, a, b, **k)),
+        aten.mm: rec("mm", torch.mm),
+        aten.bmm: rec("bmm", torch.bmm),
+        aten._softmax: rec("_softmax", lambda x, d, h: torch.softmax(x, d)),
+        aten.gelu: rec("gelu", lambda x, approximate="none": torch.nn.functional.gelu(x, approximate=approximate)),
+        aten.argmax: rec("argmax", torch.argmax),
+    }
+
+    def ln(x, shape, w, b, eps):
+        log.append("ln_first_only" if af._only_first_output_used() else "ln_all")
+        return torch.native_layer_norm(x, shape, w, b, eps)
+
+    fake[aten.native_layer_norm] = ln
+    for k, v in fake.items():
+        monkeypatch.setitem(MAPPING_TORCH_ATEN_TO_MOJO, k, v)
+    # the fusion pass keys on the built-in entries; point it at the stand-ins
+    monkeypatch.setattr(compiler, "_BUILTIN_ADDMM", fake[aten.addmm])
+    monkeypatch.setattr(compiler, "_BUILTIN_GELU", fake[aten.gelu])
+    monkeypatch.setattr(af, "addmm_gelu",
+                        rec("addmm_gelu", lambda i, a, b, approx: torch.nn.functional.gelu(
+                            torch.addmm(i, a, b), approximate=approx)))
+    return log
+
+
+def test_executor_runs_a_model_and_fuses_bias_gelu(cpu_hot_ops):
+    torch.manual_seed(0)
+    mlp = torch.nn.Sequential(torch.nn.LayerNorm(16), torch.nn.Linear(16, 32),
+                              torch.nn.GELU(approximate="tanh"), torch.nn.Linear(32, 8)).eval()
+    x = torch.randn(2, 5, 16)
+    with torch.no_grad():
+        want = mlp(x)
+        got = torch.compile(mlp, backend=mojo_backend, fullgraph=True)(x)
+    torch.testing.assert_close(got, want)
+    assert "addmm_gelu" in cpu_hot_ops and "gelu" not in cpu_hot_ops
+    assert cpu_hot_ops.count("addmm") == 1          # the second Linear
+    assert "ln_first_only" in cpu_hot_ops           # inference graph: statistics are dead
+
+
+def test_fusion_can_be_switched_off(cpu_hot_ops, monkeypatch):
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_FUSION", "1")
+    lin = torch.nn.Sequential(torch.nn.Linear(8, 8), torch.nn.GELU()).eval()
+    x = torch.randn(3, 8)
+    with torch.no_grad():
+        torch.testing.assert_close(torch.compile(lin, backend=mojo_backend)(x), lin(x))
+    assert "gelu" in cpu_hot_ops and "addmm_gelu" not in cpu_hot_ops
+
+
+def test_layer_norm_statistics_kept_when_used(cpu_hot_ops):
+    def fn(x, w, b):
+        out, mean, rstd = torch.native_layer_norm(x, [8], w, b, 1e-5)
+        return out, mean, rstd
+
+    x, w, b = torch.randn(4, 8), torch.randn(8), torch.randn(8)
+    got = torch.compile(fn, backend=mojo_backend)(x, w, b)
+    want = fn(x, w, b)
+    for g, t in zip(got, want):
+        torch.testing.assert_close(g, t)
+    assert "ln_all" in cpu_hot_ops
+
+
+def test_outputs_none_ints_and_dynamic_shapes(cpu_hot_ops):
+    def fn(x):
+        return x.shape[0] * 2, None, x + 1
+
+    compiled = torch.compile(fn, backend=mojo_backend, dynamic=True)
+    for n in (3, 5, 9):
+        size, nothing, y = compiled(torch.zeros(n, 2))
+        assert size == 2 * n and nothing is None and y.shape == (n, 2) and bool((y == 1).all())
+
+
+def test_intermediates_are_released_after_their_last_use():
+    gm = torch.fx.symbolic_trace(lambda x: torch.ops.aten.add.Tensor(
+        torch.ops.aten.mul.Tensor(x, 2), torch.ops.aten.mul.Tensor(x, 3)))
+    program = compiler._GraphFactory().create_graph(gm.graph)
+    released = [slot for step in program.steps for slot in step.release]
+    # both products and the input are dropped once the add has run; the result is kept
+    assert sorted(released) == [0, 1, 2]
+    assert program.steps[-1].out not in released

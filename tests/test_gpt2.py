@@ -1,0 +1,84 @@
+"""End-to-end: the GPT-2-small-shaped forward through torch.compile(backend=mojo_backend) on the
+HIP kernels, against PyTorch CPU eager float32 of the same seeded module (the reference's
+check_functions_are_equivalent, torch_mojo_backend/testing.py:139-166)."""
+
+import pytest
+import torch
+
+from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+def _hot_counts():
+    from torch_mojo_backend import aten_functions as af
+    return {f.__name__: f.call_count for f in (af.aten_addmm, af.aten_mm, af.aten_bmm,
+                                               af.aten__softmax, af.aten_native_layer_norm,
+                                               af.aten_argmax, af.aten_gelu)}
+
+
+def test_gpt2_small_fp32_batch1_seq128_matches_cpu_eager():
+    """Workload: 12 layers, d 768, 12 heads, B=1, T=128, float32, seed 0."""
+    from torch_mojo_backend import mojo_backend
+
+    model = build_gpt2_small(seed=0)
+    idx = seeded_tokens(1, 128, seed=0)
+    with torch.no_grad():
+        want_logits, want_next = model(idx)
+    gpu_model = build_gpt2_small(seed=0).to("cuda")
+    compiled = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)
+    before = _hot_counts()
+    with torch.no_grad():
+        logits, nxt = compiled(idx.to("cuda"))
+    after = _hot_counts()
+    assert logits.shape == (1, 128, 50257) and logits.dtype == torch.float32
+    # every hot op of the graph went through the HIP mapping functions
+    # (c_fc's addmm and its gelu are one fused kernel: 12 of the 48 addmm run through it)
+    assert after["aten_addmm"] - before["aten_addmm"] == 36
+    assert after["aten_bmm"] - before["aten_bmm"] == 24
+    assert after["aten__softmax"] - before["aten__softmax"] == 12
+    assert after["aten_native_layer_norm"] - before["aten_native_layer_norm"] == 25
+    assert after["aten_mm"] - before["aten_mm"] == 1
+    assert after["aten_argmax"] - before["aten_argmax"] == 1
+    # float32 end to end: 25 layer norms and 97 GEMMs deep, so a few 1e-5 relative
+    torch.testing.assert_close(logits.cpu(), want_logits, rtol=1e-4, atol=1e-4)
+    # argmax is exact on the backend's own logits ...
+    assert torch.equal(nxt.cpu(), torch.argmax(logits[:, -1, :], dim=-1).cpu())
+    # ... and agrees with the oracle wherever the oracle's top-2 margin exceeds the tolerance
+    top2 = want_logits[:, -1, :].topk(2, dim=-1).values
+    if (top2[:, 0] - top2[:, 1]).min() > 2e-4:
+        assert torch.equal(nxt.cpu(), want_next)
+
+
+def test_gpt2_small_bf16_logits_within_2e_2_of_fp32_oracle():
+    """bf16 weights/activations on the GPU vs float32 CPU eager on the same bf16-rounded weights."""
+    from torch_mojo_backend import mojo_backend
+
+    model = build_gpt2_small(seed=0)
+    model = model.to(torch.bfloat16).to(torch.float32)   # weights rounded to bf16, math in fp32
+    idx = seeded_tokens(2, 256, seed=1)
+    with torch.no_grad():
+        want_logits, _ = model(idx)
+    gpu_model = build_gpt2_small(seed=0).to(torch.bfloat16).to("cuda")
+    compiled = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)
+    with torch.no_grad():
+        logits, nxt = compiled(idx.to("cuda"))
+    assert logits.dtype == torch.bfloat16
+    err = (logits.float().cpu() - want_logits).abs().max().item()
+    assert err <= 2e-2, f"max-abs logit error {err}"
+    assert torch.equal(nxt.cpu(), torch.argmax(logits[:, -1, :], dim=-1).cpu())
+
+
+def test_fusion_is_bit_identical_to_unfused(monkeypatch):
+    """The addmm->gelu rewrite must not change a single bit of the logits."""
+    from torch_mojo_backend import mojo_backend
+
+    gpu_model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).to("cuda")
+    idx = seeded_tokens(2, 64, seed=2).to("cuda")
+    with torch.no_grad():
+        fused, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    torch.compiler.reset()
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_FUSION", "1")
+    with torch.no_grad():
+        unfused, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    assert torch.equal(fused, unfused)

@@ -33,11 +33,17 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
 __device__ __forceinline__ float gelu_erf_f32(float x) {
   return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
-template <int EPI>
-__device__ __forceinline__ float apply_epilogue(float v) {
-  if constexpr (EPI == TMB_EPI_GELU_TANH) return gelu_tanh_f32(v);
-  if constexpr (EPI == TMB_EPI_GELU_ERF) return gelu_erf_f32(v);
-  return v;
+// Bias has already been added in fp32. With a GELU epilogue the sum is first rounded to the
+// storage type, so that the fused kernel returns exactly what addmm followed by a separate
+// gelu returns; then one final cast.
+template <typename T, int EPI>
+__device__ __forceinline__ T finish(float v) {
+  if constexpr (EPI == TMB_EPI_NONE) {
+    return from_f32<T>(v);
+  } else {
+    const float r = to_f32(from_f32<T>(v));
+    return from_f32<T>(EPI == TMB_EPI_GELU_TANH ? gelu_tanh_f32(r) : gelu_erf_f32(r));
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -104,7 +110,7 @@ __global__ __launch_bounds__(256) void gemm_simt_kernel(
       if (gn >= n) continue;
       float v = acc[i][j];
       if (bias != nullptr) v += to_f32(bias[gn]);
-      c[gm * ldc + gn] = from_f32<T>(apply_epilogue<EPI>(v));
+      c[gm * ldc + gn] = finish<T, EPI>(v);
     }
   }
 }
@@ -367,8 +373,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g) {
       for (int e = 0; e < 16; ++e) {
         const int64_t row = row_base + 8 * (e >> 2) + (e & 3);
         if (col_ok && row < M) {
-          const float v = apply_epilogue<EPI>(acc[i][j][e] + bv);
-          C[row * g.ldc + col] = from_f32<T>(v);
+          C[row * g.ldc + col] = finish<T, EPI>(acc[i][j][e] + bv);
         }
       }
     }
@@ -461,7 +466,7 @@ __global__ void gemm_k0_kernel(T* c, const T* bias, int64_t m, int64_t n, int64_
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const int64_t r = i / n, col = i - r * n;
     const float v = bias != nullptr ? to_f32(bias[col]) : 0.0f;
-    cb[r * ldc + col] = from_f32<T>(apply_epilogue<EPI>(v));
+    cb[r * ldc + col] = finish<T, EPI>(v);
   }
 }
 
