@@ -1,0 +1,351 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot-op kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|rows|reduce|gpt2|all]
+
+Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
+accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
+W untimed warm-up steps, then exactly K steps between two ``torch.cuda.synchronize()`` calls.
+
+The same line carries
+  * ``roofline``   — the GEMM kernel against the MI355X dense bf16 MFMA peak (2.5 PFLOP/s):
+                     algorithmic FLOPs (2*M*N*K) / average launch duration from HIP events on
+                     the launch stream;
+  * ``cpu_baseline`` — the CPU oracle (a C restatement of the reference's CPU GEMM loop, OpenMP
+                     over rows) timed on this host on a bounded slab of the same product;
+  * ``sweep``      — every other row of the workload definition (remaining GEMM shapes, bmm,
+                     softmax, LayerNorm, sum/mean/amax, argmax, the GPT-2-small bf16 forward at
+                     B=32, T=1024 through ``mojo_backend``), each with absolute throughput, the
+                     fraction of its roofline (HBM 8 TB/s or MFMA 2.5 PFLOP/s) and a CPU figure.
+Memory-bound rows rotate through enough distinct buffers that the 256 MB Infinity Cache cannot
+serve them.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "torch-max-backend_amd"))
+
+PEAK_BF16_DENSE_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
+PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+
+# HBM bytes per launch of the headline GEMM kernel measured with rocprofv3 --pmc
+# (FETCH_SIZE + WRITE_SIZE, scaled by the same counters on tmb_copy_bytes); None until the
+# counter runs summarised under profiles/ exist for the current kernel.
+GEMM_TRAFFIC_BYTES = None
+
+
+def _parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--only", default="all", choices=["all", "gemm", "rows", "reduce", "gpt2"])
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    return p.parse_args()
+
+
+def main() -> int:
+    args = _parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every row of the "
+              "workload is a single-device kernel); run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 2
+    from torch_mojo_backend import eager_kernels as ek
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    ek.lib()  # fail loudly right here if the HIP library is missing
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(0)
+    host_cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    omp = int(os.environ.get("OMP_NUM_THREADS", host_cores))
+    cpu_threads = max(1, min(host_cores, omp))
+    torch.set_num_threads(cpu_threads)
+
+    def sync():
+        torch.cuda.synchronize()
+
+    def timed(fn, steps, warmup):
+        """(wall ms per step between two syncs, HIP-event ms per launch) over exactly `steps`."""
+        for _ in range(warmup):
+            fn()
+        sync()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        start.record()
+        for _ in range(steps):
+            fn()
+        end.record()
+        sync()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return wall, start.elapsed_time(end) / steps
+
+    def cpu_time(fn, iters=3, warmup=1):
+        for _ in range(warmup):
+            fn()
+        ts = []
+        for _ in range(iters):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2]
+
+    def gen(shape, seed, dtype, scale=1.0, shift=0.0):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        x = torch.randn(shape, generator=g, device=dev, dtype=torch.float32)
+        if scale != 1.0 or shift != 0.0:
+            x = x * scale + shift
+        return x.to(dtype)
+
+    sweep = {}
+    want = args.only
+
+    # ------------------------------------------------------------------ GEMM (headline)
+    M = N = K = 8192
+    a = gen((M, K), 0, torch.bfloat16)
+    b = gen((K, N), 1, torch.bfloat16)
+    bias = gen((N,), 2, torch.bfloat16)
+    flops = 2.0 * M * N * K
+    wall_ms, ev_ms = timed(lambda: hip_ops.gemm(a, b, bias), args.steps, args.warmup)
+    value = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_DENSE_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
+                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_mfma_kernel<bf16,256,256,N-major B>",
+                "launch_ms": round(ev_ms, 4), "algorithmic_flops": flops}
+
+    cpu_baseline = None
+    if not args.no_cpu:
+        import oracle  # the checker, timed here as the reported CPU baseline only
+
+        # bounded sample: the [0:1024, 0:1024] slab of the same product (1/64 of the FLOPs)
+        sm = sn = 1024
+        a_h, b_h, bias_h = a[:sm].cpu(), b[:, :sn].contiguous().cpu(), bias[:sn].cpu()
+        t = cpu_time(lambda: oracle.gemm(a_h, b_h, bias_h), iters=1, warmup=0)
+        cpu_baseline = {"value": round(2.0 * sm * sn * K / t / 1e12, 5), "unit": "TFLOP/s",
+                        "cores": cpu_threads, "kind": "port",
+                        "sample": f"C[0:{sm},0:{sn}] slab of the same 8192^3 bf16 addmm (1/64 of "
+                                  f"the work), oracle/tmb_oracle.c orc_gemm, OpenMP over rows, "
+                                  f"{t:.2f} s"}
+        # context: a tuned CPU BLAS on the same slab (PyTorch CPU, fp32 math on bf16-rounded data)
+        a32, b32, bias32 = a_h.float(), b_h.float(), bias_h.float()
+        t_blas = cpu_time(lambda: torch.addmm(bias32, a32, b32), iters=3, warmup=1)
+        cpu_baseline["torch_cpu_fp32_tflops_same_slab"] = round(2.0 * sm * sn * K / t_blas / 1e12, 4)
+        # check the GPU result on that slab against the oracle while we are here
+        got = hip_ops.gemm(a, b, bias)[:sm, :sn].float().cpu()
+        ref = oracle.gemm(a_h, b_h, bias_h).float()
+        rel = ((got - ref).norm() / ref.norm()).item()
+        cpu_baseline["gpu_vs_oracle_rel_frobenius"] = rel
+        if not rel < 1e-2:
+            print(f"bench: GEMM result deviates from the oracle (rel Frobenius {rel})", file=sys.stderr)
+            return 1
+    del a, b, bias
+
+    def gemm_row(name, m, n, k, batch=None, trans_b=False, steps=50):
+        if batch:
+            x = gen((batch, m, k), 3, torch.bfloat16)
+            w = gen((batch, k, n), 4, torch.bfloat16)
+            bs = None
+        else:
+            x = gen((m, k), 3, torch.bfloat16)
+            w = gen((n, k), 4, torch.bfloat16).t() if trans_b else gen((k, n), 4, torch.bfloat16)
+            bs = gen((n,), 5, torch.bfloat16)
+        _, ms = timed(lambda: hip_ops.gemm(x, w, bs), steps, 10)
+        bt = batch or 1
+        fl = 2.0 * bt * m * n * k
+        by = 2.0 * bt * (m * k + k * n + m * n) + (0 if batch else 2 * n)
+        tf, gbs = fl / ms / 1e9, by / ms / 1e6
+        sweep[name] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 2),
+                       "frac_mfma": round(tf / PEAK_BF16_DENSE_TFLOPS, 4),
+                       "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+
+    if want in ("all", "gemm"):
+        sweep["addmm_bf16_8192x8192x8192"] = {"us": round(ev_ms * 1e3, 2), "TFLOP/s": round(achieved, 2),
+                                              "frac_mfma": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4)}
+        gemm_row("addmm_bf16_8192x8192x8192_Bt", 8192, 8192, 8192, trans_b=True, steps=args.steps)
+        for (m, n, k) in ((128, 768, 768), (1024, 3072, 768), (1024, 768, 3072), (4096, 4096, 4096)):
+            gemm_row(f"addmm_bf16_{m}x{n}x{k}", m, n, k)
+        gemm_row("bmm_bf16_48x1024x64x1024", 1024, 1024, 64, batch=48)
+
+    # ------------------------------------------------------------------ memory-bound rows
+    def rotating(make, bytes_per_buffer):
+        n = max(2, math.ceil(768e6 / max(bytes_per_buffer, 1)) + 1)
+        n = min(n, 16)
+        return [make(i) for i in range(n)]
+
+    def hbm_row(name, bufs, fn, bytes_algo, steps=40, cpu_fn=None):
+        state = {"i": 0}
+
+        def step():
+            fn(bufs[state["i"] % len(bufs)])
+            state["i"] += 1
+
+        _, ms = timed(step, steps, 8)
+        gbs = bytes_algo / ms / 1e6
+        row = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+               "bytes": bytes_algo, "buffers": len(bufs)}
+        if cpu_fn is not None and not args.no_cpu:
+            t = cpu_fn()
+            row["cpu_GB/s"] = round(t[1] / t[0] / 1e9, 3)
+            row["cpu_note"] = t[2]
+        sweep[name] = row
+
+    if want in ("all", "rows"):
+        import oracle
+
+        for dtype, dn in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+            es = torch.finfo(dtype).bits // 8
+            for (B, H, S) in ((8, 12, 1024), (4, 32, 4096)):
+                rows, cols = B * H * S, S
+                nbytes = rows * cols * es
+                if nbytes > 3e9:
+                    bufs = [gen((rows, cols), 10, dtype, scale=4.0)]  # 8.6 GB: no cache can hold it
+                else:
+                    bufs = rotating(lambda i: gen((rows, cols), 10 + i, dtype, scale=4.0), nbytes)
+
+                def cpu_softmax(rows=rows, cols=cols, dtype=dtype, es=es):
+                    sub = min(rows, 8192)
+                    xh = (torch.randn(sub, cols) * 4).to(dtype)
+                    t = cpu_time(lambda: oracle.softmax_rows(xh), iters=3, warmup=1)
+                    return t, 2 * sub * cols * es, f"first {sub} rows, C oracle, {cpu_threads} threads"
+
+                hbm_row(f"softmax_{dn}_{rows}x{cols}", bufs, lambda x: hip_ops.softmax(x, -1),
+                        2 * nbytes, steps=20 if nbytes > 3e9 else 40, cpu_fn=cpu_softmax)
+                del bufs
+            for (rows, cols) in ((32768, 768), (16384, 4096)):
+                nbytes = rows * cols * es
+                g_ = gen((cols,), 1, dtype, scale=0.1, shift=1.0)
+                b_ = gen((cols,), 2, dtype, scale=0.1)
+                bufs = rotating(lambda i: gen((rows, cols), 20 + i, dtype), nbytes)
+
+                def cpu_ln(rows=rows, cols=cols, dtype=dtype, es=es):
+                    sub = min(rows, 8192)
+                    xh = torch.randn(sub, cols).to(dtype)
+                    gh, bh = torch.ones(cols).to(dtype), torch.zeros(cols).to(dtype)
+                    t = cpu_time(lambda: oracle.layer_norm_rows(xh, gh, bh, 1e-5), iters=3, warmup=1)
+                    return t, 2 * sub * cols * es, f"first {sub} rows, C oracle, {cpu_threads} threads"
+
+                hbm_row(f"layer_norm_{dn}_{rows}x{cols}", bufs,
+                        lambda x: hip_ops.layer_norm(x, [cols], g_, b_, 1e-5),
+                        2 * nbytes + 2 * cols * es + 2 * rows * 4, cpu_fn=cpu_ln)
+                del bufs
+
+    if want in ("all", "reduce"):
+        import oracle
+
+        for dtype, dn in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+            es = torch.finfo(dtype).bits // 8
+            rows, cols = 65536, 4096
+            nbytes = rows * cols * es
+            bufs = rotating(lambda i: gen((rows, cols), 30 + i, dtype), nbytes)
+            for opname, op in (("sum", ek.SUM), ("mean", ek.MEAN), ("amax", ek.AMAX)):
+                def cpu_red(op=op, dtype=dtype, es=es, cols=cols):
+                    sub = 4096
+                    xh = torch.randn(sub, cols).to(dtype)
+                    t = cpu_time(lambda: oracle.reduce_rows(xh, op), iters=3, warmup=1)
+                    return t, sub * cols * es, f"first {sub} rows, C oracle, {cpu_threads} threads"
+
+                hbm_row(f"{opname}_{dn}_rows_{rows}x{cols}", bufs,
+                        lambda x, op=op: hip_ops.reduce(x, [1], False, op), nbytes + rows * es,
+                        cpu_fn=cpu_red)
+                hbm_row(f"{opname}_{dn}_all_{rows}x{cols}", bufs,
+                        lambda x, op=op: hip_ops.reduce(x, [0, 1], False, op), nbytes + es)
+            del bufs
+        rows, cols = 512, 50257
+        bufs = rotating(lambda i: gen((rows, cols), 40 + i, torch.float32), rows * cols * 4)
+
+        def cpu_argmax():
+            xh = torch.randn(rows, cols)
+            t = cpu_time(lambda: oracle.argmax_rows(xh), iters=3, warmup=1)
+            return t, rows * cols * 4, f"all {rows} rows, C oracle, {cpu_threads} threads"
+
+        hbm_row(f"argmax_fp32_{rows}x{cols}", bufs, lambda x: hip_ops.argmax(x, 1, False),
+                rows * cols * 4 + rows * 8, steps=100, cpu_fn=cpu_argmax)
+        del bufs
+
+    # ------------------------------------------------------------------ GPT-2 forward
+    if want in ("all", "gpt2"):
+        from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+        from torch_mojo_backend import aten_functions as af
+        from torch_mojo_backend import mojo_backend
+        from torch_mojo_backend.torch_compile_backend import compiler
+
+        B, T = 32, 1024
+        model = build_gpt2_small(seed=0).to(torch.bfloat16).to(dev)
+        idx = seeded_tokens(B, T, seed=0).to(dev)
+        compiled = torch.compile(model, backend=mojo_backend, fullgraph=True)
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            compiled(idx)
+            sync()
+            compile_s = time.perf_counter() - t0
+
+            def fwd():
+                out = compiled(idx)
+                del out
+
+            wall, ev = timed(fwd, 10, 3)
+            compiler.COLLECT_OP_TIMINGS = True
+            compiled(idx)
+            sync()
+            compiler.COLLECT_OP_TIMINGS = False
+        breakdown = compiler.summarize_op_timings()
+        gemm_flops = 12 * (2 * B * T * 7077888) + 12 * (2 * 2 * B * 12 * T * T * 64) + 2 * B * T * 768 * 50257
+        row = {"tokens/s": round(B * T / (wall * 1e-3), 1), "ms_per_forward": round(wall, 3),
+               "gemm_TFLOP/s_over_whole_forward": round(gemm_flops / (wall * 1e-3) / 1e12, 2),
+               "compile_s": round(compile_s, 2), "batch": B, "seq": T, "dtype": "bf16",
+               "per_op_ms": breakdown}
+        if not args.no_cpu:
+            cpu_model = build_gpt2_small(seed=0)
+            cb, ct = 1, 128
+            cidx = seeded_tokens(cb, ct, seed=0)
+            with torch.no_grad():
+                t = cpu_time(lambda: cpu_model(cidx), iters=3, warmup=1)
+            row["cpu_tokens/s"] = round(cb * ct / t, 1)
+            row["cpu_note"] = (f"PyTorch CPU eager fp32 of the same module at B={cb}, T={ct} "
+                               f"(the workload's CPU configuration), {cpu_threads} threads")
+        sweep[f"gpt2_small_fwd_bf16_B{B}_T{T}"] = row
+        del model, compiled
+
+    line = {
+        "metric": "GEMM TFLOP/s (bf16 addmm M=N=K=8192, fp32 accumulate)",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "standalone op sweep: aten.addmm bf16, (M,N,K)=(8192,8192,8192), "
+                               "bias [N], seeded N(0,1) inputs resident in HBM",
+                   "device": props.name, "compute_units": props.multi_processor_count,
+                   "host_threads": cpu_threads},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "sweep": sweep,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

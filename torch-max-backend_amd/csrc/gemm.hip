@@ -23,16 +23,6 @@ namespace tmb {
 // ---------------------------------------------------------------------------
 // Epilogue math
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_tanh_f32(float x) {
-  constexpr float kAlpha = 0.7978845608028654f;  // sqrt(2/pi)
-  const float u = kAlpha * (x + 0.044715f * x * x * x);
-  // tanh(u) = 1 - 2/(exp(2u)+1): saturates cleanly to +-1 for large |u|.
-  const float t = 1.0f - 2.0f / (exp_f32(2.0f * u) + 1.0f);
-  return 0.5f * x * (1.0f + t);
-}
-__device__ __forceinline__ float gelu_erf_f32(float x) {
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
-}
 // Bias has already been added in fp32. With a GELU epilogue the sum is first rounded to the
 // storage type, so that the fused kernel returns exactly what addmm followed by a separate
 // gelu returns; then one final cast.

@@ -3,16 +3,6 @@
 
 namespace tmb {
 
-__device__ __forceinline__ float gelu_tanh_scalar(float x) {
-  constexpr float kAlpha = 0.7978845608028654f;  // sqrt(2/pi)
-  const float u = kAlpha * (x + 0.044715f * x * x * x);
-  const float t = 1.0f - 2.0f / (exp_f32(2.0f * u) + 1.0f);
-  return 0.5f * x * (1.0f + t);
-}
-__device__ __forceinline__ float gelu_erf_scalar(float x) {
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
-}
-
 // Grid-stride over 16-byte vectors; scalar tail. `in`/`out` must be 16-byte aligned for the
 // vector body (the launcher checks and otherwise runs everything through the scalar loop).
 template <typename T, bool TANH>
@@ -27,13 +17,13 @@ __global__ __launch_bounds__(256) void gelu_kernel(T* __restrict__ out, const T*
 #pragma unroll
     for (int e = 0; e < EPV; ++e) {
       const float x = to_f32(v.v[e]);
-      y[e] = TANH ? gelu_tanh_scalar(x) : gelu_erf_scalar(x);
+      y[e] = TANH ? gelu_tanh_f32(x) : gelu_erf_f32(x);
     }
     store_converted<T, EPV>(out + i * EPV, y);
   }
   for (int64_t i = nvec * EPV + tid; i < numel; i += stride) {
     const float x = to_f32(in[i]);
-    out[i] = from_f32<T>(TANH ? gelu_tanh_scalar(x) : gelu_erf_scalar(x));
+    out[i] = from_f32<T>(TANH ? gelu_tanh_f32(x) : gelu_erf_f32(x));
   }
 }
 

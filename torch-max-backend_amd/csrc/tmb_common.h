@@ -65,6 +65,7 @@ __device__ __forceinline__ void store_converted(TOut* p, const float (&x)[N]) {
 // x*log2(e) is formed as hi+lo so the result keeps ~1-2 ulp even for |x|~80.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float exp_f32(float x) {
+#pragma clang fp contract(off)
   constexpr float kLog2eHi = 1.44269502162933349609375f;   // float(log2 e)
   constexpr float kLog2eLo = 1.92596299112661746e-08f;     // log2 e - hi
   constexpr float kLn2 = 0.693147180559945309417f;
@@ -75,6 +76,24 @@ __device__ __forceinline__ float exp_f32(float x) {
   float r = __builtin_fmaf(e, lo * kLn2, e);
   // exp(-inf) must be exactly 0 (0 * nan hazards: lo is nan when x is -inf).
   return (x == -__builtin_inff()) ? 0.0f : r;
+}
+
+// ---------------------------------------------------------------------------
+// GELU, shared by the GEMM epilogue and the standalone kernel. Floating-point contraction is
+// switched off inside so that both users execute the same instruction sequence and a fused
+// GEMM+GELU is bit-identical to the GEMM followed by the elementwise kernel.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+#pragma clang fp contract(off)
+  constexpr float kAlpha = 0.7978845608028654f;  // sqrt(2/pi)
+  const float u = kAlpha * (x + 0.044715f * x * x * x);
+  // tanh(u) = 1 - 2/(exp(2u)+1): saturates cleanly to +-1 for large |u|.
+  const float t = 1.0f - 2.0f / (exp_f32(2.0f * u) + 1.0f);
+  return 0.5f * x * (1.0f + t);
+}
+__device__ __forceinline__ float gelu_erf_f32(float x) {
+#pragma clang fp contract(off)
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
 // ---------------------------------------------------------------------------

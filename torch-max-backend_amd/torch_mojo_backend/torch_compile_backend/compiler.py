@@ -66,6 +66,34 @@ def gather_stats_on_graph(gm: torch.fx.GraphModule) -> None:
         print(f"  {name}: {count}")
 
 
+# Per-op device timing (the reference's per-op breakdown comes from a Kineto trace grouped by
+# aten op, profile_gpt2_generate_aten.py:151-286). When COLLECT_OP_TIMINGS is set the executor
+# brackets every step with HIP events on the current stream; `summarize_op_timings()` waits for
+# the stream and returns {op: {"ms": total, "calls": n}} sorted by time.
+COLLECT_OP_TIMINGS = False
+_OP_EVENTS: list = []
+
+
+def summarize_op_timings() -> dict:
+    torch.cuda.synchronize()
+    totals: dict = {}
+    for name, start, end in _OP_EVENTS:
+        entry = totals.setdefault(name, {"ms": 0.0, "calls": 0})
+        entry["ms"] += start.elapsed_time(end)
+        entry["calls"] += 1
+    _OP_EVENTS.clear()
+    return {k: {"ms": round(v["ms"], 3), "calls": v["calls"]}
+            for k, v in sorted(totals.items(), key=lambda kv: -kv[1]["ms"])}
+
+
+def _step_name(step) -> str:
+    if step.fn is _identity:
+        return "fused-away"
+    if step.fn is _FUSED_ADDMM_GELU:
+        return "aten.addmm+gelu (fused)"
+    return str(step.key)
+
+
 def _fusion_enabled() -> bool:
     return os.environ.get("TORCH_MOJO_BACKEND_NO_FUSION", "0").lower() not in ("1", "true", "yes")
 
@@ -294,12 +322,19 @@ class BaseMaxCompiler:
             a = _materialize(step.args, env) if step.dynamic_args else step.args
             kw = _materialize(step.kwargs, env) if step.dynamic_kwargs else step.kwargs
             token = CURRENT_FX_NODE.set(step.node)
+            if COLLECT_OP_TIMINGS:
+                ev0 = torch.cuda.Event(enable_timing=True)
+                ev0.record()
             try:
                 out = step.fn(*a, **kw)
             except Exception as exc:  # noqa: BLE001 - re-raised with the node's context
                 self._fail(step, a, kw, exc)
             finally:
                 CURRENT_FX_NODE.reset(token)
+            if COLLECT_OP_TIMINGS:
+                ev1 = torch.cuda.Event(enable_timing=True)
+                ev1.record()
+                _OP_EVENTS.append((_step_name(step), ev0, ev1))
             if check:
                 _compare_with_torch(step, a, kw, out)
             env[step.out] = out
