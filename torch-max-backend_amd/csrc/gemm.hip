@@ -28,6 +28,7 @@ namespace tmb {
 // gelu returns; then one final cast.
 template <typename T, int EPI>
 __device__ __forceinline__ T finish(float v) {
+  v = pin_f32(v);  // acc + bias is an fp32 sum; it is rounded to T as a separate step
   if constexpr (EPI == TMB_EPI_NONE) {
     return from_f32<T>(v);
   } else {

@@ -74,8 +74,19 @@ __device__ __forceinline__ float exp_f32(float x) {
   float e = __builtin_amdgcn_exp2f(hi);
   // 2^(hi+lo) = 2^hi * (1 + lo*ln2 + ...), |lo| < 1e-5 so first order is exact to fp32.
   float r = __builtin_fmaf(e, lo * kLn2, e);
-  // exp(-inf) must be exactly 0 (0 * nan hazards: lo is nan when x is -inf).
+  // Overflow: e is +inf and inf*lo + inf would be NaN for negative lo; keep the +inf.
+  r = (e == __builtin_inff()) ? e : r;
+  // exp(-inf) must be exactly 0 (lo is NaN when x is -inf).
   return (x == -__builtin_inff()) ? 0.0f : r;
+}
+
+// Pins a value in a VGPR as an fp32 number. The compiler otherwise folds an fp32 multiply or
+// add into the following fp32->fp16 conversion (v_fma_mixlo_f16: one rounding instead of two),
+// and whether it does so depends on the surrounding code — which would make the same formula
+// round differently in two kernels.
+__device__ __forceinline__ float pin_f32(float v) {
+  asm volatile("" : "+v"(v));
+  return v;
 }
 
 // ---------------------------------------------------------------------------
@@ -89,11 +100,11 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
   const float u = kAlpha * (x + 0.044715f * x * x * x);
   // tanh(u) = 1 - 2/(exp(2u)+1): saturates cleanly to +-1 for large |u|.
   const float t = 1.0f - 2.0f / (exp_f32(2.0f * u) + 1.0f);
-  return 0.5f * x * (1.0f + t);
+  return pin_f32(0.5f * x * (1.0f + t));
 }
 __device__ __forceinline__ float gelu_erf_f32(float x) {
 #pragma clang fp contract(off)
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+  return pin_f32(0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)));
 }
 
 // ---------------------------------------------------------------------------
