@@ -1,0 +1,214 @@
+"""The eager ``mojo`` device surface.
+
+GPU part: tensors move to ``mojo``, the hot aten ops dispatch through PrivateUse1 to
+``fast_aten_*`` and the HIP kernels, results match PyTorch CPU eager (the reference's
+``check_outputs``). Host part (no GPU): the NOT_HANDLED ladder of ``aten_fast`` with stand-in
+tensors, the reference's own fake-backend pattern (tests/test_tensor_spec_oom.py:14-143)."""
+
+import types
+
+import pytest
+import torch
+
+import torch_mojo_backend
+from torch_mojo_backend import register_mojo_devices
+from torch_mojo_backend.eager_kernels import aten_fast
+from torch_mojo_backend.mojo_device import mojo_device_aten_ops as reg
+
+register_mojo_devices()
+
+
+# ---------------------------------------------------------------------------
+# host logic (runs anywhere)
+# ---------------------------------------------------------------------------
+def _fake(shape, dtype=torch.float32, device="cuda:0"):
+    numel = 1
+    for s in shape:
+        numel *= s
+    return types.SimpleNamespace(_shape=tuple(shape), _dtype=dtype, _numel=numel,
+                                 _device=torch.device(device), _holder=None)
+
+
+@pytest.fixture()
+def fake_backend(monkeypatch):
+    """aten_fast sees stand-in tensors; any kernel launch or wrap is recorded, not executed."""
+    launched = []
+    monkeypatch.setattr(aten_fast, "_t", lambda x: x if isinstance(x, types.SimpleNamespace) else None)
+    monkeypatch.setattr(aten_fast, "_wrap", lambda holder: ("wrapped", holder))
+    for name in ("gemm", "softmax", "layer_norm", "reduce", "argmax", "gelu"):
+        monkeypatch.setattr(aten_fast.hip_ops, name,
+                            lambda *a, _n=name, **k: launched.append(_n) or (_n, _n, _n))
+    return launched
+
+
+def test_registration_helpers_collect_the_hot_ops():
+    names = [n for n, _ in reg._aten_ops_registry]
+    for op in ("aten::mm", "aten::addmm", "aten::bmm", "aten::linear", "aten::_softmax",
+               "aten::softmax.int", "aten::_log_softmax", "aten::native_layer_norm",
+               "aten::sum.dim_IntList", "aten::mean", "aten::mean.dim", "aten::amax",
+               "aten::argmax", "aten::gelu"):
+        assert op in names
+        assert hasattr(reg.EAGER_CALL_COUNTERS[op], "call_count")
+    for name in ("fast_aten_mm", "fast_aten_addmm", "fast_aten_linear", "fast_aten_bmm",
+                 "fast_aten__softmax", "fast_aten_softmax", "fast_aten__log_softmax",
+                 "fast_aten_native_layer_norm", "fast_aten_sum", "fast_aten_mean",
+                 "fast_aten_amax", "fast_aten_argmax"):
+        assert hasattr(getattr(aten_fast, name), "call_count")
+    assert torch_mojo_backend.TorchMojoTensor is not None
+
+
+def test_not_handled_becomes_a_named_not_implemented_error():
+    impl = reg._eager_impl("fast_aten_mm", "aten::mm")
+    with pytest.raises(NotImplementedError) as info:
+        impl(torch.randn(2, 3), torch.randn(3, 2))
+    text = str(info.value)
+    assert "aten::mm is not supported by mojo eager mode for these inputs" in text
+    assert "(2, 3):torch.float32:cpu" in text
+
+
+def test_addmm_rules(fake_backend):
+    a, b = _fake((4, 8)), _fake((8, 6))
+    assert aten_fast.fast_aten_addmm(_fake((6,)), a, b) != aten_fast.NOT_HANDLED
+    assert fake_backend == ["gemm"]
+    assert aten_fast.fast_aten_addmm(_fake((6,)), a, b, beta=0.5) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_addmm(_fake((6,)), a, b, alpha=2) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_addmm(_fake((5,)), a, b) is aten_fast.NOT_HANDLED          # bad bias
+    assert aten_fast.fast_aten_addmm(_fake((6,), torch.bfloat16), a, b) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_addmm(_fake((6,)), a, _fake((7, 6))) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_addmm(_fake((6,)), a, _fake((8, 6), device="cuda:1")) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_mm(_fake((4, 8), torch.int64), _fake((8, 6), torch.int64)) is aten_fast.NOT_HANDLED
+    assert fake_backend == ["gemm"]  # nothing was launched for any rejected call
+
+
+def test_softmax_rules(fake_backend):
+    x = _fake((4, 8))
+    assert aten_fast.fast_aten__softmax(x, -1) != aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten__softmax(x, 2) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten__softmax(_fake((0, 8)), -1) is aten_fast.NOT_HANDLED        # numel == 0
+    assert aten_fast.fast_aten__softmax(_fake((4, 8), torch.int64), -1) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten__softmax(x, -1, True) is aten_fast.NOT_HANDLED              # fp32 + half_to_float
+    assert aten_fast.fast_aten__softmax(_fake((4, 8), torch.bfloat16), -1, True) != aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten__log_softmax(_fake((4, 8), torch.bfloat16), -1, True) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten__log_softmax(_fake((4, 8), torch.float16), -1, True) != aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_softmax(x, -1, torch.float32) is aten_fast.NOT_HANDLED      # dtype= unsupported
+
+
+def test_layer_norm_rejects_metadata_before_materializing(fake_backend):
+    x = _fake((2, 3, 8))
+    ok = aten_fast.fast_aten_native_layer_norm(x, [8], _fake((8,)), _fake((8,)), 1e-5)
+    assert ok != aten_fast.NOT_HANDLED and fake_backend == ["layer_norm"]
+    bad = [
+        (x, [7], None, None),                                   # trailing dims do not match
+        (x, [], None, None),                                    # k < 1
+        (x, [8], _fake((7,)), None),                            # weight shape
+        (x, [8], _fake((8,), torch.bfloat16), None),            # weight dtype
+        (x, [8], None, _fake((8,), device="cuda:1")),           # bias device
+        (_fake((0, 8)), [8], None, None),                       # empty
+        (_fake((2, 8), torch.int32), [8], None, None),          # dtype
+    ]
+    for inp, shape, w, b in bad:
+        assert aten_fast.fast_aten_native_layer_norm(inp, shape, w, b, 1e-5) is aten_fast.NOT_HANDLED
+    assert fake_backend == ["layer_norm"]
+
+
+def test_reduce_dim_rules():
+    n = aten_fast._norm_reduce_dims
+    assert n(None, 3, True) == [0, 1, 2]
+    assert n([], 3, True) == [0, 1, 2] and n([], 3, False) == []
+    assert n(-1, 3, True) == [2] and n([2, 0], 3, True) == [0, 2]
+    assert n([0, 0], 3, True) is None and n([3], 3, True) is None and n([True], 3, True) is None
+    assert n("x", 3, True) is None
+    assert aten_fast._reduced_shape((4, 5, 6), [0, 2], True) == (1, 5, 1)
+    assert aten_fast._reduced_shape((4, 5, 6), [0, 2], False) == (5,)
+
+
+def test_reduction_dtype_rules(fake_backend):
+    assert aten_fast.fast_aten_mean(_fake((4, 8), torch.int64)) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_amax(_fake((4, 8), torch.int16), [1]) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_argmax(_fake((0, 8)), 1) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_argmax(_fake((4, 8)), 2) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_sum(_fake((4, 8)), [0, 0]) is aten_fast.NOT_HANDLED
+    assert fake_backend == []
+
+
+# ---------------------------------------------------------------------------
+# on the GPU
+# ---------------------------------------------------------------------------
+gpu = pytest.mark.gpu
+
+
+def _close(got, want, rtol=None, atol=None):
+    assert isinstance(got, torch_mojo_backend.TorchMojoTensor)
+    assert got.device.type == "mojo" and got.dtype == want.dtype and got.shape == want.shape
+    torch.testing.assert_close(got.cpu(), want, rtol=rtol, atol=atol)
+
+
+@gpu
+def test_roundtrip_views_and_payload():
+    x = torch.randn(4, 6)
+    m = x.to("mojo")
+    assert isinstance(m, torch_mojo_backend.TorchMojoTensor) and m.device == torch.device("mojo:0")
+    assert m._shape == (4, 6) and m._strides == (6, 1) and m._is_contiguous and m._itemsize == 4
+    assert m._ptr == m._holder.data_ptr() and m._numel == 24
+    assert torch.equal(m.cpu(), x)
+    t = m.t()
+    assert t._strides == (1, 6) and not t._is_contiguous and t._ptr == m._ptr   # zero-copy view
+    assert torch.equal(t.cpu(), x.t())
+    assert torch.equal(m.view(2, 12).cpu(), x.view(2, 12))
+    assert torch.equal(m[1:3].cpu(), x[1:3])
+    assert torch.equal(m.to(torch.bfloat16).cpu(), x.to(torch.bfloat16))
+
+
+@gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 5e-2)])
+def test_eager_gemm_family(dtype, tol):
+    a, b, bias = torch.randn(33, 64).to(dtype), torch.randn(64, 48).to(dtype), torch.randn(48).to(dtype)
+    am, bm, cm = a.to("mojo"), b.to("mojo"), bias.to("mojo")
+    before = aten_fast.fast_aten_addmm.call_count
+    _close(torch.addmm(cm, am, bm), torch.addmm(bias, a, b), rtol=tol, atol=tol)
+    assert aten_fast.fast_aten_addmm.call_count == before + 1
+    _close(torch.mm(am, bm), torch.mm(a, b), rtol=tol, atol=tol)
+    w = torch.randn(48, 64).to(dtype)
+    x3 = torch.randn(2, 5, 64).to(dtype)
+    _close(torch.nn.functional.linear(x3.to("mojo"), w.to("mojo"), cm),
+           torch.nn.functional.linear(x3, w, bias), rtol=tol, atol=tol)
+    a3, b3 = torch.randn(3, 9, 16).to(dtype), torch.randn(3, 16, 11).to(dtype)
+    _close(torch.bmm(a3.to("mojo"), b3.to("mojo")), torch.bmm(a3, b3), rtol=tol, atol=tol)
+    with pytest.raises(NotImplementedError, match="aten::addmm is not supported by mojo eager"):
+        torch.addmm(cm, am, bm, beta=0.5)
+
+
+@gpu
+def test_eager_softmax_layer_norm_reductions():
+    x = torch.randn(6, 10, 12)
+    m = x.to("mojo")
+    for dim in (0, 1, 2, -1):
+        _close(torch.softmax(m, dim), torch.softmax(x, dim), rtol=1e-5, atol=1e-6)
+        _close(torch.log_softmax(m, dim), torch.log_softmax(x, dim), rtol=1e-5, atol=1e-5)
+    w, b = torch.randn(12), torch.randn(12)
+    got = torch.native_layer_norm(m, [12], w.to("mojo"), b.to("mojo"), 1e-5)
+    want = torch.native_layer_norm(x, [12], w, b, 1e-5)
+    for g, t, tol in zip(got, want, (1e-5, 1e-5, 1e-4)):
+        _close(g, t, rtol=tol, atol=tol)
+    assert got[1].shape == (6, 10, 1) and got[1].dtype == torch.float32
+    _close(torch.nn.functional.layer_norm(m, [12]), torch.nn.functional.layer_norm(x, [12]),
+           rtol=1e-5, atol=1e-5)
+    _close(m.sum(), x.sum(), rtol=1e-5, atol=1e-4)
+    _close(m.sum(dim=1), x.sum(dim=1), rtol=1e-5, atol=1e-5)
+    _close(m.mean(dim=(0, 2), keepdim=True), x.mean(dim=(0, 2), keepdim=True), rtol=1e-5, atol=1e-6)
+    _close(m.mean(), x.mean(), rtol=1e-5, atol=1e-6)
+    _close(torch.amax(m, dim=-1), torch.amax(x, dim=-1), rtol=0, atol=0)
+    _close(torch.argmax(m, dim=1), torch.argmax(x, dim=1), rtol=0, atol=0)
+    _close(torch.argmax(m), torch.argmax(x), rtol=0, atol=0)
+    ints = torch.randint(-5, 5, (7, 9), dtype=torch.int32)
+    _close(ints.to("mojo").sum(dim=1), ints.sum(dim=1), rtol=0, atol=0)
+    _close(torch.nn.functional.gelu(m, approximate="tanh"),
+           torch.nn.functional.gelu(x, approximate="tanh"), rtol=1e-5, atol=1e-6)
+
+
+@gpu
+def test_eager_argmax_vocab_planted_max():
+    x = torch.randn(256, 50257)
+    planted = torch.randint(0, 50257, (256,))
+    x[torch.arange(256), planted] = 100.0
+    assert torch.equal(torch.argmax(x.to("mojo"), dim=-1).cpu(), planted)

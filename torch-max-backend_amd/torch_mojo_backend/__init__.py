@@ -9,6 +9,8 @@ Public names follow torch_mojo_backend/__init__.py:11-33 of the reference.
 """
 
 from torch_mojo_backend.mojo_device.log_aten_calls import log_aten_calls
+from torch_mojo_backend.mojo_device.register import register_mojo_devices
+from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
 from torch_mojo_backend.torch_compile_backend.compiler import (
     MAPPING_TORCH_ATEN_TO_MOJO,
     MojoCompilerError,
@@ -21,5 +23,7 @@ __all__ = [
     "get_accelerators",
     "MAPPING_TORCH_ATEN_TO_MOJO",
     "MojoCompilerError",
+    "register_mojo_devices",
+    "TorchMojoTensor",
     "log_aten_calls",
 ]

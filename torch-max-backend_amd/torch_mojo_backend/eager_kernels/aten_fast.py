@@ -1,0 +1,339 @@
+"""ATen-signature eager implementations of the hot ops over ``TorchMojoTensor``.
+
+Counterpart of the reference's ``torch_mojo_backend/eager_kernels/aten_fast.py`` for the hot
+path. Each ``fast_aten_*`` takes the ATen schema's arguments, validates metadata *before*
+allocating or materialising anything (reference :2741-2742), and returns a tensor (or tuple)
+or the ``NOT_HANDLED`` sentinel (reference :46) — which the dispatcher turns into a
+``NotImplementedError`` naming the op (mojo_device_aten_ops.py:94-119). Supported cases launch
+the gfx950 kernels through ``hip_ops``; there is no other route.
+"""
+
+from __future__ import annotations
+
+import functools
+import math
+
+import torch
+
+import torch_mojo_backend.is_running_tests
+from torch_mojo_backend import eager_kernels as _ek
+from torch_mojo_backend.eager_kernels import hip_ops
+from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
+
+NOT_HANDLED = object()
+
+_FLOAT_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+_ROW_REDUCE_DTYPES = _FLOAT_DTYPES + (torch.int64, torch.int32)
+_CAST_DTYPES = _FLOAT_DTYPES + (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8,
+                                torch.bool)
+
+
+def _t(x):
+    """The mojo tensor behind ``x`` or None."""
+    return x if isinstance(x, TorchMojoTensor) else None
+
+
+def _wrap(holder: torch.Tensor) -> TorchMojoTensor:
+    return TorchMojoTensor._wrap(holder)
+
+
+def fast_filled(shape, value, dtype, device) -> TorchMojoTensor:
+    return _wrap(torch.full(tuple(shape), value, dtype=dtype, device=device))
+
+
+def _same_device(*tensors) -> bool:
+    devs = {t._device for t in tensors if t is not None}
+    return len(devs) <= 1
+
+
+# ---------------------------------------------------------------------------
+# Matmul family (reference :4853-5059)
+# ---------------------------------------------------------------------------
+def _gemm_operands_ok(a, b, rank) -> bool:
+    return (a is not None and b is not None and len(a._shape) == rank and len(b._shape) == rank
+            and a._dtype == b._dtype and a._dtype in _FLOAT_DTYPES and _same_device(a, b)
+            and a._shape[-1] == b._shape[-2])
+
+
+def fast_aten_mm(x, y):
+    a, b = _t(x), _t(y)
+    if not _gemm_operands_ok(a, b, 2):
+        return NOT_HANDLED
+    return _wrap(hip_ops.gemm(a._holder, b._holder))
+
+
+def fast_aten_addmm(input, mat1, mat2, *, beta=1.0, alpha=1.0):
+    # beta/alpha scaling is not implemented by the fast path (reference :4864-4876).
+    if beta != 1 or alpha != 1:
+        return NOT_HANDLED
+    bias, a, b = _t(input), _t(mat1), _t(mat2)
+    if bias is None or not _gemm_operands_ok(a, b, 2) or not _same_device(a, bias):
+        return NOT_HANDLED
+    n = b._shape[1]
+    if bias._dtype != a._dtype:
+        return NOT_HANDLED
+    if tuple(bias._shape) == (n,):
+        return _wrap(hip_ops.gemm(a._holder, b._holder, bias._holder))
+    if tuple(bias._shape) in ((a._shape[0], n), (1, n)):
+        # full-matrix input: matmul, then the broadcast add (two roundings, as ATen does)
+        prod = hip_ops.gemm(a._holder, b._holder)
+        return _wrap(bias._holder + prod)
+    return NOT_HANDLED
+
+
+def fast_aten_linear(input, weight, bias=None):
+    """``input @ weight.T + bias``; the weight is read K-major in place, leading dims of the
+    input are flattened as a zero-copy view (reference :4798-4812, :4879-4936)."""
+    a, w = _t(input), _t(weight)
+    bs = _t(bias) if bias is not None else None
+    if a is None or w is None or (bias is not None and bs is None):
+        return NOT_HANDLED
+    if len(w._shape) != 2 or len(a._shape) < 1 or a._shape[-1] != w._shape[1]:
+        return NOT_HANDLED
+    if a._dtype != w._dtype or a._dtype not in _FLOAT_DTYPES or not _same_device(a, w, bs):
+        return NOT_HANDLED
+    out_features = w._shape[0]
+    if bs is not None and (tuple(bs._shape) != (out_features,) or bs._dtype != a._dtype):
+        return NOT_HANDLED
+    lead = tuple(a._shape[:-1])
+    k = a._shape[-1]
+    rows = math.prod(lead)
+    if out_features == 0 or rows == 0:
+        return _wrap(torch.empty(lead + (out_features,), dtype=a._dtype, device=a._device))
+    if k == 0:  # reference :4923-4928
+        if bs is not None:
+            return _wrap(bs._holder.expand(lead + (out_features,)).clone())
+        return fast_filled(lead + (out_features,), 0.0, a._dtype, a._device)
+    x2 = a._holder.reshape(rows, k)
+    out = hip_ops.gemm(x2, w._holder.t(), None if bs is None else bs._holder)
+    return _wrap(out.view(lead + (out_features,)))
+
+
+def fast_aten_bmm(input, mat2):
+    a, b = _t(input), _t(mat2)
+    if not _gemm_operands_ok(a, b, 3) or a._shape[0] != b._shape[0]:
+        return NOT_HANDLED
+    return _wrap(hip_ops.gemm(a._holder, b._holder))
+
+
+def _fast_aten_bmm_transpose_b(input, mat2):
+    """``input @ mat2.transpose(-2, -1)`` without a transpose copy (reference :5045-5059)."""
+    a, b = _t(input), _t(mat2)
+    if a is None or b is None or len(b._shape) != 3:
+        return NOT_HANDLED
+    return fast_aten_bmm(a, _wrap(b._holder.transpose(-2, -1)))
+
+
+# ---------------------------------------------------------------------------
+# Softmax family (reference :5294-5328, :3201-3234)
+# ---------------------------------------------------------------------------
+def fast_aten__softmax(input, dim, half_to_float=False):
+    t = _t(input)
+    if t is None or t._numel == 0 or t._dtype not in _FLOAT_DTYPES or not isinstance(dim, int) \
+            or isinstance(dim, bool):
+        return NOT_HANDLED
+    if half_to_float and t._dtype not in (torch.float16, torch.bfloat16):
+        return NOT_HANDLED
+    rank = len(t._shape)
+    if rank == 0:
+        return fast_filled((), 1.0, torch.float32 if half_to_float else t._dtype, t._device)
+    if not -rank <= dim < rank:
+        return NOT_HANDLED
+    return _wrap(hip_ops.softmax(t._holder, dim % rank, half_to_float=bool(half_to_float)))
+
+
+def fast_aten_softmax(input, dim=-1, dtype=None):
+    if dtype is not None:
+        return NOT_HANDLED
+    return fast_aten__softmax(input, dim, False)
+
+
+def fast_aten__log_softmax(input, dim, half_to_float=False):
+    t = _t(input)
+    if t is None or t._numel == 0 or t._dtype not in _FLOAT_DTYPES or not isinstance(dim, int) \
+            or isinstance(dim, bool):
+        return NOT_HANDLED
+    if half_to_float and t._dtype != torch.float16:  # fp16 only (reference :3213)
+        return NOT_HANDLED
+    rank = len(t._shape)
+    if rank == 0:
+        if dim not in (-1, 0):
+            return NOT_HANDLED
+        return fast_filled((), 0.0, torch.float32 if half_to_float else t._dtype, t._device)
+    if not -rank <= dim < rank:
+        return NOT_HANDLED
+    return _wrap(hip_ops.softmax(t._holder, dim % rank, half_to_float=bool(half_to_float), log=True))
+
+
+# ---------------------------------------------------------------------------
+# Layer norm (reference :2704-2794)
+# ---------------------------------------------------------------------------
+def fast_aten_native_layer_norm(input, normalized_shape, weight, bias, eps):
+    a = _t(input)
+    normalized_shape = tuple(int(s) for s in normalized_shape)
+    k = len(normalized_shape)
+    if a is None or a._numel == 0 or a._dtype not in _FLOAT_DTYPES or k < 1 \
+            or len(a._shape) < k or tuple(a._shape[-k:]) != normalized_shape:
+        return NOT_HANDLED
+    gamma = beta = None
+    if weight is not None:
+        gamma = _t(weight)
+        if gamma is None or gamma._dtype != a._dtype or gamma._device != a._device \
+                or tuple(gamma._shape) != normalized_shape:
+            return NOT_HANDLED
+    if bias is not None:
+        beta = _t(bias)
+        if beta is None or beta._dtype != a._dtype or beta._device != a._device \
+                or tuple(beta._shape) != normalized_shape:
+            return NOT_HANDLED
+    out, mean, rstd = hip_ops.layer_norm(a._holder, normalized_shape,
+                                         None if gamma is None else gamma._holder,
+                                         None if beta is None else beta._holder, float(eps))
+    return _wrap(out), _wrap(mean), _wrap(rstd)
+
+
+# ---------------------------------------------------------------------------
+# Reductions (reference :2944-3133)
+# ---------------------------------------------------------------------------
+def _norm_reduce_dims(dim, rank, empty_is_all):
+    """Sorted unique normalised reduce dims, or None if invalid (reference :2944-2973)."""
+    if dim is None:
+        return list(range(rank))
+    if isinstance(dim, int) and not isinstance(dim, bool):
+        dims = [dim]
+    elif isinstance(dim, (list, tuple)):
+        dims = list(dim)
+    else:
+        return None
+    if len(dims) == 0:
+        return list(range(rank)) if empty_is_all else []
+    seen, out = set(), []
+    for d in dims:
+        if not isinstance(d, int) or isinstance(d, bool) or not -rank <= d < rank:
+            return None
+        d %= rank
+        if d in seen:
+            return None
+        seen.add(d)
+        out.append(d)
+    return sorted(out)
+
+
+def _reduced_shape(shape, reduce_dims, keepdim):
+    rset = set(reduce_dims)
+    if keepdim:
+        return tuple(1 if i in rset else s for i, s in enumerate(shape))
+    return tuple(s for i, s in enumerate(shape) if i not in rset)
+
+
+def _cast(t: TorchMojoTensor, dtype):
+    if t._dtype == dtype:
+        return t
+    if t._dtype not in _CAST_DTYPES or dtype not in _CAST_DTYPES:
+        return None
+    return _wrap(t._holder.to(dtype))
+
+
+def _reduce(a: TorchMojoTensor, rdims, keepdim, op):
+    if a._numel == 0:
+        return None
+    if len(a._shape) == 0:
+        return _wrap(hip_ops.reduce(a._holder.reshape(1), [0], False, op).reshape(()))
+    return _wrap(hip_ops.reduce(a._holder, rdims, bool(keepdim), op))
+
+
+def fast_aten_sum(input, dim=None, keepdim=False, *, dtype=None):
+    a = _t(input)
+    if a is None:
+        return NOT_HANDLED
+    if dtype is not None:
+        a = _cast(a, dtype)
+        if a is None:
+            return NOT_HANDLED
+    elif not a._dtype.is_floating_point and a._dtype != torch.int64:
+        a = _cast(a, torch.int64)  # torch promotes bool/integer sums to int64
+        if a is None:
+            return NOT_HANDLED
+    if a._dtype not in _FLOAT_DTYPES + (torch.int64,):
+        return NOT_HANDLED
+    rdims = _norm_reduce_dims(dim, len(a._shape), empty_is_all=True)
+    if rdims is None:
+        return NOT_HANDLED
+    if a._numel == 0:  # empty reduction: torch defines it as 0 (reference :3033-3037)
+        return fast_filled(_reduced_shape(a._shape, rdims, keepdim), 0, a._dtype, a._device)
+    out = _reduce(a, rdims, keepdim, _ek.SUM)
+    return out if out is not None else NOT_HANDLED
+
+
+def fast_aten_mean(input, dim=None, keepdim=False, *, dtype=None):
+    a = _t(input)
+    if a is None:
+        return NOT_HANDLED
+    if dtype is not None:
+        if dtype not in _FLOAT_DTYPES:
+            return NOT_HANDLED
+        a = _cast(a, dtype)
+        if a is None:
+            return NOT_HANDLED
+    if a._dtype not in _FLOAT_DTYPES:
+        return NOT_HANDLED
+    rdims = _norm_reduce_dims(dim, len(a._shape), empty_is_all=True)
+    if rdims is None:
+        return NOT_HANDLED
+    out = _reduce(a, rdims, keepdim, _ek.MEAN)
+    return out if out is not None else NOT_HANDLED
+
+
+def fast_aten_amax(input, dim=(), keepdim=False):
+    a = _t(input)
+    if a is None or a._dtype not in _ROW_REDUCE_DTYPES:
+        return NOT_HANDLED
+    rdims = _norm_reduce_dims(dim, len(a._shape), empty_is_all=True)
+    if rdims is None:
+        return NOT_HANDLED
+    out = _reduce(a, rdims, keepdim, _ek.AMAX)
+    return out if out is not None else NOT_HANDLED
+
+
+def fast_aten_argmax(input, dim=None, keepdim=False):
+    a = _t(input)
+    if a is None or a._numel == 0 or a._dtype not in _ROW_REDUCE_DTYPES:
+        return NOT_HANDLED
+    rank = len(a._shape)
+    if dim is None:
+        return _wrap(hip_ops.argmax(a._holder, None, bool(keepdim)))
+    if not (isinstance(dim, int) and not isinstance(dim, bool) and rank > 0 and -rank <= dim < rank):
+        return NOT_HANDLED
+    return _wrap(hip_ops.argmax(a._holder, dim % rank, bool(keepdim)))
+
+
+def fast_aten_gelu(input, approximate="none"):
+    a = _t(input)
+    if a is None or a._dtype not in _FLOAT_DTYPES or approximate not in ("none", "tanh"):
+        return NOT_HANDLED
+    return _wrap(hip_ops.gelu(a._holder, approximate))
+
+
+# ---------------------------------------------------------------------------
+# Call counting under TORCH_MOJO_BACKEND_TESTING=1 (reference :5499-5522)
+# ---------------------------------------------------------------------------
+def _instrument_call_counts():
+    module = globals()
+    for name, fn in list(module.items()):
+        if not (name.startswith("fast_aten") or name.startswith("_fast_aten")) or not callable(fn):
+            continue
+
+        def make(fn):
+            @functools.wraps(fn)
+            def counted(*args, **kwargs):
+                counted.call_count += 1
+                return fn(*args, **kwargs)
+
+            counted.call_count = 0
+            return counted
+
+        module[name] = make(fn)
+
+
+if torch_mojo_backend.is_running_tests.IS_RUNNING_TESTS:
+    _instrument_call_counts()

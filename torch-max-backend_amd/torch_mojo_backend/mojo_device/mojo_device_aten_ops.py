@@ -1,0 +1,207 @@
+"""Eager ``mojo`` device op registrations.
+
+Same mechanism as the reference's ``mojo_device/mojo_device_aten_ops.py``:
+``register_aten_op(name)`` collects ``(op_name, fn)`` pairs (:42-64) that
+``register_mojo_devices()`` hands to ``torch.library.impl(op_name, "privateuseone")``;
+``_register_fast(op_name, fast_name)`` binds an op lazily to ``aten_fast.<fast_name>`` and
+raises ``NotImplementedError`` naming the op when that returns ``NOT_HANDLED`` (:84-135).
+
+Hot ops go to the HIP kernels through ``aten_fast``. The handful of runtime ops a tensor needs
+to exist at all (allocation, host/device copies, zero-copy views) act on the holder directly.
+"""
+
+from __future__ import annotations
+
+import functools
+from collections.abc import Callable
+
+import torch
+
+import torch_mojo_backend.is_running_tests
+from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor, hip_device_of
+
+_aten_ops_registry: list = []
+EAGER_CALL_COUNTERS: dict = {}
+
+
+def register_aten_op(op_name: str):
+    """Decorator marking a function as the ``mojo`` implementation of ``op_name``."""
+
+    def decorator(func: Callable) -> Callable:
+        if torch_mojo_backend.is_running_tests.IS_RUNNING_TESTS:
+
+            @functools.wraps(func)
+            def counted(*args, **kwargs):
+                counted.call_count += 1
+                return func(*args, **kwargs)
+
+            counted.call_count = 0
+            EAGER_CALL_COUNTERS[op_name] = counted
+            _aten_ops_registry.append((op_name, counted))
+            return counted
+        _aten_ops_registry.append((op_name, func))
+        return func
+
+    return decorator
+
+
+_aten_fast_module = None
+
+
+def _fast():
+    global _aten_fast_module
+    if _aten_fast_module is None:
+        from torch_mojo_backend.eager_kernels import aten_fast
+
+        _aten_fast_module = aten_fast
+    return _aten_fast_module
+
+
+def _describe_args(args, kwargs) -> str:
+    descs = []
+    for a in list(args) + list(kwargs.values()):
+        if isinstance(a, TorchMojoTensor):
+            descs.append(f"{tuple(a._shape)}:{a._dtype}")
+        elif isinstance(a, torch.Tensor):
+            descs.append(f"{tuple(a.shape)}:{a.dtype}:{a.device}")
+    return ", ".join(descs) or "none"
+
+
+def _unsupported(op_name: str, args=(), kwargs=None) -> NotImplementedError:
+    return NotImplementedError(
+        f"{op_name} is not supported by mojo eager mode for these inputs "
+        f"(tensor args: {_describe_args(args, kwargs or {})}). There is no fallback; add a fast "
+        "kernel in torch_mojo_backend/eager_kernels/ or open an issue."
+    )
+
+
+def _eager_impl(fast_name: str, op_name: str) -> Callable:
+    """Bind an op to its aten_fast implementation; raise on NOT_HANDLED."""
+    fast_fn = None
+    not_handled = None
+
+    def dispatcher(*args, **kwargs):
+        nonlocal fast_fn, not_handled
+        if fast_fn is None:
+            aten_fast = _fast()
+            fast_fn = getattr(aten_fast, fast_name)
+            not_handled = aten_fast.NOT_HANDLED
+        result = fast_fn(*args, **kwargs)
+        if result is not_handled:
+            raise _unsupported(op_name, args, kwargs)
+        return result
+
+    return dispatcher
+
+
+def _not_implemented(op_name: str) -> Callable:
+    def raiser(*args, **kwargs):
+        raise _unsupported(op_name, args, kwargs)
+
+    return raiser
+
+
+def _register_fast(op_name: str, fast_name: str):
+    register_aten_op(op_name)(_eager_impl(fast_name, op_name))
+
+
+def _register_missing(op_name: str):
+    register_aten_op(op_name)(_not_implemented(op_name))
+
+
+# ---------------------------------------------------------------------------
+# The hot ops (same op names as the reference registers, :860-1021)
+# ---------------------------------------------------------------------------
+_register_fast("aten::_log_softmax", "fast_aten__log_softmax")
+_register_fast("aten::_softmax", "fast_aten__softmax")
+_register_fast("aten::addmm", "fast_aten_addmm")
+_register_fast("aten::amax", "fast_aten_amax")
+_register_fast("aten::argmax", "fast_aten_argmax")
+_register_fast("aten::bmm", "fast_aten_bmm")
+_register_fast("aten::gelu", "fast_aten_gelu")
+_register_fast("aten::linear", "fast_aten_linear")
+_register_fast("aten::mean", "fast_aten_mean")
+_register_fast("aten::mean.dim", "fast_aten_mean")
+_register_fast("aten::mm", "fast_aten_mm")
+_register_fast("aten::native_layer_norm", "fast_aten_native_layer_norm")
+_register_fast("aten::softmax.int", "fast_aten_softmax")
+_register_fast("aten::sum.dim_IntList", "fast_aten_sum")
+
+
+@register_aten_op("aten::sum")
+def _sum_default(self, *, dtype=None):
+    result = _fast().fast_aten_sum(self, None, False, dtype=dtype)
+    if result is _fast().NOT_HANDLED:
+        raise _unsupported("aten::sum", (self,), {})
+    return result
+
+
+# ---------------------------------------------------------------------------
+# Runtime plumbing: allocation, copies, views (act on the holder; no arithmetic)
+# ---------------------------------------------------------------------------
+def _holder(x):
+    return x._holder if isinstance(x, TorchMojoTensor) else x
+
+
+@register_aten_op("aten::empty.memory_format")
+def _empty(size, *, dtype=None, layout=None, device=None, pin_memory=None, memory_format=None):
+    dtype = dtype or torch.get_default_dtype()
+    return TorchMojoTensor._wrap(torch.empty(tuple(size), dtype=dtype, device=hip_device_of(device)))
+
+
+@register_aten_op("aten::empty_strided")
+def _empty_strided(size, stride, *, dtype=None, layout=None, device=None, pin_memory=None):
+    dtype = dtype or torch.get_default_dtype()
+    return TorchMojoTensor._wrap(
+        torch.empty_strided(tuple(size), tuple(stride), dtype=dtype, device=hip_device_of(device)))
+
+
+@register_aten_op("aten::_copy_from")
+def _copy_from(self, dst, non_blocking=False):
+    """copy_(dst, self): host -> mojo, mojo -> host, mojo -> mojo."""
+    src_h, dst_h = _holder(self), _holder(dst)
+    dst_h.copy_(src_h, non_blocking=bool(non_blocking))
+    return dst
+
+
+@register_aten_op("aten::_to_copy")
+def _to_copy(self, *, dtype=None, layout=None, device=None, pin_memory=None, non_blocking=False,
+             memory_format=None):
+    src = _holder(self)
+    target = torch.device(device) if device is not None else self.device
+    dtype = dtype or src.dtype
+    if target.type == "mojo":
+        return TorchMojoTensor._wrap(src.to(device=hip_device_of(target), dtype=dtype, copy=True))
+    return src.to(device=target, dtype=dtype, copy=True)
+
+
+@register_aten_op("aten::_local_scalar_dense")
+def _local_scalar_dense(self):
+    return self._holder.item()
+
+
+def _view_op(op_name: str, fn: Callable):
+    @register_aten_op(op_name)
+    def view(self, *args, **kwargs):
+        return TorchMojoTensor._wrap(fn(self._holder, *args, **kwargs))
+
+    return view
+
+
+_view_op("aten::view", lambda h, size: h.view(size))
+_view_op("aten::_unsafe_view", lambda h, size: h.view(size))
+_view_op("aten::_reshape_alias", lambda h, size, stride: h.as_strided(size, stride))
+_view_op("aten::as_strided", lambda h, size, stride, storage_offset=None:
+         h.as_strided(size, stride, h.storage_offset() if storage_offset is None else storage_offset))
+_view_op("aten::t", lambda h: h.t())
+_view_op("aten::transpose.int", lambda h, d0, d1: h.transpose(d0, d1))
+_view_op("aten::permute", lambda h, dims: h.permute(dims))
+_view_op("aten::expand", lambda h, size, implicit=False: h.expand(size))
+_view_op("aten::unsqueeze", lambda h, dim: h.unsqueeze(dim))
+_view_op("aten::squeeze.dim", lambda h, dim: h.squeeze(dim))
+_view_op("aten::select.int", lambda h, dim, index: h.select(dim, index))
+_view_op("aten::slice.Tensor", lambda h, dim=0, start=None, end=None, step=1:
+         h[(slice(None),) * (dim % max(h.dim(), 1)) + (slice(start, end, step),)])
+_view_op("aten::alias", lambda h: h.alias() if hasattr(h, "alias") else h.view(h.shape))
+_view_op("aten::detach", lambda h: h.detach())
+_view_op("aten::clone", lambda h, memory_format=None: h.clone())

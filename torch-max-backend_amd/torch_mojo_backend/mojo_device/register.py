@@ -1,0 +1,27 @@
+"""``register_mojo_devices()``: enable the eager ``mojo`` device
+(reference: torch_mojo_backend/mojo_device/register.py:141-198)."""
+
+from __future__ import annotations
+
+import torch
+
+_registered = False
+
+
+def register_mojo_devices() -> None:
+    """Rename PrivateUse1 to ``mojo``, install the device module and register every collected
+    aten op with ``torch.library.impl(op_name, "privateuseone")`` (reference :180-181)."""
+    global _registered
+    if _registered:
+        return
+    from torch.utils.backend_registration import _setup_privateuseone_for_python_backend
+
+    from . import torch_mojo_device_module
+    from .mojo_device_aten_ops import _aten_ops_registry
+
+    # Tied parameters (GPT-2's wte / lm_head) must stay one Parameter through .to("mojo").
+    torch.__future__.set_swap_module_params_on_conversion(True)
+    _setup_privateuseone_for_python_backend("mojo", backend_module=torch_mojo_device_module)
+    for op_name, func in _aten_ops_registry:
+        torch.library.impl(op_name, "privateuseone")(func)
+    _registered = True

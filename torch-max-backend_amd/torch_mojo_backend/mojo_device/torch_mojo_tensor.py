@@ -1,0 +1,80 @@
+"""``TorchMojoTensor``: the eager ``mojo`` tensor.
+
+Same shape as the reference's class (torch_mojo_backend/mojo_device/torch_mojo_tensor.py:255-588):
+a storage-less ``PrivateUse1`` wrapper subclass whose payload is a ``_holder`` owning the device
+allocation plus layout metadata as plain attributes (``_ptr``, ``_shape``, ``_strides``,
+``_offset``, ``_dtype``, ``_numel``, ``_itemsize``, ``_device``, ``_is_contiguous``). Views share
+the holder's allocation. Here the holder is a PyTorch-ROCm tensor (its caching allocator is
+stream-ordered, the job the reference's ``TensorHolder`` does, op_utils/__init__.mojo:250-263),
+already viewed with this tensor's shape/strides/offset, so kernels take ``_ptr`` directly.
+"""
+
+from __future__ import annotations
+
+import torch
+
+MAX_RANK = 8  # reference :243
+
+
+class TorchMojoTensor(torch.Tensor):
+    @classmethod
+    def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+        # Let higher-priority wrappers (FakeTensor, FunctionalTensor) handle mixed calls, then
+        # continue into the ordinary PrivateUse1 kernels with the exact overload PyTorch chose.
+        if not all(issubclass(cls, t) for t in types):
+            return NotImplemented
+        with torch._C._DisableTorchDispatch():
+            return func(*args, **(kwargs or {}))
+
+    @classmethod
+    def _wrap(cls, holder: torch.Tensor) -> "TorchMojoTensor":
+        """Adopt a HIP tensor (zero-copy) as a mojo tensor with the same view."""
+        if holder.device.type != "cuda":
+            raise TypeError(f"a mojo tensor is backed by HIP memory, got {holder.device}")
+        if holder.dim() > MAX_RANK:
+            raise NotImplementedError(f"mojo tensors support at most rank {MAX_RANK}, got {holder.dim()}")
+        holder = holder.detach()
+        res = torch.Tensor._make_wrapper_subclass(
+            cls, holder.shape, strides=holder.stride(), storage_offset=holder.storage_offset(),
+            dtype=holder.dtype, layout=torch.strided,
+            device=torch.device("mojo", holder.device.index or 0), requires_grad=False)
+        res._holder = holder
+        res._ptr = holder.data_ptr()
+        res._shape = tuple(holder.shape)
+        res._strides = tuple(holder.stride())
+        res._offset = holder.storage_offset()
+        res._dtype = holder.dtype
+        res._itemsize = holder.element_size()
+        res._numel = holder.numel()
+        res._device = holder.device
+        res._is_contiguous = holder.is_contiguous()
+        return res
+
+    @classmethod
+    def _alloc(cls, shape, dtype: torch.dtype, device) -> "TorchMojoTensor":
+        """A new contiguous uninitialised tensor (one device allocation)."""
+        return cls._wrap(torch.empty(tuple(shape), dtype=dtype, device=hip_device_of(device)))
+
+    def __reduce_ex__(self, protocol):
+        # Pickles as a plain CPU tensor (reference :498-509).
+        return self._holder.cpu().__reduce_ex__(protocol)
+
+    def __repr__(self, *, tensor_contents=None):
+        return f"TorchMojoTensor({self._holder.cpu()!r}, device='{self.device}')"
+
+
+def hip_device_of(device) -> torch.device:
+    """``mojo:i`` (or an int, or a HIP device) -> the HIP device backing it."""
+    if isinstance(device, int):
+        return torch.device("cuda", device)
+    device = torch.device(device)
+    if device.type == "cuda":
+        return device
+    if device.type == "mojo":
+        index = device.index or 0
+        if index >= max(torch.cuda.device_count(), 1):
+            raise RuntimeError(
+                f"{device} does not name a HIP device; the CPU entry of get_accelerators() has "
+                "no kernels in this build")
+        return torch.device("cuda", index)
+    raise TypeError(f"not a mojo device: {device}")
