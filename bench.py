@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot-op kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|rows|reduce|gpt2|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|gpt2|all]
 
 Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
@@ -48,7 +48,7 @@ def _parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--only", default="all", choices=["all", "gemm", "rows", "reduce", "gpt2"])
+    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "gpt2"])
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return p.parse_args()
 
@@ -183,22 +183,30 @@ def main() -> int:
         gemm_row("bmm_bf16_48x1024x64x1024", 1024, 1024, 64, batch=48)
 
     # ------------------------------------------------------------------ memory-bound rows
+    # Launched straight through the C ABI with preallocated outputs, so the timed region holds
+    # kernel launches only (the PyTorch-side allocation of outputs costs more host time than
+    # the smaller kernels run for).
+    lib = ek.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+
     def rotating(make, bytes_per_buffer):
         n = max(2, math.ceil(768e6 / max(bytes_per_buffer, 1)) + 1)
         n = min(n, 16)
         return [make(i) for i in range(n)]
 
-    def hbm_row(name, bufs, fn, bytes_algo, steps=40, cpu_fn=None):
+    def hbm_row(name, nbuf, launch, bytes_algo, steps=40, cpu_fn=None):
         state = {"i": 0}
 
         def step():
-            fn(bufs[state["i"] % len(bufs)])
+            rc = launch(state["i"] % nbuf)
+            if rc != 0:
+                raise RuntimeError(f"{name}: launch failed with {ek.status_string(rc)}")
             state["i"] += 1
 
         _, ms = timed(step, steps, 8)
         gbs = bytes_algo / ms / 1e6
         row = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
-               "bytes": bytes_algo, "buffers": len(bufs)}
+               "bytes": bytes_algo, "buffers": nbuf}
         if cpu_fn is not None and not args.no_cpu:
             t = cpu_fn()
             row["cpu_GB/s"] = round(t[1] / t[0] / 1e9, 3)
@@ -210,6 +218,7 @@ def main() -> int:
 
         for dtype, dn in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             es = torch.finfo(dtype).bits // 8
+            code = hip_ops.code_of(dtype)
             for (B, H, S) in ((8, 12, 1024), (4, 32, 4096)):
                 rows, cols = B * H * S, S
                 nbytes = rows * cols * es
@@ -217,6 +226,8 @@ def main() -> int:
                     bufs = [gen((rows, cols), 10, dtype, scale=4.0)]  # 8.6 GB: no cache can hold it
                 else:
                     bufs = rotating(lambda i: gen((rows, cols), 10 + i, dtype, scale=4.0), nbytes)
+                outs = [torch.empty_like(b_) for b_ in bufs]
+                ptrs = [(o.data_ptr(), b_.data_ptr()) for o, b_ in zip(outs, bufs)]
 
                 def cpu_softmax(rows=rows, cols=cols, dtype=dtype, es=es):
                     sub = min(rows, 8192)
@@ -224,14 +235,21 @@ def main() -> int:
                     t = cpu_time(lambda: oracle.softmax_rows(xh), iters=3, warmup=1)
                     return t, 2 * sub * cols * es, f"first {sub} rows, C oracle, {cpu_threads} threads"
 
-                hbm_row(f"softmax_{dn}_{rows}x{cols}", bufs, lambda x: hip_ops.softmax(x, -1),
+                hbm_row(f"softmax_{dn}_{rows}x{cols}", len(bufs),
+                        lambda i: lib.tmb_softmax_rows(ptrs[i][0], ptrs[i][1], rows, cols, code, code, 0, stream),
                         2 * nbytes, steps=20 if nbytes > 3e9 else 40, cpu_fn=cpu_softmax)
-                del bufs
+                # spot-check the raw launch against the tensor-level op
+                assert torch.equal(outs[0], hip_ops.softmax(bufs[0], -1))
+                del bufs, outs
             for (rows, cols) in ((32768, 768), (16384, 4096)):
                 nbytes = rows * cols * es
                 g_ = gen((cols,), 1, dtype, scale=0.1, shift=1.0)
                 b_ = gen((cols,), 2, dtype, scale=0.1)
                 bufs = rotating(lambda i: gen((rows, cols), 20 + i, dtype), nbytes)
+                outs = [torch.empty_like(x_) for x_ in bufs]
+                mean = torch.empty(rows, dtype=torch.float32, device=dev)
+                rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+                ptrs = [(o.data_ptr(), x_.data_ptr()) for o, x_ in zip(outs, bufs)]
 
                 def cpu_ln(rows=rows, cols=cols, dtype=dtype, es=es):
                     sub = min(rows, 8192)
@@ -240,19 +258,28 @@ def main() -> int:
                     t = cpu_time(lambda: oracle.layer_norm_rows(xh, gh, bh, 1e-5), iters=3, warmup=1)
                     return t, 2 * sub * cols * es, f"first {sub} rows, C oracle, {cpu_threads} threads"
 
-                hbm_row(f"layer_norm_{dn}_{rows}x{cols}", bufs,
-                        lambda x: hip_ops.layer_norm(x, [cols], g_, b_, 1e-5),
+                hbm_row(f"layer_norm_{dn}_{rows}x{cols}", len(bufs),
+                        lambda i: lib.tmb_layer_norm_rows(ptrs[i][0], mean.data_ptr(), rstd.data_ptr(),
+                                                          ptrs[i][1], g_.data_ptr(), b_.data_ptr(),
+                                                          rows, cols, 1e-5, code, stream),
                         2 * nbytes + 2 * cols * es + 2 * rows * 4, cpu_fn=cpu_ln)
-                del bufs
+                assert torch.equal(outs[0], hip_ops.layer_norm(bufs[0], [cols], g_, b_, 1e-5)[0])
+                del bufs, outs
 
     if want in ("all", "reduce"):
         import oracle
 
         for dtype, dn in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             es = torch.finfo(dtype).bits // 8
+            code = hip_ops.code_of(dtype)
             rows, cols = 65536, 4096
             nbytes = rows * cols * es
             bufs = rotating(lambda i: gen((rows, cols), 30 + i, dtype), nbytes)
+            in_ptrs = [x_.data_ptr() for x_ in bufs]
+            out_rows = torch.empty(rows, dtype=dtype, device=dev)
+            out_all = torch.empty(1, dtype=dtype, device=dev)
+            ws_bytes = lib.tmb_reduce_workspace_bytes(1, rows * cols, code)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
             for opname, op in (("sum", ek.SUM), ("mean", ek.MEAN), ("amax", ek.AMAX)):
                 def cpu_red(op=op, dtype=dtype, es=es, cols=cols):
                     sub = 4096
@@ -260,22 +287,33 @@ def main() -> int:
                     t = cpu_time(lambda: oracle.reduce_rows(xh, op), iters=3, warmup=1)
                     return t, sub * cols * es, f"first {sub} rows, C oracle, {cpu_threads} threads"
 
-                hbm_row(f"{opname}_{dn}_rows_{rows}x{cols}", bufs,
-                        lambda x, op=op: hip_ops.reduce(x, [1], False, op), nbytes + rows * es,
-                        cpu_fn=cpu_red)
-                hbm_row(f"{opname}_{dn}_all_{rows}x{cols}", bufs,
-                        lambda x, op=op: hip_ops.reduce(x, [0, 1], False, op), nbytes + es)
+                hbm_row(f"{opname}_{dn}_rows_{rows}x{cols}", len(bufs),
+                        lambda i, op=op: lib.tmb_reduce_rows(out_rows.data_ptr(), in_ptrs[i], rows, cols, op,
+                                                             code, None, 0, stream),
+                        nbytes + rows * es, cpu_fn=cpu_red)
+                hbm_row(f"{opname}_{dn}_all_{rows}x{cols}", len(bufs),
+                        lambda i, op=op: lib.tmb_reduce_rows(out_all.data_ptr(), in_ptrs[i], 1, rows * cols,
+                                                             op, code, ws.data_ptr(), ws_bytes, stream),
+                        nbytes + es)
+            assert torch.equal(out_all.reshape(()), hip_ops.reduce(bufs[(39 + 8) % len(bufs)], [0, 1], False, ek.AMAX))
             del bufs
         rows, cols = 512, 50257
         bufs = rotating(lambda i: gen((rows, cols), 40 + i, torch.float32), rows * cols * 4)
+        in_ptrs = [x_.data_ptr() for x_ in bufs]
+        out_idx = torch.empty(rows, dtype=torch.int64, device=dev)
+        ws_bytes = lib.tmb_reduce_workspace_bytes(rows, cols, ek.F32)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
 
         def cpu_argmax():
             xh = torch.randn(rows, cols)
             t = cpu_time(lambda: oracle.argmax_rows(xh), iters=3, warmup=1)
             return t, rows * cols * 4, f"all {rows} rows, C oracle, {cpu_threads} threads"
 
-        hbm_row(f"argmax_fp32_{rows}x{cols}", bufs, lambda x: hip_ops.argmax(x, 1, False),
+        hbm_row(f"argmax_fp32_{rows}x{cols}", len(bufs),
+                lambda i: lib.tmb_argmax_rows(out_idx.data_ptr(), in_ptrs[i], rows, cols, ek.F32,
+                                              ws.data_ptr(), ws_bytes, stream),
                 rows * cols * 4 + rows * 8, steps=100, cpu_fn=cpu_argmax)
+        assert torch.equal(out_idx, torch.argmax(bufs[(99 + 8) % len(bufs)], dim=1))
         del bufs
 
     # ------------------------------------------------------------------ GPT-2 forward

@@ -16,27 +16,15 @@
 //
 // Arithmetic contract: fp32 accumulate, bias added in fp32 before the single down-cast
 // (torch_mojo_backend/eager_kernels/matmul_ops.mojo:2651-2720).
-#include "tmb_common.h"
+#include <type_traits>
+
+#include "gemm_mfma.h"
 
 namespace tmb {
 
 // ---------------------------------------------------------------------------
 // Epilogue math
 // ---------------------------------------------------------------------------
-// Bias has already been added in fp32. With a GELU epilogue the sum is first rounded to the
-// storage type, so that the fused kernel returns exactly what addmm followed by a separate
-// gelu returns; then one final cast.
-template <typename T, int EPI>
-__device__ __forceinline__ T finish(float v) {
-  v = pin_f32(v);  // acc + bias is an fp32 sum; it is rounded to T as a separate step
-  if constexpr (EPI == TMB_EPI_NONE) {
-    return from_f32<T>(v);
-  } else {
-    const float r = to_f32(from_f32<T>(v));
-    return from_f32<T>(EPI == TMB_EPI_GELU_TANH ? gelu_tanh_f32(r) : gelu_erf_f32(r));
-  }
-}
-
 // ---------------------------------------------------------------------------
 // SIMT fallback: any dtype / stride / alignment. 64x64 tile, BK = 16, 4x4 per thread.
 // ---------------------------------------------------------------------------
@@ -106,297 +94,12 @@ __global__ __launch_bounds__(256) void gemm_simt_kernel(
   }
 }
 
-// ---------------------------------------------------------------------------
-// MFMA path
-// ---------------------------------------------------------------------------
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
-typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
-
-template <typename T>
-struct Mfma;
-template <>
-struct Mfma<bf16_t> {
-  static __device__ __forceinline__ f32x16_t run(u32x4_t a, u32x4_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  }
-};
-template <>
-struct Mfma<f16_t> {
-  static __device__ __forceinline__ f32x16_t run(u32x4_t a, u32x4_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
-                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-  }
-};
-
-constexpr int kBK = 64;          // K extent of one LDS stage (64 x 2 bytes = one 128-byte line)
-constexpr int kLineBytes = 128;
-
-// Byte offset of 16-byte chunk `chunk` (0..7) of line `row` inside a swizzled tile.
-__device__ __forceinline__ int lds_offset(int row, int chunk) {
-  return row * kLineBytes + (((chunk ^ row ^ (row >> 3)) & 7) << 4);
-}
-
-struct GemmArgs {
-  void* c;
-  const void* a;
-  const void* b;
-  const void* bias;
-  int64_t m, n, k;
-  int64_t lda, ldb, ldc;
-  int64_t stride_a, stride_b, stride_c;
-  int tiles_m, tiles_n;
-};
-
-// Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
-// 8 XCDs round-robin) works on a contiguous run of tiles, walked in column-major groups of
-// `kGroupM` tile rows.
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int kXcds = 8;
-  constexpr int kGroupM = 8;
-  const int total = tiles_m * tiles_n;
-  const int q = total / kXcds, r = total % kXcds;
-  const int xcd = pid % kXcds, idx = pid / kXcds;
-  const int tile = xcd * q + (xcd < r ? xcd : r) + idx;
-  const int per_group = kGroupM * tiles_n;
-  const int group = tile / per_group;
-  const int first_m = group * kGroupM;
-  const int gsz = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
-  const int in_group = tile - group * per_group;
-  tm = first_m + in_group % gsz;
-  tn = in_group / gsz;
-}
-
-// B_KMAJOR: B is stored [N, K] (ldb = row pitch of an N-row); otherwise [K, N].
-template <typename T, int BM, int BN, bool B_KMAJOR, int EPI>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmArgs g) {
-  constexpr int WM = BM / 2, WN = BN / 2;   // wave tile
-  constexpr int TM = WM / 32, TN = WN / 32;  // 32x32 MFMA tiles per wave
-  constexpr int A_BYTES = BM * kLineBytes, B_BYTES = BN * kLineBytes;
-  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int A_LOADS = BM / 32;  // 16-byte chunks per thread per stage
-  constexpr int B_LOADS = BN / 32;
-  constexpr int B_BLOCKS = (BN + 255) / 256;  // 8x8 transpose blocks per thread (N-major B)
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-
-  int tile_m, tile_n;
-  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
-  const int64_t m0 = static_cast<int64_t>(tile_m) * BM;
-  const int64_t n0 = static_cast<int64_t>(tile_n) * BN;
-  const int64_t batch = blockIdx.y;
-  const T* __restrict__ A = static_cast<const T*>(g.a) + batch * g.stride_a;
-  const T* __restrict__ B = static_cast<const T*>(g.b) + batch * g.stride_b;
-  T* __restrict__ C = static_cast<T*>(g.c) + batch * g.stride_c;
-  const int64_t M = g.m, N = g.n, K = g.k;
-
-  // ---- global -> register staging -------------------------------------------------------
-  u32x4_t a_stage[A_LOADS];
-  u32x4_t b_stage[B_KMAJOR ? B_LOADS : B_BLOCKS * 8];
-  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-
-  const int ld_row = tid >> 3;   // 0..31
-  const int ld_chunk = tid & 7;  // 16-byte chunk inside the 128-byte line
-
-  auto load_a = [&](int64_t k0) {
-    const int64_t kk = k0 + ld_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) {
-      int64_t row = m0 + ld_row + j * 32;
-      row = row < M ? row : M - 1;
-      a_stage[j] = (kk < K) ? *reinterpret_cast<const u32x4_t*>(A + row * g.lda + kk) : zero4;
-    }
-  };
-  auto load_b = [&](int64_t k0) {
-    if constexpr (B_KMAJOR) {
-      const int64_t kk = k0 + ld_chunk * 8;
-#pragma unroll
-      for (int j = 0; j < B_LOADS; ++j) {
-        int64_t row = n0 + ld_row + j * 32;
-        row = row < N ? row : N - 1;
-        b_stage[j] = (kk < K) ? *reinterpret_cast<const u32x4_t*>(B + row * g.ldb + kk) : zero4;
-      }
-    } else {
-      // Thread owns an 8(k) x 8(n) block: k-chunk kc = blk / (BN/8), n-group ng = blk % (BN/8).
-#pragma unroll
-      for (int q = 0; q < B_BLOCKS; ++q) {
-        const int blk = tid + q * 256;
-        const int kc = blk / (BN / 8), ng = blk % (BN / 8);
-        const int64_t nn = n0 + ng * 8;
-        const bool active = blk < BN;  // BN blocks in total (8 k-chunks x BN/8 n-groups)
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          const int64_t kk = k0 + kc * 8 + r;
-          u32x4_t v = zero4;
-          if (active && kk < K) {
-            const T* src = B + kk * g.ldb + nn;
-            if (nn + 8 <= N) {
-              v = *reinterpret_cast<const u32x4_t*>(src);
-            } else {
-              // ragged right edge: element-wise, never past column N-1
-              unsigned short e[8];
-#pragma unroll
-              for (int t = 0; t < 8; ++t)
-                e[t] = (nn + t < N) ? reinterpret_cast<const unsigned short*>(src)[t]
-                                    : static_cast<unsigned short>(0);
-              v[0] = e[0] | (static_cast<uint32_t>(e[1]) << 16);
-              v[1] = e[2] | (static_cast<uint32_t>(e[3]) << 16);
-              v[2] = e[4] | (static_cast<uint32_t>(e[5]) << 16);
-              v[3] = e[6] | (static_cast<uint32_t>(e[7]) << 16);
-            }
-          }
-          b_stage[q * 8 + r] = v;
-        }
-      }
-    }
-  };
-  auto store_stage = [&](int buf) {
-    unsigned char* sa = smem + buf * STAGE_BYTES;
-    unsigned char* sb = sa + A_BYTES;
-#pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) {
-      const int row = ld_row + j * 32;
-      *reinterpret_cast<u32x4_t*>(sa + lds_offset(row, ld_chunk)) = a_stage[j];
-    }
-    if constexpr (B_KMAJOR) {
-#pragma unroll
-      for (int j = 0; j < B_LOADS; ++j) {
-        const int row = ld_row + j * 32;
-        *reinterpret_cast<u32x4_t*>(sb + lds_offset(row, ld_chunk)) = b_stage[j];
-      }
-    } else {
-#pragma unroll
-      for (int q = 0; q < B_BLOCKS; ++q) {
-        const int blk = tid + q * 256;
-        if (blk < BN) {
-          const int kc = blk / (BN / 8), ng = blk % (BN / 8);
-          // 8x8 transpose of 16-bit elements: out[i] holds k = 0..7 for column i.
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            u32x4_t o;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const uint32_t lo = b_stage[q * 8 + 2 * j][i >> 1];
-              const uint32_t hi = b_stage[q * 8 + 2 * j + 1][i >> 1];
-              o[j] = (i & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-            }
-            const int row = ng * 8 + i;
-            *reinterpret_cast<u32x4_t*>(sb + lds_offset(row, kc)) = o;
-          }
-        }
-      }
-    }
-  };
-
-  // ---- accumulators ---------------------------------------------------------------------
-  f32x16_t acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  const int frag_row = lane & 31;
-  const int frag_half = lane >> 5;  // which 8-wide K half of the 16-wide MFMA step
-
-  auto compute_stage = [&](int buf) {
-    const unsigned char* sa = smem + buf * STAGE_BYTES;
-    const unsigned char* sb = sa + A_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      u32x4_t af[TM], bf[TN];
-      const int chunk = ks * 2 + frag_half;
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = wm * WM + i * 32 + frag_row;
-        af[i] = *reinterpret_cast<const u32x4_t*>(sa + lds_offset(row, chunk));
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int row = wn * WN + j * 32 + frag_row;
-        bf[j] = *reinterpret_cast<const u32x4_t*>(sb + lds_offset(row, chunk));
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(af[i], bf[j], acc[i][j]);
-    }
-  };
-
-  // ---- main loop ------------------------------------------------------------------------
-  const int64_t k_tiles = (K + kBK - 1) / kBK;
-  load_a(0);
-  load_b(0);
-  store_stage(0);
-  __syncthreads();
-  for (int64_t kt = 0; kt < k_tiles; ++kt) {
-    const int buf = static_cast<int>(kt & 1);
-    const bool more = kt + 1 < k_tiles;
-    if (more) {
-      load_a((kt + 1) * kBK);
-      load_b((kt + 1) * kBK);
-    }
-    compute_stage(buf);
-    if (more) store_stage(buf ^ 1);
-    __syncthreads();
-  }
-
-  // ---- epilogue -------------------------------------------------------------------------
-  // MFMA 32x32 result layout: lane holds column (lane & 31); register e holds row
-  // 8*(e/4) + 4*(lane>>5) + (e&3).
-  const T* __restrict__ bias = static_cast<const T*>(g.bias);
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int64_t col = n0 + wn * WN + j * 32 + (lane & 31);
-    const bool col_ok = col < N;
-    const float bv = (bias != nullptr && col_ok) ? to_f32(bias[col]) : 0.0f;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int64_t row_base = m0 + wm * WM + i * 32 + 4 * (lane >> 5);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int64_t row = row_base + 8 * (e >> 2) + (e & 3);
-        if (col_ok && row < M) {
-          C[row * g.ldc + col] = finish<T, EPI>(acc[i][j][e] + bv);
-        }
-      }
-    }
-  }
-}
-
-template <typename T, int BM, int BN, bool B_KMAJOR, int EPI>
-static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) {
-  constexpr int SMEM = 2 * (BM + BN) * kLineBytes;
-  static bool configured = false;
-  auto kernel = gemm_mfma_kernel<T, BM, BN, B_KMAJOR, EPI>;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-    if (e != hipSuccess) return static_cast<int>(e);
-    configured = true;
-  }
-  GemmArgs g = base;
-  g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
-  g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
-  const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
-  if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
-  kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(256), SMEM, stream>>>(g);
-  return check_launch();
-}
-
 template <typename T, bool B_KMAJOR, int EPI>
 static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) {
   // Big tiles when they still fill the 256 CUs, otherwise the 128x128 tile.
   const int64_t big_tiles = ((g.m + 255) / 256) * ((g.n + 255) / 256) * batch;
-  if (big_tiles >= 192) return launch_mfma<T, 256, 256, B_KMAJOR, EPI>(g, batch, stream);
-  return launch_mfma<T, 128, 128, B_KMAJOR, EPI>(g, batch, stream);
+  if (big_tiles >= 192) return launch_mfma<T, 256, 256, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
 }
 
 template <typename T, int EPI>
@@ -420,6 +123,9 @@ static bool mfma_eligible(const GemmArgs& g, int64_t batch, int trans_a, int tra
   if (!aligned16(g.a) || !aligned16(g.b)) return false;
   if (batch > 1 && (g.stride_a % 8 != 0 || g.stride_b % 8 != 0)) return false;
   if (g.m < 1 || g.n < 1 || g.k < 8) return false;
+  // the kernel addresses operands with 32-bit byte offsets from their base
+  const int64_t a_span = g.m * g.lda * 2, b_span = (trans_b ? g.n : g.k) * g.ldb * 2;
+  if (a_span >= (int64_t{1} << 32) || b_span >= (int64_t{1} << 32)) return false;
   (void)trans_b;
   return true;
 }
@@ -482,7 +188,7 @@ extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias,
   }
   if (batch > 65535) return TMB_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0};
+  GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0, 0};
   if (k == 0) {
     const unsigned blocks = static_cast<unsigned>((m * n + 255) / 256 > 4096 ? 4096 : (m * n + 255) / 256);
     dim3 grid(blocks, static_cast<unsigned>(batch));

@@ -1,0 +1,386 @@
+// MFMA GEMM kernel for gfx950 (bf16 / fp16 storage, fp32 accumulation).
+//
+// One workgroup of WAVES_M x WAVES_N waves owns a BM x BN tile of C and walks K in stages of 64.
+// Stage k+1 is fetched from global memory into registers while stage k is multiplied out of LDS;
+// after the multiply the registers are written to the other LDS buffer, one barrier closes the
+// stage, and the first operand fragments of the next stage are fetched from LDS *before* the
+// last quarter of the current stage's MFMAs is issued, so that the LDS latency after the
+// barrier is covered by matrix work. Operand fragments are double-buffered in registers.
+//
+// LDS layout: K-major, one 128-byte line (64 K-values) per matrix row; the eight 16-byte chunks
+// of a line are XOR-swizzled with (row ^ row>>3) so that ds_read_b128 fragment fetches, the
+// workgroup's row-wise stores and the transposed stores of an N-major B are all bank-conflict
+// free.
+//
+// The MFMA is issued with the operands swapped (B fragment first): the 32x32 result then holds,
+// per lane, one row m of C and four consecutive columns n per register quad, which the epilogue
+// turns into 8-byte stores after adding the bias in fp32 (and the optional GELU).
+#pragma once
+
+#include "tmb_common.h"
+
+namespace tmb {
+
+// Bias has already been added in fp32. With a GELU epilogue the sum is first rounded to the
+// storage type, so that the fused kernel returns exactly what addmm followed by a separate
+// gelu returns; then one final cast.
+template <typename T, int EPI>
+__device__ __forceinline__ T finish(float v) {
+  v = pin_f32(v);  // acc + bias is an fp32 sum; it is rounded to T as a separate step
+  if constexpr (EPI == TMB_EPI_NONE) {
+    return from_f32<T>(v);
+  } else {
+    const float r = to_f32(from_f32<T>(v));
+    return from_f32<T>(EPI == TMB_EPI_GELU_TANH ? gelu_tanh_f32(r) : gelu_erf_f32(r));
+  }
+}
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+
+template <typename T>
+struct Mfma;
+template <>
+struct Mfma<bf16_t> {
+  static __device__ __forceinline__ f32x16_t run(u32x4_t a, u32x4_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<f16_t> {
+  static __device__ __forceinline__ f32x16_t run(u32x4_t a, u32x4_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+};
+
+constexpr int kBK = 64;  // K extent of one LDS stage (64 x 2 bytes = one 128-byte line)
+constexpr int kLineBytes = 128;
+
+// Byte offset of 16-byte chunk `chunk` (0..7) of line `row` inside a swizzled tile.
+__device__ __forceinline__ int lds_offset(int row, int chunk) {
+  return row * kLineBytes + (((chunk ^ row ^ (row >> 3)) & 7) << 4);
+}
+
+struct GemmArgs {
+  void* c;
+  const void* a;
+  const void* b;
+  const void* bias;
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc;
+  int64_t stride_a, stride_b, stride_c;
+  int tiles_m, tiles_n;
+  int vec_store;  // C rows allow aligned 8-byte stores
+};
+
+// Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
+// 8 XCDs round-robin) works on a contiguous run of tiles, walked in column-major groups of
+// `kGroupM` tile rows.
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  constexpr int kXcds = 8;
+  constexpr int kGroupM = 8;
+  const int total = tiles_m * tiles_n;
+  const int q = total / kXcds, r = total % kXcds;
+  const int xcd = pid % kXcds, idx = pid / kXcds;
+  const int tile = xcd * q + (xcd < r ? xcd : r) + idx;
+  const int per_group = kGroupM * tiles_n;
+  const int group = tile / per_group;
+  const int first_m = group * kGroupM;
+  const int gsz = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
+  const int in_group = tile - group * per_group;
+  tm = first_m + in_group % gsz;
+  tn = in_group / gsz;
+}
+
+// B_KMAJOR: B is stored [N, K] (ldb = pitch of an N-row); otherwise [K, N].
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmArgs g) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wave
+  constexpr int A_BYTES = BM * kLineBytes, B_BYTES = BN * kLineBytes;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int ROWS_PER_PASS = NT / 8;           // rows covered by one 16-byte load per thread
+  constexpr int A_LOADS = BM / ROWS_PER_PASS;
+  constexpr int B_LOADS = BN / ROWS_PER_PASS;
+  constexpr int B_BLOCKS = (BN + NT - 1) / NT;    // 8x8 transpose blocks per thread (N-major B)
+  constexpr int KSTEPS = kBK / 16;
+  static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile/threads mismatch");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+  const int64_t m0 = static_cast<int64_t>(tile_m) * BM;
+  const int64_t n0 = static_cast<int64_t>(tile_n) * BN;
+  const int64_t batch = blockIdx.y;
+  const T* __restrict__ A = static_cast<const T*>(g.a) + batch * g.stride_a;
+  const T* __restrict__ B = static_cast<const T*>(g.b) + batch * g.stride_b;
+  T* __restrict__ C = static_cast<T*>(g.c) + batch * g.stride_c;
+  const int64_t M = g.m, N = g.n, K = g.k;
+
+  // ---- global -> register staging -------------------------------------------------------
+  const int ld_row = tid >> 3;   // row inside one pass
+  const int ld_chunk = tid & 7;  // 16-byte chunk inside the 128-byte line
+  u32x4_t a_stage[A_LOADS];
+  u32x4_t b_stage[B_KMAJOR ? B_LOADS : B_BLOCKS * 8];
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+
+  // Per-lane byte offsets from the (wave-uniform) operand base are computed once, with rows
+  // clamped to the last valid one (results of such rows are never stored), so the main loop
+  // needs no predication and addresses are "uniform base + 32-bit lane offset".
+  const unsigned char* a_base = reinterpret_cast<const unsigned char*>(A);
+  const unsigned char* b_base = reinterpret_cast<const unsigned char*>(B);
+  uint32_t a_off[A_LOADS];
+#pragma unroll
+  for (int j = 0; j < A_LOADS; ++j) {
+    int64_t row = m0 + ld_row + j * ROWS_PER_PASS;
+    row = row < M ? row : M - 1;
+    a_off[j] = static_cast<uint32_t>((row * g.lda + ld_chunk * 8) * 2);
+  }
+  uint32_t b_off[B_KMAJOR ? B_LOADS : 1];
+  if constexpr (B_KMAJOR) {
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) {
+      int64_t row = n0 + ld_row + j * ROWS_PER_PASS;
+      row = row < N ? row : N - 1;
+      b_off[j] = static_cast<uint32_t>((row * g.ldb + ld_chunk * 8) * 2);
+    }
+  }
+
+  // FULL: every 16-byte chunk of the stage lies below K (no predication).
+  auto load_stage = [&](int64_t k0, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    const bool k_ok = FULL || (k0 + ld_chunk * 8 < K);
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j)
+      a_stage[j] = k_ok ? *reinterpret_cast<const u32x4_t*>(a_base + k0 * 2 + a_off[j]) : zero4;
+    if constexpr (B_KMAJOR) {
+#pragma unroll
+      for (int j = 0; j < B_LOADS; ++j)
+        b_stage[j] = k_ok ? *reinterpret_cast<const u32x4_t*>(b_base + k0 * 2 + b_off[j]) : zero4;
+    } else {
+      // Thread owns 8(k) x 8(n) blocks: k-chunk kc = blk / (BN/8), n-group ng = blk % (BN/8).
+#pragma unroll
+      for (int q = 0; q < B_BLOCKS; ++q) {
+        const int blk = tid + q * NT;
+        const int kc = blk / (BN / 8), ng = blk % (BN / 8);
+        const int64_t nn = n0 + ng * 8;
+        const bool active = (BN % NT == 0) || (blk < BN);
+        const bool whole = nn + 8 <= N;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const int64_t kk = k0 + kc * 8 + r;
+          u32x4_t v = zero4;
+          if (active && (FULL || kk < K)) {
+            const T* src = B + kk * g.ldb + nn;
+            if (whole) {
+              v = *reinterpret_cast<const u32x4_t*>(src);
+            } else {
+              // ragged right edge: element-wise, never past column N-1
+              unsigned short e[8];
+#pragma unroll
+              for (int t = 0; t < 8; ++t)
+                e[t] = (nn + t < N) ? reinterpret_cast<const unsigned short*>(src)[t]
+                                    : static_cast<unsigned short>(0);
+              v[0] = e[0] | (static_cast<uint32_t>(e[1]) << 16);
+              v[1] = e[2] | (static_cast<uint32_t>(e[3]) << 16);
+              v[2] = e[4] | (static_cast<uint32_t>(e[5]) << 16);
+              v[3] = e[6] | (static_cast<uint32_t>(e[7]) << 16);
+            }
+          }
+          b_stage[q * 8 + r] = v;
+        }
+      }
+    }
+  };
+  auto store_stage = [&](int buf) {
+    unsigned char* sa = smem + buf * STAGE_BYTES;
+    unsigned char* sb = sa + A_BYTES;
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) {
+      const int row = ld_row + j * ROWS_PER_PASS;
+      *reinterpret_cast<u32x4_t*>(sa + lds_offset(row, ld_chunk)) = a_stage[j];
+    }
+    if constexpr (B_KMAJOR) {
+#pragma unroll
+      for (int j = 0; j < B_LOADS; ++j) {
+        const int row = ld_row + j * ROWS_PER_PASS;
+        *reinterpret_cast<u32x4_t*>(sb + lds_offset(row, ld_chunk)) = b_stage[j];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < B_BLOCKS; ++q) {
+        const int blk = tid + q * NT;
+        if ((BN % NT == 0) || (blk < BN)) {
+          const int kc = blk / (BN / 8), ng = blk % (BN / 8);
+          // 8x8 transpose of 16-bit elements: out[i] holds k = 0..7 for column i.
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            u32x4_t o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const uint32_t lo = b_stage[q * 8 + 2 * j][i >> 1];
+              const uint32_t hi = b_stage[q * 8 + 2 * j + 1][i >> 1];
+              o[j] = (i & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+            }
+            const int row = ng * 8 + i;
+            *reinterpret_cast<u32x4_t*>(sb + lds_offset(row, kc)) = o;
+          }
+        }
+      }
+    }
+  };
+
+  // ---- accumulators and fragments -------------------------------------------------------
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int frag_row = lane & 31;
+  const int frag_half = lane >> 5;  // which 8-wide K half of the 16-wide MFMA step
+  u32x4_t af[2][TM], bf[2][TN];
+
+  auto load_frags = [&](int buf, int ks, int slot) {
+    const unsigned char* sa = smem + buf * STAGE_BYTES;
+    const unsigned char* sb = sa + A_BYTES;
+    const int chunk = ks * 2 + frag_half;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm * WM + i * 32 + frag_row;
+      af[slot][i] = *reinterpret_cast<const u32x4_t*>(sa + lds_offset(row, chunk));
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn * WN + j * 32 + frag_row;
+      bf[slot][j] = *reinterpret_cast<const u32x4_t*>(sb + lds_offset(row, chunk));
+    }
+  };
+  auto mfma_step = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[slot][j], af[slot][i], acc[i][j]);
+  };
+
+  // ---- main loop ------------------------------------------------------------------------
+  const int64_t k_tiles = (K + kBK - 1) / kBK;
+  const int64_t full_tiles = K / kBK;  // stages that need no K predication
+  if (full_tiles > 0) {
+    load_stage(0, std::true_type{});
+  } else {
+    load_stage(0, std::false_type{});
+  }
+  store_stage(0);
+  __syncthreads();
+  load_frags(0, 0, 0);
+  for (int64_t kt = 0; kt < k_tiles; ++kt) {
+    const int buf = static_cast<int>(kt & 1);
+    const bool more = kt + 1 < k_tiles;
+    if (more) {
+      if (kt + 1 < full_tiles) {
+        load_stage((kt + 1) * kBK, std::true_type{});
+      } else {
+        load_stage((kt + 1) * kBK, std::false_type{});
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS - 1; ++ks) {
+      load_frags(buf, ks + 1, (ks + 1) & 1);
+      mfma_step(ks & 1);
+    }
+    if (more) store_stage(buf ^ 1);
+    __syncthreads();
+    if (more) load_frags(buf ^ 1, 0, 0);  // KSTEPS is even: slot 0 is free again
+    mfma_step((KSTEPS - 1) & 1);
+  }
+
+  // ---- epilogue -------------------------------------------------------------------------
+  // Swapped-operand 32x32 result layout: lane holds row m = lane & 31 of the sub-tile;
+  // register e holds column n = 8*(e/4) + 4*(lane>>5) + (e&3).
+  const T* __restrict__ bias = static_cast<const T*>(g.bias);
+  const bool vec = g.vec_store != 0;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = m0 + wm * WM + i * 32 + (lane & 31);
+    if (row >= M) continue;
+    T* crow = C + row * g.ldc;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = n0 + wn * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+        if (col >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+        if (col + 4 <= N) {
+          if (bias != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += to_f32(bias[col + e]);
+          }
+          T o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(v[e]);
+          if (vec) {
+            u32x2_t packed;
+            packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
+                        (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
+            packed[1] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[2])) |
+                        (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[3])) << 16);
+            *reinterpret_cast<u32x2_t*>(crow + col) = packed;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) crow[col + e] = o[e];
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (col + e < N) {
+              const float b = bias != nullptr ? to_f32(bias[col + e]) : 0.0f;
+              crow[col + e] = finish<T, EPI>(v[e] + b);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
+static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) {
+  constexpr int SMEM = 2 * (BM + BN) * kLineBytes;
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  static bool configured = false;
+  auto kernel = gemm_mfma_kernel<T, BM, BN, WAVES_M, WAVES_N, B_KMAJOR, EPI>;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+    if (e != hipSuccess) return static_cast<int>(e);
+    configured = true;
+  }
+  GemmArgs g = base;
+  g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
+  g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
+  g.vec_store = (g.ldc % 4 == 0) && (g.stride_c % 4 == 0 || batch == 1) &&
+                ((reinterpret_cast<uintptr_t>(g.c) & 7u) == 0);
+  const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
+  if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
+  kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), SMEM, stream>>>(g);
+  return check_launch();
+}
+
+}  // namespace tmb

@@ -10,97 +10,148 @@
 
 namespace tmb {
 
-template <typename T, int WPR, int VPL, int BLOCK>
+// Same work decomposition as the softmax kernel: WPR waves per row, or (WPR == 1) RPW rows per
+// wave with all loads issued up front. gamma/beta are fetched before the statistics so their
+// latency hides behind the reductions.
+//
+// AFFINE_LDS (long rows): gamma and beta are copied into LDS once per workgroup, the workgroup
+// then walks many rows (grid-stride), so the affine parameters cost LDS reads instead of a
+// second and third pass through L2 for every row.
+template <typename T, int WPR, int VPL, int RPW, bool STREAM, bool AFFINE_LDS, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void layer_norm_regs_kernel(
     T* __restrict__ out, float* __restrict__ mean_out, float* __restrict__ rstd_out,
     const T* __restrict__ in, const T* __restrict__ gamma, const T* __restrict__ beta,
     int64_t rows, int cols, float eps) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int WAVES = BLOCK / kWave;
-  constexpr int ROWS_PER_BLOCK = WAVES / WPR;
+  constexpr int GROUPS = WAVES / WPR;
+  static_assert(WPR == 1 || RPW == 1, "several rows per wave only without cross-wave reductions");
   __shared__ float slot[WAVES];
 
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int group = wave / WPR;
   const int wave_in_row = wave - group * WPR;
-  int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + group;
-  const bool valid = row < rows;
-  if (!valid) row = rows - 1;
-
   const int nvec = cols / EPV;
-  const T* src = in + row * static_cast<int64_t>(cols);
-  T* dst = out + row * static_cast<int64_t>(cols);
+  const float n = static_cast<float>(cols);
 
-  float x[VPL][EPV];
-#pragma unroll
-  for (int v = 0; v < VPL; ++v) {
-    const int vi = (v * WPR + wave_in_row) * kWave + lane;
-    if (vi < nvec) {
-      Vec16<T> t = load_vec16(src + static_cast<int64_t>(vi) * EPV);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[v][e] = to_f32(t.v[e]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[v][e] = 0.0f;
+  extern __shared__ __attribute__((aligned(16))) unsigned char affine_lds[];
+  T* lds_gamma = reinterpret_cast<T*>(affine_lds);
+  T* lds_beta = lds_gamma + cols;
+  if constexpr (AFFINE_LDS) {
+    for (int vi = threadIdx.x; vi < nvec; vi += BLOCK) {
+      if (gamma != nullptr) store_vec16(lds_gamma + vi * EPV, load_vec16(gamma + vi * EPV));
+      if (beta != nullptr) store_vec16(lds_beta + vi * EPV, load_vec16(beta + vi * EPV));
     }
+    __syncthreads();
   }
 
-  float s = 0.0f;
-#pragma unroll
-  for (int v = 0; v < VPL; ++v)
-#pragma unroll
-    for (int e = 0; e < EPV; ++e) s += x[v][e];
-  s = wave_sum(s);
-  s = group_reduce(s, slot, wave, group * WPR, WPR, SumOp{});
-  float mean = s / static_cast<float>(cols);
+  const int64_t rows_per_block = static_cast<int64_t>(GROUPS) * RPW;
+  for (int64_t block_row = static_cast<int64_t>(blockIdx.x) * rows_per_block; block_row < rows;
+       block_row += static_cast<int64_t>(gridDim.x) * rows_per_block) {
+  const int64_t row0 = block_row + static_cast<int64_t>(group) * RPW;
 
-  float q = 0.0f;
+  float x[RPW][VPL][EPV];
 #pragma unroll
-  for (int v = 0; v < VPL; ++v) {
-    const int vi = (v * WPR + wave_in_row) * kWave + lane;
-    if (vi < nvec) {
+  for (int r = 0; r < RPW; ++r) {
+    int64_t row = row0 + r;
+    if (row >= rows) row = rows - 1;
+    const T* src = in + row * static_cast<int64_t>(cols);
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) {
-        const float d = x[v][e] - mean;
-        x[v][e] = d;
-        q += d * d;
+    for (int v = 0; v < VPL; ++v) {
+      // Lanes past the end of the row re-read vector 0 (always valid) and discard it: no
+      // branch, so all of a wave's loads are issued back to back.
+      const int vi = (v * WPR + wave_in_row) * kWave + lane;
+      const bool ok = vi < nvec;
+      const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
+      const Vec16<T> t = STREAM ? load_vec16_stream(src + at) : load_vec16(src + at);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) x[r][v][e] = ok ? to_f32(t.v[e]) : 0.0f;
+    }
+  }
+  // Short rows: fetch gamma/beta now so their latency hides behind the reductions. Long rows
+  // would pay for that with occupancy; they fetch them (from L2) in groups of four vectors
+  // right before use.
+  constexpr bool PREFETCH_AFFINE = !AFFINE_LDS && VPL <= 4;
+  constexpr int AFF = PREFETCH_AFFINE ? VPL : (VPL < 4 ? VPL : 4);  // vectors held at a time
+  Vec16<T> gv[AFF], bv[AFF];
+  auto load_affine = [&](int v_first) {
+#pragma unroll
+    for (int u = 0; u < AFF; ++u) {
+      const int vi = ((v_first + u) * WPR + wave_in_row) * kWave + lane;
+      const int64_t at = static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
+      if constexpr (AFFINE_LDS) {
+        if (gamma != nullptr) gv[u] = load_vec16(lds_gamma + at);
+        if (beta != nullptr) bv[u] = load_vec16(lds_beta + at);
+      } else {
+        if (gamma != nullptr) gv[u] = load_vec16(gamma + at);
+        if (beta != nullptr) bv[u] = load_vec16(beta + at);
       }
     }
-  }
-  q = wave_sum(q);
-  q = group_reduce(q, slot, wave, group * WPR, WPR, SumOp{});
-  const float var = q / static_cast<float>(cols);
-  const float rstd = 1.0f / sqrtf(var + eps);
-  if (var != var) mean = var;
+  };
+  if constexpr (PREFETCH_AFFINE) load_affine(0);
 
-  if (valid) {
-    if (wave_in_row == 0 && lane == 0) {
-      if (mean_out) mean_out[row] = mean;
-      if (rstd_out) rstd_out[row] = rstd;
-    }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    float s = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) s += x[r][v][e];
+    s = wave_sum(s);
+    s = group_reduce(s, slot, wave, group * WPR, WPR, SumOp{});
+    float mean = s / n;
+
+    float q = 0.0f;
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
       const int vi = (v * WPR + wave_in_row) * kWave + lane;
-      if (vi < nvec) {
-        float y[EPV];
-        if (gamma != nullptr) {
-          Vec16<T> g = load_vec16(gamma + static_cast<int64_t>(vi) * EPV);
+      const bool ok = vi < nvec;
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) y[e] = x[v][e] * rstd * to_f32(g.v[e]);
-        } else {
+      for (int e = 0; e < EPV; ++e) {
+        const float d = ok ? x[r][v][e] - mean : 0.0f;
+        x[r][v][e] = d;
+        q += d * d;
+      }
+    }
+    q = wave_sum(q);
+    q = group_reduce(q, slot, wave, group * WPR, WPR, SumOp{});
+    const float var = q / n;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    if (var != var) mean = var;
+
+    const int64_t row = row0 + r;
+    if (row < rows) {
+      if (wave_in_row == 0 && lane == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (rstd_out) rstd_out[row] = rstd;
+      }
+      T* dst = out + row * static_cast<int64_t>(cols);
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) y[e] = x[v][e] * rstd;
+      for (int v0 = 0; v0 < VPL; v0 += AFF) {
+        if constexpr (!PREFETCH_AFFINE) load_affine(v0);
+#pragma unroll
+        for (int u = 0; u < AFF; ++u) {
+          const int v = v0 + u;
+          const int vi = (v * WPR + wave_in_row) * kWave + lane;
+          float y[EPV];
+          if (gamma != nullptr) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) y[e] = x[r][v][e] * rstd * to_f32(gv[u].v[e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) y[e] = x[r][v][e] * rstd;
+          }
+          if (beta != nullptr) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) y[e] += to_f32(bv[u].v[e]);
+          }
+          if (vi < nvec) store_converted<T, EPV, STREAM>(dst + static_cast<int64_t>(vi) * EPV, y);
         }
-        if (beta != nullptr) {
-          Vec16<T> b = load_vec16(beta + static_cast<int64_t>(vi) * EPV);
-#pragma unroll
-          for (int e = 0; e < EPV; ++e) y[e] += to_f32(b.v[e]);
-        }
-        store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, y);
       }
     }
   }
+  }  // grid-stride over row groups
 }
 
 template <typename T>
@@ -145,11 +196,34 @@ __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
 template <typename T, int WPR, int VPL, int BLOCK>
 static int launch_ln(T* out, float* mean, float* rstd, const T* x, const T* g, const T* b,
                      int64_t rows, int64_t cols, float eps, hipStream_t stream) {
-  constexpr int ROWS_PER_BLOCK = (BLOCK / kWave) / WPR;
-  const int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
-  layer_norm_regs_kernel<T, WPR, VPL, BLOCK>
-      <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(
-          out, mean, rstd, x, g, b, rows, static_cast<int>(cols), eps);
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int FLOATS = VPL * EPV;
+  constexpr int RPW = (WPR > 1 || FLOATS >= 64) ? 1 : (FLOATS >= 32 ? 2 : 4);
+  constexpr int ROWS_PER_BLOCK = (BLOCK / kWave) / WPR * RPW;
+  int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  const bool stream_hint = rows * cols * static_cast<int64_t>(2 * sizeof(T)) >= (int64_t{256} << 20);
+  const dim3 block(BLOCK);
+  const int c = static_cast<int>(cols);
+  // Long rows with affine parameters: stage gamma/beta in LDS, few persistent workgroups.
+  const size_t lds_bytes = static_cast<size_t>(cols) * sizeof(T) * 2;
+  // (16-bit rows only: for fp32 the LDS reads would cost as much as the L2 re-reads they replace)
+  if constexpr (VPL >= 8 && sizeof(T) == 2) {
+    if ((g != nullptr || b != nullptr) && lds_bytes <= 65536) {
+      const int64_t persistent = 256 * (BLOCK >= 1024 ? 2 : 8);
+      if (blocks > persistent) blocks = persistent;
+      const dim3 grid(static_cast<unsigned>(blocks));
+      if (stream_hint)
+        layer_norm_regs_kernel<T, WPR, VPL, RPW, true, true, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
+      else
+        layer_norm_regs_kernel<T, WPR, VPL, RPW, false, true, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
+      return check_launch();
+    }
+  }
+  const dim3 grid(static_cast<unsigned>(blocks));
+  if (stream_hint)
+    layer_norm_regs_kernel<T, WPR, VPL, RPW, true, false, BLOCK><<<grid, block, 0, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
+  else
+    layer_norm_regs_kernel<T, WPR, VPL, RPW, false, false, BLOCK><<<grid, block, 0, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
   return check_launch();
 }
 
@@ -162,20 +236,27 @@ static int layer_norm_dispatch(void* out_, float* mean, float* rstd, const void*
   const T* g = static_cast<const T*>(g_);
   const T* b = static_cast<const T*>(b_);
   constexpr int EPV = Vec16<T>::N;
+  constexpr int MAXV = 64 / EPV;  // at most 64 fp32 values of a row per lane
   const bool vec_ok = (cols % EPV == 0) && aligned16(x) && aligned16(out) &&
                       (g == nullptr || aligned16(g)) && (b == nullptr || aligned16(b)) &&
                       rows < (int64_t{1} << 31);
   const int64_t nvec = cols / EPV;
-  if (vec_ok && nvec <= 8192) {
-    if (nvec <= 64) return launch_ln<T, 1, 1, 256>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    if (nvec <= 128) return launch_ln<T, 1, 2, 256>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    if (nvec <= 256) return launch_ln<T, 1, 4, 256>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    if (nvec <= 512) return launch_ln<T, 1, 8, 256>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    if (nvec <= 1024) return launch_ln<T, 4, 4, 256>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    if (nvec <= 2048) return launch_ln<T, 4, 8, 256>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    if (nvec <= 4096) return launch_ln<T, 16, 4, 1024>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
-    return launch_ln<T, 16, 8, 1024>(out, mean, rstd, x, g, b, rows, cols, eps, stream);
+#define TMB_LN(WPR, VPL, BLOCK) \
+  return launch_ln<T, WPR, VPL, BLOCK>(out, mean, rstd, x, g, b, rows, cols, eps, stream)
+  if (vec_ok && nvec <= 16 * 64 * MAXV) {
+    if (nvec <= 64) TMB_LN(1, 1, 256);
+    if (nvec <= 128) TMB_LN(1, 2, 256);
+    if (nvec <= 256) TMB_LN(1, 4, 256);
+    if (nvec <= 512) TMB_LN(1, 8, 256);
+    if constexpr (MAXV >= 16) {
+      if (nvec <= 1024) TMB_LN(1, 16, 256);
+    }
+    if (nvec <= 4 * 64 * MAXV / 2) TMB_LN(4, MAXV / 2, 256);
+    if (nvec <= 4 * 64 * MAXV) TMB_LN(4, MAXV, 256);
+    if (nvec <= 16 * 64 * MAXV / 2) TMB_LN(16, MAXV / 2, 1024);
+    TMB_LN(16, MAXV, 1024);
   }
+#undef TMB_LN
   const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
   layer_norm_generic_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(
       out, mean, rstd, x, g, b, rows, cols, eps);

@@ -26,7 +26,7 @@ struct SplitPlan {
 // Must stay a pure function of (rows, cols): the Python side sizes the workspace from it and
 // reproducibility relies on it.
 static SplitPlan plan_splits(int64_t rows, int64_t cols) {
-  constexpr int64_t kTargetBlocks = 2048;   // 8 workgroups per CU on 256 CUs
+  constexpr int64_t kTargetBlocks = 8192;   // 32 chunks per CU on 256 CUs: dynamic balance
   constexpr int64_t kMinChunk = 16384;      // elements; below this a split is not worth a launch
   constexpr int64_t kMaxChunk = int64_t{1} << 30;
   int64_t splits = 1;
@@ -38,7 +38,7 @@ static SplitPlan plan_splits(int64_t rows, int64_t cols) {
   }
   const int64_t need = (cols + kMaxChunk - 1) / kMaxChunk;
   if (splits < need) splits = need;
-  if (splits > 4096) splits = 4096;
+  if (splits > 8192) splits = 8192;
   int64_t chunk = (cols + splits - 1) / splits;
   if (splits > 1) {
     chunk = (chunk + 63) / 64 * 64;
@@ -250,20 +250,30 @@ __global__ __launch_bounds__(kRedBlock) void reduce_wave_kernel(T* __restrict__ 
   if ((threadIdx.x & 63) == 0) out[row] = finalize<T>(acc, op, cols);
 }
 
-// Second stage: combines the `splits` partials of each row in chunk order.
-template <typename Policy, typename T>
-__global__ __launch_bounds__(kWave) void reduce_final_kernel(T* __restrict__ out,
-                                                             const void* __restrict__ ws,
-                                                             int64_t rows, int64_t cols,
-                                                             int splits, int op) {
+// Second stage: combines the `splits` partials of each row. Thread t takes partials t, t+NT, ...
+// (independent loads, all in flight at once), then the usual wave tree and a fixed-order
+// combine across waves.
+template <typename Policy, typename T, int kFinalBlock>
+__global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(T* __restrict__ out,
+                                                                  const void* __restrict__ ws,
+                                                                  int64_t rows, int64_t cols,
+                                                                  int splits, int op) {
   using A = typename Policy::acc_t;
+  constexpr int WAVES = kFinalBlock / kWave;
+  __shared__ A slot[WAVES];
   const int64_t row = blockIdx.x;
-  const int lane = threadIdx.x;
   A acc = Policy::identity();
-  for (int i = lane; i < splits; i += kWave)
+  for (int i = threadIdx.x; i < splits; i += kFinalBlock)
     acc = Policy::combine(acc, AccStore<A>::get(ws, row * splits + i));
   acc = wave_combine<Policy>(acc);
-  if (lane == 0) out[row] = finalize<T>(acc, op, cols);
+  if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    A r = slot[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) r = Policy::combine(r, slot[w]);
+    out[row] = finalize<T>(r, op, cols);
+  }
 }
 
 template <typename Policy, typename T, bool IMAX>
@@ -288,8 +298,13 @@ static int launch_reduce(void* out_, const void* in_, int64_t rows, int64_t cols
       out, ws, in, rows, cols, plan.splits, plan.chunk, op);
   int rc = check_launch();
   if (rc != 0 || plan.splits == 1) return rc;
-  reduce_final_kernel<Policy, T><<<dim3(static_cast<unsigned>(rows)), dim3(kWave), 0, stream>>>(
-      out, ws, rows, cols, plan.splits, op);
+  if (plan.splits > 256) {
+    reduce_final_kernel<Policy, T, 1024><<<dim3(static_cast<unsigned>(rows)), dim3(1024), 0, stream>>>(
+        out, ws, rows, cols, plan.splits, op);
+  } else {
+    reduce_final_kernel<Policy, T, 64><<<dim3(static_cast<unsigned>(rows)), dim3(64), 0, stream>>>(
+        out, ws, rows, cols, plan.splits, op);
+  }
   return check_launch();
 }
 
@@ -376,14 +391,15 @@ __device__ __forceinline__ Best<typename ArgTraits<T>::val_t> argmax_range(const
   const T* body = p + head;
   const int nvec = static_cast<int>((n - head) / EPV);
   int i = tid;
-  for (; i + NT < nvec; i += 2 * NT) {
-    const Vec16<T> v0 = load_vec16(body + static_cast<int64_t>(i) * EPV);
-    const Vec16<T> v1 = load_vec16(body + static_cast<int64_t>(i + NT) * EPV);
+  for (; i + 3 * NT < nvec; i += 4 * NT) {  // four 16-byte loads in flight per lane
+    Vec16<T> v[4];
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) scan_one(best, off, ArgTraits<T>::conv(v0.v[e]), head + i * EPV + e);
+    for (int u = 0; u < 4; ++u) v[u] = load_vec16(body + static_cast<int64_t>(i + u * NT) * EPV);
 #pragma unroll
-    for (int e = 0; e < EPV; ++e)
-      scan_one(best, off, ArgTraits<T>::conv(v1.v[e]), head + (i + NT) * EPV + e);
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e)
+        scan_one(best, off, ArgTraits<T>::conv(v[u].v[e]), head + (i + u * NT) * EPV + e);
   }
   for (; i < nvec; i += NT) {
     const Vec16<T> v0 = load_vec16(body + static_cast<int64_t>(i) * EPV);
@@ -444,19 +460,28 @@ __global__ __launch_bounds__(kRedBlock) void argmax_chunk_kernel(int64_t* __rest
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(kWave) void argmax_final_kernel(int64_t* __restrict__ out,
-                                                             const void* __restrict__ ws,
-                                                             int64_t rows, int splits) {
+template <typename T, int kFinalBlock>
+__global__ __launch_bounds__(kFinalBlock) void argmax_final_kernel(int64_t* __restrict__ out,
+                                                                  const void* __restrict__ ws,
+                                                                  int64_t rows, int splits) {
   using V = typename ArgTraits<T>::val_t;
+  constexpr int WAVES = kFinalBlock / kWave;
+  __shared__ BestSlot<V> slot[WAVES];
   const int64_t row = blockIdx.x;
   Best<V> b{V(0), int64_t{-1}};
-  for (int i = threadIdx.x; i < splits; i += kWave) {
+  for (int i = threadIdx.x; i < splits; i += kFinalBlock) {
     const BestSlot<V> s = static_cast<const BestSlot<V>*>(ws)[row * splits + i];
     b = best_combine(b, Best<V>{s.val, s.idx});
   }
   b = wave_best(b);
-  if (threadIdx.x == 0) out[row] = b.idx;
+  if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = BestSlot<V>{b.idx, b.val};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Best<V> r{slot[0].val, slot[0].idx};
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) r = best_combine(r, Best<V>{slot[w].val, slot[w].idx});
+    out[row] = r.idx;
+  }
 }
 
 template <typename T>
@@ -473,8 +498,13 @@ static int launch_argmax(int64_t* out, const void* in_, int64_t rows, int64_t co
       out, ws, in, rows, cols, plan.splits, plan.chunk);
   int rc = check_launch();
   if (rc != 0 || plan.splits == 1) return rc;
-  argmax_final_kernel<T><<<dim3(static_cast<unsigned>(rows)), dim3(kWave), 0, stream>>>(
-      out, ws, rows, plan.splits);
+  if (plan.splits > 256) {
+    argmax_final_kernel<T, 1024><<<dim3(static_cast<unsigned>(rows)), dim3(1024), 0, stream>>>(
+        out, ws, rows, plan.splits);
+  } else {
+    argmax_final_kernel<T, 64><<<dim3(static_cast<unsigned>(rows)), dim3(64), 0, stream>>>(
+        out, ws, rows, plan.splits);
+  }
   return check_launch();
 }
 

@@ -14,85 +14,96 @@
 
 namespace tmb {
 
-template <typename TIn, typename TOut, int WPR, int VPL, bool LOG, int BLOCK>
+// WPR waves cooperate on a row (WPR > 1: one row per group of waves); with WPR == 1 every wave
+// owns RPW independent rows whose loads are all issued before any arithmetic, which keeps more
+// bytes in flight for short rows. STREAM selects non-temporal loads/stores (tensors larger than
+// the Infinity Cache).
+template <typename TIn, typename TOut, int WPR, int VPL, int RPW, bool LOG, bool STREAM, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(TOut* __restrict__ out,
                                                              const TIn* __restrict__ in,
                                                              int64_t rows, int cols) {
   constexpr int EPV = Vec16<TIn>::N;
   constexpr int WAVES = BLOCK / kWave;
-  constexpr int ROWS_PER_BLOCK = WAVES / WPR;
+  constexpr int GROUPS = WAVES / WPR;
+  static_assert(WPR == 1 || RPW == 1, "several rows per wave only without cross-wave reductions");
   __shared__ float slot[WAVES];
 
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int group = wave / WPR;
   const int wave_in_row = wave - group * WPR;
-  int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + group;
-  const bool valid = row < rows;
-  if (!valid) row = rows - 1;  // stay in lock-step with the block's barriers; stores are masked
-
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * GROUPS + group) * RPW;
   const int nvec = cols / EPV;
-  const TIn* src = in + row * static_cast<int64_t>(cols);
-  TOut* dst = out + row * static_cast<int64_t>(cols);
-
-  float x[VPL][EPV];
   const float neg_inf = -__builtin_inff();
-#pragma unroll
-  for (int v = 0; v < VPL; ++v) {
-    const int vi = (v * WPR + wave_in_row) * kWave + lane;
-    if (vi < nvec) {
-      Vec16<TIn> t = load_vec16(src + static_cast<int64_t>(vi) * EPV);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[v][e] = to_f32(t.v[e]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[v][e] = neg_inf;
-    }
-  }
 
-  float m = neg_inf;
+  float x[RPW][VPL][EPV];
 #pragma unroll
-  for (int v = 0; v < VPL; ++v)
-#pragma unroll
-    for (int e = 0; e < EPV; ++e) m = fmaxf(m, x[v][e]);
-  m = wave_max(m);
-  m = group_reduce(m, slot, wave, group * WPR, WPR, MaxOp{});
-
-  float s = 0.0f;
-#pragma unroll
-  for (int v = 0; v < VPL; ++v)
-#pragma unroll
-    for (int e = 0; e < EPV; ++e) {
-      const float ex = exp_f32(x[v][e] - m);
-      if (LOG) {
-        x[v][e] = x[v][e] - m;
-      } else {
-        x[v][e] = ex;
-      }
-      s += ex;
-    }
-  s = wave_sum(s);
-  s = group_reduce(s, slot, wave, group * WPR, WPR, SumOp{});
-
-  if (LOG) {
-    const float lg = logf(s);
-#pragma unroll
-    for (int v = 0; v < VPL; ++v)
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[v][e] -= lg;
-  } else {
-    const float inv = 1.0f / s;
-#pragma unroll
-    for (int v = 0; v < VPL; ++v)
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[v][e] *= inv;
-  }
-
-  if (valid) {
+  for (int r = 0; r < RPW; ++r) {
+    int64_t row = row0 + r;
+    if (row >= rows) row = rows - 1;  // keep lock-step; stores are masked below
+    const TIn* src = in + row * static_cast<int64_t>(cols);
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
+      // Lanes past the end of the row re-read vector 0 (always valid) and discard it: no
+      // branch, so all of a wave's loads are issued back to back.
       const int vi = (v * WPR + wave_in_row) * kWave + lane;
-      if (vi < nvec) store_converted<TOut, EPV>(dst + static_cast<int64_t>(vi) * EPV, x[v]);
+      const bool ok = vi < nvec;
+      const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
+      const Vec16<TIn> t = STREAM ? load_vec16_stream(src + at) : load_vec16(src + at);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) x[r][v][e] = ok ? to_f32(t.v[e]) : neg_inf;
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    float m = neg_inf;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) m = fmaxf(m, x[r][v][e]);
+    m = wave_max(m);
+    m = group_reduce(m, slot, wave, group * WPR, WPR, MaxOp{});
+
+    float s = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float ex = exp_f32(x[r][v][e] - m);
+        if (LOG) {
+          x[r][v][e] = x[r][v][e] - m;
+        } else {
+          x[r][v][e] = ex;
+        }
+        s += ex;
+      }
+    s = wave_sum(s);
+    s = group_reduce(s, slot, wave, group * WPR, WPR, SumOp{});
+
+    if (LOG) {
+      const float lg = logf(s);
+#pragma unroll
+      for (int v = 0; v < VPL; ++v)
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) x[r][v][e] -= lg;
+    } else {
+      const float inv = 1.0f / s;
+#pragma unroll
+      for (int v = 0; v < VPL; ++v)
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) x[r][v][e] *= inv;
+    }
+
+    const int64_t row = row0 + r;
+    if (row < rows) {
+      TOut* dst = out + row * static_cast<int64_t>(cols);
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) {
+        const int vi = (v * WPR + wave_in_row) * kWave + lane;
+        if (vi < nvec)
+          store_converted<TOut, EPV, STREAM>(dst + static_cast<int64_t>(vi) * EPV, x[r][v]);
+      }
     }
   }
 }
@@ -129,11 +140,20 @@ __global__ __launch_bounds__(256) void softmax_generic_kernel(TOut* __restrict__
 
 template <typename TIn, typename TOut, bool LOG, int WPR, int VPL, int BLOCK>
 static int launch_regs(TOut* out, const TIn* in, int64_t rows, int64_t cols, hipStream_t stream) {
-  constexpr int ROWS_PER_BLOCK = (BLOCK / kWave) / WPR;
+  constexpr int EPV = Vec16<TIn>::N;
+  constexpr int FLOATS = VPL * EPV;
+  constexpr int RPW = (WPR > 1 || FLOATS >= 64) ? 1 : (FLOATS >= 32 ? 2 : 4);
+  constexpr int ROWS_PER_BLOCK = (BLOCK / kWave) / WPR * RPW;
   const int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
-  softmax_regs_kernel<TIn, TOut, WPR, VPL, LOG, BLOCK>
-      <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows,
-                                                                         static_cast<int>(cols));
+  // Streams when the tensor cannot live in the 256 MB Infinity Cache anyway.
+  const bool stream_hint = rows * cols * static_cast<int64_t>(sizeof(TIn) + sizeof(TOut)) >= (int64_t{256} << 20);
+  if (stream_hint) {
+    softmax_regs_kernel<TIn, TOut, WPR, VPL, RPW, LOG, true, BLOCK>
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows, static_cast<int>(cols));
+  } else {
+    softmax_regs_kernel<TIn, TOut, WPR, VPL, RPW, LOG, false, BLOCK>
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows, static_cast<int>(cols));
+  }
   return check_launch();
 }
 
@@ -141,19 +161,25 @@ template <typename TIn, typename TOut, bool LOG>
 static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols,
                             hipStream_t stream) {
   constexpr int EPV = Vec16<TIn>::N;
+  constexpr int MAXV = 64 / EPV;  // at most 64 fp32 values of a row per lane
   const bool vec_ok = (cols % EPV == 0) && aligned16(in) && aligned16(out) &&
                       rows < (int64_t{1} << 31);
   const int64_t nvec = cols / EPV;
-  if (vec_ok && nvec <= 8192) {
+  if (vec_ok && nvec <= 16 * 64 * MAXV) {
     if (nvec <= 64) return launch_regs<TIn, TOut, LOG, 1, 1, 256>(out, in, rows, cols, stream);
     if (nvec <= 128) return launch_regs<TIn, TOut, LOG, 1, 2, 256>(out, in, rows, cols, stream);
     if (nvec <= 256) return launch_regs<TIn, TOut, LOG, 1, 4, 256>(out, in, rows, cols, stream);
     if (nvec <= 512) return launch_regs<TIn, TOut, LOG, 1, 8, 256>(out, in, rows, cols, stream);
-    if (nvec <= 1024) return launch_regs<TIn, TOut, LOG, 4, 4, 256>(out, in, rows, cols, stream);
-    if (nvec <= 2048) return launch_regs<TIn, TOut, LOG, 4, 8, 256>(out, in, rows, cols, stream);
-    if (nvec <= 4096)
-      return launch_regs<TIn, TOut, LOG, 16, 4, 1024>(out, in, rows, cols, stream);
-    return launch_regs<TIn, TOut, LOG, 16, 8, 1024>(out, in, rows, cols, stream);
+    if constexpr (MAXV >= 16) {
+      if (nvec <= 1024) return launch_regs<TIn, TOut, LOG, 1, 16, 256>(out, in, rows, cols, stream);
+    }
+    if (nvec <= 4 * 64 * MAXV / 2)
+      return launch_regs<TIn, TOut, LOG, 4, MAXV / 2, 256>(out, in, rows, cols, stream);
+    if (nvec <= 4 * 64 * MAXV)
+      return launch_regs<TIn, TOut, LOG, 4, MAXV, 256>(out, in, rows, cols, stream);
+    if (nvec <= 16 * 64 * MAXV / 2)
+      return launch_regs<TIn, TOut, LOG, 16, MAXV / 2, 1024>(out, in, rows, cols, stream);
+    return launch_regs<TIn, TOut, LOG, 16, MAXV, 1024>(out, in, rows, cols, stream);
   }
   const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
   softmax_generic_kernel<TIn, TOut, LOG>

@@ -45,9 +45,22 @@ __device__ __forceinline__ void store_vec16(T* p, const Vec16<T>& v) {
   *reinterpret_cast<Vec16<T>*>(p) = v;
 }
 
+// Streaming variants: data that is touched exactly once is moved with the non-temporal hint so
+// it does not displace reusable lines (gamma/beta, partials) from L2 / Infinity Cache.
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t raw16_t;
+template <typename T>
+__device__ __forceinline__ Vec16<T> load_vec16_stream(const T* p) {
+  const raw16_t r = __builtin_nontemporal_load(reinterpret_cast<const raw16_t*>(p));
+  return __builtin_bit_cast(Vec16<T>, r);
+}
+template <typename T>
+__device__ __forceinline__ void store_vec16_stream(T* p, const Vec16<T>& v) {
+  __builtin_nontemporal_store(__builtin_bit_cast(raw16_t, v), reinterpret_cast<raw16_t*>(p));
+}
+
 // Stores N = 16/sizeof(TIn) fp32 values as TOut elements. When TOut is wider
 // than TIn (half_to_float softmax) this issues several 16-byte stores.
-template <typename TOut, int N>
+template <typename TOut, int N, bool STREAM = false>
 __device__ __forceinline__ void store_converted(TOut* p, const float (&x)[N]) {
   constexpr int OUT_PER_VEC = 16 / sizeof(TOut);
   static_assert(N % OUT_PER_VEC == 0, "vector width mismatch");
@@ -56,7 +69,11 @@ __device__ __forceinline__ void store_converted(TOut* p, const float (&x)[N]) {
     Vec16<TOut> o;
 #pragma unroll
     for (int e = 0; e < OUT_PER_VEC; ++e) o.v[e] = from_f32<TOut>(x[c * OUT_PER_VEC + e]);
-    store_vec16(p + c * OUT_PER_VEC, o);
+    if (STREAM) {
+      store_vec16_stream(p + c * OUT_PER_VEC, o);
+    } else {
+      store_vec16(p + c * OUT_PER_VEC, o);
+    }
   }
 }
 
