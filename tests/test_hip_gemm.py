@@ -86,12 +86,15 @@ def test_mm_fp32(mnk):
 
 
 @pytest.mark.parametrize("mnk", [(4096, 4096, 4096), (8192, 8192, 8192)])
-def test_addmm_bf16_large_sampled_rows(mnk):
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_addmm_bf16_large_sampled_rows(mnk, trans_b):
     """Benchmark sizes: float64 check on 64 sampled rows + linearity over the whole product."""
     m, n, k = mnk
     g = torch.Generator(device="cuda").manual_seed(0)
     a = torch.randn(m, k, generator=g, device="cuda").bfloat16()
     b = torch.randn(k, n, generator=g, device="cuda").bfloat16()
+    if trans_b:
+        b = b.t().contiguous().t()
     bias = torch.randn(n, generator=g, device="cuda").bfloat16()
     got = _ops().gemm(a, b, bias)
     rows = torch.randperm(m, generator=torch.Generator().manual_seed(1))[:64]
@@ -122,6 +125,40 @@ def test_bmm(dtype):
     assert_close64(scores, as64(ref), rtol=2e-5, atol=1e-4, rounded_want=True, what="vs C oracle")
 
 
+# K-major B with K a multiple of 128 takes the direct-to-LDS kernel; the shapes are chosen so
+# that each of its tile sizes runs, with ragged M and N edges: 256x256 (256 tiles, one round of
+# the 256 CUs), 256x128 (528 tiles), 128x128 (few tiles), and a single K revolution (K = 128).
+KMAJOR = [(3900, 4000, 256), (4000, 4100, 256), (300, 1000, 384), (1000, 5000, 128), (130, 70, 1152)]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", KMAJOR)
+def test_addmm_kmajor_b_tiles(mnk, dtype):
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
+    w = torch.randn(n, k, generator=g, device="cuda").to(dtype)      # weight [n, k]; B = w.t()
+    bias = torch.randn(n, generator=g, device="cuda").to(dtype)
+    got = _ops().gemm(a, w.t(), bias)
+    want = (a.double() @ w.double().t() + bias.double()).cpu().numpy()
+    assert rel_frobenius(got, want) <= 1e-2
+    assert_close64(got, want, rtol=2e-5, atol=1e-3, what=f"addmm K-major B {mnk} {dtype}")
+    # same product through the N-major path (other kernel, same fp32 accumulation order per
+    # output is not guaranteed, so compare to the same bound rather than bit-for-bit)
+    got_nn = _ops().gemm(a, w.t().contiguous(), bias)
+    assert_close64(got_nn, want, rtol=2e-5, atol=1e-3, what=f"addmm N-major B {mnk} {dtype}")
+
+
+def test_bmm_kmajor_b_direct_to_lds():
+    a = seeded((12, 300, 128), seed=1, dtype=torch.bfloat16)
+    b = seeded((12, 200, 128), seed=2, dtype=torch.bfloat16)
+    got = _ops().gemm(_dev(a), _dev(b).transpose(1, 2))
+    want = torch.bmm(a.double(), b.double().transpose(1, 2)).numpy()
+    assert_close64(got, want, rtol=2e-5, atol=1e-4, what="bmm K-major B, K=128")
+    assert_close64(got, as64(oracle.gemm(a, b.transpose(1, 2))), rtol=2e-5, atol=1e-4,
+                   rounded_want=True, what="vs C oracle")
+
+
 def test_bmm_benchmark_shape_bf16():
     a = seeded((48, 1024, 64), seed=1, dtype=torch.bfloat16)
     b = seeded((48, 64, 1024), seed=2, dtype=torch.bfloat16)
@@ -133,11 +170,14 @@ def test_bmm_benchmark_shape_bf16():
 
 @pytest.mark.parametrize("dtype", [torch.float32] + HALF)
 @pytest.mark.parametrize("approximate", ["tanh", "none"])
-def test_gelu_epilogue_equals_unfused(dtype, approximate):
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gelu_epilogue_equals_unfused(dtype, approximate, trans_b):
     """The fused epilogue must be bit-identical to addmm followed by the standalone GELU."""
     m, n, k = 200, 3072, 768
     a, b, bias = _abc(m, n, k, dtype, seed=9)
     b = (b * 0.05).to(dtype)
+    if trans_b:
+        b = b.t().contiguous().t()
     ek = _ek()
     epi = ek.EPI_GELU_TANH if approximate == "tanh" else ek.EPI_GELU_ERF
     fused = _ops().gemm(_dev(a), _dev(b), _dev(bias), epilogue=epi)

@@ -19,6 +19,7 @@
 #include <type_traits>
 
 #include "gemm_mfma.h"
+#include "gemm_ring.h"
 
 namespace tmb {
 
@@ -94,12 +95,31 @@ __global__ __launch_bounds__(256) void gemm_simt_kernel(
   }
 }
 
+// Tile choice. 256x256 has the best reuse per byte staged through LDS, but it runs one workgroup
+// per CU; narrow outputs and short-K products (attention's q.k^T and att.v) are load/store bound
+// and want more, smaller workgroups in flight.
 template <typename T, bool B_KMAJOR, int EPI>
 static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) {
-  // Big tiles when they still fill the 256 CUs, otherwise the 128x128 tile.
-  const int64_t big_tiles = ((g.m + 255) / 256) * ((g.n + 255) / 256) * batch;
-  if (big_tiles >= 192) return launch_mfma<T, 256, 256, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
-  return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  auto tiles = [&](int64_t bm, int64_t bn) { return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn) * batch; };
+  if constexpr (B_KMAJOR) {
+    // Both operands K-major and K a whole number of ring revolutions: direct-to-LDS kernel.
+    // 256x256 (8 waves) has the best steady state; it is used when its tiles fill the 256 CUs
+    // in nearly whole rounds, otherwise smaller tiles cut the idle tail.
+    if (g.k % 128 == 0 && g.n > 64) {
+      const int64_t t256 = tiles(256, 256);
+      const int64_t rounds = (t256 + 255) / 256;
+      if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9)
+        return launch_ring<T, 256, 256, 2, 4, EPI>(g, batch, stream);
+      if (tiles(256, 128) >= 512) return launch_ring<T, 256, 128, 4, 2, EPI>(g, batch, stream);
+      if (tiles(128, 128) >= 32) return launch_ring<T, 128, 128, 2, 2, EPI>(g, batch, stream);
+    }
+  }
+  if (g.n <= 64) return launch_mfma<T, 256, 64, 4, 1, B_KMAJOR, EPI>(g, batch, stream);
+  if (g.k <= 128) return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  if (tiles(256, 256) >= 768) return launch_mfma<T, 256, 256, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  if (g.n <= 128 && tiles(256, 128) >= 128) return launch_mfma<T, 256, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  if (tiles(128, 128) >= 128) return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  return launch_mfma<T, 64, 64, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
 }
 
 template <typename T, int EPI>

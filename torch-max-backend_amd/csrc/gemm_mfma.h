@@ -97,6 +97,54 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = in_group / gsz;
 }
 
+// Epilogue of one 32x32 MFMA result. Swapped-operand layout: the lane holds one row of C
+// (`crow`, valid when `row_ok`) and register e holds column col0 + 8*(e/4) + (e&3).
+// Adds the bias in fp32, applies the activation, casts once, stores 8 bytes per register quad
+// when the row allows it. Kept out of line: sixteen inlined copies of the GELU epilogue exceed
+// the unroller's budget, and a rolled loop would index the accumulators dynamically.
+template <typename T, int EPI>
+__device__ __noinline__ void store_tile(f32x16_t acc, T* __restrict__ crow, bool row_ok,
+                                        int64_t col0, int64_t N, const T* __restrict__ bias,
+                                        bool vec) {
+  if (!row_ok) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int64_t col = col0 + 8 * q;
+    if (col >= N) continue;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = acc[4 * q + e];
+    if (col + 4 <= N) {
+      if (bias != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += to_f32(bias[col + e]);
+      }
+      T o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(v[e]);
+      if (vec) {
+        u32x2_t packed;
+        packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
+                    (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
+        packed[1] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[2])) |
+                    (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[3])) << 16);
+        *reinterpret_cast<u32x2_t*>(crow + col) = packed;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) crow[col + e] = o[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (col + e < N) {
+          const float b = bias != nullptr ? to_f32(bias[col + e]) : 0.0f;
+          crow[col + e] = finish<T, EPI>(v[e] + b);
+        }
+      }
+    }
+  }
+}
+
 // B_KMAJOR: B is stored [N, K] (ldb = pitch of an N-row); otherwise [K, N].
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmArgs g) {
@@ -309,53 +357,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmAr
   }
 
   // ---- epilogue -------------------------------------------------------------------------
-  // Swapped-operand 32x32 result layout: lane holds row m = lane & 31 of the sub-tile;
-  // register e holds column n = 8*(e/4) + 4*(lane>>5) + (e&3).
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
-  const bool vec = g.vec_store != 0;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int64_t row = m0 + wm * WM + i * 32 + (lane & 31);
-    if (row >= M) continue;
-    T* crow = C + row * g.ldc;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t col = n0 + wn * WN + j * 32 + 8 * q + 4 * (lane >> 5);
-        if (col >= N) continue;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-        if (col + 4 <= N) {
-          if (bias != nullptr) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += to_f32(bias[col + e]);
-          }
-          T o[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(v[e]);
-          if (vec) {
-            u32x2_t packed;
-            packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
-                        (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
-            packed[1] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[2])) |
-                        (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[3])) << 16);
-            *reinterpret_cast<u32x2_t*>(crow + col) = packed;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) crow[col + e] = o[e];
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (col + e < N) {
-              const float b = bias != nullptr ? to_f32(bias[col + e]) : 0.0f;
-              crow[col + e] = finish<T, EPI>(v[e] + b);
-            }
-          }
-        }
-      }
+      const int64_t col0 = n0 + wn * WN + j * 32 + 4 * (lane >> 5);
+      store_tile<T, EPI>(acc[i][j], C + (row < M ? row : 0) * g.ldc, row < M, col0, N, bias,
+                         g.vec_store != 0);
     }
   }
 }

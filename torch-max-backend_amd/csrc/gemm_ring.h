@@ -1,0 +1,209 @@
+// MFMA GEMM with direct-to-LDS loads for gfx950: A [M,K] and B [N,K] both K-major.
+//
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS (lane l
+// of a wave lands at base + 16*l), so no staging registers and no ds_write instructions are
+// spent on the operands. K is walked in stages of 32; four stages form a ring in LDS and up to
+// three of them are in flight while one is multiplied. Each wave waits only for its own
+// loads of the stage needed next (s_waitcnt vmcnt(N) with N = the loads of the two younger
+// stages), then one s_barrier makes every wave's part of that stage visible.
+//
+// LDS stage layout: 64-byte lines (32 K-values) per matrix row, the four 16-byte chunks of a
+// line XOR-swizzled with (row>>1)&3: ds_read_b128 fragment fetches of 8 consecutive rows then
+// touch 8 distinct 16-byte bank groups. The swizzle is applied on the global side: each lane
+// of a load picks the source chunk that belongs at its LDS slot.
+//
+// The four stages are distinct __shared__ arrays and the ring is unrolled by hand, so that the
+// compiler can tell a stage being filled from the stage being read and does not serialise them.
+#pragma once
+
+#include <type_traits>
+
+#include "gemm_mfma.h"
+
+namespace tmb {
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+constexpr int kRingBK = 32;
+constexpr int kRingLine = 64;  // bytes per row per stage
+
+__device__ __forceinline__ int ring_offset(int row, int chunk) {
+  return row * kRingLine + (((chunk ^ (row >> 1)) & 3) << 4);
+}
+
+// s_waitcnt with vmcnt = VM, lgkmcnt = 0 (expcnt left at its maximum).
+template <int VM>
+__device__ __forceinline__ void wait_vm_lgkm0() {
+  static_assert(VM >= 0 && VM < 64, "vmcnt is a 6-bit field");
+  __builtin_amdgcn_s_waitcnt((VM & 0xF) | (7 << 4) | (0 << 8) | ((VM >> 4) << 14));
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_BYTES = BM * kRingLine, B_BYTES = BN * kRingLine;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_GROUPS = BM / 16 / NW, B_GROUPS = BN / 16 / NW;  // 16-row (1 KiB) loads per wave
+  constexpr int PER_STAGE = A_GROUPS + B_GROUPS;
+  static_assert(A_GROUPS >= 1 && B_GROUPS >= 1 && BM % (16 * NW) == 0 && BN % (16 * NW) == 0,
+                "tile does not split into whole 1 KiB loads per wave");
+  __shared__ __attribute__((aligned(1024))) unsigned char st0[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char st1[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char st2[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char st3[STAGE_BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+  const int64_t m0 = static_cast<int64_t>(tile_m) * BM;
+  const int64_t n0 = static_cast<int64_t>(tile_n) * BN;
+  const int64_t batch = blockIdx.y;
+  const int64_t M = g.m, N = g.n;
+  T* __restrict__ C = static_cast<T*>(g.c) + batch * g.stride_c;
+  const unsigned char* a_base =
+      reinterpret_cast<const unsigned char*>(static_cast<const T*>(g.a) + batch * g.stride_a);
+  const unsigned char* b_base =
+      reinterpret_cast<const unsigned char*>(static_cast<const T*>(g.b) + batch * g.stride_b);
+
+  // Lane -> (row inside a 16-row load, LDS slot); the source chunk is slot ^ swizzle(row).
+  // Rows past the edge re-read the last valid row; their results are never stored.
+  const int r_in = lane >> 2, slot = lane & 3;
+  uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
+#pragma unroll
+  for (int j = 0; j < A_GROUPS; ++j) {
+    const int row = (wave * A_GROUPS + j) * 16 + r_in;
+    const int chunk = (slot ^ (row >> 1)) & 3;
+    int64_t grow = m0 + row;
+    grow = grow < M ? grow : M - 1;
+    a_off[j] = static_cast<uint32_t>((grow * g.lda + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int j = 0; j < B_GROUPS; ++j) {
+    const int row = (wave * B_GROUPS + j) * 16 + r_in;
+    const int chunk = (slot ^ (row >> 1)) & 3;
+    int64_t grow = n0 + row;
+    grow = grow < N ? grow : N - 1;
+    b_off[j] = static_cast<uint32_t>((grow * g.ldb + chunk * 8) * 2);
+  }
+
+  auto fetch_stage = [&](unsigned char* stage, int64_t k0) {
+#pragma unroll
+    for (int j = 0; j < A_GROUPS; ++j)
+      __builtin_amdgcn_global_load_lds(a_base + k0 * 2 + a_off[j],
+                                       (lds_void_t*)(stage + (wave * A_GROUPS + j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < B_GROUPS; ++j)
+      __builtin_amdgcn_global_load_lds(
+          b_base + k0 * 2 + b_off[j],
+          (lds_void_t*)(stage + A_BYTES + (wave * B_GROUPS + j) * 1024), 16, 0, 0);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  u32x4_t af[2][TM], bf[2][TN];
+  auto load_frags = [&](const unsigned char* stage, int ks, int s) {
+    const int chunk = ks * 2 + frag_half;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      af[s][i] = *reinterpret_cast<const u32x4_t*>(
+          stage + ring_offset(wm * WM + i * 32 + frag_row, chunk));
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      bf[s][j] = *reinterpret_cast<const u32x4_t*>(
+          stage + A_BYTES + ring_offset(wn * WN + j * 32 + frag_row, chunk));
+  };
+  auto mfma_step = [&](int s) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[s][j], af[s][i], acc[i][j]);
+  };
+
+  // One ring step. `cur` is multiplied (its first fragments are already in slot 0), `nxt`
+  // follows it, `pre` (multiplied in the previous step, so free) is refilled three stages ahead.
+  // ISSUE and INFLIGHT (stages younger than `nxt` that may still be in flight) are compile-time
+  // so that the loop body stays straight-line code: with run-time flags the register allocator
+  // starts moving accumulators between register files and spills.
+  auto step = [&](unsigned char* cur, unsigned char* nxt, unsigned char* pre, int64_t k_pre,
+                  auto issue_tag, auto inflight_tag) {
+    constexpr bool ISSUE = decltype(issue_tag)::value;
+    constexpr int INFLIGHT = decltype(inflight_tag)::value;
+    if constexpr (ISSUE) fetch_stage(pre, k_pre);
+    load_frags(cur, 1, 1);
+    mfma_step(0);
+    wait_vm_lgkm0<INFLIGHT * PER_STAGE>();
+    __builtin_amdgcn_s_barrier();
+    load_frags(nxt, 0, 0);
+    mfma_step(1);
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+
+  // The launcher guarantees k % 128 == 0 and k >= 128: a whole number of ring revolutions.
+  const int64_t k_tiles = g.k / kRingBK;
+  fetch_stage(st0, 0);
+  fetch_stage(st1, kRingBK);
+  fetch_stage(st2, 2 * kRingBK);
+  wait_vm_lgkm0<2 * PER_STAGE>();
+  __builtin_amdgcn_s_barrier();
+  load_frags(st0, 0, 0);
+  int64_t kt = 0;
+#pragma unroll 1
+  for (; kt + 4 < k_tiles; kt += 4) {
+    step(st0, st1, st3, (kt + 3) * kRingBK, Yes{}, I2{});
+    step(st1, st2, st0, (kt + 4) * kRingBK, Yes{}, I2{});
+    step(st2, st3, st1, (kt + 5) * kRingBK, Yes{}, I2{});
+    step(st3, st0, st2, (kt + 6) * kRingBK, Yes{}, I2{});
+  }
+  // last revolution: only its fourth stage is still to be requested
+  step(st0, st1, st3, (kt + 3) * kRingBK, Yes{}, I2{});
+  step(st1, st2, st0, 0, No{}, I1{});
+  step(st2, st3, st1, 0, No{}, I0{});
+  load_frags(st3, 1, 1);
+  mfma_step(0);
+  mfma_step(1);
+
+  const T* __restrict__ bias = static_cast<const T*>(g.bias);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = m0 + wm * WM + i * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int64_t col0 = n0 + wn * WN + j * 32 + 4 * (lane >> 5);
+      store_tile<T, EPI>(acc[i][j], C + (row < M ? row : 0) * g.ldc, row < M, col0, N, bias,
+                         g.vec_store != 0);
+    }
+  }
+#endif
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {
+  GemmArgs g = base;
+  g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
+  g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
+  g.vec_store = (g.ldc % 4 == 0) && (g.stride_c % 4 == 0 || batch == 1) &&
+                ((reinterpret_cast<uintptr_t>(g.c) & 7u) == 0);
+  const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
+  if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
+  gemm_ring_kernel<T, BM, BN, WAVES_M, WAVES_N, EPI>
+      <<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)),
+         dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
+  return check_launch();
+}
+
+}  // namespace tmb
