@@ -126,7 +126,7 @@ def main() -> int:
     achieved = flops / (ev_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_DENSE_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
-                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_mfma_kernel<bf16,256,256,N-major B>",
+                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_ring_kernel<bf16,256,256,2x4 waves,N-major B>",
                 "launch_ms": round(ev_ms, 4), "algorithmic_flops": flops}
 
     cpu_baseline = None

@@ -1,4 +1,5 @@
-// MFMA GEMM with direct-to-LDS loads for gfx950: A [M,K] and B [N,K] both K-major.
+// MFMA GEMM with direct-to-LDS loads for gfx950: A [M,K] K-major; B either [N,K] (K-major, the
+// transposed view of a weight) or [K,N] (N-major).
 //
 // global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS (lane l
 // of a wave lands at base + 16*l), so no staging registers and no ds_write instructions are
@@ -11,6 +12,12 @@
 // line XOR-swizzled with (row>>1)&3: ds_read_b128 fragment fetches of 8 consecutive rows then
 // touch 8 distinct 16-byte bank groups. The swizzle is applied on the global side: each lane
 // of a load picks the source chunk that belongs at its LDS slot.
+//
+// N-major B is staged as it lies in memory, [32 k][BN n], and its fragments are fetched with
+// ds_read_b64_tr_b16: sixteen lanes read a 4(k) x 16(n) block as 8-byte row pieces and get it
+// back transposed (lane = n, four consecutive k), which is the MFMA operand layout, so no
+// shuffle or repacking is spent on the transpose. Its 16-byte chunks are XOR-swizzled with
+// 4*(k%4), which spreads the four k-rows of such a block over distinct banks.
 //
 // The four stages are distinct __shared__ arrays and the ring is unrolled by hand, so that the
 // compiler can tell a stage being filled from the stage being read and does not serialise them.
@@ -38,7 +45,10 @@ __device__ __forceinline__ void wait_vm_lgkm0() {
   __builtin_amdgcn_s_waitcnt((VM & 0xF) | (7 << 4) | (0 << 8) | ((VM >> 4) << 14));
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NW = WAVES_M * WAVES_N;
@@ -83,12 +93,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   }
 #pragma unroll
   for (int j = 0; j < B_GROUPS; ++j) {
-    const int row = (wave * B_GROUPS + j) * 16 + r_in;
-    const int chunk = (slot ^ (row >> 1)) & 3;
-    int64_t grow = n0 + row;
-    grow = grow < N ? grow : N - 1;
-    b_off[j] = static_cast<uint32_t>((grow * g.ldb + chunk * 8) * 2);
+    if constexpr (B_KMAJOR) {
+      const int row = (wave * B_GROUPS + j) * 16 + r_in;
+      const int chunk = (slot ^ (row >> 1)) & 3;
+      int64_t grow = n0 + row;
+      grow = grow < N ? grow : N - 1;
+      b_off[j] = static_cast<uint32_t>((grow * g.ldb + chunk * 8) * 2);
+    } else {
+      // stage bytes [group*1024 + 16*lane] = k-row (BN*2 bytes each), swizzled 16-byte slot
+      const int at = (wave * B_GROUPS + j) * 1024 + lane * 16;
+      const int krow = at / (BN * 2);
+      const int chunk = ((at % (BN * 2)) >> 4) ^ ((krow & 3) << 2);
+      int64_t col = n0 + chunk * 8;
+      col = col < N ? col : n0;  // columns past the edge: any valid address, never stored
+      b_off[j] = static_cast<uint32_t>((krow * g.ldb + col) * 2);
+    }
   }
+  const int64_t b_kstep = B_KMAJOR ? 2 : g.ldb * 2;  // bytes per unit of k in B
 
   auto fetch_stage = [&](unsigned char* stage, int64_t k0) {
 #pragma unroll
@@ -98,7 +119,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 #pragma unroll
     for (int j = 0; j < B_GROUPS; ++j)
       __builtin_amdgcn_global_load_lds(
-          b_base + k0 * 2 + b_off[j],
+          b_base + k0 * b_kstep + b_off[j],
           (lds_void_t*)(stage + A_BYTES + (wave * B_GROUPS + j) * 1024), 16, 0, 0);
   };
 
@@ -111,6 +132,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   const int frag_row = lane & 31, frag_half = lane >> 5;
+  // N-major B: this lane's source piece of the transposed read. Within 16 lanes, lane j16 reads
+  // k-row j16/4 and the 4 columns starting at 4*(j16%4); lanes 16..31 take the next 16 columns
+  // and lanes 32..63 the upper eight k of the MFMA step.
+  int bt_off[TN];
+  if constexpr (!B_KMAJOR) {
+    const int j16 = lane & 15, q = j16 >> 2, nsub = (lane >> 4) & 1;
+    const int krow = frag_half * 8 + q;  // + 16*ks + 4*r, which leave krow % 4 == q
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int ncol = wn * WN + j * 32 + nsub * 16 + (j16 & 3) * 4;
+      bt_off[j] = A_BYTES + krow * (BN * 2) + (((ncol >> 3) ^ (q << 2)) << 4) + (ncol & 7) * 2;
+    }
+  }
   u32x4_t af[2][TM], bf[2][TN];
   auto load_frags = [&](const unsigned char* stage, int ks, int s) {
     const int chunk = ks * 2 + frag_half;
@@ -119,9 +153,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
       af[s][i] = *reinterpret_cast<const u32x4_t*>(
           stage + ring_offset(wm * WM + i * 32 + frag_row, chunk));
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-      bf[s][j] = *reinterpret_cast<const u32x4_t*>(
-          stage + A_BYTES + ring_offset(wn * WN + j * 32 + frag_row, chunk));
+    for (int j = 0; j < TN; ++j) {
+      if constexpr (B_KMAJOR) {
+        bf[s][j] = *reinterpret_cast<const u32x4_t*>(
+            stage + A_BYTES + ring_offset(wn * WN + j * 32 + frag_row, chunk));
+      } else {
+        const unsigned char* src = stage + bt_off[j] + ks * 16 * (BN * 2);
+        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
+        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src + 4 * (BN * 2)));
+        typedef short i16x8_t __attribute__((ext_vector_type(8)));
+        const i16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        bf[s][j] = __builtin_bit_cast(u32x4_t, both);
+      }
+    }
   };
   auto mfma_step = [&](int s) {
 #pragma unroll
@@ -191,7 +235,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 #endif
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
 static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
@@ -200,7 +244,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
                 ((reinterpret_cast<uintptr_t>(g.c) & 7u) == 0);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
-  gemm_ring_kernel<T, BM, BN, WAVES_M, WAVES_N, EPI>
+  gemm_ring_kernel<T, BM, BN, WAVES_M, WAVES_N, B_KMAJOR, EPI>
       <<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();
