@@ -9,9 +9,11 @@
 // stages), then one s_barrier makes every wave's part of that stage visible.
 //
 // LDS stage layout: 64-byte lines (32 K-values) per matrix row, the four 16-byte chunks of a
-// line XOR-swizzled with (row>>1)&3: ds_read_b128 fragment fetches of 8 consecutive rows then
-// touch 8 distinct 16-byte bank groups. The swizzle is applied on the global side: each lane
-// of a load picks the source chunk that belongs at its LDS slot.
+// line XOR-swizzled with (row>>2)&3: a ds_read_b128 is served sixteen lanes at a time from 64
+// banks (256 bytes), and the fragment fetch of 16 consecutive rows then touches 16 distinct
+// 16-byte bank groups (row%4 picks the line's quarter of the bank window, the swizzle the slot
+// inside it). The swizzle is applied on the global side: each lane of a load picks the source
+// chunk that belongs at its LDS slot.
 //
 // N-major B is staged as it lies in memory, [32 k][BN n], and its fragments are fetched with
 // ds_read_b64_tr_b16: sixteen lanes read a 4(k) x 16(n) block as 8-byte row pieces and get it
@@ -19,8 +21,8 @@
 // shuffle or repacking is spent on the transpose. Its 16-byte chunks are XOR-swizzled with
 // 4*(k%4), which spreads the four k-rows of such a block over distinct banks.
 //
-// The four stages are distinct __shared__ arrays and the ring is unrolled by hand, so that the
-// compiler can tell a stage being filled from the stage being read and does not serialise them.
+// The ring is unrolled by hand (stage indices are compile-time), so every fragment read is a
+// per-lane base register plus an immediate offset.
 #pragma once
 
 #include <type_traits>
@@ -35,7 +37,7 @@ constexpr int kRingBK = 32;
 constexpr int kRingLine = 64;  // bytes per row per stage
 
 __device__ __forceinline__ int ring_offset(int row, int chunk) {
-  return row * kRingLine + (((chunk ^ (row >> 1)) & 3) << 4);
+  return row * kRingLine + (((chunk ^ (row >> 2)) & 3) << 4);
 }
 
 // s_waitcnt with vmcnt = VM, lgkmcnt = 0 (expcnt left at its maximum).
@@ -60,10 +62,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   constexpr int PER_STAGE = A_GROUPS + B_GROUPS;
   static_assert(A_GROUPS >= 1 && B_GROUPS >= 1 && BM % (16 * NW) == 0 && BN % (16 * NW) == 0,
                 "tile does not split into whole 1 KiB loads per wave");
-  __shared__ __attribute__((aligned(1024))) unsigned char st0[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char st1[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char st2[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char st3[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[4 * STAGE_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -86,7 +85,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 #pragma unroll
   for (int j = 0; j < A_GROUPS; ++j) {
     const int row = (wave * A_GROUPS + j) * 16 + r_in;
-    const int chunk = (slot ^ (row >> 1)) & 3;
+    const int chunk = (slot ^ (row >> 2)) & 3;
     int64_t grow = m0 + row;
     grow = grow < M ? grow : M - 1;
     a_off[j] = static_cast<uint32_t>((grow * g.lda + chunk * 8) * 2);
@@ -95,7 +94,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   for (int j = 0; j < B_GROUPS; ++j) {
     if constexpr (B_KMAJOR) {
       const int row = (wave * B_GROUPS + j) * 16 + r_in;
-      const int chunk = (slot ^ (row >> 1)) & 3;
+      const int chunk = (slot ^ (row >> 2)) & 3;
       int64_t grow = n0 + row;
       grow = grow < N ? grow : N - 1;
       b_off[j] = static_cast<uint32_t>((grow * g.ldb + chunk * 8) * 2);
@@ -111,16 +110,30 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   }
   const int64_t b_kstep = B_KMAJOR ? 2 : g.ldb * 2;  // bytes per unit of k in B
 
-  auto fetch_stage = [&](unsigned char* stage, int64_t k0) {
+  // The loads are written as inline assembly: M0 carries the LDS destination of the wave's
+  // 1 KiB, the SGPR pair the tile's base at this k, the VGPR the lane's byte offset. Issued
+  // through the compiler's own builtin, every later LDS wait in the loop degrades to
+  // lgkmcnt(0) (it orders the DMA against all LDS traffic), which stalls each MFMA group on
+  // loads issued for the next one. The compiler does not see these loads at all, so the
+  // vmcnt waits below are placed by hand.
+  typedef __attribute__((address_space(3))) unsigned char lds_u8;
+  const uint32_t ring_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_u8*)ring));
+  const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const uint32_t a_m0 = ring_lds + wave_s * (A_GROUPS * 1024);
+  const uint32_t b_m0 = ring_lds + A_BYTES + wave_s * (B_GROUPS * 1024);
+  auto dma16 = [](uint32_t m0, uint32_t voff, const unsigned char* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0), "v"(voff), "s"(sbase)
+                 : "memory");
+  };
+  auto fetch_stage = [&](int stage, int64_t k0) {
+    const unsigned char* ak = a_base + k0 * 2;
+    const unsigned char* bk = b_base + k0 * b_kstep;
 #pragma unroll
-    for (int j = 0; j < A_GROUPS; ++j)
-      __builtin_amdgcn_global_load_lds(a_base + k0 * 2 + a_off[j],
-                                       (lds_void_t*)(stage + (wave * A_GROUPS + j) * 1024), 16, 0, 0);
+    for (int j = 0; j < A_GROUPS; ++j) dma16(a_m0 + stage * STAGE_BYTES + j * 1024, a_off[j], ak);
 #pragma unroll
-    for (int j = 0; j < B_GROUPS; ++j)
-      __builtin_amdgcn_global_load_lds(
-          b_base + k0 * b_kstep + b_off[j],
-          (lds_void_t*)(stage + A_BYTES + (wave * B_GROUPS + j) * 1024), 16, 0, 0);
+    for (int j = 0; j < B_GROUPS; ++j) dma16(b_m0 + stage * STAGE_BYTES + j * 1024, b_off[j], bk);
   };
 
   f32x16_t acc[TM][TN];
@@ -131,34 +144,45 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+  // Fragment addresses as LDS byte offsets inside a stage: one per-lane register per k-step
+  // (the XOR swizzle is not additive in the k chunk) and, for N-major B, per 32-column tile;
+  // everything else (stage, 32-row tile) is a compile-time offset the ds_read encodes itself.
+  // (row>>2)&3 does not change when a multiple of 32 rows is added, so one swizzle per lane.
   const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int frag_swz = (frag_row >> 2) & 3;
+  int a_lane[2], b_lane[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    const int slot16 = ((ks * 2 + frag_half) ^ frag_swz) << 4;
+    a_lane[ks] = (wm * WM + frag_row) * kRingLine + slot16;
+    b_lane[ks] = A_BYTES + (wn * WN + frag_row) * kRingLine + slot16;
+  }
   // N-major B: this lane's source piece of the transposed read. Within 16 lanes, lane j16 reads
   // k-row j16/4 and the 4 columns starting at 4*(j16%4); lanes 16..31 take the next 16 columns
   // and lanes 32..63 the upper eight k of the MFMA step.
-  int bt_off[TN];
+  int bt_lane[TN];
   if constexpr (!B_KMAJOR) {
     const int j16 = lane & 15, q = j16 >> 2, nsub = (lane >> 4) & 1;
     const int krow = frag_half * 8 + q;  // + 16*ks + 4*r, which leave krow % 4 == q
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int ncol = wn * WN + j * 32 + nsub * 16 + (j16 & 3) * 4;
-      bt_off[j] = A_BYTES + krow * (BN * 2) + (((ncol >> 3) ^ (q << 2)) << 4) + (ncol & 7) * 2;
+      bt_lane[j] = A_BYTES + krow * (BN * 2) + (((ncol >> 3) ^ (q << 2)) << 4) + (ncol & 7) * 2;
     }
   }
+  typedef __attribute__((address_space(3))) u32x4_t lds_u32x4_t;
   u32x4_t af[2][TM], bf[2][TN];
-  auto load_frags = [&](const unsigned char* stage, int ks, int s) {
-    const int chunk = ks * 2 + frag_half;
+  auto load_frags = [&](int stage_index, int ks, int s) {
+    lds_u8* stage = (lds_u8*)ring + stage_index * STAGE_BYTES;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      af[s][i] = *reinterpret_cast<const u32x4_t*>(
-          stage + ring_offset(wm * WM + i * 32 + frag_row, chunk));
+      af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (32 * kRingLine));
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if constexpr (B_KMAJOR) {
-        bf[s][j] = *reinterpret_cast<const u32x4_t*>(
-            stage + A_BYTES + ring_offset(wn * WN + j * 32 + frag_row, chunk));
+        bf[s][j] = *(const lds_u32x4_t*)(stage + b_lane[ks] + j * (32 * kRingLine));
       } else {
-        const unsigned char* src = stage + bt_off[j] + ks * 16 * (BN * 2);
+        lds_u8* src = stage + bt_lane[j] + ks * 16 * (BN * 2);
         const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
         const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src + 4 * (BN * 2)));
         typedef short i16x8_t __attribute__((ext_vector_type(8)));
@@ -179,17 +203,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   // ISSUE and INFLIGHT (stages younger than `nxt` that may still be in flight) are compile-time
   // so that the loop body stays straight-line code: with run-time flags the register allocator
   // starts moving accumulators between register files and spills.
-  auto step = [&](unsigned char* cur, unsigned char* nxt, unsigned char* pre, int64_t k_pre,
-                  auto issue_tag, auto inflight_tag) {
+  auto step = [&](int cur, int nxt, int pre, int64_t k_pre, auto issue_tag, auto inflight_tag) {
     constexpr bool ISSUE = decltype(issue_tag)::value;
     constexpr int INFLIGHT = decltype(inflight_tag)::value;
+    // sched_barrier(0): nothing is scheduled across. Left alone, the scheduler sinks each
+    // fragment load to just before its MFMA and reuses one register for all of them, which
+    // puts the LDS latency back on the critical path.
     if constexpr (ISSUE) fetch_stage(pre, k_pre);
     load_frags(cur, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
     mfma_step(0);
+    __builtin_amdgcn_sched_barrier(0);
     wait_vm_lgkm0<INFLIGHT * PER_STAGE>();
     __builtin_amdgcn_s_barrier();
     load_frags(nxt, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
     mfma_step(1);
+    __builtin_amdgcn_sched_barrier(0);
   };
   using Yes = std::true_type;
   using No = std::false_type;
@@ -199,25 +229,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 
   // The launcher guarantees k % 128 == 0 and k >= 128: a whole number of ring revolutions.
   const int64_t k_tiles = g.k / kRingBK;
-  fetch_stage(st0, 0);
-  fetch_stage(st1, kRingBK);
-  fetch_stage(st2, 2 * kRingBK);
+  fetch_stage(0, 0);
+  fetch_stage(1, kRingBK);
+  fetch_stage(2, 2 * kRingBK);
   wait_vm_lgkm0<2 * PER_STAGE>();
   __builtin_amdgcn_s_barrier();
-  load_frags(st0, 0, 0);
+  load_frags(0, 0, 0);
   int64_t kt = 0;
 #pragma unroll 1
   for (; kt + 4 < k_tiles; kt += 4) {
-    step(st0, st1, st3, (kt + 3) * kRingBK, Yes{}, I2{});
-    step(st1, st2, st0, (kt + 4) * kRingBK, Yes{}, I2{});
-    step(st2, st3, st1, (kt + 5) * kRingBK, Yes{}, I2{});
-    step(st3, st0, st2, (kt + 6) * kRingBK, Yes{}, I2{});
+    step(0, 1, 3, (kt + 3) * kRingBK, Yes{}, I2{});
+    step(1, 2, 0, (kt + 4) * kRingBK, Yes{}, I2{});
+    step(2, 3, 1, (kt + 5) * kRingBK, Yes{}, I2{});
+    step(3, 0, 2, (kt + 6) * kRingBK, Yes{}, I2{});
   }
   // last revolution: only its fourth stage is still to be requested
-  step(st0, st1, st3, (kt + 3) * kRingBK, Yes{}, I2{});
-  step(st1, st2, st0, 0, No{}, I1{});
-  step(st2, st3, st1, 0, No{}, I0{});
-  load_frags(st3, 1, 1);
+  step(0, 1, 3, (kt + 3) * kRingBK, Yes{}, I2{});
+  step(1, 2, 0, 0, No{}, I1{});
+  step(2, 3, 1, 0, No{}, I0{});
+  load_frags(3, 1, 1);
+  __builtin_amdgcn_sched_barrier(0);
   mfma_step(0);
   mfma_step(1);
 
