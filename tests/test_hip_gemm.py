@@ -125,10 +125,13 @@ def test_bmm(dtype):
     assert_close64(scores, as64(ref), rtol=2e-5, atol=1e-4, rounded_want=True, what="vs C oracle")
 
 
-# K-major B with K a multiple of 128 takes the direct-to-LDS kernel; the shapes are chosen so
-# that each of its tile sizes runs, with ragged M and N edges: 256x256 (256 tiles, one round of
-# the 256 CUs), 256x128 (528 tiles), 128x128 (few tiles), and a single K revolution (K = 128).
-KMAJOR = [(3900, 4000, 256), (4000, 4100, 256), (300, 1000, 384), (1000, 5000, 128), (130, 70, 1152)]
+# K >= 256 takes the direct-to-LDS ring kernel; the shapes are chosen so that each of its tile
+# configurations runs, with ragged M and N edges: 256x256 with 64-deep stages (256 tiles = one
+# round of the 256 CUs; K = 320 is five stages), 256x128 (528 tiles), 128x128 with 32-deep stages
+# (K = 352 is not a multiple of 64), and shapes that stay on the register-staged kernel
+# (few tiles, K < 256).
+KMAJOR = [(3900, 4000, 320), (4000, 4100, 256), (4000, 4104, 448), (600, 1000, 352),
+          (1000, 5000, 128), (130, 70, 1152)]
 
 
 @pytest.mark.parametrize("dtype", HALF)
@@ -150,11 +153,11 @@ def test_addmm_kmajor_b_tiles(mnk, dtype):
 
 
 def test_bmm_kmajor_b_direct_to_lds():
-    a = seeded((12, 300, 128), seed=1, dtype=torch.bfloat16)
-    b = seeded((12, 200, 128), seed=2, dtype=torch.bfloat16)
+    a = seeded((12, 300, 256), seed=1, dtype=torch.bfloat16)
+    b = seeded((12, 200, 256), seed=2, dtype=torch.bfloat16)
     got = _ops().gemm(_dev(a), _dev(b).transpose(1, 2))
     want = torch.bmm(a.double(), b.double().transpose(1, 2)).numpy()
-    assert_close64(got, want, rtol=2e-5, atol=1e-4, what="bmm K-major B, K=128")
+    assert_close64(got, want, rtol=2e-5, atol=1e-4, what="bmm K-major B, K=256")
     assert_close64(got, as64(oracle.gemm(a, b.transpose(1, 2))), rtol=2e-5, atol=1e-4,
                    rounded_want=True, what="vs C oracle")
 

@@ -101,18 +101,22 @@ __global__ __launch_bounds__(256) void gemm_simt_kernel(
 template <typename T, bool B_KMAJOR, int EPI>
 static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) {
   auto tiles = [&](int64_t bm, int64_t bn) { return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn) * batch; };
-  // K a whole number of ring revolutions: direct-to-LDS kernel. 256x256 (8 waves) has the best
-  // steady state; it is used when its tiles fill the 256 CUs in nearly whole rounds, otherwise
-  // smaller tiles cut the idle tail. N-major B is staged in whole 16-byte column chunks, so N
-  // must be a multiple of 8 there (nothing past column N-1 is ever read).
-  if (g.k % 128 == 0 && g.n > 64 && (B_KMAJOR || g.n % 8 == 0)) {
-    const int64_t t256 = tiles(256, 256);
-    const int64_t rounds = (t256 + 255) / 256;
-    if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9)
-      return launch_ring<T, 256, 256, 2, 4, B_KMAJOR, EPI>(g, batch, stream);
-    if (B_KMAJOR && tiles(256, 128) >= 512)
-      return launch_ring<T, 256, 128, 4, 2, B_KMAJOR, EPI>(g, batch, stream);
-    if (tiles(128, 128) >= 32) return launch_ring<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  // Direct-to-LDS ring kernel for long enough K. 256x256 (8 waves, 64-deep stages: every row
+  // of a K-major operand is fetched as one whole 128-byte line) has the best steady state; it
+  // is used when its tiles fill the 256 CUs in nearly whole rounds, otherwise smaller tiles cut
+  // the idle tail. N-major B is staged in whole 16-byte column chunks, so N must be a multiple
+  // of 8 there (nothing past column N-1 is ever read).
+  if (g.k >= 256 && g.n > 64 && (B_KMAJOR || g.n % 8 == 0)) {
+    if (g.k % 64 == 0) {
+      const int64_t t256 = tiles(256, 256);
+      const int64_t rounds = (t256 + 255) / 256;
+      if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9)
+        return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI>(g, batch, stream);
+      if (tiles(256, 128) >= 512)
+        return launch_ring<T, 256, 128, 64, 4, 2, 3, B_KMAJOR, EPI>(g, batch, stream);
+    }
+    if (g.k % 32 == 0 && tiles(128, 128) >= 32)
+      return launch_ring<T, 128, 128, 32, 2, 2, 4, B_KMAJOR, EPI>(g, batch, stream);
   }
   if (g.n <= 64) return launch_mfma<T, 256, 64, 4, 1, B_KMAJOR, EPI>(g, batch, stream);
   if (g.k <= 128) return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);

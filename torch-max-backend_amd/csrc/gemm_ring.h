@@ -26,6 +26,7 @@
 #pragma once
 
 #include <type_traits>
+#include <utility>
 
 #include "gemm_mfma.h"
 
@@ -33,11 +34,23 @@ namespace tmb {
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-constexpr int kRingBK = 32;
-constexpr int kRingLine = 64;  // bytes per row per stage
+// XOR swizzle of the 16-byte chunks of a K-major LDS line of LINE bytes (64 or 128). A
+// ds_read_b128 is served sixteen lanes at a time from 64 banks (a 256-byte window); 256/LINE
+// consecutive rows share a window, so the swizzle must differ between rows that are a multiple
+// of 256/LINE apart: (row / (256/LINE)) mod (LINE/16). Adding 32 rows leaves it unchanged.
+template <int LINE>
+__device__ __forceinline__ int ring_swizzle(int row) {
+  return (row / (256 / LINE)) & (LINE / 16 - 1);
+}
 
-__device__ __forceinline__ int ring_offset(int row, int chunk) {
-  return row * kRingLine + (((chunk ^ (row >> 2)) & 3) << 4);
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), unrolled at compile time.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
 // s_waitcnt with vmcnt = VM, lgkmcnt = 0 (expcnt left at its maximum).
@@ -50,19 +63,26 @@ __device__ __forceinline__ void wait_vm_lgkm0() {
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int A_BYTES = BM * kRingLine, B_BYTES = BN * kRingLine;
+  constexpr int LINE = BK * 2;         // bytes of one row of a K-major operand per stage
+  constexpr int KSTEPS = BK / 16;      // MFMA k-steps per stage
+  constexpr int LPR = LINE / 16;       // lanes (16-byte chunks) per row of a load
+  constexpr int RPG = 1024 / LINE;     // rows per 1 KiB load
+  constexpr int A_BYTES = BM * LINE, B_BYTES = BN * LINE;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int A_GROUPS = BM / 16 / NW, B_GROUPS = BN / 16 / NW;  // 16-row (1 KiB) loads per wave
+  constexpr int A_GROUPS = A_BYTES / 1024 / NW, B_GROUPS = B_BYTES / 1024 / NW;  // loads per wave
   constexpr int PER_STAGE = A_GROUPS + B_GROUPS;
-  static_assert(A_GROUPS >= 1 && B_GROUPS >= 1 && BM % (16 * NW) == 0 && BN % (16 * NW) == 0,
+  static_assert(BK == 32 || BK == 64, "a stage is 32 or 64 deep");
+  static_assert(R >= 2 && R * STAGE_BYTES <= 160 * 1024, "ring does not fit the 160 KB LDS");
+  static_assert(A_GROUPS >= 1 && B_GROUPS >= 1 && A_BYTES % (1024 * NW) == 0 &&
+                    B_BYTES % (1024 * NW) == 0,
                 "tile does not split into whole 1 KiB loads per wave");
-  __shared__ __attribute__((aligned(1024))) unsigned char ring[4 * STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[R * STAGE_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -78,14 +98,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   const unsigned char* b_base =
       reinterpret_cast<const unsigned char*>(static_cast<const T*>(g.b) + batch * g.stride_b);
 
-  // Lane -> (row inside a 16-row load, LDS slot); the source chunk is slot ^ swizzle(row).
+  // Lane -> (row inside a 1 KiB load, LDS slot); the source chunk is slot ^ swizzle(row).
   // Rows past the edge re-read the last valid row; their results are never stored.
-  const int r_in = lane >> 2, slot = lane & 3;
+  const int r_in = lane / LPR, slot = lane % LPR;
   uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
 #pragma unroll
   for (int j = 0; j < A_GROUPS; ++j) {
-    const int row = (wave * A_GROUPS + j) * 16 + r_in;
-    const int chunk = (slot ^ (row >> 2)) & 3;
+    const int row = (wave * A_GROUPS + j) * RPG + r_in;
+    const int chunk = slot ^ ring_swizzle<LINE>(row);
     int64_t grow = m0 + row;
     grow = grow < M ? grow : M - 1;
     a_off[j] = static_cast<uint32_t>((grow * g.lda + chunk * 8) * 2);
@@ -93,8 +113,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 #pragma unroll
   for (int j = 0; j < B_GROUPS; ++j) {
     if constexpr (B_KMAJOR) {
-      const int row = (wave * B_GROUPS + j) * 16 + r_in;
-      const int chunk = (slot ^ (row >> 2)) & 3;
+      const int row = (wave * B_GROUPS + j) * RPG + r_in;
+      const int chunk = slot ^ ring_swizzle<LINE>(row);
       int64_t grow = n0 + row;
       grow = grow < N ? grow : N - 1;
       b_off[j] = static_cast<uint32_t>((grow * g.ldb + chunk * 8) * 2);
@@ -127,13 +147,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
                  : "s"(m0), "v"(voff), "s"(sbase)
                  : "memory");
   };
-  auto fetch_stage = [&](int stage, int64_t k0) {
+  auto fetch_stage = [&](uint32_t stage_off, int64_t k0) {
     const unsigned char* ak = a_base + k0 * 2;
     const unsigned char* bk = b_base + k0 * b_kstep;
 #pragma unroll
-    for (int j = 0; j < A_GROUPS; ++j) dma16(a_m0 + stage * STAGE_BYTES + j * 1024, a_off[j], ak);
+    for (int j = 0; j < A_GROUPS; ++j) dma16(a_m0 + stage_off + j * 1024, a_off[j], ak);
 #pragma unroll
-    for (int j = 0; j < B_GROUPS; ++j) dma16(b_m0 + stage * STAGE_BYTES + j * 1024, b_off[j], bk);
+    for (int j = 0; j < B_GROUPS; ++j) dma16(b_m0 + stage_off + j * 1024, b_off[j], bk);
   };
 
   f32x16_t acc[TM][TN];
@@ -146,16 +166,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 
   // Fragment addresses as LDS byte offsets inside a stage: one per-lane register per k-step
   // (the XOR swizzle is not additive in the k chunk) and, for N-major B, per 32-column tile;
-  // everything else (stage, 32-row tile) is a compile-time offset the ds_read encodes itself.
-  // (row>>2)&3 does not change when a multiple of 32 rows is added, so one swizzle per lane.
+  // the 32-row tile index (and the k-step of N-major B) is an immediate offset of the ds_read.
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  const int frag_swz = (frag_row >> 2) & 3;
-  int a_lane[2], b_lane[2];
+  const int frag_swz = ring_swizzle<LINE>(frag_row);
+  int a_lane[KSTEPS], b_lane[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
+  for (int ks = 0; ks < KSTEPS; ++ks) {
     const int slot16 = ((ks * 2 + frag_half) ^ frag_swz) << 4;
-    a_lane[ks] = (wm * WM + frag_row) * kRingLine + slot16;
-    b_lane[ks] = A_BYTES + (wn * WN + frag_row) * kRingLine + slot16;
+    a_lane[ks] = (wm * WM + frag_row) * LINE + slot16;
+    b_lane[ks] = A_BYTES + (wn * WN + frag_row) * LINE + slot16;
   }
   // N-major B: this lane's source piece of the transposed read. Within 16 lanes, lane j16 reads
   // k-row j16/4 and the 4 columns starting at 4*(j16%4); lanes 16..31 take the next 16 columns
@@ -172,15 +191,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   }
   typedef __attribute__((address_space(3))) u32x4_t lds_u32x4_t;
   u32x4_t af[2][TM], bf[2][TN];
-  auto load_frags = [&](int stage_index, int ks, int s) {
-    lds_u8* stage = (lds_u8*)ring + stage_index * STAGE_BYTES;
+  // ks is a compile-time constant at every call site (the k-step loop is unrolled).
+  auto load_frags = [&](uint32_t stage_off, int ks, int s) {
+    lds_u8* stage = (lds_u8*)ring + stage_off;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (32 * kRingLine));
+      af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (32 * LINE));
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if constexpr (B_KMAJOR) {
-        bf[s][j] = *(const lds_u32x4_t*)(stage + b_lane[ks] + j * (32 * kRingLine));
+        bf[s][j] = *(const lds_u32x4_t*)(stage + b_lane[ks] + j * (32 * LINE));
       } else {
         lds_u8* src = stage + bt_lane[j] + ks * 16 * (BN * 2);
         const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
@@ -198,59 +218,75 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
       for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[s][j], af[s][i], acc[i][j]);
   };
 
-  // One ring step. `cur` is multiplied (its first fragments are already in slot 0), `nxt`
-  // follows it, `pre` (multiplied in the previous step, so free) is refilled three stages ahead.
-  // ISSUE and INFLIGHT (stages younger than `nxt` that may still be in flight) are compile-time
-  // so that the loop body stays straight-line code: with run-time flags the register allocator
-  // starts moving accumulators between register files and spills.
-  auto step = [&](int cur, int nxt, int pre, int64_t k_pre, auto issue_tag, auto inflight_tag) {
+  // Ring position as a byte offset that lives in an SGPR (every wave computes the same value).
+  auto next_stage = [](uint32_t off) {
+    return off + STAGE_BYTES == R * STAGE_BYTES ? 0u : off + STAGE_BYTES;
+  };
+
+  // One ring step: tile t sits in stage `cur` with its first fragments already in slot 0; the
+  // stage before `cur` was multiplied in the previous step and is refilled with tile t+R-1.
+  // INFLIGHT = tiles younger than t+1 whose loads may still be outstanding when t+1 is waited
+  // for. sched_barrier(0): nothing is scheduled across. Left alone, the scheduler sinks each
+  // fragment load to just before its MFMA and reuses one register for all of them, which puts
+  // the LDS latency back on the critical path.
+  auto step = [&](uint32_t cur, uint32_t nxt, uint32_t pre, int64_t k_pre, auto issue_tag,
+                  auto inflight_tag) {
     constexpr bool ISSUE = decltype(issue_tag)::value;
     constexpr int INFLIGHT = decltype(inflight_tag)::value;
-    // sched_barrier(0): nothing is scheduled across. Left alone, the scheduler sinks each
-    // fragment load to just before its MFMA and reuses one register for all of them, which
-    // puts the LDS latency back on the critical path.
     if constexpr (ISSUE) fetch_stage(pre, k_pre);
-    load_frags(cur, 1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_step(0);
-    __builtin_amdgcn_sched_barrier(0);
+    static_for<KSTEPS - 1>([&](auto ks_tag) {
+      constexpr int ks = decltype(ks_tag)::value;
+      load_frags(cur, ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step(ks & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    });
     wait_vm_lgkm0<INFLIGHT * PER_STAGE>();
     __builtin_amdgcn_s_barrier();
     load_frags(nxt, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step(1);
+    mfma_step((KSTEPS - 1) & 1);
     __builtin_amdgcn_sched_barrier(0);
   };
-  using Yes = std::true_type;
-  using No = std::false_type;
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
 
-  // The launcher guarantees k % 128 == 0 and k >= 128: a whole number of ring revolutions.
-  const int64_t k_tiles = g.k / kRingBK;
-  fetch_stage(0, 0);
-  fetch_stage(1, kRingBK);
-  fetch_stage(2, 2 * kRingBK);
-  wait_vm_lgkm0<2 * PER_STAGE>();
+  // The launcher guarantees k % BK == 0 and at least R-1 stages of k.
+  const int64_t k_tiles = g.k / BK;
+  {
+    uint32_t off = 0;
+#pragma unroll
+    for (int t = 0; t < R - 1; ++t) {
+      fetch_stage(off, t * BK);
+      off += STAGE_BYTES;
+    }
+  }
+  wait_vm_lgkm0<(R - 2) * PER_STAGE>();
   __builtin_amdgcn_s_barrier();
   load_frags(0, 0, 0);
-  int64_t kt = 0;
+  uint32_t cur = 0, pre = (R - 1) * STAGE_BYTES;
+  // main part: every step also requests tile t+R-1
 #pragma unroll 1
-  for (; kt + 4 < k_tiles; kt += 4) {
-    step(0, 1, 3, (kt + 3) * kRingBK, Yes{}, I2{});
-    step(1, 2, 0, (kt + 4) * kRingBK, Yes{}, I2{});
-    step(2, 3, 1, (kt + 5) * kRingBK, Yes{}, I2{});
-    step(3, 0, 2, (kt + 6) * kRingBK, Yes{}, I2{});
+  for (int64_t t = 0; t + (R - 1) < k_tiles; ++t) {
+    const uint32_t nxt = next_stage(cur);
+    step(cur, nxt, pre, (t + (R - 1)) * BK, std::true_type{},
+         std::integral_constant<int, R - 2>{});
+    pre = cur;
+    cur = nxt;
   }
-  // last revolution: only its fourth stage is still to be requested
-  step(0, 1, 3, (kt + 3) * kRingBK, Yes{}, I2{});
-  step(1, 2, 0, 0, No{}, I1{});
-  step(2, 3, 1, 0, No{}, I0{});
-  load_frags(3, 1, 1);
-  __builtin_amdgcn_sched_barrier(0);
-  mfma_step(0);
-  mfma_step(1);
+  // the last R-1 tiles are already in flight or resident; the in-flight count runs down
+  static_for<R - 2>([&](auto s) {
+    const uint32_t nxt = next_stage(cur);
+    step(cur, nxt, pre, 0, std::false_type{}, std::integral_constant<int, R - 3 - decltype(s)::value>{});
+    pre = cur;
+    cur = nxt;
+  });
+  static_for<KSTEPS - 1>([&](auto ks_tag) {
+    constexpr int ks = decltype(ks_tag)::value;
+    load_frags(cur, ks + 1, (ks + 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(ks & 1);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+  mfma_step((KSTEPS - 1) & 1);
 
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
 #pragma unroll
@@ -266,7 +302,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
 #endif
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
 static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
@@ -275,7 +311,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
                 ((reinterpret_cast<uintptr_t>(g.c) & 7u) == 0);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
-  gemm_ring_kernel<T, BM, BN, WAVES_M, WAVES_N, B_KMAJOR, EPI>
+  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI>
       <<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();
