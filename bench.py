@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot-op kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|gpt2|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|gpt2|copy|all]
 
 Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
@@ -37,10 +37,10 @@ sys.path.insert(0, os.path.join(ROOT, "torch-max-backend_amd"))
 PEAK_BF16_DENSE_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 
-# HBM bytes per launch of the headline GEMM kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE + WRITE_SIZE, scaled by the same counters on tmb_copy_bytes); None until the
-# counter runs summarised under profiles/ exist for the current kernel.
-GEMM_TRAFFIC_BYTES = None
+# Bytes per launch of the headline GEMM kernel between L2 and the memory side, measured with
+# rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the factors being what the same
+# counters read for tmb_copy_bytes moving 1 GiB: `--only copy`).
+GEMM_TRAFFIC_BYTES = 1.879e9
 
 
 def _parse():
@@ -48,7 +48,7 @@ def _parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "gpt2"])
+    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "gpt2", "copy"])
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return p.parse_args()
 
@@ -115,6 +115,20 @@ def main() -> int:
     sweep = {}
     want = args.only
 
+    if want == "copy":
+        # Calibration workload for the HBM counters: tmb_copy_bytes moves exactly 1 GiB in and
+        # 1 GiB out per launch, so FETCH_SIZE / WRITE_SIZE of this kernel give the counters'
+        # scale. Not a bench line.
+        nbytes = 1 << 30
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        wall_ms, ev_ms = timed(lambda: hip_ops.copy_bytes(dst, src), args.steps, args.warmup)
+        assert torch.equal(dst, src)
+        print(json.dumps({"workload": "tmb_copy_bytes 1 GiB", "bytes_read": nbytes,
+                          "bytes_written": nbytes, "launch_ms": round(ev_ms, 4),
+                          "GB/s": round(2 * nbytes / (ev_ms * 1e-3) / 1e9, 1)}))
+        return 0
+
     # ------------------------------------------------------------------ GEMM (headline)
     M = N = K = 8192
     a = gen((M, K), 0, torch.bfloat16)
@@ -126,7 +140,7 @@ def main() -> int:
     achieved = flops / (ev_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_DENSE_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
-                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_ring_kernel<bf16,256,256,2x4 waves,N-major B>",
+                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_ring_kernel<bf16,256x256x64,2x4 waves,2 stages,N-major B>",
                 "launch_ms": round(ev_ms, 4), "algorithmic_flops": flops}
 
     cpu_baseline = None
