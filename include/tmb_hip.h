@@ -61,6 +61,17 @@ const char* tmb_status_string(int code);
 int tmb_softmax_rows(void* out, const void* in, int64_t rows, int64_t cols, int in_dtype,
                      int out_dtype, int log_mode, void* stream);
 
+/* Attention form of the row softmax: y = softmax_j(x[r][j] * scale), and with q_len > 0 only
+ * columns j <= r % q_len take part (causal mask of a [.., q_len, cols] score tensor flattened
+ * to rows); the masked columns are written as exact zeros and their input is not read.
+ * `round_scaled` != 0 rounds x*scale to `dtype` before the max, i.e. reproduces the bits of a
+ * separate `mul` kernel followed by masked_fill(-inf) and softmax. `dtype` in {F32,F16,BF16},
+ * output of the same type.
+ * Replaces nn_ops.mojo:413-493 (`_softmax_rows(scale, causal, q_len)`: m = max(x*scale),
+ * denom = sum exp(x*scale - m), causal zeroes j > r % q_len). */
+int tmb_softmax_rows_scaled(void* out, const void* in, int64_t rows, int64_t cols, int dtype,
+                            float scale, int round_scaled, int64_t q_len, void* stream);
+
 /* Layer norm over the last dimension of [rows, cols]: two-pass fp32 statistics
  * (mean = sum(x)/cols, var = sum((x-mean)^2)/cols biased, rstd = 1/sqrt(var+eps)),
  * out = (x-mean)*rstd*gamma + beta cast once. `gamma`/`beta` may be NULL (no affine);

@@ -68,6 +68,8 @@ def lib() -> ctypes.CDLL:
         i64, vp, ci, dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_double
         L.orc_gemm.argtypes = [vp, vp, vp, vp] + [i64] * 10 + [ci] * 4
         L.orc_softmax.argtypes = [vp, vp, i64, i64, ci, ci, ci]
+        L.orc_softmax_scaled.argtypes = [vp, vp, i64, i64, ci, ctypes.c_float, ci, i64]
+        L.orc_softmax_scaled.restype = ci
         L.orc_layer_norm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ci]
         L.orc_reduce.argtypes = [vp, vp, i64, i64, ci, ci]
         L.orc_argmax.argtypes = [vp, vp, i64, i64, ci]
@@ -156,6 +158,19 @@ def softmax_rows(x: torch.Tensor, *, log: bool = False,
     if x.numel():
         _check(lib().orc_softmax(out.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1],
                                  _code(x.dtype), _code(out.dtype), int(log)), "softmax")
+    return out
+
+
+def softmax_scaled(x: torch.Tensor, scale: float, causal_q_len: int = 0,
+                   round_scaled: bool = False) -> torch.Tensor:
+    """softmax(x*scale) over the last dim; rows are flattened, causal rows keep j <= r % q_len."""
+    x = _cpu(x).contiguous()
+    out = torch.empty_like(x)
+    cols = x.shape[-1]
+    if x.numel():
+        _check(lib().orc_softmax_scaled(out.data_ptr(), x.data_ptr(), x.numel() // cols, cols,
+                                        _code(x.dtype), float(scale), int(bool(round_scaled)),
+                                        int(causal_q_len)), "softmax_scaled")
     return out
 
 

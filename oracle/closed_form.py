@@ -16,6 +16,17 @@ def softmax(x: np.ndarray, axis: int = -1) -> np.ndarray:
     return e / e.sum(axis=axis, keepdims=True)
 
 
+def softmax_scaled_causal(x: np.ndarray, scale: float, causal: bool) -> np.ndarray:
+    """float64 softmax(x*scale) over the last axis of [..., q, cols]; causal keeps j <= query row."""
+    z = x.astype(np.float64) * scale
+    if causal:
+        q, cols = z.shape[-2], z.shape[-1]
+        keep = np.arange(cols)[None, :] <= np.arange(q)[:, None]
+        z = np.where(keep, z, -np.inf)
+    e = np.exp(z - z.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
 def log_softmax(x: np.ndarray, axis: int = -1) -> np.ndarray:
     x = x.astype(np.float64)
     s = x - x.max(axis=axis, keepdims=True)

@@ -9,6 +9,8 @@
  *                                               bias added in fp32, one cast) and :2651-2657
  *   orc_softmax     nn_ops.mojo:428-455        (max, sum of exp(x-m), exp(x-m)/denom; fp32)
  *                   reduction_ops.mojo:874-895 (log-softmax: x - m - log(denom))
+ *   orc_softmax_scaled nn_ops.mojo:413-493     (`_softmax_rows(scale, causal, q_len)`: x*scale, causal
+ *                                               rows keep j <= r % q_len, the rest is zero)
  *   orc_layer_norm  nn_ops.mojo:299-326        (two-pass mean / centered variance, fp32) with the
  *                                               NaN-mean rule of normalization_forward_kernels.mojo:60-70
  *   orc_reduce      reduction_ops.mojo:161-194 (fp32 accumulator for floats, own type for ints,
@@ -153,6 +155,41 @@ int orc_softmax(void* out, const void* in, int64_t rows, int64_t cols, int in_dt
     } else {
       for (int64_t j = 0; j < cols; ++j)
         store_f(out, base + j, out_dtype, expf(load_f(in, base + j, in_dtype) - m) / denom);
+    }
+  }
+  return 0;
+}
+
+/* Attention softmax: y = softmax_j(x*scale) over the columns j <= r % q_len (all columns when
+ * q_len == 0); masked columns give 0. round_scaled rounds x*scale to the storage type first
+ * (the value a separate mul would have stored). */
+int orc_softmax_scaled(void* out, const void* in, int64_t rows, int64_t cols, int dtype,
+                       float scale, int round_scaled, int64_t q_len) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * cols;
+    const int64_t last = q_len > 0 ? r % q_len : cols - 1;
+    float m = -INFINITY;
+    for (int64_t j = 0; j <= last && j < cols; ++j) {
+      float x = load_f(in, base + j, dtype) * scale;
+      if (round_scaled) { store_f(out, base + j, dtype, x); x = load_f(out, base + j, dtype); }
+      if (x > m) m = x;
+      if (x != x) m = x;
+    }
+    float denom = 0.0f;
+    for (int64_t j = 0; j <= last && j < cols; ++j) {
+      float x = load_f(in, base + j, dtype) * scale;
+      if (round_scaled) { store_f(out, base + j, dtype, x); x = load_f(out, base + j, dtype); }
+      denom += expf(x - m);
+    }
+    for (int64_t j = 0; j < cols; ++j) {
+      float y = 0.0f;
+      if (j <= last) {
+        float x = load_f(in, base + j, dtype) * scale;
+        if (round_scaled) { store_f(out, base + j, dtype, x); x = load_f(out, base + j, dtype); }
+        y = expf(x - m) / denom;
+      }
+      store_f(out, base + j, dtype, y);
     }
   }
   return 0;

@@ -196,3 +196,80 @@ def test_intermediates_are_released_after_their_last_use():
     # both products and the input are dropped once the add has run; the result is kept
     assert sorted(released) == [0, 1, 2]
     assert program.steps[-1].out not in released
+
+
+class _Attn(torch.nn.Module):
+    """Score pipeline of a decoder block, as demo_scripts/gpt2.py writes it."""
+
+    def __init__(self, block=16, causal=True):
+        super().__init__()
+        mask = torch.tril(torch.ones(block, block)) if causal else (torch.rand(block, block) > 0.3).float()
+        mask[:, 0] = 1.0  # no fully masked row
+        self.register_buffer("bias", mask.view(1, 1, block, block), persistent=False)
+
+    def forward(self, q, k):
+        t = q.shape[-2]
+        att = (q @ k.transpose(-2, -1)) * 0.25
+        att = att.masked_fill(self.bias[:, :, :t, :t] == 0, float("-inf"))
+        return torch.softmax(att, dim=-1)
+
+
+def test_masked_softmax_rewrite_plans_one_fused_step(cpu_hot_ops, monkeypatch):
+    monkeypatch.setattr(compiler, "_BUILTIN_SOFTMAX", MAPPING_TORCH_ATEN_TO_MOJO[aten._softmax])
+    programs = []
+    real = compiler._GraphFactory.create_graph
+
+    def spy(self, graph):
+        programs.append(real(self, graph))
+        return programs[-1]
+
+    monkeypatch.setattr(compiler._GraphFactory, "create_graph", spy)
+    model = _Attn().eval()
+    q, k = torch.randn(2, 3, 8, 4), torch.randn(2, 3, 8, 4)
+    with torch.no_grad():
+        want = model(q, k)
+        got = torch.compile(model, backend=mojo_backend, fullgraph=True)(q, k)
+    # host tensors take the unfused branch inside the fused step: same numbers as eager
+    torch.testing.assert_close(got, want)
+    program = programs[-1]
+    names = [compiler._step_name(s) for s in program.steps]
+    assert names.count("aten.mul+masked_fill+_softmax (fused)") == 1
+    fused = next(s for s in program.steps if s.fn is compiler._FUSED_MASKED_SOFTMAX)
+    skipped = {str(s.node.target) for s in program.steps if s.fn is compiler._skipped}
+    assert {"aten.mul.Tensor", "aten.masked_fill.Scalar", "aten.eq.Scalar",
+            "aten.slice.Tensor"} <= skipped
+    assert fused.args[1] == 0.25 and fused.args[3] == ((2, 0, 8, 1), (3, 0, 8, 1))
+    # the scores stay alive until the fused step has read them, then go
+    scores_slot = fused.args[0].index
+    assert scores_slot in fused.release
+    for s in program.steps:
+        if s is not fused:
+            assert scores_slot not in s.release
+
+
+def test_masked_softmax_rewrite_leaves_other_patterns_alone(cpu_hot_ops, monkeypatch):
+    monkeypatch.setattr(compiler, "_BUILTIN_SOFTMAX", MAPPING_TORCH_ATEN_TO_MOJO[aten._softmax])
+
+    def shared_product(q, k, mask):
+        att = (q @ k.transpose(-2, -1)) * 0.5
+        return torch.softmax(att.masked_fill(mask == 0, float("-inf")), dim=-1), att  # mul has 2 users
+
+    def finite_fill(q, k, mask):
+        att = (q @ k.transpose(-2, -1)) * 0.5
+        return torch.softmax(att.masked_fill(mask == 0, -1e9), dim=-1)
+
+    q, k = torch.randn(2, 6, 4), torch.randn(2, 6, 4)
+    mask = torch.tril(torch.ones(6, 6))
+    for fn in (shared_product, finite_fill):
+        want = fn(q, k, mask)
+        got = torch.compile(fn, backend=mojo_backend, fullgraph=True)(q, k, mask)
+        torch.testing.assert_close(got, want)
+        torch.compiler.reset()
+    assert cpu_hot_ops.count("_softmax") == 2
+
+
+def test_causal_verdict_is_cached_and_follows_the_buffer():
+    mask = torch.tril(torch.ones(1, 1, 8, 8))
+    x = torch.zeros(2, 2, 8, 8)
+    # host tensors never qualify (the fused kernel is a device kernel)
+    assert compiler._causal_q_len(mask, ((2, 0, 8, 1), (3, 0, 8, 1)), x) == 0

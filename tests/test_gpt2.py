@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+from helpers import seeded
 
 pytestmark = pytest.mark.gpu
 
@@ -36,7 +37,8 @@ def test_gpt2_small_fp32_batch1_seq128_matches_cpu_eager():
     # (c_fc's addmm and its gelu are one fused kernel: 12 of the 48 addmm run through it)
     assert after["aten_addmm"] - before["aten_addmm"] == 36
     assert after["aten_bmm"] - before["aten_bmm"] == 24
-    assert after["aten__softmax"] - before["aten__softmax"] == 12
+    # mul + masked_fill + _softmax run as one fused step that launches the kernel directly
+    assert after["aten__softmax"] - before["aten__softmax"] == 0
     assert after["aten_native_layer_norm"] - before["aten_native_layer_norm"] == 25
     assert after["aten_mm"] - before["aten_mm"] == 1
     assert after["aten_argmax"] - before["aten_argmax"] == 1
@@ -97,3 +99,65 @@ def test_fusion_is_bit_identical_to_unfused(monkeypatch):
     with torch.no_grad():
         unfused, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
     assert torch.equal(fused, unfused)
+
+
+class _Scores(torch.nn.Module):
+    def __init__(self, block, causal):
+        super().__init__()
+        mask = torch.tril(torch.ones(block, block))
+        if not causal:
+            mask = (torch.rand(block, block, generator=torch.Generator().manual_seed(3)) > 0.4).float()
+            mask[:, 0] = 1.0
+        self.register_buffer("bias", mask.view(1, 1, block, block), persistent=False)
+
+    def forward(self, q, k):
+        t = q.shape[-2]
+        att = (q @ k.transpose(-2, -1)) * (1.0 / 8.0)
+        att = att.masked_fill(self.bias[:, :, :t, :t] == 0, float("-inf"))
+        return torch.softmax(att, dim=-1)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_masked_softmax_fusion_on_device(causal, monkeypatch):
+    """Causal buffer -> one fused kernel; any other mask -> the unfused ops inside the same
+    step. Either way the result has the bits of the unfused graph."""
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    model = _Scores(128, causal).to("cuda").eval()
+    q = seeded((2, 4, 96, 64), seed=1, dtype=torch.bfloat16).to("cuda")
+    k = seeded((2, 4, 96, 64), seed=2, dtype=torch.bfloat16).to("cuda")
+    calls = []
+    real = compiler.aten_functions.hip_ops.softmax_scaled
+    monkeypatch.setattr(compiler.aten_functions.hip_ops, "softmax_scaled",
+                        lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    with torch.no_grad():
+        fused = torch.compile(model, backend=mojo_backend, fullgraph=True)(q, k)
+    assert bool(calls) == causal
+    torch.compiler.reset()
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_FUSION", "1")
+    with torch.no_grad():
+        unfused = torch.compile(model, backend=mojo_backend, fullgraph=True)(q, k)
+    assert torch.equal(fused, unfused)
+    want = model.float().cpu()(q.float().cpu(), k.float().cpu())
+    assert (fused.float().cpu() - want).abs().max().item() <= 2e-2
+
+
+def test_causal_verdict_follows_the_buffer_not_its_address():
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    x = torch.zeros(1, 1, 64, 64, device="cuda")
+    mask = torch.tril(torch.ones(1, 1, 64, 64, device="cuda"))
+    assert compiler._causal_q_len(mask, (), x) == 64
+    assert compiler._causal_q_len(mask, (), x) == 64            # cached
+    mask[0, 0, 3, 40] = 1.0                                      # in-place edit: no longer causal
+    assert compiler._causal_q_len(mask, (), x) == 0
+    addr = mask.data_ptr()
+    del mask
+    other = torch.ones(1, 1, 64, 64, device="cuda")              # likely the same block again
+    assert compiler._causal_q_len(other, (), x) == 0
+    assert other.data_ptr() == addr or True
+    # a sliced view of a larger causal buffer
+    big = torch.tril(torch.ones(1, 1, 128, 128, device="cuda"))
+    assert compiler._causal_q_len(big, ((2, 0, 64, 1), (3, 0, 64, 1)), x) == 64
+    assert compiler._causal_q_len(big, ((2, 0, 64, 1), (3, 1, 65, 1)), x) == 0

@@ -161,3 +161,62 @@ def test_row_kernels_are_deterministic():
     outs = [_ops().softmax(x, -1) for _ in range(3)]
     torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+
+
+# ---------------------------------------------------------------- attention softmax (scale, causal)
+# widths pick every kernel family: one wave per row (64, 128, 1024), several waves per row
+# (4096 fp32), the generic kernel (77: not a whole number of 16-byte vectors)
+SCALED_SHAPES = [(2, 3, 64, 64), (1, 2, 128, 128), (3, 1000, 1000), (2, 1024, 1024), (1, 77, 77),
+                 (1, 300, 4096)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", SCALED_SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_softmax_scaled_matches_oracle(shape, dtype, causal):
+    q_len = shape[-2]  # (300, 4096) is rectangular: keys beyond the query index are masked too
+    x = seeded(shape, seed=31, scale=4.0, dtype=dtype)
+    scale = 0.125
+    got = _ops().softmax_scaled(_dev(x), scale, causal_q_len=q_len if causal else 0)
+    assert got.dtype == dtype and got.shape == x.shape
+    want = cf.softmax_scaled_causal(as64(x), scale, causal)
+    cols = shape[-1]
+    assert_close64(got, want, rtol=1e-5, atol=1e-6 + cols * 2.0 ** -24 * 1e-2, what="vs closed form")
+    ref = oracle.softmax_scaled(x, scale, causal_q_len=q_len if causal else 0)
+    assert_close64(got, as64(ref), rtol=1e-5, atol=1e-6 + cols * 2.0 ** -24, rounded_want=True,
+                   what="vs C oracle")
+    if causal:
+        upper = torch.ones(shape[-2], shape[-1], dtype=torch.bool).triu(1)
+        assert bool((got.cpu()[..., upper] == 0).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_softmax_scaled_rounding_reproduces_the_three_op_pipeline(dtype):
+    """round_scaled: bit-identical to mul -> masked_fill(-inf) -> softmax run one after another."""
+    x = _dev(seeded((4, 6, 256, 256), seed=32, scale=3.0, dtype=dtype))
+    mask = _dev(torch.tril(torch.ones(256, 256)) == 0)
+    scale = 1.0 / 8.0 + 1.0 / 64.0  # not a power of two: the product really rounds
+    unfused = _ops().softmax((x * scale).masked_fill(mask, float("-inf")), -1)
+    fused = _ops().softmax_scaled(x, scale, causal_q_len=256, round_scaled=True)
+    assert torch.equal(fused, unfused)
+
+
+def test_softmax_scaled_full_size_invariants():
+    """BASELINE attention shape [32*12, 1024, 1024] bf16: rows sum to one, zeros above the
+    diagonal, first row is exactly [1, 0, ...]."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = (torch.randn(96, 1024, 1024, generator=g, device="cuda") * 4).bfloat16()
+    y = _ops().softmax_scaled(x, 0.125, causal_q_len=1024)
+    sums = y.float().sum(-1)
+    assert (sums - 1).abs().max().item() <= 2e-2
+    assert bool((y[:, 0, 0] == 1).all()) and bool((y[:, 0, 1:] == 0).all())
+    assert bool((y.triu(1) == 0).all())
+    assert torch.equal(y, _ops().softmax_scaled(x, 0.125, causal_q_len=1024))
+
+
+def test_softmax_scaled_rejects_bad_arguments():
+    x = _dev(seeded((2, 8, 8), dtype=torch.float32))
+    with pytest.raises(ValueError):
+        _ops().softmax_scaled(x, 1.0, causal_q_len=4)      # q_len must be the query dimension
+    with pytest.raises(TypeError, match="no CPU path"):
+        _ops().softmax_scaled(x.cpu(), 1.0)

@@ -359,3 +359,45 @@ def test_oracle_reproduces_golden_fixtures():
     sx = _t(g["sum_x"], "float32")
     torch.testing.assert_close(oracle.aten_sum(sx, [1]), _t(g["sum_rows"], "float32"), rtol=1e-5, atol=1e-4)
     torch.testing.assert_close(oracle.aten_amax(sx, [1]), _t(g["amax_rows"], "float32"), rtol=0, atol=0)
+
+
+# ---------------------------------------------------------------- attention softmax (scale, causal)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_softmax_scaled_closed_form_and_invariants(dtype, causal):
+    x = seeded((3, 2, 37, 37), seed=21, scale=3.0, dtype=dtype)
+    scale = 0.125
+    got = oracle.softmax_scaled(x, scale, causal_q_len=37 if causal else 0)
+    want = cf.softmax_scaled_causal(as64(x), scale, causal)
+    tol = {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 5e-4}[dtype]
+    assert np.abs(as64(got) - want).max() <= tol
+    np.testing.assert_allclose(as64(got).sum(-1), 1.0, atol=37 * tol)
+    if causal:
+        upper = np.triu(np.ones((37, 37), dtype=bool), 1)
+        assert (as64(got)[..., upper] == 0).all()          # exact zeros above the diagonal
+        assert (as64(got)[..., 0, 0] == 1.0).all()          # first query row sees one key
+
+
+def test_softmax_scaled_reduces_to_plain_softmax_and_to_torch_pipeline():
+    x = seeded((5, 64, 64), seed=22, scale=2.0, dtype=torch.bfloat16)
+    # scale 1, no mask: the very same arithmetic as orc_softmax
+    assert torch.equal(oracle.softmax_scaled(x, 1.0), oracle.softmax_rows(x.reshape(-1, 64)).reshape(x.shape))
+    # rounded product + causal mask == what PyTorch's three separate ops compute (bf16 storage
+    # between them); torch's CPU softmax rounds once from fp32 as well
+    mask = torch.tril(torch.ones(64, 64)) == 0
+    want = torch.softmax((x * 0.3).masked_fill(mask, float("-inf")), dim=-1)
+    got = oracle.softmax_scaled(x, 0.3, causal_q_len=64, round_scaled=True)
+    assert np.abs(as64(got) - as64(want)).max() <= 2 ** -8
+    # without the rounding the result differs from it only by the bf16 rounding of the product
+    free = oracle.softmax_scaled(x, 0.3, causal_q_len=64, round_scaled=False)
+    assert np.abs(as64(free) - as64(got)).max() <= 3e-2
+
+
+def test_softmax_scaled_brute_force_tiny():
+    x = torch.tensor([[[1.0, 2.0, 3.0], [0.5, -1.0, 4.0], [2.0, 2.0, 2.0]]])
+    got = as64(oracle.softmax_scaled(x, 2.0, causal_q_len=3))
+    rows = []
+    for r in range(3):
+        e = [math.exp(2.0 * x[0, r, j].item()) if j <= r else 0.0 for j in range(3)]
+        rows.append([v / sum(e) for v in e])
+    np.testing.assert_allclose(got[0], np.array(rows), rtol=1e-6)

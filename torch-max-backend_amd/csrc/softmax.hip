@@ -18,10 +18,26 @@ namespace tmb {
 // owns RPW independent rows whose loads are all issued before any arithmetic, which keeps more
 // bytes in flight for short rows. STREAM selects non-temporal loads/stores (tensors larger than
 // the Infinity Cache).
-template <typename TIn, typename TOut, int WPR, int VPL, int RPW, bool LOG, bool STREAM, int BLOCK>
+//
+// SCALED: the attention form of the reference kernel (nn_ops.mojo:413-493, `_softmax_rows(scale,
+// causal, q_len)`): x*scale before the max, and with q_len > 0 column j of row r takes part only
+// if j <= r % q_len (the rest comes out as exact zeros). round_scaled rounds x*scale to the
+// storage type first, which is what a separate `mul` kernel in front of the softmax would have
+// stored: a graph that fuses mul + masked_fill + softmax into this kernel then gets the bits
+// of the unfused pipeline. Vectors that are masked out entirely are not fetched (their lanes
+// re-read vector 0 of the row), so a causal softmax reads about half of its input.
+struct SoftmaxScale {
+  float scale;
+  int round_scaled;
+  int q_len;
+};
+
+template <typename TIn, typename TOut, int WPR, int VPL, int RPW, bool LOG, bool STREAM, bool SCALED,
+          int BLOCK>
 __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(TOut* __restrict__ out,
                                                              const TIn* __restrict__ in,
-                                                             int64_t rows, int cols) {
+                                                             int64_t rows, int cols,
+                                                             SoftmaxScale sc) {
   constexpr int EPV = Vec16<TIn>::N;
   constexpr int WAVES = BLOCK / kWave;
   constexpr int GROUPS = WAVES / WPR;
@@ -42,16 +58,26 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(TOut* __restrict__ 
     int64_t row = row0 + r;
     if (row >= rows) row = rows - 1;  // keep lock-step; stores are masked below
     const TIn* src = in + row * static_cast<int64_t>(cols);
+    // last column that takes part (causal), or the whole row
+    const int last_col = (SCALED && sc.q_len > 0) ? static_cast<int>(row % sc.q_len) : cols - 1;
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
       // Lanes past the end of the row re-read vector 0 (always valid) and discard it: no
       // branch, so all of a wave's loads are issued back to back.
       const int vi = (v * WPR + wave_in_row) * kWave + lane;
-      const bool ok = vi < nvec;
+      const bool ok = SCALED ? (vi < nvec && vi * EPV <= last_col) : vi < nvec;
       const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
       const Vec16<TIn> t = STREAM ? load_vec16_stream(src + at) : load_vec16(src + at);
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) x[r][v][e] = ok ? to_f32(t.v[e]) : neg_inf;
+      for (int e = 0; e < EPV; ++e) {
+        if constexpr (SCALED) {
+          float xs = to_f32(t.v[e]) * sc.scale;
+          if (sc.round_scaled) xs = to_f32(from_f32<TIn>(xs));
+          x[r][v][e] = (ok && vi * EPV + e <= last_col) ? xs : neg_inf;
+        } else {
+          x[r][v][e] = ok ? to_f32(t.v[e]) : neg_inf;
+        }
+      }
     }
   }
 
@@ -109,37 +135,51 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(TOut* __restrict__ 
 }
 
 // Any width / alignment. One block per row.
-template <typename TIn, typename TOut, bool LOG>
+template <typename TIn, typename TOut, bool LOG, bool SCALED>
 __global__ __launch_bounds__(256) void softmax_generic_kernel(TOut* __restrict__ out,
                                                               const TIn* __restrict__ in,
-                                                              int64_t rows, int64_t cols) {
+                                                              int64_t rows, int64_t cols,
+                                                              SoftmaxScale sc) {
   __shared__ float slot[4];
   const int wave = threadIdx.x >> 6;
+  const float neg_inf = -__builtin_inff();
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const TIn* src = in + row * cols;
     TOut* dst = out + row * cols;
-    float m = -__builtin_inff();
-    for (int64_t j = threadIdx.x; j < cols; j += 256) m = fmaxf(m, to_f32(src[j]));
+    const int64_t last_col = (SCALED && sc.q_len > 0) ? row % sc.q_len : cols - 1;
+    auto value = [&](int64_t j) {
+      if constexpr (SCALED) {
+        if (j > last_col) return neg_inf;
+        float xs = to_f32(src[j]) * sc.scale;
+        if (sc.round_scaled) xs = to_f32(from_f32<TIn>(xs));
+        return xs;
+      } else {
+        return to_f32(src[j]);
+      }
+    };
+    float m = neg_inf;
+    for (int64_t j = threadIdx.x; j < cols; j += 256) m = fmaxf(m, value(j));
     m = wave_max(m);
     m = group_reduce(m, slot, wave, 0, 4, MaxOp{});
     float s = 0.0f;
-    for (int64_t j = threadIdx.x; j < cols; j += 256) s += exp_f32(to_f32(src[j]) - m);
+    for (int64_t j = threadIdx.x; j < cols; j += 256) s += exp_f32(value(j) - m);
     s = wave_sum(s);
     s = group_reduce(s, slot, wave, 0, 4, SumOp{});
     if (LOG) {
       const float lg = logf(s);
       for (int64_t j = threadIdx.x; j < cols; j += 256)
-        dst[j] = from_f32<TOut>(to_f32(src[j]) - m - lg);
+        dst[j] = from_f32<TOut>(value(j) - m - lg);
     } else {
       const float inv = 1.0f / s;
       for (int64_t j = threadIdx.x; j < cols; j += 256)
-        dst[j] = from_f32<TOut>(exp_f32(to_f32(src[j]) - m) * inv);
+        dst[j] = from_f32<TOut>(exp_f32(value(j) - m) * inv);
     }
   }
 }
 
-template <typename TIn, typename TOut, bool LOG, int WPR, int VPL, int BLOCK>
-static int launch_regs(TOut* out, const TIn* in, int64_t rows, int64_t cols, hipStream_t stream) {
+template <typename TIn, typename TOut, bool LOG, bool SCALED, int WPR, int VPL, int BLOCK>
+static int launch_regs(TOut* out, const TIn* in, int64_t rows, int64_t cols, SoftmaxScale sc,
+                       hipStream_t stream) {
   constexpr int EPV = Vec16<TIn>::N;
   constexpr int FLOATS = VPL * EPV;
   constexpr int RPW = (WPR > 1 || FLOATS >= 64) ? 1 : (FLOATS >= 32 ? 2 : 4);
@@ -148,17 +188,17 @@ static int launch_regs(TOut* out, const TIn* in, int64_t rows, int64_t cols, hip
   // Streams when the tensor cannot live in the 256 MB Infinity Cache anyway.
   const bool stream_hint = rows * cols * static_cast<int64_t>(sizeof(TIn) + sizeof(TOut)) >= (int64_t{256} << 20);
   if (stream_hint) {
-    softmax_regs_kernel<TIn, TOut, WPR, VPL, RPW, LOG, true, BLOCK>
-        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows, static_cast<int>(cols));
+    softmax_regs_kernel<TIn, TOut, WPR, VPL, RPW, LOG, true, SCALED, BLOCK>
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows, static_cast<int>(cols), sc);
   } else {
-    softmax_regs_kernel<TIn, TOut, WPR, VPL, RPW, LOG, false, BLOCK>
-        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows, static_cast<int>(cols));
+    softmax_regs_kernel<TIn, TOut, WPR, VPL, RPW, LOG, false, SCALED, BLOCK>
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(out, in, rows, static_cast<int>(cols), sc);
   }
   return check_launch();
 }
 
-template <typename TIn, typename TOut, bool LOG>
-static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols,
+template <typename TIn, typename TOut, bool LOG, bool SCALED>
+static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols, SoftmaxScale sc,
                             hipStream_t stream) {
   constexpr int EPV = Vec16<TIn>::N;
   constexpr int MAXV = 64 / EPV;  // at most 64 fp32 values of a row per lane
@@ -166,40 +206,42 @@ static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols
                       rows < (int64_t{1} << 31);
   const int64_t nvec = cols / EPV;
   if (vec_ok && nvec <= 16 * 64 * MAXV) {
-    if (nvec <= 64) return launch_regs<TIn, TOut, LOG, 1, 1, 256>(out, in, rows, cols, stream);
-    if (nvec <= 128) return launch_regs<TIn, TOut, LOG, 1, 2, 256>(out, in, rows, cols, stream);
-    if (nvec <= 256) return launch_regs<TIn, TOut, LOG, 1, 4, 256>(out, in, rows, cols, stream);
-    if (nvec <= 512) return launch_regs<TIn, TOut, LOG, 1, 8, 256>(out, in, rows, cols, stream);
+    if (nvec <= 64) return launch_regs<TIn, TOut, LOG, SCALED, 1, 1, 256>(out, in, rows, cols, sc, stream);
+    if (nvec <= 128) return launch_regs<TIn, TOut, LOG, SCALED, 1, 2, 256>(out, in, rows, cols, sc, stream);
+    if (nvec <= 256) return launch_regs<TIn, TOut, LOG, SCALED, 1, 4, 256>(out, in, rows, cols, sc, stream);
+    if (nvec <= 512) return launch_regs<TIn, TOut, LOG, SCALED, 1, 8, 256>(out, in, rows, cols, sc, stream);
     if constexpr (MAXV >= 16) {
-      if (nvec <= 1024) return launch_regs<TIn, TOut, LOG, 1, 16, 256>(out, in, rows, cols, stream);
+      if (nvec <= 1024) return launch_regs<TIn, TOut, LOG, SCALED, 1, 16, 256>(out, in, rows, cols, sc, stream);
     }
     if (nvec <= 4 * 64 * MAXV / 2)
-      return launch_regs<TIn, TOut, LOG, 4, MAXV / 2, 256>(out, in, rows, cols, stream);
+      return launch_regs<TIn, TOut, LOG, SCALED, 4, MAXV / 2, 256>(out, in, rows, cols, sc, stream);
     if (nvec <= 4 * 64 * MAXV)
-      return launch_regs<TIn, TOut, LOG, 4, MAXV, 256>(out, in, rows, cols, stream);
+      return launch_regs<TIn, TOut, LOG, SCALED, 4, MAXV, 256>(out, in, rows, cols, sc, stream);
     if (nvec <= 16 * 64 * MAXV / 2)
-      return launch_regs<TIn, TOut, LOG, 16, MAXV / 2, 1024>(out, in, rows, cols, stream);
-    return launch_regs<TIn, TOut, LOG, 16, MAXV, 1024>(out, in, rows, cols, stream);
+      return launch_regs<TIn, TOut, LOG, SCALED, 16, MAXV / 2, 1024>(out, in, rows, cols, sc, stream);
+    return launch_regs<TIn, TOut, LOG, SCALED, 16, MAXV, 1024>(out, in, rows, cols, sc, stream);
   }
   const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
-  softmax_generic_kernel<TIn, TOut, LOG>
-      <<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(out, in, rows, cols);
+  softmax_generic_kernel<TIn, TOut, LOG, SCALED>
+      <<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(out, in, rows, cols, sc);
   return check_launch();
 }
 
-template <bool LOG>
+template <bool LOG, bool SCALED>
 static int softmax_by_dtype(void* out, const void* in, int64_t rows, int64_t cols, int in_dtype,
-                            int out_dtype, hipStream_t s) {
+                            int out_dtype, SoftmaxScale sc, hipStream_t s) {
   if (in_dtype == TMB_F32 && out_dtype == TMB_F32)
-    return softmax_dispatch<float, float, LOG>((float*)out, (const float*)in, rows, cols, s);
+    return softmax_dispatch<float, float, LOG, SCALED>((float*)out, (const float*)in, rows, cols, sc, s);
   if (in_dtype == TMB_F16 && out_dtype == TMB_F16)
-    return softmax_dispatch<f16_t, f16_t, LOG>((f16_t*)out, (const f16_t*)in, rows, cols, s);
+    return softmax_dispatch<f16_t, f16_t, LOG, SCALED>((f16_t*)out, (const f16_t*)in, rows, cols, sc, s);
   if (in_dtype == TMB_BF16 && out_dtype == TMB_BF16)
-    return softmax_dispatch<bf16_t, bf16_t, LOG>((bf16_t*)out, (const bf16_t*)in, rows, cols, s);
-  if (in_dtype == TMB_F16 && out_dtype == TMB_F32)
-    return softmax_dispatch<f16_t, float, LOG>((float*)out, (const f16_t*)in, rows, cols, s);
-  if (in_dtype == TMB_BF16 && out_dtype == TMB_F32)
-    return softmax_dispatch<bf16_t, float, LOG>((float*)out, (const bf16_t*)in, rows, cols, s);
+    return softmax_dispatch<bf16_t, bf16_t, LOG, SCALED>((bf16_t*)out, (const bf16_t*)in, rows, cols, sc, s);
+  if constexpr (!SCALED) {  // widening outputs exist for the plain form only
+    if (in_dtype == TMB_F16 && out_dtype == TMB_F32)
+      return softmax_dispatch<f16_t, float, LOG, false>((float*)out, (const f16_t*)in, rows, cols, sc, s);
+    if (in_dtype == TMB_BF16 && out_dtype == TMB_F32)
+      return softmax_dispatch<bf16_t, float, LOG, false>((float*)out, (const bf16_t*)in, rows, cols, sc, s);
+  }
   return TMB_ERR_UNSUPPORTED;
 }
 
@@ -211,6 +253,20 @@ extern "C" int tmb_softmax_rows(void* out, const void* in, int64_t rows, int64_t
   if (rows == 0 || cols == 0) return TMB_OK;
   if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return log_mode ? tmb::softmax_by_dtype<true>(out, in, rows, cols, in_dtype, out_dtype, s)
-                  : tmb::softmax_by_dtype<false>(out, in, rows, cols, in_dtype, out_dtype, s);
+  const tmb::SoftmaxScale none{1.0f, 0, 0};
+  return log_mode
+             ? tmb::softmax_by_dtype<true, false>(out, in, rows, cols, in_dtype, out_dtype, none, s)
+             : tmb::softmax_by_dtype<false, false>(out, in, rows, cols, in_dtype, out_dtype, none, s);
+}
+
+extern "C" int tmb_softmax_rows_scaled(void* out, const void* in, int64_t rows, int64_t cols,
+                                       int dtype, float scale, int round_scaled, int64_t q_len,
+                                       void* stream) {
+  if (rows < 0 || cols < 0 || q_len < 0 || q_len > 0x7fffffff) return TMB_ERR_INVALID_ARGUMENT;
+  if (!(scale == scale)) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || cols == 0) return TMB_OK;
+  if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const tmb::SoftmaxScale sc{scale, round_scaled ? 1 : 0, static_cast<int>(q_len)};
+  return tmb::softmax_by_dtype<false, true>(out, in, rows, cols, dtype, dtype, sc, s);
 }

@@ -22,10 +22,12 @@ EPI_NONE, EPI_GELU_TANH, EPI_GELU_ERF = 0, 1, 2
 
 # Every symbol include/tmb_hip.h declares, with its ctypes signature.
 _i64, _vp, _ci, _sz, _dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_double
+_flt = ctypes.c_float
 SIGNATURES = {
     "tmb_version": (_ci, []),
     "tmb_status_string": (ctypes.c_char_p, [_ci]),
     "tmb_softmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _ci, _vp]),
+    "tmb_softmax_rows_scaled": (_ci, [_vp, _vp, _i64, _i64, _ci, _flt, _ci, _i64, _vp]),
     "tmb_layer_norm_rows": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _dbl, _ci, _vp]),
     "tmb_reduce_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),

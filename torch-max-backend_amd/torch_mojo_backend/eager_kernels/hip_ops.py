@@ -161,6 +161,30 @@ def softmax(x: torch.Tensor, dim: int, half_to_float: bool = False, log: bool = 
     return out.movedim(-1, dim) if moved else out
 
 
+def softmax_scaled(x: torch.Tensor, scale: float, causal_q_len: int = 0,
+                   round_scaled: bool = False) -> torch.Tensor:
+    """softmax(x * scale) over the last dimension; with ``causal_q_len`` = q > 0 the tensor is
+    read as [..., q, cols] and column j of query row r takes part only if j <= r (the
+    reference's ``_softmax_rows(scale, causal, q_len)``, nn_ops.mojo:413-493)."""
+    require_hip(x)
+    if x.dtype not in FLOAT_DTYPES:
+        raise TypeError(f"softmax_scaled: unsupported dtype {x.dtype}")
+    if x.dim() < 1:
+        raise ValueError("softmax_scaled needs at least one dimension")
+    if causal_q_len < 0 or (causal_q_len and (x.dim() < 2 or x.shape[-2] != causal_q_len)):
+        raise ValueError(f"softmax_scaled: causal_q_len {causal_q_len} does not match input "
+                         f"{tuple(x.shape)}")
+    xc = x if x.is_contiguous() else x.contiguous()
+    out = torch.empty_like(xc)
+    cols = xc.shape[-1]
+    if out.numel():
+        rc = _ek.lib().tmb_softmax_rows_scaled(out.data_ptr(), xc.data_ptr(), xc.numel() // cols,
+                                               cols, code_of(x.dtype), float(scale),
+                                               int(bool(round_scaled)), int(causal_q_len), _stream())
+        _check("tmb_softmax_rows_scaled", rc)
+    return out
+
+
 def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optional[torch.Tensor],
                bias: Optional[torch.Tensor], eps: float, need_stats: bool = True):
     """(out, mean, rstd); mean/rstd are float32 with shape ``x.shape[:-k] + (1,)*k`` or None

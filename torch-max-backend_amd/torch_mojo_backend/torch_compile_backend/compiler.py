@@ -30,6 +30,7 @@ import operator
 import os
 import time
 import traceback
+import weakref
 from typing import Any, Callable, List, Optional
 
 import torch
@@ -91,6 +92,10 @@ def _step_name(step) -> str:
         return "fused-away"
     if step.fn is _FUSED_ADDMM_GELU:
         return "aten.addmm+gelu (fused)"
+    if step.fn is _FUSED_MASKED_SOFTMAX:
+        return "aten.mul+masked_fill+_softmax (fused)"
+    if step.fn is _skipped:
+        return "fused-away"
     return str(step.key)
 
 
@@ -100,6 +105,24 @@ def _fusion_enabled() -> bool:
 
 def _identity(x, *args, **kwargs):
     return x
+
+
+def _skipped(*args, **kwargs):
+    """Stands in for a node whose work a later fused step does."""
+    return None
+
+
+def _nodes_in(value):
+    if isinstance(value, torch.fx.Node):
+        yield value
+    elif isinstance(value, (list, tuple)):
+        for v in value:
+            yield from _nodes_in(v)
+    elif isinstance(value, dict):
+        for v in value.values():
+            yield from _nodes_in(v)
+    elif isinstance(value, slice):
+        yield from _nodes_in((value.start, value.stop, value.step))
 
 
 class _Slot:
@@ -212,12 +235,82 @@ class _GraphFactory:
             rewrites[node] = None
         return rewrites
 
+    @staticmethod
+    def _fuse_masked_softmax(graph: torch.fx.Graph) -> dict:
+        """mul(x, python scalar) -> masked_fill(., eq(slice*(buffer), 0), -inf) -> _softmax(., last
+        dim), each with a single user: the attention-score pipeline of a decoder block. The
+        _softmax node becomes one fused step over (x, scale, buffer, slices); mul, masked_fill
+        and the mask nodes that nothing else uses are skipped. Whether the buffer really is a
+        causal mask is decided at run time, with the unfused ops as the other branch.
+        Returns {node: None (skip) | ("softmax", x, scale, root, slices, dim)}."""
+        rewrites: dict = {}
+        builtin = ((aten._softmax, _BUILTIN_SOFTMAX), (aten.masked_fill, _BUILTIN_MASKED_FILL),
+                   (aten.mul, _BUILTIN_MUL), (aten.eq, _BUILTIN_EQ), (aten.slice, _BUILTIN_SLICE),
+                   (aten.alias, _BUILTIN_ALIAS))
+        if any(MAPPING_TORCH_ATEN_TO_MOJO.get(op) is not fn for op, fn in builtin):
+            return rewrites  # a user replaced one of the ops: leave the graph alone
+        for node in graph.nodes:
+            if node.op != "call_function" or node.target is not aten._softmax.default:
+                continue
+            fill, dim, half_to_float = node.args[0], node.args[1], node.args[2]
+            val = node.meta.get("val")
+            if half_to_float or val is None or val.dim() < 2 or dim not in (-1, val.dim() - 1):
+                continue
+            if not (isinstance(fill, torch.fx.Node) and fill.op == "call_function"
+                    and fill.target is aten.masked_fill.Scalar and len(fill.users) == 1
+                    and fill.args[2] == float("-inf")):
+                continue
+            mul, mask = fill.args[0], fill.args[1]
+            if not (isinstance(mul, torch.fx.Node) and mul.op == "call_function"
+                    and mul.target is aten.mul.Tensor and len(mul.users) == 1
+                    and isinstance(mul.args[0], torch.fx.Node)
+                    and isinstance(mul.args[1], (int, float)) and not isinstance(mul.args[1], bool)):
+                continue
+            if not (isinstance(mask, torch.fx.Node) and mask.op == "call_function"
+                    and mask.target is aten.eq.Scalar and mask.args[1] == 0):
+                continue
+            chain, root, slices = [mask], mask.args[0], []
+            while isinstance(root, torch.fx.Node) and root.op == "call_function" \
+                    and root.target in (aten.slice.Tensor, aten.alias.default):
+                if root.target is aten.slice.Tensor:
+                    a = list(root.args) + [None] * (5 - len(root.args))
+                    slices.append((a[1] if a[1] is not None else 0, a[2], a[3],
+                                   a[4] if a[4] is not None else 1))
+                chain.append(root)  # a full-range slice reaches the graph as an alias
+                root = root.args[0]
+            if not (isinstance(root, torch.fx.Node) and root.op in ("placeholder", "get_attr")):
+                continue
+            if any(isinstance(v, torch.fx.Node) for sl in slices for v in sl):
+                continue  # symbolic slice bounds: not handled
+            rewrites[node] = ("softmax", mul.args[0], float(mul.args[1]), root,
+                              tuple(reversed(slices)), dim)
+            rewrites[mul] = None
+            rewrites[fill] = None
+            # mask nodes are skipped from the masked_fill upwards while nothing else uses them
+            live_users = {fill}
+            for link in chain:
+                if all(u in live_users or rewrites.get(u, 0) is None for u in link.users):
+                    rewrites[link] = None
+                    live_users.add(link)
+                else:
+                    break
+        return rewrites
+
     def create_graph(self, graph: torch.fx.Graph):
         rewrites = self._fuse_bias_gelu(graph) if _fusion_enabled() else {}
+        softmax_rewrites = self._fuse_masked_softmax(graph) if _fusion_enabled() else {}
         nodes = list(graph.nodes)
+        # what each node reads after the rewrites (liveness must follow the rewritten program)
+        reads: dict = {}
+        for node in nodes:
+            if node in softmax_rewrites:
+                plan = softmax_rewrites[node]
+                reads[node] = [] if plan is None else [plan[1], plan[3]]
+            else:
+                reads[node] = list(node.all_input_nodes)
         last_use: dict = {}
         for idx, node in enumerate(nodes):
-            for used in node.all_input_nodes:
+            for used in reads[node]:
                 last_use[used.name] = idx
         for idx, node in enumerate(nodes):
             if node.op == "placeholder":
@@ -233,7 +326,14 @@ class _GraphFactory:
             elif node.op == "call_function":
                 key, fn = self.resolve(idx, node)
                 args, kwargs = node.args, dict(node.kwargs)
-                if node in rewrites:
+                if node in softmax_rewrites:
+                    plan = softmax_rewrites[node]
+                    if plan is None:
+                        fn, args, kwargs = _skipped, (), {}
+                    else:
+                        fn, kwargs = _FUSED_MASKED_SOFTMAX, {}
+                        args = (plan[1], plan[2], plan[3], plan[4], plan[5])
+                elif node in rewrites:
                     if rewrites[node] is None:
                         fn, args, kwargs = _identity, (node.args[0],), {}
                     else:
@@ -258,7 +358,7 @@ class _GraphFactory:
                 raise MojoCompilerError(f"Unsupported FX node kind {node.op!r} ({node.name})")
         # Release each value after the step that uses it last (never graph outputs).
         output_node = nodes[-1]
-        keep = {n.name for n in output_node.all_input_nodes}
+        keep = {n.name for n in _nodes_in(output_node.args)}
         step_of_idx = {s.node_idx: s for s in self.steps}
         for name, idx in last_use.items():
             if name in keep or idx not in step_of_idx:
@@ -277,9 +377,63 @@ def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none"):
     return _BUILTIN_GELU(_BUILTIN_ADDMM(input, mat1, mat2), approximate=approximate)
 
 
+# id(buffer) -> (weak reference, version, slices and shapes, verdict); verdict = query length if
+# the sliced buffer is a causal mask (nonzero exactly where column <= row), else 0. Checking
+# costs one device sync, once per buffer object and shape. The weak reference guards against a
+# new tensor reusing the id (or the address) of a dead one, the version counter against
+# in-place edits of the buffer.
+_CAUSAL_VERDICTS: dict = {}
+
+
+def _causal_q_len(root: torch.Tensor, slices: tuple, x: torch.Tensor) -> int:
+    if not (isinstance(root, torch.Tensor) and root.is_cuda and x.is_cuda and x.dim() >= 2):
+        return 0
+    what = (tuple(root.shape), tuple(root.stride()), root.dtype, root.data_ptr(), slices,
+            tuple(x.shape[-2:]))
+    entry = _CAUSAL_VERDICTS.get(id(root))
+    if entry is not None and entry[0]() is root and entry[1] == root._version and entry[2] == what:
+        return entry[3]
+    sub = root
+    for dim, start, end, step in slices:
+        sub = sub[(slice(None),) * (dim % sub.dim()) + (slice(start, end, step),)]
+    q, cols = x.shape[-2], x.shape[-1]
+    verdict = 0
+    if sub.dim() >= 2 and tuple(sub.shape[-2:]) == (q, cols) and sub.numel() == q * cols:
+        keep = torch.ones(q, cols, dtype=torch.bool, device=sub.device).tril()
+        if bool(torch.equal(sub.reshape(q, cols) != 0, keep)):
+            verdict = q
+    if len(_CAUSAL_VERDICTS) > 256:
+        _CAUSAL_VERDICTS.clear()
+    _CAUSAL_VERDICTS[id(root)] = (weakref.ref(root), root._version, what, verdict)
+    return verdict
+
+
+def _fused_masked_softmax(x, scale, root, slices, dim):
+    """softmax(masked_fill(x * scale, sliced(root) == 0, -inf), dim=-1)."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    if isinstance(x, torch.Tensor) and x.is_cuda and x.dtype in hip_ops.FLOAT_DTYPES:
+        q_len = _causal_q_len(root, slices, x)
+        if q_len:
+            # round_scaled: same bits as the separate mul kernel would have handed on
+            return hip_ops.softmax_scaled(x, scale, causal_q_len=q_len, round_scaled=True)
+    sub = root
+    for d, start, end, step in slices:
+        sub = _BUILTIN_SLICE(sub, d, start, end, step)
+    filled = _BUILTIN_MASKED_FILL(_BUILTIN_MUL(x, scale), _BUILTIN_EQ(sub, 0), float("-inf"))
+    return _BUILTIN_SOFTMAX(filled, dim, False)
+
+
 _BUILTIN_ADDMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.addmm]
 _BUILTIN_GELU = MAPPING_TORCH_ATEN_TO_MOJO[aten.gelu]
+_BUILTIN_SOFTMAX = MAPPING_TORCH_ATEN_TO_MOJO[aten._softmax]
+_BUILTIN_MASKED_FILL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.masked_fill)
+_BUILTIN_MUL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.mul)
+_BUILTIN_EQ = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.eq)
+_BUILTIN_SLICE = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.slice)
+_BUILTIN_ALIAS = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.alias)
 _FUSED_ADDMM_GELU = _fused_addmm_gelu
+_FUSED_MASKED_SOFTMAX = _fused_masked_softmax
 
 
 class BaseMaxCompiler:
