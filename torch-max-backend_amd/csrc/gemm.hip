@@ -118,11 +118,10 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
     if (g.k % 32 == 0 && tiles(128, 128) >= 32)
       return launch_ring<T, 128, 128, 32, 2, 2, 4, B_KMAJOR, EPI>(g, batch, stream);
   }
+  // Register-staged kernel for the rest (short K, K not a multiple of 32, ragged N-major N).
   if (g.n <= 64) return launch_mfma<T, 256, 64, 4, 1, B_KMAJOR, EPI>(g, batch, stream);
-  if (g.k <= 128) return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
-  if (tiles(256, 256) >= 768) return launch_mfma<T, 256, 256, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
-  if (g.n <= 128 && tiles(256, 128) >= 128) return launch_mfma<T, 256, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
-  if (tiles(128, 128) >= 128) return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
+  if (g.k <= 128 || tiles(128, 128) >= 128)
+    return launch_mfma<T, 128, 128, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
   return launch_mfma<T, 64, 64, 2, 2, B_KMAJOR, EPI>(g, batch, stream);
 }
 

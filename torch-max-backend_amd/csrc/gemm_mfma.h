@@ -75,7 +75,7 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int64_t stride_a, stride_b, stride_c;
   int tiles_m, tiles_n;
-  int vec_store;  // C rows allow aligned 8-byte stores
+  int vec_store;  // C rows start on 16-byte boundaries: 8 columns per store
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
@@ -97,51 +97,121 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = in_group / gsz;
 }
 
-// Epilogue of one 32x32 MFMA result. Swapped-operand layout: the lane holds one row of C
-// (`crow`, valid when `row_ok`) and register e holds column col0 + 8*(e/4) + (e&3).
-// Adds the bias in fp32, applies the activation, casts once, stores 8 bytes per register quad
-// when the row allows it. Kept out of line: sixteen inlined copies of the GELU epilogue exceed
-// the unroller's budget, and a rolled loop would index the accumulators dynamically.
+// Epilogue. A lane of the (operand-swapped) MFMA result holds, for row lane%32 of a 32x32 tile,
+// columns 8q + 4*(lane/32) + {0..3}, q = 0..3: stored straight from there, every store
+// instruction would scatter 8-byte pieces over 32 rows and memory would see partial lines
+// (measured: 1.9x the output bytes written). So a wave stages one 32-row band of its tile in
+// LDS (the operand buffers are free by then) and writes it out row by row: 16 bytes per lane,
+// consecutive lanes along a row, whole 128-byte lines per row where the tile is 64 wide.
+//
+// stage_tile: +bias (fp32) -> optional GELU -> one cast, 4 x 8 bytes into the band. Kept out of
+// line: sixteen inlined copies of the GELU epilogue exceed the unroller's budget, and a rolled
+// loop would index the accumulators dynamically.
+typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
+typedef __attribute__((address_space(3))) u32x2_t lds_u32x2_t;
+typedef __attribute__((address_space(3))) u32x4_t lds_u32x4v_t;
+
+template <int WN>
+struct BandLayout {
+  static constexpr int PITCH = WN * 2 + 16;  // bytes; the pad spreads the rows over the banks
+  static constexpr int BYTES = 32 * PITCH;
+};
+
 template <typename T, int EPI>
-__device__ __noinline__ void store_tile(f32x16_t acc, T* __restrict__ crow, bool row_ok,
-                                        int64_t col0, int64_t N, const T* __restrict__ bias,
-                                        bool vec) {
-  if (!row_ok) return;
+__device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, int64_t col0, int64_t N,
+                                        const T* __restrict__ bias) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int64_t col = col0 + 8 * q;
-    if (col >= N) continue;
     float v[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = acc[4 * q + e];
-    if (col + 4 <= N) {
-      if (bias != nullptr) {
+    if (bias != nullptr) {
+      if (col + 4 <= N) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] += to_f32(bias[col + e]);
-      }
-      T o[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(v[e]);
-      if (vec) {
-        u32x2_t packed;
-        packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
-                    (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
-        packed[1] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[2])) |
-                    (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[3])) << 16);
-        *reinterpret_cast<u32x2_t*>(crow + col) = packed;
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) crow[col + e] = o[e];
+        for (int e = 0; e < 4; ++e)
+          if (col + e < N) v[e] += to_f32(bias[col + e]);  // columns past N are never stored
       }
-    } else {
+    }
+    T o[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (col + e < N) {
-          const float b = bias != nullptr ? to_f32(bias[col + e]) : 0.0f;
-          crow[col + e] = finish<T, EPI>(v[e] + b);
+    for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(v[e]);
+    u32x2_t packed;
+    packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
+                (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
+    packed[1] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[2])) |
+                (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[3])) << 16);
+    *(lds_u32x2_t*)(dst + 16 * q) = packed;
+  }
+}
+
+// Writes the staged 32 x WN band to C. vec16: rows of C start on 16-byte boundaries (pitch and
+// base), so a lane stores 8 columns at once; otherwise lanes store single elements, still
+// consecutive along the row.
+template <typename T, int WN>
+__device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict__ C, int64_t ldc,
+                                           int64_t row0, int64_t col0, int64_t M, int64_t N,
+                                           bool vec16, int lane) {
+  constexpr int PITCH = BandLayout<WN>::PITCH;
+  if (vec16) {
+    constexpr int LPR = WN / 8;    // lanes per row
+    constexpr int RPP = 64 / LPR;  // rows per pass
+#pragma unroll
+    for (int p = 0; p < 32 / RPP; ++p) {
+      const int r = p * RPP + lane / LPR;
+      const int c = (lane % LPR) * 8;
+      const u32x4_t v = *(const lds_u32x4v_t*)(band + r * PITCH + c * 2);
+      const int64_t row = row0 + r, col = col0 + c;
+      if (row < M && col < N) {
+        T* dst = C + row * ldc + col;
+        if (col + 8 <= N) {
+          *reinterpret_cast<u32x4_t*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N)
+              dst[e] = __builtin_bit_cast(T, static_cast<unsigned short>(v[e >> 1] >> (16 * (e & 1))));
         }
       }
     }
+  } else {
+    typedef __attribute__((address_space(3))) unsigned short lds_u16_t;
+#pragma unroll 4
+    for (int r = 0; r < 32; ++r) {
+      const int64_t row = row0 + r;
+      if (row >= M) break;
+#pragma unroll
+      for (int c0 = 0; c0 < WN; c0 += 64) {
+        const int c = c0 + lane;
+        if (c < WN && col0 + c < N)
+          C[row * ldc + col0 + c] =
+              __builtin_bit_cast(T, *(const lds_u16_t*)(band + r * PITCH + c * 2));
+      }
+    }
+  }
+}
+
+// The whole wave tile (TM x TN tiles of 32x32), one 32-row band at a time through `band`
+// (wave-private, BandLayout<WN>::BYTES). The caller has synchronised the workgroup so that
+// nobody still reads operands from the LDS that `band` overlays.
+template <typename T, int EPI, int TM, int TN>
+__device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
+                                                T* __restrict__ C, int64_t ldc, int64_t row0,
+                                                int64_t col0, int64_t M, int64_t N,
+                                                const T* __restrict__ bias, bool vec16, int lane) {
+  constexpr int WN = TN * 32;
+  constexpr int PITCH = BandLayout<WN>::PITCH;
+  lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    if (row0 + i * 32 >= M) break;  // wave-uniform
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      stage_tile<T, EPI>(acc[i][j], mine + j * 64, col0 + j * 32 + 4 * (lane >> 5), N, bias);
+    flush_band<T, WN>(band, C, ldc, row0 + i * 32, col0, M, N, vec16, lane);
   }
 }
 
@@ -358,16 +428,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmAr
 
   // ---- epilogue -------------------------------------------------------------------------
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int64_t row = m0 + wm * WM + i * 32 + (lane & 31);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int64_t col0 = n0 + wn * WN + j * 32 + 4 * (lane >> 5);
-      store_tile<T, EPI>(acc[i][j], C + (row < M ? row : 0) * g.ldc, row < M, col0, N, bias,
-                         g.vec_store != 0);
-    }
-  }
+  __syncthreads();  // every wave is done with the operand buffers: reuse them for the output
+  static_assert(WAVES_M * WAVES_N * BandLayout<WN>::BYTES <= 2 * STAGE_BYTES, "band staging");
+  lds_byte_t* band = (lds_byte_t*)smem + wave * BandLayout<WN>::BYTES;
+  store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
+                                  g.vec_store != 0, lane);
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
@@ -385,8 +450,8 @@ static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
-  g.vec_store = (g.ldc % 4 == 0) && (g.stride_c % 4 == 0 || batch == 1) &&
-                ((reinterpret_cast<uintptr_t>(g.c) & 7u) == 0);
+  g.vec_store = (g.ldc % 8 == 0) && (g.stride_c % 8 == 0 || batch == 1) &&
+                ((reinterpret_cast<uintptr_t>(g.c) & 15u) == 0);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), SMEM, stream>>>(g);

@@ -289,16 +289,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmAr
   mfma_step((KSTEPS - 1) & 1);
 
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int64_t row = m0 + wm * WM + i * 32 + (lane & 31);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int64_t col0 = n0 + wn * WN + j * 32 + 4 * (lane >> 5);
-      store_tile<T, EPI>(acc[i][j], C + (row < M ? row : 0) * g.ldc, row < M, col0, N, bias,
-                         g.vec_store != 0);
-    }
-  }
+  __syncthreads();  // every wave is done with the ring: reuse it for the output
+  static_assert(NW * BandLayout<WN>::BYTES <= R * STAGE_BYTES, "band staging");
+  lds_byte_t* band = (lds_byte_t*)ring + wave * BandLayout<WN>::BYTES;
+  store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
+                                  g.vec_store != 0, lane);
 #endif
 }
 
@@ -307,8 +302,8 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
-  g.vec_store = (g.ldc % 4 == 0) && (g.stride_c % 4 == 0 || batch == 1) &&
-                ((reinterpret_cast<uintptr_t>(g.c) & 7u) == 0);
+  g.vec_store = (g.ldc % 8 == 0) && (g.stride_c % 8 == 0 || batch == 1) &&
+                ((reinterpret_cast<uintptr_t>(g.c) & 15u) == 0);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI>
