@@ -117,6 +117,25 @@ int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t ba
              int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
              int epilogue, void* stream);
 
+/* Fused attention forward: out[b,t,h,:] = softmax_j(scale * q[b,h,t,:] . k[b,h,j,:]) v[b,h,j,:],
+ * with `causal` != 0 only keys j <= t take part. The [batch, heads, q_len, kv_len] scores never
+ * reach memory (online softmax over blocks of 64 keys). `dtype` in {F16,BF16}; head_dim must
+ * be 64 and contiguous; every tensor is described by three element strides {batch, head,
+ * token}, multiples of 8 (q, k, v; 16-byte aligned bases) or 4 (out; 8-byte aligned), so q, k
+ * and v may be slices of one packed [batch, q_len, 3*heads*64] projection and out may be laid
+ * out [batch, q_len, heads, 64]. fp32 scores and statistics; probabilities are rounded to
+ * `dtype` before they multiply v; `round_like_unfused` != 0 also rounds the scores and the
+ * scaled scores to `dtype`, as a separate bmm and mul kernel would have stored them.
+ * Returns TMB_ERR_UNSUPPORTED for other head sizes, kv_len == 0 or unaligned layouts (the
+ * caller then runs the unfused chain).
+ * Replaces aten_functions.py:443-677 (`aten__scaled_dot_product_*`, built from matmul, softmax
+ * and matmul graph ops) and aten_fast.py:5177-5285 (`fast_aten_scaled_dot_product_attention`). */
+int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v, int64_t batch,
+                      int64_t heads, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                      const int64_t* q_strides, const int64_t* k_strides,
+                      const int64_t* v_strides, const int64_t* out_strides, float scale,
+                      int causal, int round_like_unfused, int dtype, void* stream);
+
 /* Elementwise GELU over `numel` contiguous elements, fp32 inside, one cast.
  * `approximate_tanh` != 0 selects the tanh form. Replaces activation_forward_kernels.mojo:22-56
  * (used when the GELU cannot be fused into the producing GEMM's epilogue). */

@@ -70,6 +70,8 @@ def lib() -> ctypes.CDLL:
         L.orc_softmax.argtypes = [vp, vp, i64, i64, ci, ci, ci]
         L.orc_softmax_scaled.argtypes = [vp, vp, i64, i64, ci, ctypes.c_float, ci, i64]
         L.orc_softmax_scaled.restype = ci
+        L.orc_attention.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, ctypes.c_float, ci, ci]
+        L.orc_attention.restype = ci
         L.orc_layer_norm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ci]
         L.orc_reduce.argtypes = [vp, vp, i64, i64, ci, ci]
         L.orc_argmax.argtypes = [vp, vp, i64, i64, ci]
@@ -171,6 +173,19 @@ def softmax_scaled(x: torch.Tensor, scale: float, causal_q_len: int = 0,
         _check(lib().orc_softmax_scaled(out.data_ptr(), x.data_ptr(), x.numel() // cols, cols,
                                         _code(x.dtype), float(scale), int(bool(round_scaled)),
                                         int(causal_q_len)), "softmax_scaled")
+    return out
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+              causal: bool) -> torch.Tensor:
+    """[B,H,T,D] x [B,H,S,D] x [B,H,S,D] -> [B,T,H,D], stage by stage like the unfused graph."""
+    q, k, v = (_cpu(x).contiguous() for x in (q, k, v))
+    b, h, t, d = q.shape
+    out = torch.empty((b, t, h, d), dtype=q.dtype)
+    if out.numel():
+        _check(lib().orc_attention(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), b, h,
+                                   t, k.shape[2], d, float(scale), int(bool(causal)),
+                                   _code(q.dtype)), "attention")
     return out
 
 

@@ -27,6 +27,13 @@ def softmax_scaled_causal(x: np.ndarray, scale: float, causal: bool) -> np.ndarr
     return e / e.sum(axis=-1, keepdims=True)
 
 
+def attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, causal: bool) -> np.ndarray:
+    """float64 softmax(scale q k^T [+ causal]) v for [B,H,T,D],[B,H,S,D],[B,H,S,D] -> [B,T,H,D]."""
+    s = np.einsum("bhtd,bhsd->bhts", q.astype(np.float64), k.astype(np.float64))
+    p = softmax_scaled_causal(s, scale, causal)
+    return np.einsum("bhts,bhsd->bthd", p, v.astype(np.float64))
+
+
 def log_softmax(x: np.ndarray, axis: int = -1) -> np.ndarray:
     x = x.astype(np.float64)
     s = x - x.max(axis=axis, keepdims=True)

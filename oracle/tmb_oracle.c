@@ -11,6 +11,9 @@
  *                   reduction_ops.mojo:874-895 (log-softmax: x - m - log(denom))
  *   orc_softmax_scaled nn_ops.mojo:413-493     (`_softmax_rows(scale, causal, q_len)`: x*scale, causal
  *                                               rows keep j <= r % q_len, the rest is zero)
+ *   orc_attention   aten_functions.py:443-677  (scaled dot product attention as the reference builds
+ *                                               it: matmul, *scale, causal mask, softmax, matmul;
+ *                                               every stage stored in the tensor dtype)
  *   orc_layer_norm  nn_ops.mojo:299-326        (two-pass mean / centered variance, fp32) with the
  *                                               NaN-mean rule of normalization_forward_kernels.mojo:60-70
  *   orc_reduce      reduction_ops.mojo:161-194 (fp32 accumulator for floats, own type for ints,
@@ -190,6 +193,42 @@ int orc_softmax_scaled(void* out, const void* in, int64_t rows, int64_t cols, in
         y = expf(x - m) / denom;
       }
       store_f(out, base + j, dtype, y);
+    }
+  }
+  return 0;
+}
+
+/* out[b,t,h,:] = softmax_j(scale * q[b,h,t,:].k[b,h,j,:]) v[b,h,j,:]; q,k,v are [B,H,T|S,D]
+ * contiguous, out is [B,T,H,D] contiguous. Stage by stage like the unfused graph: scores
+ * (fp32 accumulate) rounded to dtype, times scale rounded to dtype, masked, softmax in fp32
+ * rounded to dtype, second product accumulated in fp32 and rounded once. */
+int orc_attention(void* out, const void* q, const void* k, const void* v, int64_t B, int64_t H,
+                  int64_t T, int64_t S, int64_t D, float scale, int causal, int dtype) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t bh = 0; bh < B * H; ++bh) {
+    for (int64_t t = 0; t < T; ++t) {
+      const int64_t b = bh / H, h = bh % H;
+      float sc[S > 0 ? S : 1];
+      const int64_t last = causal ? (t < S - 1 ? t : S - 1) : S - 1;
+      float m = -INFINITY;
+      for (int64_t j = 0; j <= last; ++j) {
+        float acc = 0.0f;
+        for (int64_t d = 0; d < D; ++d)
+          acc += load_f(q, (bh * T + t) * D + d, dtype) * load_f(k, (bh * S + j) * D + d, dtype);
+        acc = round_to(acc, dtype);
+        acc = round_to(acc * scale, dtype);
+        sc[j] = acc;
+        if (acc > m) m = acc;
+        if (acc != acc) m = acc;
+      }
+      float denom = 0.0f;
+      for (int64_t j = 0; j <= last; ++j) denom += expf(sc[j] - m);
+      for (int64_t j = 0; j <= last; ++j) sc[j] = round_to(expf(sc[j] - m) / denom, dtype);
+      for (int64_t d = 0; d < D; ++d) {
+        float acc = 0.0f;
+        for (int64_t j = 0; j <= last; ++j) acc += sc[j] * load_f(v, (bh * S + j) * D + d, dtype);
+        store_f(out, ((b * T + t) * H + h) * D + d, dtype, acc);
+      }
     }
   }
   return 0;

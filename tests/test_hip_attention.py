@@ -1,0 +1,110 @@
+"""GPU parity of the fused attention forward (scores never reach memory)."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import closed_form as cf
+from helpers import as64, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from torch_mojo_backend.eager_kernels import hip_ops
+    return hip_ops
+
+
+def _qkv(b, h, t, s, dtype, seed=0):
+    return (seeded((b, h, t, 64), seed=seed, dtype=dtype), seeded((b, h, s, 64), seed=seed + 1, dtype=dtype),
+            seeded((b, h, s, 64), seed=seed + 2, dtype=dtype))
+
+
+# query/key counts around the 128-query workgroup, the 32-query wave and the 64-key block
+SHAPES = [(1, 1, 1, 1), (2, 3, 33, 33), (1, 2, 64, 64), (2, 2, 65, 65), (1, 3, 128, 128),
+          (1, 2, 129, 129), (2, 4, 200, 200), (1, 2, 77, 150), (1, 2, 150, 77), (1, 12, 512, 512)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("btsh", SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_matches_closed_form_and_oracle(btsh, dtype, causal):
+    b, h, t, s = btsh
+    q, k, v = _qkv(b, h, t, s, dtype, seed=t + s)
+    scale = 0.125
+    got = _ops().attention(q.cuda(), k.cuda(), v.cuda(), scale, causal)
+    assert got.shape == (b, t, h, 64) and got.dtype == dtype and got.is_contiguous()
+    want = cf.attention(as64(q), as64(k), as64(v), scale, causal)
+    # probabilities are stored with the storage type's 8 (bf16) / 11 (fp16) bit significand and
+    # the output once more: |error| <= 2 ulp of the largest |v| that is averaged (about 4.5)
+    tol = {torch.bfloat16: 3e-2, torch.float16: 4e-3}[dtype]
+    err = np.abs(as64(got) - want)
+    assert err.max() <= tol, f"max err {err.max():.3e}"
+    assert err.mean() <= tol / 8
+    ref = oracle.attention(q, k, v, scale, causal)
+    assert np.abs(as64(got) - as64(ref)).max() <= 2 * tol
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_special_cases(causal):
+    # identical keys -> uniform weights -> running mean of the values (causal) or their mean
+    v = seeded((1, 2, 96, 64), seed=3, dtype=torch.float16)
+    k = torch.ones(1, 2, 96, 64, dtype=torch.float16)
+    q = seeded((1, 2, 96, 64), seed=4, dtype=torch.float16) * 0.01
+    got = as64(_ops().attention(q.cuda(), k.cuda(), v.cuda(), 1.0, causal))
+    v64 = as64(v)
+    if causal:
+        want = np.cumsum(v64, axis=2) / np.arange(1, 97)[None, None, :, None]
+    else:
+        want = np.broadcast_to(v64.mean(axis=2, keepdims=True), v64.shape)
+    np.testing.assert_allclose(got, want.transpose(0, 2, 1, 3), atol=3e-3)
+    # huge scores must not overflow: one dominant key per query
+    q2 = torch.zeros(1, 1, 64, 64, dtype=torch.bfloat16)
+    k2 = torch.zeros(1, 1, 64, 64, dtype=torch.bfloat16)
+    q2[..., 0] = 200.0
+    k2[0, 0, 0, 0] = 200.0                  # key 0 scores 40000 * scale, the rest 0
+    v2 = seeded((1, 1, 64, 64), seed=5, dtype=torch.bfloat16)
+    got2 = _ops().attention(q2.cuda(), k2.cuda(), v2.cuda(), 1.0, causal).cpu()
+    assert torch.isfinite(got2).all()
+    assert torch.equal(got2[0, :, 0], v2[0, 0, 0].expand(64, 64))
+
+
+def test_attention_reads_a_packed_projection_in_place():
+    """q, k, v as strided slices of one [B, T, 3*H*64] tensor, exactly as a decoder block holds
+    them: no copies, same numbers as the contiguous call."""
+    b, t, h = 2, 256, 12
+    qkv = seeded((b, t, 3 * h * 64), seed=9, dtype=torch.bfloat16).cuda()
+    q, k, v = (x.view(b, t, h, 64).transpose(1, 2) for x in qkv.split(h * 64, dim=2))
+    assert not q.is_contiguous() and _ops().attention_supported(q, k, v)
+    got = _ops().attention(q, k, v, 0.125, True)
+    same = _ops().attention(q.contiguous(), k.contiguous(), v.contiguous(), 0.125, True)
+    assert torch.equal(got, same)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.float().cpu(), k.float().cpu(), v.float().cpu(), is_causal=True, scale=0.125)
+    assert (got.float().cpu() - want.transpose(1, 2)).abs().max().item() <= 3e-2
+
+
+def test_attention_benchmark_shape_and_determinism():
+    """GPT-2 small at B=32, T=1024: [32, 12, 1024, 64] bf16, causal. Checked on sampled
+    (batch, head) pairs against float64 and for bit-identical repeats."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+    qkv = torch.randn(32, 1024, 2304, generator=g, device="cuda").bfloat16()
+    q, k, v = (x.view(32, 1024, 12, 64).transpose(1, 2) for x in qkv.split(768, dim=2))
+    got = _ops().attention(q, k, v, 0.125, True, round_like_unfused=True)
+    assert torch.equal(got, _ops().attention(q, k, v, 0.125, True, round_like_unfused=True))
+    for (bi, hi) in ((0, 0), (17, 5), (31, 11)):
+        want = cf.attention(as64(q[bi:bi + 1, hi:hi + 1]), as64(k[bi:bi + 1, hi:hi + 1]),
+                            as64(v[bi:bi + 1, hi:hi + 1]), 0.125, True)
+        err = np.abs(as64(got[bi:bi + 1, :, hi:hi + 1]) - want)
+        assert err.max() <= 3e-2 and err.mean() <= 3e-3
+
+
+def test_attention_rejects_what_it_cannot_take():
+    ops = _ops()
+    q, k, v = (x.cuda() for x in _qkv(1, 1, 8, 8, torch.bfloat16))
+    assert not ops.attention_supported(q.float(), k.float(), v.float())
+    assert not ops.attention_supported(q[..., :32], k[..., :32], v[..., :32])
+    assert not ops.attention_supported(q.cpu(), k.cpu(), v.cpu())
+    with pytest.raises(ValueError):
+        ops.attention(q[..., :32], k[..., :32], v[..., :32], 1.0, True)

@@ -401,3 +401,39 @@ def test_softmax_scaled_brute_force_tiny():
         e = [math.exp(2.0 * x[0, r, j].item()) if j <= r else 0.0 for j in range(3)]
         rows.append([v / sum(e) for v in e])
     np.testing.assert_allclose(got[0], np.array(rows), rtol=1e-6)
+
+
+# ---------------------------------------------------------------- attention (unfused chain)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_oracle_vs_closed_form_and_torch(dtype, causal):
+    q = seeded((2, 3, 33, 16), seed=41, dtype=dtype)
+    k = seeded((2, 3, 33, 16), seed=42, dtype=dtype)
+    v = seeded((2, 3, 33, 16), seed=43, dtype=dtype)
+    got = oracle.attention(q, k, v, 0.25, causal)
+    assert got.shape == (2, 33, 3, 16)
+    want = cf.attention(as64(q), as64(k), as64(v), 0.25, causal)
+    tol = {torch.float32: 5e-6, torch.bfloat16: 3e-2, torch.float16: 4e-3}[dtype]
+    assert np.abs(as64(got) - want).max() <= tol
+    # PyTorch's own fused op on the CPU, same inputs (what the reference's tests compare with)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(),
+                                                           is_causal=causal, scale=0.25)
+    assert np.abs(as64(got) - as64(ref.transpose(1, 2))).max() <= tol
+
+
+def test_attention_oracle_special_cases():
+    # one key: the output is that key's value row, whatever the scores
+    q = seeded((1, 2, 5, 8), seed=1)
+    k = seeded((1, 2, 1, 8), seed=2)
+    v = seeded((1, 2, 1, 8), seed=3)
+    got = oracle.attention(q, k, v, 3.0, False)
+    np.testing.assert_allclose(as64(got), np.broadcast_to(as64(v).transpose(0, 2, 1, 3), (1, 5, 2, 8)), rtol=1e-6)
+    # causal: query 0 sees only key 0
+    k2, v2 = seeded((1, 2, 5, 8), seed=4), seeded((1, 2, 5, 8), seed=5)
+    got2 = oracle.attention(q, k2, v2, 1.0, True)
+    np.testing.assert_allclose(as64(got2)[:, 0], as64(v2)[:, :, 0], rtol=1e-6)
+    # identical keys: uniform weights -> the mean of the values
+    k3 = torch.ones(1, 1, 4, 8)
+    v3 = seeded((1, 1, 4, 8), seed=6)
+    got3 = oracle.attention(seeded((1, 1, 2, 8), seed=7), k3, v3, 1.0, False)
+    np.testing.assert_allclose(as64(got3)[0, :, 0], np.broadcast_to(as64(v3)[0, 0].mean(0), (2, 8)), rtol=1e-6)

@@ -1,0 +1,303 @@
+// Fused attention forward for gfx950: out = softmax(scale * q k^T [+ causal mask]) v without the
+// [batch, heads, q_len, kv_len] score tensor ever reaching memory.
+//
+// One workgroup = 128 queries of one (batch, head): 4 waves x 32 queries. Keys and values are
+// walked in blocks of 64; a block's K and V rows (128 bytes each: head_dim 64 x 2 bytes) go
+// global -> LDS with global_load_lds_dwordx4 into a double buffer, the next block in flight
+// while the current one is multiplied. Per block and wave:
+//   S^T = K_blk Q^T    v_mfma_f32_32x32x16 with the keys as rows: a lane then holds 32 scores of
+//                      ONE query (column lane%32), so the row max / row sum of the softmax are
+//                      in-lane reductions plus one exchange between lanes l and l^32;
+//   online softmax     running max m and sum l per query, accumulator rescaled by exp(m - m');
+//   O^T += V_blk^T P^T the exponentials, rounded to the storage type, are already laid out as
+//                      the MFMA's B operand (k = keys, in the order the score registers hold
+//                      them); V^T comes from ds_read_b64_tr_b16 in that same key order.
+// Q stays in registers for the whole kernel (loaded once, straight from global memory).
+//
+// Arithmetic follows the reference's unfused chain (aten_functions.py:443-677 builds
+// softmax(q k^T * scale + mask) v from the same pieces; eager twin aten_fast.py:5177-5285):
+// fp32 scores, fp32 softmax statistics, probabilities rounded to the storage type before they
+// multiply V. With round_like_unfused the scores and their scaled value are rounded to the
+// storage type too, as a separate bmm and mul kernel would have stored them. The one
+// difference that remains is that probabilities are rounded before, not after, the division by
+// the row sum.
+#include "gemm_mfma.h"
+
+namespace tmb {
+
+typedef __attribute__((address_space(3))) unsigned char attn_lds_u8;
+typedef __attribute__((address_space(3))) u32x4_t attn_lds_u32x4_t;
+typedef short attn_i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) attn_i16x4_t attn_lds_i16x4_t;
+
+struct AttnArgs {
+  void* out;
+  const void* q;
+  const void* k;
+  const void* v;
+  int64_t q_sb, q_sh, q_st;  // element strides: batch, head, token (head_dim is contiguous)
+  int64_t k_sb, k_sh, k_st;
+  int64_t v_sb, v_sh, v_st;
+  int64_t o_sb, o_sh, o_st;
+  int heads, q_len, kv_len;
+  float scale;
+  int causal;
+  int round_like_unfused;
+};
+
+constexpr int kAttnBQ = 128;     // queries per workgroup
+constexpr int kAttnBKV = 64;     // keys per block
+constexpr int kAttnRow = 128;    // bytes of one K or V row (head_dim 64)
+constexpr int kAttnTile = kAttnBKV * kAttnRow;  // 8 KiB: one K or V block
+constexpr int kAttnBuf = 2 * kAttnTile;         // K + V
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, from_f32<T>(lo))) |
+         (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, from_f32<T>(hi))) << 16);
+}
+
+__device__ __forceinline__ float other_half(float x, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2,
+                                                                __builtin_bit_cast(int, x)));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attention_fwd_kernel(AttnArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kAttnBuf];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+  // heavy (late) query blocks first: under a causal mask they have the most key blocks
+  const int qb = gridDim.x - 1 - blockIdx.x;
+  const int b = blockIdx.y / a.heads, h = blockIdx.y % a.heads;
+  const int q0 = qb * kAttnBQ, qw0 = q0 + wave * 32;
+  const int qi = qw0 + (lane & 31);
+  const float neg_inf = -__builtin_inff();
+
+  const T* qp = static_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh;
+  const unsigned char* kp =
+      reinterpret_cast<const unsigned char*>(static_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh);
+  const unsigned char* vp =
+      reinterpret_cast<const unsigned char*>(static_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh);
+
+  // Q as the B operand of S^T = K Q^T: column = query lane%32, k = head-dim 16s + 8*half + 0..7
+  u32x4_t qf[4];
+  {
+    const int qrow = qi < a.q_len ? qi : a.q_len - 1;  // rows past the end are never stored
+    const T* src = qp + static_cast<int64_t>(qrow) * a.q_st + 8 * half;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const u32x4_t*>(src + 16 * s);
+  }
+
+  int n_blocks = (a.kv_len + kAttnBKV - 1) / kAttnBKV;
+  if (a.causal) {
+    const int last_q = (q0 + kAttnBQ < a.q_len ? q0 + kAttnBQ : a.q_len) - 1;
+    const int need = last_q / kAttnBKV + 1;  // keys 0..last_q
+    n_blocks = n_blocks < need ? n_blocks : need;
+  }
+
+  // DMA plan: a 1 KiB load covers 8 rows; the wave issues loads 2w and 2w+1 of K and of V.
+  // Lane -> (row inside the load, 16-byte slot); the source chunk is the slot un-swizzled.
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((attn_lds_u8*)lds));
+  const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int ld_row = lane >> 3, ld_slot = lane & 7;
+  auto dma16 = [](uint32_t m0, uint32_t voff, const unsigned char* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0), "v"(voff), "s"(sbase)
+                 : "memory");
+  };
+  auto fetch_block = [&](int blk, uint32_t buf_off) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int row = (wave * 2 + j) * 8 + ld_row;  // key inside the block
+      int key = blk * kAttnBKV + row;
+      key = key < a.kv_len ? key : a.kv_len - 1;    // masked later; any valid row will do
+      const int k_chunk = ld_slot ^ ((row >> 1) & 7);
+      const int v_chunk = ld_slot ^ (((row >> 1) & 1) << 2);
+      const uint32_t k_off = static_cast<uint32_t>((static_cast<int64_t>(key) * a.k_st + k_chunk * 8) * 2);
+      const uint32_t v_off = static_cast<uint32_t>((static_cast<int64_t>(key) * a.v_st + v_chunk * 8) * 2);
+      const uint32_t dst = lds_base + buf_off + (wave_s * 2 + j) * 1024;
+      dma16(dst, k_off, kp);
+      dma16(dst + kAttnTile, v_off, vp);
+    }
+  };
+
+  // fragment addresses (bytes inside a buffer)
+  int k_lane[4];  // K rows as the A operand: row = key lane%32, chunk 2s + half, swizzled
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+    k_lane[s] = (lane & 31) * kAttnRow + (((2 * s + half) ^ (((lane & 31) >> 1) & 7)) << 4);
+  int v_lane[2];  // V^T through the transposed read, per 32-wide head-dim tile
+  {
+    const int j16 = lane & 15, qq = j16 >> 2, nsub = (lane >> 4) & 1;
+    const int key = 4 * half + qq;  // + 16s + 8r
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt) {
+      const int d0 = dt * 32 + nsub * 16 + (j16 & 3) * 4;
+      v_lane[dt] = kAttnTile + key * kAttnRow + ((((d0 >> 3) ^ (((qq >> 1) & 1) << 2))) << 4) +
+                   (d0 & 7) * 2;
+    }
+  }
+
+  f32x16_t acc_o[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc_o[dt][e] = 0.0f;
+  float m_run = neg_inf, l_run = 0.0f;
+
+  fetch_block(0, 0);
+  for (int blk = 0; blk < n_blocks; ++blk) {
+    const uint32_t buf_off = (blk & 1) * kAttnBuf;
+    // block `blk` is the only load in flight; once every wave has it, the other buffer (read
+    // in the previous iteration) is free for block blk+1
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    if (blk + 1 < n_blocks) fetch_block(blk + 1, kAttnBuf - buf_off);
+
+    const int kb = blk * kAttnBKV;
+    if (a.causal && kb > qw0 + 31) continue;  // wave-uniform: every key lies above the diagonal
+    attn_lds_u8* buf = (attn_lds_u8*)lds + buf_off;
+
+    f32x16_t acc_s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc_s[kt][e] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4_t kf = *(const attn_lds_u32x4_t*)(buf + k_lane[s] + kt * 32 * kAttnRow);
+        acc_s[kt] = Mfma<T>::run(kf, qf[s], acc_s[kt]);
+      }
+    }
+
+    // scores of query qi: register r of tile kt is key kb + 32kt + 8(r/4) + 4*half + r%4
+    const bool need_mask = (a.causal && kb + kAttnBKV - 1 > qw0) || kb + kAttnBKV > a.kv_len;
+    float m_blk = neg_inf;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float x = acc_s[kt][r];
+        if (a.round_like_unfused) {
+          x = to_f32(from_f32<T>(x));
+          x = to_f32(from_f32<T>(x * a.scale));
+        } else {
+          x = x * a.scale;
+        }
+        if (need_mask) {
+          const int key = kb + kt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          if ((a.causal && key > qi) || key >= a.kv_len) x = neg_inf;
+        }
+        acc_s[kt][r] = x;
+        m_blk = fmaxf(m_blk, x);
+      }
+    m_blk = fmaxf(m_blk, other_half(m_blk, lane));
+    const float m_new = fmaxf(m_run, m_blk);
+    const float m_use = m_new == neg_inf ? 0.0f : m_new;  // nothing visible yet: keep exp finite
+    const float alpha = exp_f32(m_run - m_use);           // m_run = -inf gives 0
+    float l_blk = 0.0f;
+    uint32_t pf[2][8];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const float p0 = exp_f32(acc_s[kt][r] - m_use);
+        const float p1 = exp_f32(acc_s[kt][r + 1] - m_use);
+        l_blk += p0 + p1;
+        pf[kt][r >> 1] = pack2<T>(p0, p1);
+      }
+    l_blk += other_half(l_blk, lane);
+    l_run = l_run * alpha + l_blk;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc_o[dt][e] *= alpha;
+
+    // O^T += V^T P^T over the 64 keys: k-step s covers keys 16s..16s+15 in the order
+    // (half, i) -> 16s + 8(i/4) + 4*half + i%4, which is how the score registers are ordered
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      u32x4_t pb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pb[e] = pf[s >> 1][4 * (s & 1) + e];
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt) {
+        attn_lds_u8* src = buf + v_lane[dt] + s * 16 * kAttnRow;
+        const attn_i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_i16x4_t*)src);
+        const attn_i16x4_t hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((attn_lds_i16x4_t*)(src + 8 * kAttnRow));
+        typedef short i16x8_t __attribute__((ext_vector_type(8)));
+        const i16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        acc_o[dt] = Mfma<T>::run(__builtin_bit_cast(u32x4_t, both), pb, acc_o[dt]);
+      }
+    }
+  }
+
+  // out[b, qi, h, d]: register r of tile dt is d = 32dt + 8(r/4) + 4*half + r%4
+  if (qi < a.q_len) {
+    const float inv = 1.0f / l_run;
+    T* dst = static_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + static_cast<int64_t>(qi) * a.o_st;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2_t packed;
+        packed[0] = pack2<T>(acc_o[dt][4 * g] * inv, acc_o[dt][4 * g + 1] * inv);
+        packed[1] = pack2<T>(acc_o[dt][4 * g + 2] * inv, acc_o[dt][4 * g + 3] * inv);
+        *reinterpret_cast<u32x2_t*>(dst + dt * 32 + g * 8 + half * 4) = packed;
+      }
+  }
+#endif
+}
+
+}  // namespace tmb
+
+extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v,
+                                 int64_t batch, int64_t heads, int64_t q_len, int64_t kv_len,
+                                 int64_t head_dim, const int64_t* q_strides,
+                                 const int64_t* k_strides, const int64_t* v_strides,
+                                 const int64_t* out_strides, float scale, int causal,
+                                 int round_like_unfused, int dtype, void* stream) {
+  using namespace tmb;
+  if (batch < 0 || heads < 0 || q_len < 0 || kv_len < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (dtype != TMB_F16 && dtype != TMB_BF16) return TMB_ERR_UNSUPPORTED;
+  if (head_dim != 64) return TMB_ERR_UNSUPPORTED;
+  if (!(scale == scale)) return TMB_ERR_INVALID_ARGUMENT;
+  if (batch == 0 || heads == 0 || q_len == 0) return TMB_OK;
+  if (kv_len == 0) return TMB_ERR_UNSUPPORTED;  // every row empty: left to the caller
+  if (!out || !q || !k || !v || !q_strides || !k_strides || !v_strides || !out_strides)
+    return TMB_ERR_INVALID_ARGUMENT;
+  if (batch * heads > 65535 || q_len >= (int64_t{1} << 30) || kv_len >= (int64_t{1} << 30))
+    return TMB_ERR_UNSUPPORTED;
+  // 16-byte loads of q/k/v rows and 8-byte stores of out rows
+  auto aligned = [](const void* p, const int64_t* s, int64_t mult, uintptr_t mask) {
+    return (reinterpret_cast<uintptr_t>(p) & mask) == 0 && s[0] % mult == 0 && s[1] % mult == 0 &&
+           s[2] % mult == 0 && s[0] >= 0 && s[1] >= 0 && s[2] >= 0;
+  };
+  if (!aligned(q, q_strides, 8, 15) || !aligned(k, k_strides, 8, 15) ||
+      !aligned(v, v_strides, 8, 15) || !aligned(out, out_strides, 4, 7))
+    return TMB_ERR_UNSUPPORTED;
+  // K and V rows are addressed with 32-bit byte offsets from the (batch, head) base
+  if ((kv_len * k_strides[2] + 64) * 2 >= (int64_t{1} << 32) ||
+      (kv_len * v_strides[2] + 64) * 2 >= (int64_t{1} << 32))
+    return TMB_ERR_UNSUPPORTED;
+  AttnArgs a{out, q, k, v,
+             q_strides[0], q_strides[1], q_strides[2],
+             k_strides[0], k_strides[1], k_strides[2],
+             v_strides[0], v_strides[1], v_strides[2],
+             out_strides[0], out_strides[1], out_strides[2],
+             static_cast<int>(heads), static_cast<int>(q_len), static_cast<int>(kv_len),
+             scale, causal ? 1 : 0, round_like_unfused ? 1 : 0};
+  const dim3 grid(static_cast<unsigned>((q_len + kAttnBQ - 1) / kAttnBQ),
+                  static_cast<unsigned>(batch * heads));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == TMB_BF16) {
+    attention_fwd_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(a);
+  } else {
+    attention_fwd_kernel<f16_t><<<grid, dim3(256), 0, s>>>(a);
+  }
+  return check_launch();
+}

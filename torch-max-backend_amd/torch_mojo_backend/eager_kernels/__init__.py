@@ -33,6 +33,8 @@ SIGNATURES = {
     "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
     "tmb_argmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_gemm": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp]),
+    "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
+                                _flt, _ci, _ci, _ci, _vp]),
     "tmb_gelu": (_ci, [_vp, _vp, _i64, _ci, _ci, _vp]),
     "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
 }

@@ -11,6 +11,7 @@ Inputs must live on a HIP device. CPU tensors are rejected: there is no CPU rout
 
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Optional, Sequence, Tuple
 
@@ -182,6 +183,49 @@ def softmax_scaled(x: torch.Tensor, scale: float, causal_q_len: int = 0,
                                                cols, code_of(x.dtype), float(scale),
                                                int(bool(round_scaled)), int(causal_q_len), _stream())
         _check("tmb_softmax_rows_scaled", rc)
+    return out
+
+
+def attention_supported(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> bool:
+    """True when `attention` can take these [batch, heads, tokens, 64] tensors as they are."""
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        return False
+    if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        return False
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        return False
+    b, h, t, d = q.shape
+    if d != 64 or tuple(k.shape) != (b, h, k.shape[2], 64) or tuple(v.shape) != tuple(k.shape):
+        return False
+    if k.shape[2] == 0 or b * h > 65535 or b * h * t == 0:
+        return False
+    for x in (q, k, v):
+        if x.stride(3) != 1 or any(s % 8 or s < 0 for s in x.stride()[:3]) or x.data_ptr() % 16:
+            return False
+        if (x.shape[2] * x.stride(2) + 64) * 2 >= 1 << 32:
+            return False
+    return True
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool,
+              round_like_unfused: bool = False) -> torch.Tensor:
+    """softmax(scale * q k^T [causal]) v for [batch, heads, tokens, 64] tensors (any strides
+    `attention_supported` accepts). Returns a [batch, q_len, heads, 64] contiguous tensor, i.e.
+    the layout `y.transpose(1, 2).contiguous()` would have produced."""
+    require_hip(q, k, v)
+    if not attention_supported(q, k, v):
+        raise ValueError(f"attention: unsupported operands q{tuple(q.shape)} {q.dtype} "
+                         f"strides {q.stride()} / k{tuple(k.shape)} / v{tuple(v.shape)}")
+    b, h, t, d = q.shape
+    out = torch.empty((b, t, h, d), dtype=q.dtype, device=q.device)
+    i64x3 = ctypes.c_int64 * 3
+    strides = [i64x3(x.stride(0), x.stride(1), x.stride(2)) for x in (q, k, v)]
+    o_str = i64x3(out.stride(0), out.stride(2), out.stride(1))
+    rc = _ek.lib().tmb_attention_fwd(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                     b, h, t, k.shape[2], d, strides[0], strides[1], strides[2],
+                                     o_str, float(scale), int(bool(causal)),
+                                     int(bool(round_like_unfused)), code_of(q.dtype), _stream())
+    _check("tmb_attention_fwd", rc)
     return out
 
 
