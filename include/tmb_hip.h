@@ -126,7 +126,7 @@ int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t ba
  * out [batch, q_len, heads, 64]. fp32 scores and statistics; probabilities are rounded to
  * `dtype` before they multiply v; `round_like_unfused` != 0 also rounds the scores and the
  * scaled scores to `dtype`, as a separate bmm and mul kernel would have stored them.
- * Returns TMB_ERR_UNSUPPORTED for other head sizes, kv_len == 0 or unaligned layouts (the
+ * Returns TMB_ERR_UNSUPPORTED for other head sizes, scale <= 0, kv_len == 0 or unaligned layouts (the
  * caller then runs the unfused chain).
  * Replaces aten_functions.py:443-677 (`aten__scaled_dot_product_*`, built from matmul, softmax
  * and matmul graph ops) and aten_fast.py:5177-5285 (`fast_aten_scaled_dot_product_attention`). */

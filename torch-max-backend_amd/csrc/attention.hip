@@ -3,8 +3,9 @@
 //
 // One workgroup = 128 queries of one (batch, head): 4 waves x 32 queries. Keys and values are
 // walked in blocks of 64; a block's K and V rows (128 bytes each: head_dim 64 x 2 bytes) go
-// global -> LDS with global_load_lds_dwordx4 into a double buffer, the next block in flight
-// while the current one is multiplied. Per block and wave:
+// global -> LDS with global_load_lds_dwordx4 into a ring of three buffers, the next two blocks
+// in flight while the current one is multiplied (one block of lookahead leaves every iteration
+// waiting for an L2 round trip). Per block and wave:
 //   S^T = K_blk Q^T    v_mfma_f32_32x32x16 with the keys as rows: a lane then holds 32 scores of
 //                      ONE query (column lane%32), so the row max / row sum of the softmax are
 //                      in-lane reductions plus one exchange between lanes l and l^32;
@@ -50,6 +51,7 @@ constexpr int kAttnBKV = 64;     // keys per block
 constexpr int kAttnRow = 128;    // bytes of one K or V row (head_dim 64)
 constexpr int kAttnTile = kAttnBKV * kAttnRow;  // 8 KiB: one K or V block
 constexpr int kAttnBuf = 2 * kAttnTile;         // K + V
+constexpr int kAttnStages = 3;                  // LDS ring: one block in use, two in flight
 
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -63,13 +65,19 @@ __device__ __forceinline__ float other_half(float x, int lane) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void attention_fwd_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attention_fwd_kernel(
+    AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kAttnBuf];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[kAttnStages * kAttnBuf];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
-  // heavy (late) query blocks first: under a causal mask they have the most key blocks
-  const int qb = gridDim.x - 1 - blockIdx.x;
-  const int b = blockIdx.y / a.heads, h = blockIdx.y % a.heads;
+  // Workgroups are dealt to the 8 XCDs round-robin by their linear id, and under a causal mask
+  // a query block's cost grows with its index: with the query block as the fastest grid
+  // dimension and 8 of them, one XCD would get every heaviest block. Rotating the query block
+  // by the (batch, head) index gives each XCD an even mix.
+  const int n_qb = (a.q_len + kAttnBQ - 1) / kAttnBQ;
+  const int bh = blockIdx.x / n_qb;
+  const int qb = n_qb - 1 - static_cast<int>((blockIdx.x % n_qb + bh) % n_qb);
+  const int b = bh / a.heads, h = bh % a.heads;
   const int q0 = qb * kAttnBQ, qw0 = q0 + wave * 32;
   const int qi = qw0 + (lane & 31);
   const float neg_inf = -__builtin_inff();
@@ -148,17 +156,26 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnArgs a) {
   float m_run = neg_inf, l_run = 0.0f;
 
   fetch_block(0, 0);
+  if (n_blocks > 1) fetch_block(1, kAttnBuf);
+  uint32_t buf_off = 0;                 // ring position of block `blk`
+  uint32_t free_off = 2 * kAttnBuf;     // the buffer read two iterations ago
   for (int blk = 0; blk < n_blocks; ++blk) {
-    const uint32_t buf_off = (blk & 1) * kAttnBuf;
-    // block `blk` is the only load in flight; once every wave has it, the other buffer (read
-    // in the previous iteration) is free for block blk+1
-    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));  // vmcnt(0) lgkmcnt(0)
+    // Each wave has 4 loads per block in flight; block blk+1 (if any) may stay outstanding.
+    // Once every wave has block `blk`, the buffer of block blk-1 is free for block blk+2.
+    if (blk + 1 < n_blocks) {
+      __builtin_amdgcn_s_waitcnt(4 | (7 << 4) | (0 << 8) | (0 << 14));  // vmcnt(4) lgkmcnt(0)
+    } else {
+      __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));  // vmcnt(0) lgkmcnt(0)
+    }
     __builtin_amdgcn_s_barrier();
-    if (blk + 1 < n_blocks) fetch_block(blk + 1, kAttnBuf - buf_off);
+    if (blk + 2 < n_blocks) fetch_block(blk + 2, free_off);
+    const uint32_t cur_off = buf_off;
+    free_off = buf_off;
+    buf_off = buf_off + kAttnBuf == kAttnStages * kAttnBuf ? 0 : buf_off + kAttnBuf;
 
     const int kb = blk * kAttnBKV;
     if (a.causal && kb > qw0 + 31) continue;  // wave-uniform: every key lies above the diagonal
-    attn_lds_u8* buf = (attn_lds_u8*)lds + buf_off;
+    attn_lds_u8* buf = (attn_lds_u8*)lds + cur_off;
 
     f32x16_t acc_s[2];
 #pragma unroll
@@ -172,7 +189,11 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnArgs a) {
       }
     }
 
-    // scores of query qi: register r of tile kt is key kb + 32kt + 8(r/4) + 4*half + r%4
+    // scores of query qi: register r of tile kt is key kb + 32kt + 8(r/4) + 4*half + r%4.
+    // The running maximum is kept on the unscaled scores (scale > 0 keeps the order) and the
+    // scale rides in the exponent: exp(scale*(x - m)) = exp2(x*c - m*c), c = scale*log2(e),
+    // one FMA and one v_exp_f32 per score. The exponential's error (a few 1e-6 relative from
+    // the fp32 argument) disappears in the rounding of the probability to the storage type.
     const bool need_mask = (a.causal && kb + kAttnBKV - 1 > qw0) || kb + kAttnBKV > a.kv_len;
     float m_blk = neg_inf;
 #pragma unroll
@@ -181,10 +202,10 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnArgs a) {
       for (int r = 0; r < 16; ++r) {
         float x = acc_s[kt][r];
         if (a.round_like_unfused) {
+          // what a bmm kernel and then a mul kernel would have stored; the scale is applied
+          // here, so the exponent below uses log2(e) alone
           x = to_f32(from_f32<T>(x));
           x = to_f32(from_f32<T>(x * a.scale));
-        } else {
-          x = x * a.scale;
         }
         if (need_mask) {
           const int key = kb + kt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
@@ -196,15 +217,17 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnArgs a) {
     m_blk = fmaxf(m_blk, other_half(m_blk, lane));
     const float m_new = fmaxf(m_run, m_blk);
     const float m_use = m_new == neg_inf ? 0.0f : m_new;  // nothing visible yet: keep exp finite
-    const float alpha = exp_f32(m_run - m_use);           // m_run = -inf gives 0
+    const float c = a.round_like_unfused ? 1.4426950408889634f : a.scale * 1.4426950408889634f;
+    const float mc = m_use * c;
+    const float alpha = __builtin_amdgcn_exp2f(m_run * c - mc);  // m_run = -inf gives 0
     float l_blk = 0.0f;
     uint32_t pf[2][8];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        const float p0 = exp_f32(acc_s[kt][r] - m_use);
-        const float p1 = exp_f32(acc_s[kt][r + 1] - m_use);
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kt][r], c, -mc));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kt][r + 1], c, -mc));
         l_blk += p0 + p1;
         pf[kt][r >> 1] = pack2<T>(p0, p1);
       }
@@ -266,11 +289,13 @@ extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const 
   if (dtype != TMB_F16 && dtype != TMB_BF16) return TMB_ERR_UNSUPPORTED;
   if (head_dim != 64) return TMB_ERR_UNSUPPORTED;
   if (!(scale == scale)) return TMB_ERR_INVALID_ARGUMENT;
+  if (!(scale > 0.0f) || scale > 3.0e38f) return TMB_ERR_UNSUPPORTED;  // the running maximum assumes it
   if (batch == 0 || heads == 0 || q_len == 0) return TMB_OK;
   if (kv_len == 0) return TMB_ERR_UNSUPPORTED;  // every row empty: left to the caller
   if (!out || !q || !k || !v || !q_strides || !k_strides || !v_strides || !out_strides)
     return TMB_ERR_INVALID_ARGUMENT;
-  if (batch * heads > 65535 || q_len >= (int64_t{1} << 30) || kv_len >= (int64_t{1} << 30))
+  if (batch * heads * ((q_len + kAttnBQ - 1) / kAttnBQ) >= (int64_t{1} << 31) ||
+      q_len >= (int64_t{1} << 30) || kv_len >= (int64_t{1} << 30))
     return TMB_ERR_UNSUPPORTED;
   // 16-byte loads of q/k/v rows and 8-byte stores of out rows
   auto aligned = [](const void* p, const int64_t* s, int64_t mult, uintptr_t mask) {
@@ -291,8 +316,7 @@ extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const 
              out_strides[0], out_strides[1], out_strides[2],
              static_cast<int>(heads), static_cast<int>(q_len), static_cast<int>(kv_len),
              scale, causal ? 1 : 0, round_like_unfused ? 1 : 0};
-  const dim3 grid(static_cast<unsigned>((q_len + kAttnBQ - 1) / kAttnBQ),
-                  static_cast<unsigned>(batch * heads));
+  const dim3 grid(static_cast<unsigned>(((q_len + kAttnBQ - 1) / kAttnBQ) * batch * heads));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == TMB_BF16) {
     attention_fwd_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(a);

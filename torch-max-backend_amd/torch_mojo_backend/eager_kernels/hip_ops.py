@@ -197,7 +197,7 @@ def attention_supported(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> bo
     b, h, t, d = q.shape
     if d != 64 or tuple(k.shape) != (b, h, k.shape[2], 64) or tuple(v.shape) != tuple(k.shape):
         return False
-    if k.shape[2] == 0 or b * h > 65535 or b * h * t == 0:
+    if k.shape[2] == 0 or b * h * ((t + 127) // 128) >= 1 << 31 or b * h * t == 0:
         return False
     for x in (q, k, v):
         if x.stride(3) != 1 or any(s % 8 or s < 0 for s in x.stride()[:3]) or x.data_ptr() % 16:
@@ -213,6 +213,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, c
     `attention_supported` accepts). Returns a [batch, q_len, heads, 64] contiguous tensor, i.e.
     the layout `y.transpose(1, 2).contiguous()` would have produced."""
     require_hip(q, k, v)
+    if not (scale > 0.0 and math.isfinite(scale)):
+        raise ValueError(f"attention: scale must be positive and finite, got {scale}")
     if not attention_supported(q, k, v):
         raise ValueError(f"attention: unsupported operands q{tuple(q.shape)} {q.dtype} "
                          f"strides {q.stride()} / k{tuple(k.shape)} / v{tuple(v.shape)}")
