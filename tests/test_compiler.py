@@ -235,9 +235,10 @@ def test_masked_softmax_rewrite_plans_one_fused_step(cpu_hot_ops, monkeypatch):
     names = [compiler._step_name(s) for s in program.steps]
     assert names.count("aten.mul+masked_fill+_softmax (fused)") == 1
     fused = next(s for s in program.steps if s.fn is compiler._FUSED_MASKED_SOFTMAX)
-    skipped = {str(s.node.target) for s in program.steps if s.fn is compiler._skipped}
-    assert {"aten.mul.Tensor", "aten.masked_fill.Scalar", "aten.eq.Scalar",
-            "aten.slice.Tensor"} <= skipped
+    # the nodes whose work the fused step does are not in the program at all
+    remaining = {str(s.node.target) for s in program.steps}
+    assert not remaining & {"aten.mul.Tensor", "aten.masked_fill.Scalar", "aten.eq.Scalar",
+                            "aten.slice.Tensor"}
     assert fused.args[1] == 0.25 and fused.args[3] == ((2, 0, 8, 1), (3, 0, 8, 1))
     # the scores stay alive until the fused step has read them, then go
     scores_slot = fused.args[0].index
@@ -273,3 +274,43 @@ def test_causal_verdict_is_cached_and_follows_the_buffer():
     x = torch.zeros(2, 2, 8, 8)
     # host tensors never qualify (the fused kernel is a device kernel)
     assert compiler._causal_q_len(mask, ((2, 0, 8, 1), (3, 0, 8, 1)), x) == 0
+
+
+def test_attention_rewrite_plans_one_step_per_block(monkeypatch):
+    """The decoder block of demo_scripts/gpt2.py: the whole chain from the q/k/v copies to the
+    transposed copy of the context becomes one step that reads q, k, v and the mask buffer."""
+    import sys
+    sys.path.insert(0, str(__import__("pathlib").Path(__file__).resolve().parents[1] / "torch-max-backend_amd"))
+    from demo_scripts.gpt2 import GPT, GPTConfig
+    from torch._dynamo.backends.common import aot_autograd
+    from functorch.compile import make_boxed_func
+
+    programs = []
+
+    def fw(gm, example_inputs):
+        programs.append(compiler._GraphFactory().create_graph(gm.graph))
+        return make_boxed_func(gm.forward)
+
+    model = GPT(GPTConfig(block_size=16, vocab_size=50, n_layer=2, n_head=2, n_embd=8)).eval()
+    with torch.no_grad():
+        torch.compile(model, backend=aot_autograd(fw_compiler=fw, decompositions=af.DECOMPOSITION_TABLE))(
+            torch.randint(0, 50, (2, 8)))
+    program = programs[-1]
+    fused = [s for s in program.steps if s.fn is compiler._FUSED_ATTENTION]
+    assert len(fused) == 2
+    targets = [str(s.node.target) for s in program.steps]
+    assert "aten.bmm.default" not in targets and "aten._softmax.default" not in targets
+    assert "aten.clone.default" in targets          # the fused steps sit on the final clones
+    assert targets.count("aten.clone.default") == 2
+    for s in fused:
+        q, k, v, scale, root, slices = s.args
+        assert scale == 0.5 and slices == ((2, 0, 8, 1), (3, 0, 8, 1))
+        assert len({q.index, k.index, v.index, root.index}) == 4
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION", "1")
+    torch.compiler.reset()
+    with torch.no_grad():
+        torch.compile(model, backend=aot_autograd(fw_compiler=fw, decompositions=af.DECOMPOSITION_TABLE))(
+            torch.randint(0, 50, (2, 8)))
+    names = [compiler._step_name(s) for s in programs[-1].steps]
+    assert names.count("aten.mul+masked_fill+_softmax (fused)") == 2
+    assert not any(s.fn is compiler._FUSED_ATTENTION for s in programs[-1].steps)

@@ -87,9 +87,11 @@ def test_gpt2_small_bf16_logits_vs_fp32_oracle():
 
 
 def test_fusion_is_bit_identical_to_unfused(monkeypatch):
-    """The addmm->gelu rewrite must not change a single bit of the logits."""
+    """The addmm->gelu and mul+masked_fill+softmax rewrites must not change a single bit of the
+    logits (the attention rewrite reorders roundings and is checked to a tolerance below)."""
     from torch_mojo_backend import mojo_backend
 
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION", "1")
     gpu_model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).to("cuda")
     idx = seeded_tokens(2, 64, seed=2).to("cuda")
     with torch.no_grad():
@@ -161,3 +163,61 @@ def test_causal_verdict_follows_the_buffer_not_its_address():
     big = torch.tril(torch.ones(1, 1, 128, 128, device="cuda"))
     assert compiler._causal_q_len(big, ((2, 0, 64, 1), (3, 0, 64, 1)), x) == 64
     assert compiler._causal_q_len(big, ((2, 0, 64, 1), (3, 1, 65, 1)), x) == 0
+
+
+def test_attention_fusion_stays_within_the_storage_rounding(monkeypatch):
+    """Whole-block attention in one kernel against the same graph without that rewrite:
+    bf16 logits differ by the reordered roundings only."""
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    gpu_model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).to("cuda")
+    idx = seeded_tokens(2, 256, seed=2).to("cuda")
+    calls = []
+    real = compiler.aten_functions.hip_ops.attention
+    monkeypatch.setattr(compiler.aten_functions.hip_ops, "attention",
+                        lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    with torch.no_grad():
+        fused, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    assert len(calls) == 2                      # one launch per layer
+    torch.compiler.reset()
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION", "1")
+    with torch.no_grad():
+        plain, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    assert len(calls) == 2
+    # Neither is "the" answer: measure both against the float32 CPU model on the same (bf16-
+    # rounded) weights. The fused graph must be no further from it than the unfused one.
+    ref_model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).float()
+    with torch.no_grad():
+        want, _ = ref_model(idx.cpu())
+    err_fused = (fused.float().cpu() - want).abs()
+    err_plain = (plain.float().cpu() - want).abs()
+    assert err_fused.max().item() <= max(2e-2, 1.25 * err_plain.max().item())
+    assert err_fused.mean().item() <= 1.1 * err_plain.mean().item() + 1e-4
+    # and the two agree to about one bf16 spacing of a logit of magnitude ~1 (2^-7) on average
+    diff = (fused.float() - plain.float()).abs()
+    assert diff.max().item() <= 4e-2 and diff.mean().item() <= 2.0 ** -7
+
+
+def test_attention_fusion_falls_back_for_a_non_causal_buffer(monkeypatch):
+    """Same graph, but the mask buffer is not lower-triangular: the fused step must run the
+    unfused chain and give the unfused graph's bits."""
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    gpu_model = build_gpt2_small(seed=0, n_layer=1).to(torch.bfloat16).to("cuda")
+    for block in gpu_model.transformer.h:
+        block.attn.bias[0, 0, 5, 40] = 1.0      # one key above the diagonal becomes visible
+    idx = seeded_tokens(1, 128, seed=3).to("cuda")
+    calls = []
+    real = compiler.aten_functions.hip_ops.attention
+    monkeypatch.setattr(compiler.aten_functions.hip_ops, "attention",
+                        lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    with torch.no_grad():
+        fused, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    assert not calls
+    torch.compiler.reset()
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_FUSION", "1")
+    with torch.no_grad():
+        plain, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    assert torch.equal(fused, plain)

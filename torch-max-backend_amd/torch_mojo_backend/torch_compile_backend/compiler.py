@@ -94,6 +94,8 @@ def _step_name(step) -> str:
         return "aten.addmm+gelu (fused)"
     if step.fn is _FUSED_MASKED_SOFTMAX:
         return "aten.mul+masked_fill+_softmax (fused)"
+    if step.fn is _FUSED_ATTENTION:
+        return "attention: bmm+mul+masked_fill+_softmax+bmm (fused)"
     if step.fn is _skipped:
         return "fused-away"
     return str(step.key)
@@ -101,6 +103,12 @@ def _step_name(step) -> str:
 
 def _fusion_enabled() -> bool:
     return os.environ.get("TORCH_MOJO_BACKEND_NO_FUSION", "0").lower() not in ("1", "true", "yes")
+
+
+def _attention_fusion_enabled() -> bool:
+    """The attention rewrite changes rounding (online softmax); the other rewrites do not."""
+    return _fusion_enabled() and os.environ.get(
+        "TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION", "0").lower() not in ("1", "true", "yes")
 
 
 def _identity(x, *args, **kwargs):
@@ -296,16 +304,109 @@ class _GraphFactory:
                     break
         return rewrites
 
+    @staticmethod
+    def _fuse_attention(softmax_rewrites: dict) -> None:
+        """Grows a fused masked softmax into a fused attention when it sits in
+            bmm(flat(q), flat(k^T)) -> view -> [mul, masked_fill, _softmax] -> expand -> view
+              -> bmm(., flat(v)) -> view -> transpose(1, 2) -> clone(contiguous)
+        with flat(x) = _unsafe_view(clone(expand(x))) and every link used once. The clone at the
+        end becomes the fused step over (q, k, v, scale, mask buffer, slices) and returns the
+        [batch, tokens, heads, head_dim] tensor; everything in between is skipped. The plan of
+        the _softmax node is replaced in place."""
+        bmm_ops = (aten.bmm.default,)
+        if MAPPING_TORCH_ATEN_TO_MOJO.get(aten.bmm) is not _BUILTIN_BMM:
+            return
+
+        def single(node, *targets):
+            return (isinstance(node, torch.fx.Node) and node.op == "call_function"
+                    and node.target in targets and len(node.users) == 1)
+
+        def unflatten(node):
+            """_unsafe_view/view(clone(expand(x))) -> (x, [nodes])"""
+            if not single(node, aten._unsafe_view.default, aten.view.default):
+                return None
+            c = node.args[0]
+            if not single(c, aten.clone.default):
+                return None
+            e = c.args[0]
+            if not single(e, aten.expand.default):
+                return None
+            src = e.args[0]
+            val, eval_ = (src.meta.get("val") if isinstance(src, torch.fx.Node) else None), e.meta.get("val")
+            if val is None or eval_ is None or tuple(val.shape) != tuple(eval_.shape) or val.dim() != 4:
+                return None  # the expand really broadcasts: not this pattern
+            return src, [node, c, e]
+
+        for sm_node, plan in list(softmax_rewrites.items()):
+            if plan is None or plan[0] != "softmax":
+                continue
+            _, scores_view, scale, root, slices, _dim = plan
+            if not single(scores_view, aten.view.default, aten._unsafe_view.default):
+                continue
+            bmm0 = scores_view.args[0]
+            if not single(bmm0, *bmm_ops):
+                continue
+            qa, kb = unflatten(bmm0.args[0]), unflatten(bmm0.args[1])
+            if qa is None or kb is None:
+                continue
+            kt = kb[0]
+            if not (single(kt, aten.transpose.int) and
+                    {d % 4 for d in kt.args[1:3]} == {2, 3}):
+                continue
+            # forward: _softmax -> expand -> view -> bmm -> view -> transpose(1,2) -> clone
+            if len(sm_node.users) != 1:
+                continue
+            ex = next(iter(sm_node.users))
+            if not single(ex, aten.expand.default) or \
+                    tuple(ex.meta["val"].shape) != tuple(sm_node.meta["val"].shape):
+                continue
+            pv = next(iter(ex.users))
+            if not single(pv, aten.view.default, aten._unsafe_view.default):
+                continue
+            bmm1 = next(iter(pv.users))
+            if not (single(bmm1, *bmm_ops) and bmm1.args[0] is pv):
+                continue
+            va = unflatten(bmm1.args[1])
+            if va is None:
+                continue
+            ov = next(iter(bmm1.users))
+            if not single(ov, aten.view.default, aten._unsafe_view.default) or ov.meta["val"].dim() != 4:
+                continue
+            tr = next(iter(ov.users))
+            if not (single(tr, aten.transpose.int) and {d % 4 for d in tr.args[1:3]} == {1, 2}):
+                continue
+            final = next(iter(tr.users))
+            if not (isinstance(final, torch.fx.Node) and final.op == "call_function"
+                    and final.target is aten.clone.default
+                    and final.kwargs.get("memory_format", torch.contiguous_format)
+                    is torch.contiguous_format):
+                continue
+            q4, k4, v4 = qa[0], kt.args[0], va[0]
+            shapes = [tuple(n.meta["val"].shape) for n in (q4, k4, v4)]
+            if not (len(shapes[0]) == 4 and shapes[1] == shapes[2]
+                    and shapes[0][:2] == shapes[1][:2] and shapes[0][3] == shapes[1][3]):
+                continue
+            for node in [*qa[1], *kb[1], kt, bmm0, scores_view, sm_node, ex, pv, *va[1], bmm1, ov, tr]:
+                softmax_rewrites[node] = None
+            softmax_rewrites[final] = ("attention", q4, k4, v4, scale, root, slices)
+
     def create_graph(self, graph: torch.fx.Graph):
         rewrites = self._fuse_bias_gelu(graph) if _fusion_enabled() else {}
         softmax_rewrites = self._fuse_masked_softmax(graph) if _fusion_enabled() else {}
+        if softmax_rewrites and _attention_fusion_enabled():
+            self._fuse_attention(softmax_rewrites)
         nodes = list(graph.nodes)
         # what each node reads after the rewrites (liveness must follow the rewritten program)
         reads: dict = {}
         for node in nodes:
             if node in softmax_rewrites:
                 plan = softmax_rewrites[node]
-                reads[node] = [] if plan is None else [plan[1], plan[3]]
+                if plan is None:
+                    reads[node] = []
+                elif plan[0] == "softmax":
+                    reads[node] = [plan[1], plan[3]]
+                else:
+                    reads[node] = [plan[1], plan[2], plan[3], plan[5]]
             else:
                 reads[node] = list(node.all_input_nodes)
         last_use: dict = {}
@@ -330,15 +431,22 @@ class _GraphFactory:
                     plan = softmax_rewrites[node]
                     if plan is None:
                         fn, args, kwargs = _skipped, (), {}
-                    else:
+                    elif plan[0] == "softmax":
                         fn, kwargs = _FUSED_MASKED_SOFTMAX, {}
                         args = (plan[1], plan[2], plan[3], plan[4], plan[5])
+                    else:
+                        fn, kwargs = _FUSED_ATTENTION, {}
+                        args = plan[1:]
                 elif node in rewrites:
                     if rewrites[node] is None:
                         fn, args, kwargs = _identity, (node.args[0],), {}
                     else:
                         fn = _FUSED_ADDMM_GELU
                         kwargs = {"approximate": rewrites[node]}
+                if fn is _skipped:
+                    # no step at all: a fused step later does this node's work
+                    self.slots[node.name] = len(self.slots)
+                    continue
                 step = _Step()
                 step.fn = fn
                 step.key = key
@@ -385,18 +493,24 @@ def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none"):
 _CAUSAL_VERDICTS: dict = {}
 
 
-def _causal_q_len(root: torch.Tensor, slices: tuple, x: torch.Tensor) -> int:
-    if not (isinstance(root, torch.Tensor) and root.is_cuda and x.is_cuda and x.dim() >= 2):
+def _causal_q_len(root: torch.Tensor, slices: tuple, x) -> int:
+    """`x`: the score tensor, or just its last two sizes (q_len, kv_len)."""
+    if isinstance(x, torch.Tensor):
+        if not (x.is_cuda and x.dim() >= 2):
+            return 0
+        x_shape = tuple(x.shape[-2:])
+    else:
+        x_shape = tuple(x)
+    if not (isinstance(root, torch.Tensor) and root.is_cuda):
         return 0
-    what = (tuple(root.shape), tuple(root.stride()), root.dtype, root.data_ptr(), slices,
-            tuple(x.shape[-2:]))
+    what = (tuple(root.shape), tuple(root.stride()), root.dtype, root.data_ptr(), slices, x_shape)
     entry = _CAUSAL_VERDICTS.get(id(root))
     if entry is not None and entry[0]() is root and entry[1] == root._version and entry[2] == what:
         return entry[3]
     sub = root
     for dim, start, end, step in slices:
         sub = sub[(slice(None),) * (dim % sub.dim()) + (slice(start, end, step),)]
-    q, cols = x.shape[-2], x.shape[-1]
+    q, cols = x_shape
     verdict = 0
     if sub.dim() >= 2 and tuple(sub.shape[-2:]) == (q, cols) and sub.numel() == q * cols:
         keep = torch.ones(q, cols, dtype=torch.bool, device=sub.device).tril()
@@ -424,7 +538,27 @@ def _fused_masked_softmax(x, scale, root, slices, dim):
     return _BUILTIN_SOFTMAX(filled, dim, False)
 
 
+def _fused_attention(q, k, v, scale, root, slices):
+    """clone(transpose(bmm(softmax(masked_fill(bmm(q, k^T) * scale, mask == 0, -inf)), v), 1, 2))
+    for [batch, heads, tokens, head_dim] q, k, v (views of a packed projection as they come)."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    b, h, t, d = q.shape
+    s_len = k.shape[2]
+    if scale > 0 and hip_ops.attention_supported(q, k, v) and \
+            _causal_q_len(root, slices, (t, s_len)) == t:
+        return hip_ops.attention(q, k, v, scale, True)
+    # the unfused chain, op by op as the graph had it
+    flat = lambda x: x.expand(x.shape).clone(memory_format=torch.contiguous_format).view(  # noqa: E731
+        b * h, x.shape[2], x.shape[3])
+    scores = _BUILTIN_BMM(flat(q), flat(k.transpose(-2, -1))).view(b, h, t, s_len)
+    probs = _fused_masked_softmax(scores, scale, root, slices, -1)
+    ctx = _BUILTIN_BMM(probs.expand(probs.shape).view(b * h, t, s_len), flat(v)).view(b, h, t, d)
+    return ctx.transpose(1, 2).clone(memory_format=torch.contiguous_format)
+
+
 _BUILTIN_ADDMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.addmm]
+_BUILTIN_BMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.bmm]
 _BUILTIN_GELU = MAPPING_TORCH_ATEN_TO_MOJO[aten.gelu]
 _BUILTIN_SOFTMAX = MAPPING_TORCH_ATEN_TO_MOJO[aten._softmax]
 _BUILTIN_MASKED_FILL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.masked_fill)
@@ -434,6 +568,7 @@ _BUILTIN_SLICE = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.slice)
 _BUILTIN_ALIAS = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.alias)
 _FUSED_ADDMM_GELU = _fused_addmm_gelu
 _FUSED_MASKED_SOFTMAX = _fused_masked_softmax
+_FUSED_ATTENTION = _fused_attention
 
 
 class BaseMaxCompiler:
