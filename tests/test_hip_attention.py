@@ -108,3 +108,37 @@ def test_attention_rejects_what_it_cannot_take():
     assert not ops.attention_supported(q.cpu(), k.cpu(), v.cpu())
     with pytest.raises(ValueError):
         ops.attention(q[..., :32], k[..., :32], v[..., :32], 1.0, True)
+
+
+def test_registry_entry_for_scaled_dot_product_attention():
+    """aten.scaled_dot_product_attention: HIP kernel when it can take the call, PyTorch-ROCm's
+    op otherwise; same shape and layout contract ([batch, heads, tokens, head_dim])."""
+    from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO
+    fn = MAPPING_TORCH_ATEN_TO_MOJO[torch.ops.aten.scaled_dot_product_attention]
+    q, k, v = (x.cuda() for x in _qkv(2, 4, 100, 100, torch.bfloat16, seed=5))
+    got = fn(q, k, v, is_causal=True)
+    assert got.shape == (2, 4, 100, 64)
+    want = cf.attention(as64(q), as64(k), as64(v), 0.125, True).transpose(0, 2, 1, 3)
+    assert np.abs(as64(got) - want).max() <= 3e-2
+    # float32 and an explicit mask are not the kernel's: PyTorch's op answers
+    mask = torch.ones(100, 100, dtype=torch.bool, device="cuda").tril()
+    via_mask = fn(q, k, v, attn_mask=mask)
+    assert np.abs(as64(via_mask) - want).max() <= 3e-2
+    f32 = fn(q.float(), k.float(), v.float(), is_causal=True)
+    assert f32.dtype == torch.float32 and np.abs(as64(f32) - want).max() <= 1e-4
+
+
+def test_eager_device_scaled_dot_product_attention():
+    from torch_mojo_backend.eager_kernels import aten_fast
+    from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
+    q, k, v = (x.cuda() for x in _qkv(1, 2, 70, 70, torch.float16, seed=8))
+    wrap = lambda t: aten_fast._wrap(t)  # noqa: E731
+    out = aten_fast.fast_aten_scaled_dot_product_attention(wrap(q), wrap(k), wrap(v), is_causal=True)
+    assert isinstance(out, TorchMojoTensor) and tuple(out._shape) == (1, 2, 70, 64)
+    want = cf.attention(as64(q), as64(k), as64(v), 0.125, True).transpose(0, 2, 1, 3)
+    assert np.abs(as64(out._holder) - want).max() <= 4e-3
+    # what it cannot take is handed back
+    assert aten_fast.fast_aten_scaled_dot_product_attention(
+        wrap(q), wrap(k), wrap(v), dropout_p=0.1) is aten_fast.NOT_HANDLED
+    assert aten_fast.fast_aten_scaled_dot_product_attention(
+        wrap(q.float()), wrap(k.float()), wrap(v.float())) is aten_fast.NOT_HANDLED

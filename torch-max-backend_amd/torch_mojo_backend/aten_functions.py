@@ -26,6 +26,8 @@ import operator
 import os
 from typing import List, Optional
 
+import math
+
 import torch
 from torch._decomp import core_aten_decompositions
 from torch._ops import OpOverload, OpOverloadPacket
@@ -249,6 +251,22 @@ def aten_argmax(input: torch.Tensor, dim: Optional[int] = None, keepdim: bool = 
 def aten_gelu(input: torch.Tensor, approximate: str = "none") -> torch.Tensor:
     """reference :2063-2067."""
     return hip_ops.gelu(input, approximate)
+
+
+@map_to(aten.scaled_dot_product_attention)
+def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p: float = 0.0,
+                                      is_causal: bool = False, *, scale=None,
+                                      enable_gqa: bool = False) -> torch.Tensor:
+    """reference :3029-3087 (built there from matmul, softmax and matmul graph ops). The fused
+    HIP kernel takes the call when there is no explicit mask, no dropout, head_dim 64 and a
+    16-bit dtype; anything else is PyTorch-ROCm's own op."""
+    if attn_mask is None and dropout_p == 0.0 and not enable_gqa and query.dim() == 4 \
+            and hip_ops.attention_supported(query, key, value):
+        s = float(scale) if scale is not None else 1.0 / math.sqrt(query.shape[-1])
+        if s > 0.0:
+            return hip_ops.attention(query, key, value, s, bool(is_causal)).transpose(1, 2)
+    return aten.scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal,
+                                             scale=scale, enable_gqa=enable_gqa)
 
 
 HOT_OPS = (aten.mm, aten.bmm, aten.addmm, aten.linear, aten._softmax, aten.softmax,

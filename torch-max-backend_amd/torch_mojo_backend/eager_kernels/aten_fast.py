@@ -166,6 +166,23 @@ def fast_aten__log_softmax(input, dim, half_to_float=False):
 
 
 # ---------------------------------------------------------------------------
+# Attention (reference :5177-5285)
+# ---------------------------------------------------------------------------
+def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0,
+                                           is_causal=False, *, scale=None, enable_gqa=False):
+    q, k, v = _t(query), _t(key), _t(value)
+    if q is None or k is None or v is None or not _same_device(q, k, v):
+        return NOT_HANDLED
+    if attn_mask is not None or dropout_p != 0.0 or enable_gqa or len(q._shape) != 4:
+        return NOT_HANDLED
+    s = float(scale) if scale is not None else 1.0 / math.sqrt(q._shape[-1])
+    if not s > 0.0 or not hip_ops.attention_supported(q._holder, k._holder, v._holder):
+        return NOT_HANDLED
+    out = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal))
+    return _wrap(out.transpose(1, 2))  # [batch, heads, tokens, head_dim] view, as ATen returns it
+
+
+# ---------------------------------------------------------------------------
 # Layer norm (reference :2704-2794)
 # ---------------------------------------------------------------------------
 def fast_aten_native_layer_norm(input, normalized_shape, weight, bias, eps):
