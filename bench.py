@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot-op kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|gpt2|copy|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|gpt2|copy|all]
 
 Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
@@ -48,7 +48,7 @@ def _parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "gpt2", "copy"])
+    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "gpt2", "copy"])
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return p.parse_args()
 
@@ -226,6 +226,35 @@ def main() -> int:
             row["cpu_GB/s"] = round(t[1] / t[0] / 1e9, 3)
             row["cpu_note"] = t[2]
         sweep[name] = row
+
+    if want in ("all", "attn"):
+        # attention of the GPT-2 workload (B=32, H=12, T=1024, head_dim 64, bf16), q/k/v as the
+        # strided thirds of the packed projection, exactly as the compiled graph hands them over
+        Bq, Hq, Tq = 32, 12, 1024
+        qkv = gen((Bq, Tq, 3 * Hq * 64), 30, torch.bfloat16)
+        q4, k4, v4 = (x.view(Bq, Tq, Hq, 64).transpose(1, 2) for x in qkv.split(Hq * 64, dim=2))
+        _, ms = timed(lambda: hip_ops.attention(q4, k4, v4, 0.125, True), 30, 8)
+        useful = 4.0 * Bq * Hq * Tq * Tq * 64 / 2   # causal: half of the score matrix
+        algo_bytes = 4 * Bq * Hq * Tq * 64 * 2      # q, k, v in, out once
+        sweep["attention_causal_bf16_32x12x1024x64"] = {
+            "us": round(ms * 1e3, 2), "TFLOP/s": round(useful / ms / 1e9, 1),
+            "frac_mfma": round(useful / ms / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4),
+            "GB/s": round(algo_bytes / ms / 1e6, 1), "flops": useful, "bytes": algo_bytes,
+            "note": "useful FLOPs (masked half not counted); scores never reach memory"}
+        # the softmax of the same attention when it runs on its own: [B*H*T, T] scores in,
+        # probabilities out; the masked half of every row is not read
+        rows, cols = Bq * Hq * Tq, Tq
+        xs = [gen((Bq * Hq, Tq, Tq), 31 + i, torch.bfloat16, scale=4.0) for i in range(2)]
+        os_ = [torch.empty_like(x) for x in xs]
+        code = hip_ops.code_of(torch.bfloat16)
+        nbytes = rows * cols * 2
+        hbm_row("softmax_scaled_causal_bf16_393216x1024", 2,
+                lambda i: lib.tmb_softmax_rows_scaled(os_[i].data_ptr(), xs[i].data_ptr(), rows, cols,
+                                                      code, 0.125, 1, Tq, stream),
+                nbytes // 2 + nbytes, steps=30)
+        sweep["softmax_scaled_causal_bf16_393216x1024"]["note"] = \
+            "bytes = half of the input (causal) + the whole output"
+        del xs, os_, qkv
 
     if want in ("all", "rows"):
         import oracle
