@@ -128,10 +128,11 @@ def test_bmm(dtype):
 # K >= 256 takes the direct-to-LDS ring kernel; the shapes are chosen so that each of its tile
 # configurations runs, with ragged M and N edges: 256x256 with 64-deep stages (256 tiles = one
 # round of the 256 CUs; K = 320 is five stages), 256x128 (528 tiles), 128x128 with 32-deep stages
-# (K = 352 is not a multiple of 64), and shapes that stay on the register-staged kernel
-# (few tiles, K < 256).
+# (K = 352 is not a multiple of 64), the short-K rings that run two workgroups per CU (256x128x32
+# for K-major B at (8000, 2200, 352); 128x256x32 for the N-major twins of the large shapes), and
+# shapes that stay on the register-staged kernel (few tiles, K < 256).
 KMAJOR = [(3900, 4000, 320), (4000, 4100, 256), (4000, 4104, 448), (600, 1000, 352),
-          (1000, 5000, 128), (130, 70, 1152)]
+          (8000, 2200, 352), (1000, 5000, 128), (130, 70, 1152)]
 
 
 @pytest.mark.parametrize("dtype", HALF)

@@ -107,6 +107,14 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
   // the idle tail. N-major B is staged in whole 16-byte column chunks, so N must be a multiple
   // of 8 there (nothing past column N-1 is ever read).
   if (g.k >= 256 && g.n > 64 && (B_KMAJOR || g.n % 8 == 0)) {
+    // Short K: the prologue and epilogue of a tile weigh as much as its main loop, so rings that
+    // leave room for two workgroups per CU (72 KB of LDS each) win by overlapping them.
+    if (g.k % 32 == 0) {
+      if (!B_KMAJOR && g.k < 4096 && tiles(128, 256) >= 256)
+        return launch_ring<T, 128, 256, 32, 2, 4, 3, B_KMAJOR, EPI>(g, batch, stream);
+      if (B_KMAJOR && g.k <= 1024 && g.n <= 2304 && tiles(256, 128) >= 512)
+        return launch_ring<T, 256, 128, 32, 4, 2, 3, B_KMAJOR, EPI>(g, batch, stream);
+    }
     if (g.k % 64 == 0) {
       const int64_t t256 = tiles(256, 256);
       const int64_t rounds = (t256 + 255) / 256;

@@ -63,8 +63,21 @@ __device__ __forceinline__ void wait_vm_lgkm0() {
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
+// Waves per SIMD the kernel is compiled for: as many workgroups as the ring leaves room for in
+// the 160 KB LDS (at most two: a second workgroup overlaps its prologue and epilogue with the
+// first one's main loop), provided the accumulators fit the register share that leaves.
+constexpr int ring_waves_per_simd(int bm, int bn, int bk, int waves, int stages) {
+  const int lds = stages * (bm + bn) * bk * 2;
+  const int wgs = 160 * 1024 / lds >= 2 ? 2 : 1;
+  const int acc = (bm * bn) / (waves * 64);  // fp32 accumulator registers per lane
+  const int want = wgs * waves / 4;
+  return (want >= 1 && acc + 64 <= 512 / want) ? want : (waves / 4 >= 1 ? waves / 4 : 1);
+}
+
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_ring_kernel(GemmArgs g) {
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
+                             ring_waves_per_simd(BM, BN, BK, WAVES_M* WAVES_N, R))
+void gemm_ring_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
