@@ -153,10 +153,10 @@ __device__ __forceinline__ typename Policy::acc_t stream_range(const T* __restri
   const int64_t nvec = (n - head) / EPV;
   int64_t i = tid;
   for (; i + 3 * NT < nvec; i += 4 * NT) {
-    const Vec16<T> v0 = load_vec16(body + i * EPV);
-    const Vec16<T> v1 = load_vec16(body + (i + NT) * EPV);
-    const Vec16<T> v2 = load_vec16(body + (i + 2 * NT) * EPV);
-    const Vec16<T> v3 = load_vec16(body + (i + 3 * NT) * EPV);
+    const Vec16<T> v0 = load_vec16_stream(body + i * EPV);
+    const Vec16<T> v1 = load_vec16_stream(body + (i + NT) * EPV);
+    const Vec16<T> v2 = load_vec16_stream(body + (i + 2 * NT) * EPV);
+    const Vec16<T> v3 = load_vec16_stream(body + (i + 3 * NT) * EPV);
 #pragma unroll
     for (int e = 0; e < EPV; ++e) {
       acc_one<Policy, T, IMAX>(acc0, v0.v[e]);
@@ -166,7 +166,7 @@ __device__ __forceinline__ typename Policy::acc_t stream_range(const T* __restri
     }
   }
   for (; i < nvec; i += NT) {
-    const Vec16<T> v0 = load_vec16(body + i * EPV);
+    const Vec16<T> v0 = load_vec16_stream(body + i * EPV);
 #pragma unroll
     for (int e = 0; e < EPV; ++e) acc_one<Policy, T, IMAX>(acc0, v0.v[e]);
   }
@@ -394,7 +394,7 @@ __device__ __forceinline__ Best<typename ArgTraits<T>::val_t> argmax_range(const
   for (; i + 3 * NT < nvec; i += 4 * NT) {  // four 16-byte loads in flight per lane
     Vec16<T> v[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = load_vec16(body + static_cast<int64_t>(i + u * NT) * EPV);
+    for (int u = 0; u < 4; ++u) v[u] = load_vec16_stream(body + static_cast<int64_t>(i + u * NT) * EPV);
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
@@ -402,7 +402,7 @@ __device__ __forceinline__ Best<typename ArgTraits<T>::val_t> argmax_range(const
         scan_one(best, off, ArgTraits<T>::conv(v[u].v[e]), head + (i + u * NT) * EPV + e);
   }
   for (; i < nvec; i += NT) {
-    const Vec16<T> v0 = load_vec16(body + static_cast<int64_t>(i) * EPV);
+    const Vec16<T> v0 = load_vec16_stream(body + static_cast<int64_t>(i) * EPV);
 #pragma unroll
     for (int e = 0; e < EPV; ++e) scan_one(best, off, ArgTraits<T>::conv(v0.v[e]), head + i * EPV + e);
   }
