@@ -54,7 +54,7 @@ def test_addmm_small_vs_c_oracle(mnk, dtype, trans_b):
     assert_close64(got, as64(ref), extra_abs=2 * bound, rounded_want=True, what="vs C oracle")
 
 
-# BASELINE config 1 shapes that the CPU can check in seconds + the reference's awkward shapes
+# Benchmark GEMM shapes that the CPU can check in seconds + the reference's awkward shapes
 # (N=50257 / 3001 unaligned, K=1000, M=257).
 MID = [(128, 768, 768), (1024, 3072, 768), (1024, 768, 3072), (512, 2304, 768), (257, 3001, 1000),
        (512, 50257, 768), (300, 260, 264)]

@@ -202,7 +202,7 @@ def test_softmax_scaled_rounding_reproduces_the_three_op_pipeline(dtype):
 
 
 def test_softmax_scaled_full_size_invariants():
-    """BASELINE attention shape [32*12, 1024, 1024] bf16: rows sum to one, zeros above the
+    """Benchmark attention shape [32*12, 1024, 1024] bf16: rows sum to one, zeros above the
     diagonal, first row is exactly [1, 0, ...]."""
     g = torch.Generator(device="cuda").manual_seed(5)
     x = (torch.randn(96, 1024, 1024, generator=g, device="cuda") * 4).bfloat16()
