@@ -113,11 +113,15 @@ __device__ __forceinline__ float pin_f32(float v) {
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
 #pragma clang fp contract(off)
-  constexpr float kAlpha = 0.7978845608028654f;  // sqrt(2/pi)
-  const float u = kAlpha * (x + 0.044715f * x * x * x);
-  // tanh(u) = 1 - 2/(exp(2u)+1): saturates cleanly to +-1 for large |u|.
-  const float t = 1.0f - 2.0f / (exp_f32(2.0f * u) + 1.0f);
-  return pin_f32(0.5f * x * (1.0f + t));
+  // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3): no
+  // cancellation for negative x, one v_exp_f32 and one v_rcp_f32. With the constants folded,
+  // -2u log2(e) = x (c1 + c2 x^2); its three roundings cost at most 2e-7 |arg| in the exponent,
+  // i.e. < 3e-6 relative wherever the result is above 1e-7 |x|.
+  constexpr float c1 = -2.302208198144325f;   // -2 log2(e) sqrt(2/pi)
+  constexpr float c2 = -0.1029432395800235f;  // c1 * 0.044715
+  const float arg = x * __builtin_fmaf(x * x, c2, c1);
+  const float e = __builtin_amdgcn_exp2f(arg);  // +inf for very negative x: the quotient is -0
+  return pin_f32(x * __builtin_amdgcn_rcpf(1.0f + e));
 }
 __device__ __forceinline__ float gelu_erf_f32(float x) {
 #pragma clang fp contract(off)
