@@ -74,6 +74,9 @@ constexpr int ring_waves_per_simd(int bm, int bn, int bk, int waves, int stages)
   return (want >= 1 && acc + 64 <= 512 / want) ? want : (waves / 4 >= 1 ? waves / 4 : 1);
 }
 
+template <int BM, int BN, int BK, int WAVES, int R>
+constexpr bool kRingPersistent = ring_waves_per_simd(BM, BN, BK, WAVES, R) <= 2;
+
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
                              ring_waves_per_simd(BM, BN, BK, WAVES_M* WAVES_N, R))
@@ -99,10 +102,7 @@ void gemm_ring_kernel(GemmArgs g) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  int tile_m, tile_n;
-  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
-  const int64_t m0 = static_cast<int64_t>(tile_m) * BM;
-  const int64_t n0 = static_cast<int64_t>(tile_n) * BN;
+  int64_t m0 = 0, n0 = 0;  // origin of the tile being worked on (set per tile below)
   const int64_t batch = blockIdx.y;
   const int64_t M = g.m, N = g.n;
   T* __restrict__ C = static_cast<T*>(g.c) + batch * g.stride_c;
@@ -115,6 +115,7 @@ void gemm_ring_kernel(GemmArgs g) {
   // Rows past the edge re-read the last valid row; their results are never stored.
   const int r_in = lane / LPR, slot = lane % LPR;
   uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
+  auto plan_tile_loads = [&]() {
 #pragma unroll
   for (int j = 0; j < A_GROUPS; ++j) {
     const int row = (wave * A_GROUPS + j) * RPG + r_in;
@@ -141,6 +142,7 @@ void gemm_ring_kernel(GemmArgs g) {
       b_off[j] = static_cast<uint32_t>((krow * g.ldb + col) * 2);
     }
   }
+  };
   const int64_t b_kstep = B_KMAJOR ? 2 : g.ldb * 2;  // bytes per unit of k in B
 
   // The loads are written as inline assembly: M0 carries the LDS destination of the wave's
@@ -170,12 +172,6 @@ void gemm_ring_kernel(GemmArgs g) {
   };
 
   f32x16_t acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // Fragment addresses as LDS byte offsets inside a stage: one per-lane register per k-step
   // (the XOR swizzle is not additive in the k chunk) and, for N-major B, per 32-column tile;
@@ -264,6 +260,25 @@ void gemm_ring_kernel(GemmArgs g) {
 
   // The launcher guarantees k % BK == 0 and at least R-1 stages of k.
   const int64_t k_tiles = g.k / BK;
+  // Persistent workgroups: the grid covers the CUs once and each workgroup walks the tile list
+  // with the grid's stride, which hands every XCD the same sequence of tiles as one launch per
+  // tile would. The stores of a tile drain while the next tile's operands are already being
+  // fetched and multiplied.
+  const int64_t total_tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
+  auto run_tile = [&](int64_t pid) {
+  {
+    int tile_m, tile_n;
+    tile_of_block(static_cast<int>(pid), g.tiles_m, g.tiles_n, tile_m, tile_n);
+    m0 = static_cast<int64_t>(tile_m) * BM;
+    n0 = static_cast<int64_t>(tile_n) * BN;
+    plan_tile_loads();
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  }
   {
     uint32_t off = 0;
 #pragma unroll
@@ -307,7 +322,33 @@ void gemm_ring_kernel(GemmArgs g) {
   lds_byte_t* band = (lds_byte_t*)ring + wave * BandLayout<WN>::BYTES;
   store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
                                   g.vec_store != 0, lane);
+  };
+  // Configurations compiled for four waves per SIMD have no registers to spare for the loop
+  // state; their second resident workgroup already overlaps the tile boundaries.
+  if constexpr (kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R>) {
+#pragma unroll 1
+    for (int64_t pid = blockIdx.x; pid < total_tiles; pid += gridDim.x) {
+      run_tile(pid);
+      __syncthreads();  // the staging bands overlay the ring: all read back before the next fetch
+    }
+  } else {
+    run_tile(blockIdx.x);
+  }
 #endif
+}
+
+// CUs of the current device (queried once per process).
+static int compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
 }
 
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
@@ -319,8 +360,18 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
                 ((reinterpret_cast<uintptr_t>(g.c) & 15u) == 0);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
+  // as many workgroups as the device holds at once (a multiple of the 8 XCDs), shared between
+  // the batch entries; each walks the tile list
+  constexpr int kWgPerCu = ring_waves_per_simd(BM, BN, BK, WAVES_M * WAVES_N, R) * 4 /
+                                       (WAVES_M * WAVES_N) >= 2 ? 2 : 1;
+  int64_t resident = static_cast<int64_t>(compute_units()) * kWgPerCu / batch;
+  resident = resident / 8 * 8;
+  if (resident < 8) resident = 8;
+  const int64_t grid_x = (!kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R> || tiles < resident)
+                             ? tiles
+                             : resident;
   gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI>
-      <<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)),
+      <<<dim3(static_cast<unsigned>(grid_x), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();
 }
