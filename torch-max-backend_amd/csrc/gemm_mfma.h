@@ -75,7 +75,6 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int64_t stride_a, stride_b, stride_c;
   int tiles_m, tiles_n;
-  int vec_store;  // C rows start on 16-byte boundaries: 8 columns per store
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
@@ -148,47 +147,34 @@ __device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, int64_t c
   }
 }
 
-// Writes the staged 32 x WN band to C. vec16: rows of C start on 16-byte boundaries (pitch and
-// base), so a lane stores 8 columns at once; otherwise lanes store single elements, still
-// consecutive along the row.
+// Writes the staged 32 x WN band to C: a lane stores 8 columns (16 bytes) at once, consecutive
+// lanes along the row. Rows of C need not start on 16-byte boundaries (an odd pitch, as with a
+// 50257-wide vocabulary, leaves them 2-byte aligned): global memory takes unaligned vector
+// accesses on this target, and one 16-byte store per lane beats eight 2-byte ones by far.
+typedef u32x4_t __attribute__((aligned(2))) u32x4_unaligned_t;
+
 template <typename T, int WN>
 __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict__ C, int64_t ldc,
                                            int64_t row0, int64_t col0, int64_t M, int64_t N,
-                                           bool vec16, int lane) {
+                                           int lane) {
   constexpr int PITCH = BandLayout<WN>::PITCH;
-  if (vec16) {
-    constexpr int LPR = WN / 8;    // lanes per row
-    constexpr int RPP = 64 / LPR;  // rows per pass
+  constexpr int LPR = WN / 8;    // lanes per row
+  constexpr int RPP = 64 / LPR;  // rows per pass
 #pragma unroll
-    for (int p = 0; p < 32 / RPP; ++p) {
-      const int r = p * RPP + lane / LPR;
-      const int c = (lane % LPR) * 8;
-      const u32x4_t v = *(const lds_u32x4v_t*)(band + r * PITCH + c * 2);
-      const int64_t row = row0 + r, col = col0 + c;
-      if (row < M && col < N) {
-        T* dst = C + row * ldc + col;
-        if (col + 8 <= N) {
-          *reinterpret_cast<u32x4_t*>(dst) = v;
-        } else {
+  for (int p = 0; p < 32 / RPP; ++p) {
+    const int r = p * RPP + lane / LPR;
+    const int c = (lane % LPR) * 8;
+    const u32x4_t v = *(const lds_u32x4v_t*)(band + r * PITCH + c * 2);
+    const int64_t row = row0 + r, col = col0 + c;
+    if (row < M && col < N) {
+      T* dst = C + row * ldc + col;
+      if (col + 8 <= N) {
+        *reinterpret_cast<u32x4_unaligned_t*>(dst) = v;
+      } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (col + e < N)
-              dst[e] = __builtin_bit_cast(T, static_cast<unsigned short>(v[e >> 1] >> (16 * (e & 1))));
-        }
-      }
-    }
-  } else {
-    typedef __attribute__((address_space(3))) unsigned short lds_u16_t;
-#pragma unroll 4
-    for (int r = 0; r < 32; ++r) {
-      const int64_t row = row0 + r;
-      if (row >= M) break;
-#pragma unroll
-      for (int c0 = 0; c0 < WN; c0 += 64) {
-        const int c = c0 + lane;
-        if (c < WN && col0 + c < N)
-          C[row * ldc + col0 + c] =
-              __builtin_bit_cast(T, *(const lds_u16_t*)(band + r * PITCH + c * 2));
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N)
+            dst[e] = __builtin_bit_cast(T, static_cast<unsigned short>(v[e >> 1] >> (16 * (e & 1))));
       }
     }
   }
@@ -201,7 +187,7 @@ template <typename T, int EPI, int TM, int TN>
 __device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
                                                 T* __restrict__ C, int64_t ldc, int64_t row0,
                                                 int64_t col0, int64_t M, int64_t N,
-                                                const T* __restrict__ bias, bool vec16, int lane) {
+                                                const T* __restrict__ bias, int lane) {
   constexpr int WN = TN * 32;
   constexpr int PITCH = BandLayout<WN>::PITCH;
   lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
@@ -211,7 +197,7 @@ __device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byt
 #pragma unroll
     for (int j = 0; j < TN; ++j)
       stage_tile<T, EPI>(acc[i][j], mine + j * 64, col0 + j * 32 + 4 * (lane >> 5), N, bias);
-    flush_band<T, WN>(band, C, ldc, row0 + i * 32, col0, M, N, vec16, lane);
+    flush_band<T, WN>(band, C, ldc, row0 + i * 32, col0, M, N, lane);
   }
 }
 
@@ -432,7 +418,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmAr
   static_assert(WAVES_M * WAVES_N * BandLayout<WN>::BYTES <= 2 * STAGE_BYTES, "band staging");
   lds_byte_t* band = (lds_byte_t*)smem + wave * BandLayout<WN>::BYTES;
   store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  g.vec_store != 0, lane);
+                                  lane);
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
@@ -450,8 +436,6 @@ static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
-  g.vec_store = (g.ldc % 8 == 0) && (g.stride_c % 8 == 0 || batch == 1) &&
-                ((reinterpret_cast<uintptr_t>(g.c) & 15u) == 0);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), SMEM, stream>>>(g);
