@@ -219,7 +219,7 @@ extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias,
   }
   if (batch > 65535) return TMB_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0};
+  GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0, 0};
   if (k == 0) {
     const unsigned blocks = static_cast<unsigned>((m * n + 255) / 256 > 4096 ? 4096 : (m * n + 255) / 256);
     dim3 grid(blocks, static_cast<unsigned>(batch));

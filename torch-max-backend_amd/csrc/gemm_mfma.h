@@ -75,6 +75,7 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int64_t stride_a, stride_b, stride_c;
   int tiles_m, tiles_n;
+  int stream_c;  // C is larger than the 256 MB Infinity Cache: store it non-temporally
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
@@ -116,28 +117,37 @@ struct BandLayout {
   static constexpr int BYTES = 32 * PITCH;
 };
 
+typedef u32x2_t __attribute__((aligned(2))) u32x2_unaligned_t;
+
+// The four bias values a lane needs for columns col .. col+3 (zeros past N or without bias),
+// packed as stored. One 8-byte load where the row allows it.
+template <typename T>
+__device__ __forceinline__ u32x2_t load_bias4(const T* __restrict__ bias, int64_t col, int64_t N) {
+  u32x2_t out = {0u, 0u};
+  if (bias == nullptr || col >= N) return out;
+  if (col + 4 <= N) return *reinterpret_cast<const u32x2_unaligned_t*>(bias + col);
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (col + e < N)
+      out[e >> 1] |= static_cast<uint32_t>(__builtin_bit_cast(unsigned short, bias[col + e]))
+                     << (16 * (e & 1));
+  return out;
+}
+
+template <typename T>
+__device__ __forceinline__ float unpack_elem(u32x2_t v, int e) {
+  return to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(v[e >> 1] >> (16 * (e & 1)))));
+}
+
 template <typename T, int EPI>
-__device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, int64_t col0, int64_t N,
-                                        const T* __restrict__ bias) {
+__device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, u32x2_t b0, u32x2_t b1,
+                                        u32x2_t b2, u32x2_t b3) {
+  const u32x2_t bq[4] = {b0, b1, b2, b3};
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    const int64_t col = col0 + 8 * q;
-    float v[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = acc[4 * q + e];
-    if (bias != nullptr) {
-      if (col + 4 <= N) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] += to_f32(bias[col + e]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (col + e < N) v[e] += to_f32(bias[col + e]);  // columns past N are never stored
-      }
-    }
     T o[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(v[e]);
+    for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(acc[4 * q + e] + unpack_elem<T>(bq[q], e));
     u32x2_t packed;
     packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
                 (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
@@ -153,7 +163,7 @@ __device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, int64_t c
 // accesses on this target, and one 16-byte store per lane beats eight 2-byte ones by far.
 typedef u32x4_t __attribute__((aligned(2))) u32x4_unaligned_t;
 
-template <typename T, int WN>
+template <typename T, int WN, bool STREAM>
 __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict__ C, int64_t ldc,
                                            int64_t row0, int64_t col0, int64_t M, int64_t N,
                                            int lane) {
@@ -169,7 +179,13 @@ __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict
     if (row < M && col < N) {
       T* dst = C + row * ldc + col;
       if (col + 8 <= N) {
-        *reinterpret_cast<u32x4_unaligned_t*>(dst) = v;
+        // STREAM is a template parameter on purpose: as a run-time branch the two stores are
+        // merged and the non-temporal hint is lost
+        if constexpr (STREAM) {
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4_unaligned_t*>(dst));
+        } else {
+          *reinterpret_cast<u32x4_unaligned_t*>(dst) = v;
+        }
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -183,21 +199,43 @@ __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict
 // The whole wave tile (TM x TN tiles of 32x32), one 32-row band at a time through `band`
 // (wave-private, BandLayout<WN>::BYTES). The caller has synchronised the workgroup so that
 // nobody still reads operands from the LDS that `band` overlays.
-template <typename T, int EPI, int TM, int TN>
-__device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
+template <typename T, int EPI, int TM, int TN, bool STREAM>
+__device__ __forceinline__ void store_wave_tile_impl(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
                                                 T* __restrict__ C, int64_t ldc, int64_t row0,
                                                 int64_t col0, int64_t M, int64_t N,
                                                 const T* __restrict__ bias, int lane) {
   constexpr int WN = TN * 32;
   constexpr int PITCH = BandLayout<WN>::PITCH;
   lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
+  // The bias a lane adds depends on its columns only: fetched once for the whole wave tile
+  // (the operand fragments' registers are free by now).
+  u32x2_t bfrag[TN][4];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      bfrag[j][q] = load_bias4<T>(bias, col0 + j * 32 + 4 * (lane >> 5) + 8 * q, N);
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     if (row0 + i * 32 >= M) break;  // wave-uniform
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      stage_tile<T, EPI>(acc[i][j], mine + j * 64, col0 + j * 32 + 4 * (lane >> 5), N, bias);
-    flush_band<T, WN>(band, C, ldc, row0 + i * 32, col0, M, N, lane);
+      stage_tile<T, EPI>(acc[i][j], mine + j * 64, bfrag[j][0], bfrag[j][1], bfrag[j][2],
+                         bfrag[j][3]);
+    flush_band<T, WN, STREAM>(band, C, ldc, row0 + i * 32, col0, M, N, lane);
+  }
+}
+
+template <typename T, int EPI, int TM, int TN>
+__device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
+                                                T* __restrict__ C, int64_t ldc, int64_t row0,
+                                                int64_t col0, int64_t M, int64_t N,
+                                                const T* __restrict__ bias, bool stream,
+                                                int lane) {
+  if (stream) {
+    store_wave_tile_impl<T, EPI, TM, TN, true>(acc, band, C, ldc, row0, col0, M, N, bias, lane);
+  } else {
+    store_wave_tile_impl<T, EPI, TM, TN, false>(acc, band, C, ldc, row0, col0, M, N, bias, lane);
   }
 }
 
@@ -418,7 +456,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmAr
   static_assert(WAVES_M * WAVES_N * BandLayout<WN>::BYTES <= 2 * STAGE_BYTES, "band staging");
   lds_byte_t* band = (lds_byte_t*)smem + wave * BandLayout<WN>::BYTES;
   store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  lane);
+                                  g.stream_c != 0, lane);
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
@@ -436,6 +474,7 @@ static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
+  g.stream_c = g.m * g.n * batch * 2 >= (int64_t{256} << 20);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), SMEM, stream>>>(g);

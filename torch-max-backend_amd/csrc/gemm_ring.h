@@ -321,7 +321,7 @@ void gemm_ring_kernel(GemmArgs g) {
   static_assert(NW * BandLayout<WN>::BYTES <= R * STAGE_BYTES, "band staging");
   lds_byte_t* band = (lds_byte_t*)ring + wave * BandLayout<WN>::BYTES;
   store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  lane);
+                                  g.stream_c != 0, lane);
   };
   // Configurations compiled for four waves per SIMD have no registers to spare for the loop
   // state; their second resident workgroup already overlaps the tile boundaries.
@@ -356,6 +356,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
+  g.stream_c = g.m * g.n * batch * 2 >= (int64_t{256} << 20);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   // as many workgroups as the device holds at once (a multiple of the 8 XCDs), shared between
