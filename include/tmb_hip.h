@@ -117,6 +117,21 @@ int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t ba
              int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
              int epilogue, void* stream);
 
+/* tmb_gemm followed by an elementwise add of `residual` [batch][m, n] (row pitch `ldr`, batch
+ * stride `stride_r`) in the same launch: c = T(float(T(epilogue(a b + bias))) + float(residual)),
+ * rounded twice exactly as a GEMM kernel followed by an add kernel would (the residual
+ * connection of a transformer block: demo_scripts/gpt2.py:85-86 `x = x + self.attn(...)`,
+ * which reaches the graph as addmm -> view -> add). 16-bit dtypes on the MFMA path only;
+ * TMB_ERR_UNSUPPORTED otherwise (fp32, k == 0, transposed A, unaligned operands): the caller then
+ * launches tmb_gemm and adds separately.
+ * Replaces `AddF32Bf16Spec` / the residual add of aten_fast.py:657-687 together with the GEMM
+ * in front of it. */
+int tmb_gemm_residual(void* c, const void* a, const void* b, const void* bias,
+                      const void* residual, int64_t batch, int64_t m, int64_t n, int64_t k,
+                      int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr, int64_t stride_a,
+                      int64_t stride_b, int64_t stride_c, int64_t stride_r, int trans_a,
+                      int trans_b, int dtype, int epilogue, void* stream);
+
 /* Fused attention forward: out[b,t,h,:] = softmax_j(scale * q[b,h,t,:] . k[b,h,j,:]) v[b,h,j,:],
  * with `causal` != 0 only keys j <= t take part. The [batch, heads, q_len, kv_len] scores never
  * reach memory (online softmax over blocks of 64 keys). `dtype` in {F16,BF16}; head_dim must

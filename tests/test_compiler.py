@@ -314,3 +314,40 @@ def test_attention_rewrite_plans_one_step_per_block(monkeypatch):
     names = [compiler._step_name(s) for s in programs[-1].steps]
     assert names.count("aten.mul+masked_fill+_softmax (fused)") == 2
     assert not any(s.fn is compiler._FUSED_ATTENTION for s in programs[-1].steps)
+
+
+def test_residual_add_rewrite(cpu_hot_ops):
+    """x + proj(h): addmm -> view -> add becomes one step over (bias, h, w^T, x)."""
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.proj = torch.nn.Linear(16, 16)
+
+        def forward(self, x, h):
+            return x + self.proj(h), torch.tanh(self.proj(h))   # the second use stays a plain addmm
+
+    programs = []
+    real = compiler._GraphFactory.create_graph
+
+    def spy(self, graph):
+        programs.append(real(self, graph))
+        return programs[-1]
+
+    import pytest as _pytest
+    mp = _pytest.MonkeyPatch()
+    mp.setattr(compiler._GraphFactory, "create_graph", spy)
+    try:
+        block = Block().eval()
+        x, h = torch.randn(2, 5, 16), torch.randn(2, 5, 16)
+        with torch.no_grad():
+            want = block(x, h)
+            got = torch.compile(block, backend=mojo_backend, fullgraph=True)(x, h)
+    finally:
+        mp.undo()
+    torch.testing.assert_close(got[0], want[0])
+    torch.testing.assert_close(got[1], want[1])
+    names = [compiler._step_name(s) for s in programs[-1].steps]
+    assert names.count("aten.addmm+add (fused)") == 1
+    fused = next(s for s in programs[-1].steps if s.fn is compiler._FUSED_ADDMM_RESIDUAL)
+    assert fused.args[4] == (2, 5, 16)
+    assert cpu_hot_ops.count("addmm") == 2     # one inside the fused step's host branch, one plain

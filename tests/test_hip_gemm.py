@@ -247,3 +247,48 @@ def test_queued_launches_are_bit_identical():
     outs = [_ops().gemm(ad, bd, cd) for _ in range(3)]
     torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+
+
+# residual added in the GEMM's own epilogue: must give the bits of gemm(...) + residual. Shapes
+# cover the ring configurations (see KMAJOR), the register-staged kernel (K = 128) and an odd
+# row pitch; float32 has no fused path and takes the separate add inside the same call.
+RESIDUAL = [(3900, 4000, 320), (4000, 4104, 448), (600, 1000, 352), (8000, 2200, 352),
+            (1000, 5000, 128), (512, 50257, 768), (32768, 768, 768)]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", RESIDUAL)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_residual_epilogue_equals_separate_add(mnk, dtype, trans_b):
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(21)
+    a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
+    b = (torch.randn(n, k, generator=g, device="cuda") * 0.1).to(dtype)
+    b = b.t() if trans_b else b.t().contiguous()
+    bias = torch.randn(n, generator=g, device="cuda").to(dtype)
+    res = torch.randn(m, n, generator=g, device="cuda").to(dtype)
+    fused = _ops().gemm(a, b, bias, residual=res)
+    plain = _ops().gemm(a, b, bias) + res
+    assert torch.equal(fused, plain)
+
+
+def test_residual_with_gelu_batches_and_fallbacks():
+    ek = _ek()
+    g = torch.Generator(device="cuda").manual_seed(22)
+    a = torch.randn(6, 300, 256, generator=g, device="cuda").bfloat16()
+    b = (torch.randn(6, 256, 200, generator=g, device="cuda") * 0.1).bfloat16()
+    res = torch.randn(6, 300, 200, generator=g, device="cuda").bfloat16()
+    assert torch.equal(_ops().gemm(a, b, residual=res), _ops().gemm(a, b) + res)
+    a2, b2, r2 = a[0], b[0], res[0]
+    bias = torch.randn(200, generator=g, device="cuda").bfloat16()
+    fused = _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH, residual=r2)
+    assert torch.equal(fused, _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH) + r2)
+    # a residual that is a column slice of something wider (row pitch > n)
+    wide = torch.randn(300, 512, generator=g, device="cuda").bfloat16()
+    assert torch.equal(_ops().gemm(a2, b2, bias, residual=wide[:, 100:300]),
+                       _ops().gemm(a2, b2, bias) + wide[:, 100:300])
+    # float32: no fused kernel, same call, same bits as the two ops
+    a32, b32, r32 = a2.float(), b2.float(), r2.float()
+    assert torch.equal(_ops().gemm(a32, b32, residual=r32), _ops().gemm(a32, b32) + r32)
+    with pytest.raises(ValueError):
+        _ops().gemm(a2, b2, residual=r2[:, :100])

@@ -200,10 +200,11 @@ __global__ void gemm_k0_kernel(T* c, const T* bias, int64_t m, int64_t n, int64_
 
 }  // namespace tmb
 
-extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t batch,
-                        int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
-                        int64_t stride_a, int64_t stride_b, int64_t stride_c, int trans_a,
-                        int trans_b, int dtype, int epilogue, void* stream) {
+static int gemm_entry(void* c, const void* a, const void* b, const void* bias,
+                      const void* residual, int64_t batch, int64_t m, int64_t n, int64_t k,
+                      int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr, int64_t stride_a,
+                      int64_t stride_b, int64_t stride_c, int64_t stride_r, int trans_a,
+                      int trans_b, int dtype, int epilogue, void* stream) {
   using namespace tmb;
   if (batch < 0 || m < 0 || n < 0 || k < 0) return TMB_ERR_INVALID_ARGUMENT;
   if (epilogue < TMB_EPI_NONE || epilogue > TMB_EPI_GELU_ERF) return TMB_ERR_INVALID_ARGUMENT;
@@ -219,7 +220,12 @@ extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias,
   }
   if (batch > 65535) return TMB_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0, 0};
+  GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0, 0, residual, ldr, stride_r};
+  if (residual != nullptr) {
+    // only the MFMA kernels carry the second epilogue step; the caller adds separately otherwise
+    if (dtype == TMB_F32 || k == 0 || ldr < n || !mfma_eligible(g, batch, trans_a, trans_b))
+      return TMB_ERR_UNSUPPORTED;
+  }
   if (k == 0) {
     const unsigned blocks = static_cast<unsigned>((m * n + 255) / 256 > 4096 ? 4096 : (m * n + 255) / 256);
     dim3 grid(blocks, static_cast<unsigned>(batch));
@@ -238,4 +244,23 @@ extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias,
     case TMB_F16: return gemm_epi<f16_t>(g, batch, trans_a, trans_b, epilogue, s);
     default: return gemm_epi<bf16_t>(g, batch, trans_a, trans_b, epilogue, s);
   }
+}
+
+extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t batch,
+                        int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
+                        int64_t stride_a, int64_t stride_b, int64_t stride_c, int trans_a,
+                        int trans_b, int dtype, int epilogue, void* stream) {
+  return gemm_entry(c, a, b, bias, nullptr, batch, m, n, k, lda, ldb, ldc, 0, stride_a, stride_b,
+                    stride_c, 0, trans_a, trans_b, dtype, epilogue, stream);
+}
+
+extern "C" int tmb_gemm_residual(void* c, const void* a, const void* b, const void* bias,
+                                 const void* residual, int64_t batch, int64_t m, int64_t n,
+                                 int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr,
+                                 int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                                 int64_t stride_r, int trans_a, int trans_b, int dtype,
+                                 int epilogue, void* stream) {
+  if (residual == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  return gemm_entry(c, a, b, bias, residual, batch, m, n, k, lda, ldb, ldc, ldr, stride_a,
+                    stride_b, stride_c, stride_r, trans_a, trans_b, dtype, epilogue, stream);
 }

@@ -76,6 +76,10 @@ struct GemmArgs {
   int64_t stride_a, stride_b, stride_c;
   int tiles_m, tiles_n;
   int stream_c;  // C is larger than the 256 MB Infinity Cache: store it non-temporally
+  // optional second epilogue step: C = T(float(T(epilogue(acc + bias))) + float(residual)),
+  // i.e. what a separate elementwise add after the GEMM would store (MFMA kernels only)
+  const void* residual;
+  int64_t ldr, stride_r;
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
@@ -163,10 +167,20 @@ __device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, u32x2_t b
 // accesses on this target, and one 16-byte store per lane beats eight 2-byte ones by far.
 typedef u32x4_t __attribute__((aligned(2))) u32x4_unaligned_t;
 
+template <typename T>
+__device__ __forceinline__ uint32_t add_pair(uint32_t x, uint32_t r) {
+  const float x0 = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(x)));
+  const float x1 = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(x >> 16)));
+  const float r0 = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(r)));
+  const float r1 = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(r >> 16)));
+  return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, from_f32<T>(x0 + r0))) |
+         (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, from_f32<T>(x1 + r1))) << 16);
+}
+
 template <typename T, int WN, bool STREAM>
 __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict__ C, int64_t ldc,
                                            int64_t row0, int64_t col0, int64_t M, int64_t N,
-                                           int lane) {
+                                           const T* __restrict__ R, int64_t ldr, int lane) {
   constexpr int PITCH = BandLayout<WN>::PITCH;
   constexpr int LPR = WN / 8;    // lanes per row
   constexpr int RPP = 64 / LPR;  // rows per pass
@@ -174,10 +188,25 @@ __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict
   for (int p = 0; p < 32 / RPP; ++p) {
     const int r = p * RPP + lane / LPR;
     const int c = (lane % LPR) * 8;
-    const u32x4_t v = *(const lds_u32x4v_t*)(band + r * PITCH + c * 2);
+    u32x4_t v = *(const lds_u32x4v_t*)(band + r * PITCH + c * 2);
     const int64_t row = row0 + r, col = col0 + c;
     if (row < M && col < N) {
       T* dst = C + row * ldc + col;
+      if (R != nullptr) {  // wave-uniform
+        const T* rsrc = R + row * ldr + col;
+        u32x4_t rv = {0u, 0u, 0u, 0u};
+        if (col + 8 <= N) {
+          rv = *reinterpret_cast<const u32x4_unaligned_t*>(rsrc);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N)
+              rv[e >> 1] |= static_cast<uint32_t>(__builtin_bit_cast(unsigned short, rsrc[e]))
+                            << (16 * (e & 1));
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = add_pair<T>(v[e], rv[e]);
+      }
       if (col + 8 <= N) {
         // STREAM is a template parameter on purpose: as a run-time branch the two stores are
         // merged and the non-temporal hint is lost
@@ -203,7 +232,8 @@ template <typename T, int EPI, int TM, int TN, bool STREAM>
 __device__ __forceinline__ void store_wave_tile_impl(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
                                                 T* __restrict__ C, int64_t ldc, int64_t row0,
                                                 int64_t col0, int64_t M, int64_t N,
-                                                const T* __restrict__ bias, int lane) {
+                                                const T* __restrict__ bias,
+                                                const T* __restrict__ R, int64_t ldr, int lane) {
   constexpr int WN = TN * 32;
   constexpr int PITCH = BandLayout<WN>::PITCH;
   lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
@@ -222,7 +252,7 @@ __device__ __forceinline__ void store_wave_tile_impl(f32x16_t (&acc)[TM][TN], ld
     for (int j = 0; j < TN; ++j)
       stage_tile<T, EPI>(acc[i][j], mine + j * 64, bfrag[j][0], bfrag[j][1], bfrag[j][2],
                          bfrag[j][3]);
-    flush_band<T, WN, STREAM>(band, C, ldc, row0 + i * 32, col0, M, N, lane);
+    flush_band<T, WN, STREAM>(band, C, ldc, row0 + i * 32, col0, M, N, R, ldr, lane);
   }
 }
 
@@ -231,11 +261,13 @@ __device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byt
                                                 T* __restrict__ C, int64_t ldc, int64_t row0,
                                                 int64_t col0, int64_t M, int64_t N,
                                                 const T* __restrict__ bias, bool stream,
-                                                int lane) {
+                                                const T* __restrict__ R, int64_t ldr, int lane) {
   if (stream) {
-    store_wave_tile_impl<T, EPI, TM, TN, true>(acc, band, C, ldc, row0, col0, M, N, bias, lane);
+    store_wave_tile_impl<T, EPI, TM, TN, true>(acc, band, C, ldc, row0, col0, M, N, bias, R, ldr,
+                                               lane);
   } else {
-    store_wave_tile_impl<T, EPI, TM, TN, false>(acc, band, C, ldc, row0, col0, M, N, bias, lane);
+    store_wave_tile_impl<T, EPI, TM, TN, false>(acc, band, C, ldc, row0, col0, M, N, bias, R, ldr,
+                                                lane);
   }
 }
 
@@ -455,8 +487,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmAr
   __syncthreads();  // every wave is done with the operand buffers: reuse them for the output
   static_assert(WAVES_M * WAVES_N * BandLayout<WN>::BYTES <= 2 * STAGE_BYTES, "band staging");
   lds_byte_t* band = (lds_byte_t*)smem + wave * BandLayout<WN>::BYTES;
+  const T* resid = g.residual == nullptr
+                       ? nullptr
+                       : static_cast<const T*>(g.residual) + static_cast<int64_t>(blockIdx.y) * g.stride_r;
   store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  g.stream_c != 0, lane);
+                                  g.stream_c != 0, resid, g.ldr, lane);
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>

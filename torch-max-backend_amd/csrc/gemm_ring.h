@@ -320,8 +320,11 @@ void gemm_ring_kernel(GemmArgs g) {
   __syncthreads();  // every wave is done with the ring: reuse it for the output
   static_assert(NW * BandLayout<WN>::BYTES <= R * STAGE_BYTES, "band staging");
   lds_byte_t* band = (lds_byte_t*)ring + wave * BandLayout<WN>::BYTES;
+  const T* resid = g.residual == nullptr
+                       ? nullptr
+                       : static_cast<const T*>(g.residual) + batch * g.stride_r;
   store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  g.stream_c != 0, lane);
+                                  g.stream_c != 0, resid, g.ldr, lane);
   };
   // Configurations compiled for four waves per SIMD have no registers to spare for the loop
   // state; their second resident workgroup already overlaps the tile boundaries.

@@ -161,6 +161,15 @@ def addmm_gelu(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor,
     return hip_ops.gemm(mat1, mat2, input, epilogue=epi)
 
 
+def addmm_residual(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor,
+                   residual: torch.Tensor) -> torch.Tensor:
+    """``addmm(bias, mat1, mat2) + residual`` in one kernel (residual reshaped to the product's
+    [M, N]). Produced by the executor's addmm -> view -> add fusion; the sum is formed from the
+    rounded product, so the result is bit-identical to the unfused pair."""
+    m, n = mat1.shape[0], mat2.shape[-1]
+    return hip_ops.gemm(mat1, mat2, input, residual=residual.reshape(m, n))
+
+
 @map_to(aten.linear)
 def aten_linear(input: torch.Tensor, weight: torch.Tensor,
                 bias: Optional[torch.Tensor] = None) -> torch.Tensor:

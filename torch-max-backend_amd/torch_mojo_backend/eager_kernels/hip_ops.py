@@ -90,13 +90,16 @@ def _matrix_layout(t: torch.Tensor) -> Optional[Tuple[int, int]]:
 
 
 def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         epilogue: int = _ek.EPI_NONE) -> torch.Tensor:
+         epilogue: int = _ek.EPI_NONE, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``epilogue(a @ b + bias)`` for 2-D operands, or 3-D operands with equal batch sizes.
 
     Transposed views (``weight.t()``, ``k.transpose(-2, -1)``) are consumed in place through
     the kernel's transpose flags; other non-dense layouts are materialised once.
+    ``residual`` (same shape and dtype as the result) is added after the result has been rounded
+    to the storage type, in the same launch where the kernel supports it, otherwise by a separate
+    add: either way the bits of ``gemm(...) + residual``.
     """
-    require_hip(a, b, bias)
+    require_hip(a, b, bias, residual)
     if a.dtype != b.dtype or a.dtype not in FLOAT_DTYPES:
         raise TypeError(f"gemm: unsupported dtypes {a.dtype} x {b.dtype}")
     batched = a.dim() == 3
@@ -121,9 +124,24 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
         b = b.contiguous()
         lb = (0, max(n, 1))
     out = torch.empty((batch, m, n) if batched else (m, n), dtype=a.dtype, device=a.device)
+    if residual is not None and (residual.dtype != a.dtype or tuple(residual.shape) != tuple(out.shape)):
+        raise ValueError(f"gemm: residual must be {tuple(out.shape)} {a.dtype}, got "
+                         f"{tuple(residual.shape)} {residual.dtype}")
     if out.numel() == 0:
         return out
     lib = _ek.lib()
+    if residual is not None:
+        res = residual if residual.stride(-1) == 1 and residual.stride(-2) >= n else residual.contiguous()
+        rc = lib.tmb_gemm_residual(
+            out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
+            res.data_ptr(), batch, m, n, k, la[1], lb[1], n, res.stride(-2),
+            a.stride(0) if batched else 0, b.stride(0) if batched else 0, m * n,
+            res.stride(0) if batched else 0,
+            la[0], lb[0], code_of(a.dtype), epilogue, _stream())
+        if rc == _ek.ERR_UNSUPPORTED:
+            return gemm(a, b, bias, epilogue) + residual
+        _check("tmb_gemm_residual", rc)
+        return out
     rc = lib.tmb_gemm(
         out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
         batch, m, n, k, la[1], lb[1], n,

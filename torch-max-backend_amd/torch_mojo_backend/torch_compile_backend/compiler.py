@@ -92,6 +92,8 @@ def _step_name(step) -> str:
         return "fused-away"
     if step.fn is _FUSED_ADDMM_GELU:
         return "aten.addmm+gelu (fused)"
+    if step.fn is _FUSED_ADDMM_RESIDUAL:
+        return "aten.addmm+add (fused)"
     if step.fn is _FUSED_MASKED_SOFTMAX:
         return "aten.mul+masked_fill+_softmax (fused)"
     if step.fn is _FUSED_ATTENTION:
@@ -390,11 +392,57 @@ class _GraphFactory:
                 softmax_rewrites[node] = None
             softmax_rewrites[final] = ("attention", q4, k4, v4, scale, root, slices)
 
+    @staticmethod
+    def _fuse_residual_add(graph: torch.fx.Graph, taken: dict) -> dict:
+        """addmm (single user) -> optional view (single user) -> add.Tensor(x, .) or add(., x)
+        with alpha 1 and x of the viewed shape and dtype: the residual connection after a
+        projection. The add becomes the fused step; addmm and view are skipped.
+        Returns {node: None (skip) | ("residual", bias, mat1, mat2, x, out_shape)}."""
+        out: dict = {}
+        if MAPPING_TORCH_ATEN_TO_MOJO.get(aten.addmm) is not _BUILTIN_ADDMM or \
+                MAPPING_TORCH_ATEN_TO_MOJO.get(aten.add) is not _BUILTIN_ADD:
+            return out
+        for node in graph.nodes:
+            if node.op != "call_function" or node.target is not aten.add.Tensor or node in taken:
+                continue
+            if len(node.args) != 2 or node.kwargs.get("alpha", 1) != 1:
+                continue
+            for prod, other in ((node.args[0], node.args[1]), (node.args[1], node.args[0])):
+                if not (isinstance(prod, torch.fx.Node) and isinstance(other, torch.fx.Node)):
+                    continue
+                via = None
+                src = prod
+                if src.op == "call_function" and src.target in (
+                        aten.view.default, aten._unsafe_view.default) and len(src.users) == 1:
+                    via, src = src, src.args[0]
+                if not (isinstance(src, torch.fx.Node) and src.op == "call_function"
+                        and src.target is aten.addmm.default and len(src.users) == 1
+                        and src not in taken and src not in out):
+                    continue
+                if src.kwargs.get("beta", 1) != 1 or src.kwargs.get("alpha", 1) != 1:
+                    continue
+                bias_val = src.args[0].meta.get("val") if isinstance(src.args[0], torch.fx.Node) else None
+                pv, ov, nv = prod.meta.get("val"), other.meta.get("val"), node.meta.get("val")
+                if bias_val is None or bias_val.dim() != 1 or pv is None or ov is None or nv is None:
+                    continue
+                if tuple(pv.shape) != tuple(ov.shape) or pv.dtype != ov.dtype or \
+                        tuple(nv.shape) != tuple(pv.shape) or nv.dtype != pv.dtype:
+                    continue
+                out[node] = ("residual", src.args[0], src.args[1], src.args[2], other, tuple(pv.shape))
+                out[src] = None
+                if via is not None:
+                    out[via] = None
+                break
+        return out
+
     def create_graph(self, graph: torch.fx.Graph):
         rewrites = self._fuse_bias_gelu(graph) if _fusion_enabled() else {}
         softmax_rewrites = self._fuse_masked_softmax(graph) if _fusion_enabled() else {}
         if softmax_rewrites and _attention_fusion_enabled():
             self._fuse_attention(softmax_rewrites)
+        if _fusion_enabled():
+            # same bookkeeping as the softmax/attention plans: None = skipped, tuple = fused step
+            softmax_rewrites.update(self._fuse_residual_add(graph, {**rewrites, **softmax_rewrites}))
         nodes = list(graph.nodes)
         # what each node reads after the rewrites (liveness must follow the rewritten program)
         reads: dict = {}
@@ -405,6 +453,8 @@ class _GraphFactory:
                     reads[node] = []
                 elif plan[0] == "softmax":
                     reads[node] = [plan[1], plan[3]]
+                elif plan[0] == "residual":
+                    reads[node] = [plan[1], plan[2], plan[3], plan[4]]
                 else:
                     reads[node] = [plan[1], plan[2], plan[3], plan[5]]
             else:
@@ -434,6 +484,9 @@ class _GraphFactory:
                     elif plan[0] == "softmax":
                         fn, kwargs = _FUSED_MASKED_SOFTMAX, {}
                         args = (plan[1], plan[2], plan[3], plan[4], plan[5])
+                    elif plan[0] == "residual":
+                        fn, kwargs = _FUSED_ADDMM_RESIDUAL, {}
+                        args = plan[1:]
                     else:
                         fn, kwargs = _FUSED_ATTENTION, {}
                         args = plan[1:]
@@ -538,6 +591,15 @@ def _fused_masked_softmax(x, scale, root, slices, dim):
     return _BUILTIN_SOFTMAX(filled, dim, False)
 
 
+def _fused_addmm_residual(bias, mat1, mat2, residual, out_shape):
+    """add(view(addmm(bias, mat1, mat2), out_shape), residual)"""
+    n = mat2.shape[-1]
+    if isinstance(mat1, torch.Tensor) and mat1.is_cuda and bias.dim() == 1 and bias.shape[0] == n \
+            and bias.dtype == mat1.dtype and residual.dtype == mat1.dtype:
+        return aten_functions.addmm_residual(bias, mat1, mat2, residual).view(out_shape)
+    return _BUILTIN_ADD(_BUILTIN_ADDMM(bias, mat1, mat2).view(out_shape), residual)
+
+
 def _fused_attention(q, k, v, scale, root, slices):
     """clone(transpose(bmm(softmax(masked_fill(bmm(q, k^T) * scale, mask == 0, -inf)), v), 1, 2))
     for [batch, heads, tokens, head_dim] q, k, v (views of a packed projection as they come)."""
@@ -559,6 +621,7 @@ def _fused_attention(q, k, v, scale, root, slices):
 
 _BUILTIN_ADDMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.addmm]
 _BUILTIN_BMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.bmm]
+_BUILTIN_ADD = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.add)
 _BUILTIN_GELU = MAPPING_TORCH_ATEN_TO_MOJO[aten.gelu]
 _BUILTIN_SOFTMAX = MAPPING_TORCH_ATEN_TO_MOJO[aten._softmax]
 _BUILTIN_MASKED_FILL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.masked_fill)
@@ -569,6 +632,7 @@ _BUILTIN_ALIAS = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.alias)
 _FUSED_ADDMM_GELU = _fused_addmm_gelu
 _FUSED_MASKED_SOFTMAX = _fused_masked_softmax
 _FUSED_ATTENTION = _fused_attention
+_FUSED_ADDMM_RESIDUAL = _fused_addmm_residual
 
 
 class BaseMaxCompiler:
