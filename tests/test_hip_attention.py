@@ -129,7 +129,9 @@ def test_registry_entry_for_scaled_dot_product_attention():
 
 
 def test_eager_device_scaled_dot_product_attention():
+    from torch_mojo_backend import register_mojo_devices
     from torch_mojo_backend.eager_kernels import aten_fast
+    register_mojo_devices()
     from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
     q, k, v = (x.cuda() for x in _qkv(1, 2, 70, 70, torch.float16, seed=8))
     wrap = lambda t: aten_fast._wrap(t)  # noqa: E731

@@ -74,10 +74,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   // a query block's cost grows with its index: with the query block as the fastest grid
   // dimension and 8 of them, one XCD would get every heaviest block. Rotating the query block
   // by the (batch, head) index gives each XCD an even mix.
+  //
+  // Under a causal mask a workgroup takes two query blocks of one (batch, head): block
+  // n-1-u and then block u, which together always walk the same number of key blocks, so every
+  // workgroup carries the same load and its fixed costs are spread over a long key loop.
   const int n_qb = (a.q_len + kAttnBQ - 1) / kAttnBQ;
-  const int bh = blockIdx.x / n_qb;
-  const int qb = n_qb - 1 - static_cast<int>((blockIdx.x % n_qb + bh) % n_qb);
+  const bool paired = a.causal && n_qb > 1;
+  const int units = paired ? (n_qb + 1) / 2 : n_qb;
+  const int bh = blockIdx.x / units;
+  const int unit = static_cast<int>((blockIdx.x % units + bh) % units);
   const int b = bh / a.heads, h = bh % a.heads;
+  auto run_qblock = [&](const int qb) {
   const int q0 = qb * kAttnBQ, qw0 = q0 + wave * 32;
   const int qi = qw0 + (lane & 31);
   const float neg_inf = -__builtin_inff();
@@ -273,6 +280,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         *reinterpret_cast<u32x2_t*>(dst + dt * 32 + g * 8 + half * 4) = packed;
       }
   }
+  };
+  run_qblock(n_qb - 1 - unit);
+  if (paired && unit != n_qb - 1 - unit) {
+    __syncthreads();  // every wave is done with the K/V ring of the first block
+    run_qblock(unit);
+  }
 #endif
 }
 
@@ -316,7 +329,9 @@ extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const 
              out_strides[0], out_strides[1], out_strides[2],
              static_cast<int>(heads), static_cast<int>(q_len), static_cast<int>(kv_len),
              scale, causal ? 1 : 0, round_like_unfused ? 1 : 0};
-  const dim3 grid(static_cast<unsigned>(((q_len + kAttnBQ - 1) / kAttnBQ) * batch * heads));
+  const int64_t n_qb = (q_len + kAttnBQ - 1) / kAttnBQ;
+  const int64_t units = (causal && n_qb > 1) ? (n_qb + 1) / 2 : n_qb;  // query-block pairs when causal
+  const dim3 grid(static_cast<unsigned>(units * batch * heads));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == TMB_BF16) {
     attention_fwd_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(a);
