@@ -202,25 +202,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     // one FMA and one v_exp_f32 per score. The exponential's error (a few 1e-6 relative from
     // the fp32 argument) disappears in the rounding of the probability to the storage type.
     const bool need_mask = (a.causal && kb + kAttnBKV - 1 > qw0) || kb + kAttnBKV > a.kv_len;
+    // (the two optional passes are whole loops under one wave-uniform branch each: tested per
+    // element they cost an exec-mask save/restore per score)
+    if (a.round_like_unfused) {
+      // what a bmm kernel and then a mul kernel would have stored; the scale is applied here,
+      // so the exponent below uses log2(e) alone
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float x = to_f32(from_f32<T>(acc_s[kt][r]));
+          acc_s[kt][r] = to_f32(from_f32<T>(x * a.scale));
+        }
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kb + kt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          const bool hidden = (a.causal && key > qi) || key >= a.kv_len;
+          acc_s[kt][r] = hidden ? neg_inf : acc_s[kt][r];
+        }
+    }
     float m_blk = neg_inf;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = acc_s[kt][r];
-        if (a.round_like_unfused) {
-          // what a bmm kernel and then a mul kernel would have stored; the scale is applied
-          // here, so the exponent below uses log2(e) alone
-          x = to_f32(from_f32<T>(x));
-          x = to_f32(from_f32<T>(x * a.scale));
-        }
-        if (need_mask) {
-          const int key = kb + kt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-          if ((a.causal && key > qi) || key >= a.kv_len) x = neg_inf;
-        }
-        acc_s[kt][r] = x;
-        m_blk = fmaxf(m_blk, x);
-      }
+      for (int r = 0; r < 16; ++r) m_blk = fmaxf(m_blk, acc_s[kt][r]);
     m_blk = fmaxf(m_blk, other_half(m_blk, lane));
     const float m_new = fmaxf(m_run, m_blk);
     const float m_use = m_new == neg_inf ? 0.0f : m_new;  // nothing visible yet: keep exp finite
