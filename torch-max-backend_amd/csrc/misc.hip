@@ -12,7 +12,7 @@ __global__ __launch_bounds__(256) void gelu_kernel(T* __restrict__ out, const T*
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   for (int64_t i = tid; i < nvec; i += stride) {
-    const Vec16<T> v = load_vec16(in + i * EPV);
+    const Vec16<T> v = load_vec16_stream(in + i * EPV);  // read once
     float y[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; ++e) {
@@ -34,8 +34,10 @@ static int launch_gelu(void* out_, const void* in_, int64_t numel, int tanh_mode
   constexpr int EPV = Vec16<T>::N;
   const int64_t nvec = (aligned16(in) && aligned16(out)) ? numel / EPV : 0;
   int64_t work = nvec > 0 ? nvec : numel;
+  // one 16-byte vector per thread, consecutive blocks on consecutive memory: measured faster on
+  // this GPU than a capped grid whose threads stride through the tensor
   int64_t blocks = (work + 255) / 256;
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks > (int64_t{1} << 30)) blocks = int64_t{1} << 30;
   if (blocks < 1) blocks = 1;
   if (tanh_mode)
     gelu_kernel<T, true><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(out, in, numel, nvec);

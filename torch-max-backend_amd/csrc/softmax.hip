@@ -67,7 +67,8 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(TOut* __restrict__ 
       const int vi = (v * WPR + wave_in_row) * kWave + lane;
       const bool ok = SCALED ? (vi < nvec && vi * EPV <= last_col) : vi < nvec;
       const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
-      const Vec16<TIn> t = STREAM ? load_vec16_stream(src + at) : load_vec16(src + at);
+      // read once: non-temporal whatever the size; STREAM only decides how the output is stored
+      const Vec16<TIn> t = load_vec16_stream(src + at);
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
         if constexpr (SCALED) {
