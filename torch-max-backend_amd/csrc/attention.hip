@@ -53,12 +53,6 @@ constexpr int kAttnTile = kAttnBKV * kAttnRow;  // 8 KiB: one K or V block
 constexpr int kAttnBuf = 2 * kAttnTile;         // K + V
 constexpr int kAttnStages = 3;                  // LDS ring: one block in use, two in flight
 
-template <typename T>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, from_f32<T>(lo))) |
-         (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, from_f32<T>(hi))) << 16);
-}
-
 __device__ __forceinline__ float other_half(float x, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2,
                                                                 __builtin_bit_cast(int, x)));

@@ -108,9 +108,10 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 // LDS (the operand buffers are free by then) and writes it out row by row: 16 bytes per lane,
 // consecutive lanes along a row, whole 128-byte lines per row where the tile is 64 wide.
 //
-// stage_tile: +bias (fp32) -> optional GELU -> one cast, 4 x 8 bytes into the band. Kept out of
-// line: sixteen inlined copies of the GELU epilogue exceed the unroller's budget, and a rolled
-// loop would index the accumulators dynamically.
+// stage_tile: +bias (fp32) -> optional GELU -> one cast, 4 x 8 bytes into the band. The
+// epilogue is bound by its vector-ALU instruction count (both waves of a SIMD run it at the same
+// time, with the matrix pipe idle), so values are converted and packed two at a time and the
+// bias is unpacked to fp32 once per wave tile.
 typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
 typedef __attribute__((address_space(3))) u32x2_t lds_u32x2_t;
 typedef __attribute__((address_space(3))) u32x4_t lds_u32x4v_t;
@@ -143,20 +144,40 @@ __device__ __forceinline__ float unpack_elem(u32x2_t v, int e) {
   return to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(v[e >> 1] >> (16 * (e & 1)))));
 }
 
+// Two fp32 values rounded to T (nearest even) and packed, low half first. On this target the
+// bf16 form is a single v_cvt_pk_bf16_f32.
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef T tx2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, tx2_t));
+}
+
 template <typename T, int EPI>
-__device__ __noinline__ void stage_tile(f32x16_t acc, lds_byte_t* dst, u32x2_t b0, u32x2_t b1,
-                                        u32x2_t b2, u32x2_t b3) {
-  const u32x2_t bq[4] = {b0, b1, b2, b3};
+__device__ __forceinline__ uint32_t finish2(float a, float b) {
+  a = pin_f32(a);  // acc + bias is an fp32 sum; it is rounded to T as a separate step
+  b = pin_f32(b);
+  uint32_t p = pack2<T>(a, b);
+  if constexpr (EPI != TMB_EPI_NONE) {
+    const float ra = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(p)));
+    const float rb = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(p >> 16)));
+    p = EPI == TMB_EPI_GELU_TANH ? pack2<T>(gelu_tanh_f32(ra), gelu_tanh_f32(rb))
+                                 : pack2<T>(gelu_erf_f32(ra), gelu_erf_f32(rb));
+  }
+  return p;
+}
+
+// One 32x32 accumulator tile into the band: +bias (fp32) -> optional GELU -> one cast, 4 x 8
+// bytes per lane. `bias` holds the lane's 16 bias values as fp32 (zeros without a bias).
+template <typename T, int EPI>
+__device__ __forceinline__ void stage_tile(const f32x16_t& acc, lds_byte_t* dst,
+                                           const float (&bias)[16]) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    T o[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = finish<T, EPI>(acc[4 * q + e] + unpack_elem<T>(bq[q], e));
     u32x2_t packed;
-    packed[0] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[0])) |
-                (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[1])) << 16);
-    packed[1] = static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[2])) |
-                (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, o[3])) << 16);
+    packed[0] = finish2<T, EPI>(acc[4 * q + 0] + bias[4 * q + 0], acc[4 * q + 1] + bias[4 * q + 1]);
+    packed[1] = finish2<T, EPI>(acc[4 * q + 2] + bias[4 * q + 2], acc[4 * q + 3] + bias[4 * q + 3]);
     *(lds_u32x2_t*)(dst + 16 * q) = packed;
   }
 }
@@ -239,19 +260,21 @@ __device__ __forceinline__ void store_wave_tile_impl(f32x16_t (&acc)[TM][TN], ld
   lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
   // The bias a lane adds depends on its columns only: fetched once for the whole wave tile
   // (the operand fragments' registers are free by now).
-  u32x2_t bfrag[TN][4];
+  float bias_f[TN][16];
 #pragma unroll
   for (int j = 0; j < TN; ++j)
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-      bfrag[j][q] = load_bias4<T>(bias, col0 + j * 32 + 4 * (lane >> 5) + 8 * q, N);
+    for (int q = 0; q < 4; ++q) {
+      const u32x2_t b4 = load_bias4<T>(bias, col0 + j * 32 + 4 * (lane >> 5) + 8 * q, N);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bias_f[j][4 * q + e] = unpack_elem<T>(b4, e);
+    }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     if (row0 + i * 32 >= M) break;  // wave-uniform
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      stage_tile<T, EPI>(acc[i][j], mine + j * 64, bfrag[j][0], bfrag[j][1], bfrag[j][2],
-                         bfrag[j][3]);
+      stage_tile<T, EPI>(acc[i][j], mine + j * 64, bias_f[j]);
     flush_band<T, WN, STREAM>(band, C, ldc, row0 + i * 32, col0, M, N, R, ldr, lane);
   }
 }
