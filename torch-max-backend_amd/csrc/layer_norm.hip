@@ -6,6 +6,8 @@
 // (torch_mojo_backend/eager_kernels/nn_ops.mojo:299-326). A row whose variance is NaN
 // (it contains NaN or an infinity) reports NaN for the mean as well
 // (normalization_forward_kernels.mojo:60-70).
+#include <type_traits>
+
 #include "tmb_common.h"
 
 namespace tmb {
@@ -21,7 +23,7 @@ template <typename T, int WPR, int VPL, int RPW, bool STREAM, bool AFFINE_LDS, i
 __global__ __launch_bounds__(BLOCK) void layer_norm_regs_kernel(
     T* __restrict__ out, float* __restrict__ mean_out, float* __restrict__ rstd_out,
     const T* __restrict__ in, const T* __restrict__ gamma, const T* __restrict__ beta,
-    int64_t rows, int cols, float eps) {
+    int64_t rows, int cols, float eps, int64_t row_span) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int WAVES = BLOCK / kWave;
   constexpr int GROUPS = WAVES / WPR;
@@ -46,9 +48,34 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_regs_kernel(
     __syncthreads();
   }
 
+  // Short rows: gamma/beta are fetched once, before the first row's statistics (their latency
+  // hides behind the reductions), and stay in registers for every row the workgroup walks.
+  // Long rows would pay for that with occupancy; they fetch them (from LDS or L2) in groups of
+  // four vectors right before use.
+  constexpr bool PREFETCH_AFFINE = !AFFINE_LDS && VPL <= 4;
+  constexpr int AFF = PREFETCH_AFFINE ? VPL : (VPL < 4 ? VPL : 4);  // vectors held at a time
+  Vec16<T> gv[AFF], bv[AFF];
+  auto load_affine = [&](int v_first) {
+#pragma unroll
+    for (int u = 0; u < AFF; ++u) {
+      const int vi = ((v_first + u) * WPR + wave_in_row) * kWave + lane;
+      const int64_t at = static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
+      if constexpr (AFFINE_LDS) {
+        if (gamma != nullptr) gv[u] = load_vec16(lds_gamma + at);
+        if (beta != nullptr) bv[u] = load_vec16(lds_beta + at);
+      } else {
+        if (gamma != nullptr) gv[u] = load_vec16(gamma + at);
+        if (beta != nullptr) bv[u] = load_vec16(beta + at);
+      }
+    }
+  };
+  if constexpr (PREFETCH_AFFINE) load_affine(0);
+
+  // A workgroup walks `row_span` consecutive rows (a whole number of its row groups).
   const int64_t rows_per_block = static_cast<int64_t>(GROUPS) * RPW;
-  for (int64_t block_row = static_cast<int64_t>(blockIdx.x) * rows_per_block; block_row < rows;
-       block_row += static_cast<int64_t>(gridDim.x) * rows_per_block) {
+  const int64_t span_begin = static_cast<int64_t>(blockIdx.x) * row_span;
+  const int64_t span_end = span_begin + row_span < rows ? span_begin + row_span : rows;
+  for (int64_t block_row = span_begin; block_row < span_end; block_row += rows_per_block) {
   const int64_t row0 = block_row + static_cast<int64_t>(group) * RPW;
 
   float x[RPW][VPL][EPV];
@@ -71,28 +98,6 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_regs_kernel(
       for (int e = 0; e < EPV; ++e) x[r][v][e] = ok ? to_f32(t.v[e]) : 0.0f;
     }
   }
-  // Short rows: fetch gamma/beta now so their latency hides behind the reductions. Long rows
-  // would pay for that with occupancy; they fetch them (from L2) in groups of four vectors
-  // right before use.
-  constexpr bool PREFETCH_AFFINE = !AFFINE_LDS && VPL <= 4;
-  constexpr int AFF = PREFETCH_AFFINE ? VPL : (VPL < 4 ? VPL : 4);  // vectors held at a time
-  Vec16<T> gv[AFF], bv[AFF];
-  auto load_affine = [&](int v_first) {
-#pragma unroll
-    for (int u = 0; u < AFF; ++u) {
-      const int vi = ((v_first + u) * WPR + wave_in_row) * kWave + lane;
-      const int64_t at = static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
-      if constexpr (AFFINE_LDS) {
-        if (gamma != nullptr) gv[u] = load_vec16(lds_gamma + at);
-        if (beta != nullptr) bv[u] = load_vec16(lds_beta + at);
-      } else {
-        if (gamma != nullptr) gv[u] = load_vec16(gamma + at);
-        if (beta != nullptr) bv[u] = load_vec16(beta + at);
-      }
-    }
-  };
-  if constexpr (PREFETCH_AFFINE) load_affine(0);
-
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
     float s = 0.0f;
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_regs_kernel(
       }
     }
   }
-  }  // grid-stride over row groups
+  }  // rows of this workgroup's span
 }
 
 template <typename T>
@@ -199,34 +204,38 @@ template <typename T, int WPR, int VPL, int BLOCK>
 static int launch_ln(T* out, float* mean, float* rstd, const T* x, const T* g, const T* b,
                      int64_t rows, int64_t cols, float eps, hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
-  constexpr int FLOATS = VPL * EPV;
-  constexpr int RPW = (WPR > 1 || FLOATS >= 64) ? 1 : (FLOATS >= 32 ? 2 : 4);
+  constexpr int RPW = 1;
   constexpr int ROWS_PER_BLOCK = (BLOCK / kWave) / WPR * RPW;
-  int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  const int64_t groups = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;  // row groups of a workgroup
   const bool stream_hint = rows * cols * static_cast<int64_t>(2 * sizeof(T)) >= (int64_t{256} << 20);
   const dim3 block(BLOCK);
   const int c = static_cast<int>(cols);
-  // Long rows with affine parameters: stage gamma/beta in LDS, few persistent workgroups.
+  // `walk` row groups per workgroup, consecutive in memory
+  auto launch = [&](auto lds_tag, int64_t walk, size_t lds_bytes) {
+    constexpr bool LDS = decltype(lds_tag)::value;
+    const int64_t blocks = (groups + walk - 1) / walk;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    const int64_t span = walk * ROWS_PER_BLOCK;
+    if (stream_hint)
+      layer_norm_regs_kernel<T, WPR, VPL, RPW, true, LDS, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps, span);
+    else
+      layer_norm_regs_kernel<T, WPR, VPL, RPW, false, LDS, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps, span);
+    return check_launch();
+  };
+  // Long 16-bit rows with affine parameters: gamma/beta staged in LDS by a few workgroups that
+  // each walk many rows (for fp32 the LDS reads would cost as much as the L2 re-reads they
+  // replace).
   const size_t lds_bytes = static_cast<size_t>(cols) * sizeof(T) * 2;
-  // (16-bit rows only: for fp32 the LDS reads would cost as much as the L2 re-reads they replace)
   if constexpr (VPL >= 8 && sizeof(T) == 2) {
     if ((g != nullptr || b != nullptr) && lds_bytes <= 65536) {
       const int64_t persistent = 256 * (BLOCK >= 1024 ? 2 : 8);
-      if (blocks > persistent) blocks = persistent;
-      const dim3 grid(static_cast<unsigned>(blocks));
-      if (stream_hint)
-        layer_norm_regs_kernel<T, WPR, VPL, RPW, true, true, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
-      else
-        layer_norm_regs_kernel<T, WPR, VPL, RPW, false, true, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
-      return check_launch();
+      return launch(std::true_type{}, (groups + persistent - 1) / persistent, lds_bytes);
     }
   }
-  const dim3 grid(static_cast<unsigned>(blocks));
-  if (stream_hint)
-    layer_norm_regs_kernel<T, WPR, VPL, RPW, true, false, BLOCK><<<grid, block, 0, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
-  else
-    layer_norm_regs_kernel<T, WPR, VPL, RPW, false, false, BLOCK><<<grid, block, 0, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
-  return check_launch();
+  // Short rows keep gamma/beta in registers: a workgroup that walks a few consecutive row
+  // groups re-uses them (more than four measured slower: too few workgroups in flight).
+  const int64_t walk = VPL <= 4 ? (groups >= 16384 ? 4 : (groups >= 4096 ? 2 : 1)) : 1;
+  return launch(std::false_type{}, walk, 0);
 }
 
 template <typename T>
@@ -249,9 +258,13 @@ static int layer_norm_dispatch(void* out_, float* mean, float* rstd, const void*
     if (nvec <= 64) TMB_LN(1, 1, 256);
     if (nvec <= 128) TMB_LN(1, 2, 256);
     if (nvec <= 256) TMB_LN(1, 4, 256);
-    if (nvec <= 512) TMB_LN(1, 8, 256);
     if constexpr (MAXV >= 16) {
-      if (nvec <= 1024) TMB_LN(1, 16, 256);
+      // fp32: rows shared by four waves, two or four vectors per lane (measured 5-10 % faster
+      // than one wave per row)
+      if (nvec <= 512) TMB_LN(4, 2, 256);
+      if (nvec <= 1024) TMB_LN(4, 4, 256);
+    } else {
+      if (nvec <= 512) TMB_LN(1, 8, 256);  // 16-bit: gamma/beta through LDS
     }
     if (nvec <= 4 * 64 * MAXV / 2) TMB_LN(4, MAXV / 2, 256);
     if (nvec <= 4 * 64 * MAXV) TMB_LN(4, MAXV, 256);

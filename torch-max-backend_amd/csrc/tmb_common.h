@@ -97,6 +97,21 @@ __device__ __forceinline__ float exp_f32(float x) {
   return (x == -__builtin_inff()) ? 0.0f : r;
 }
 
+// exp for results that are stored in 16 bits: one multiply and v_exp_f32. The rounding of
+// x*log2(e) costs at most 6e-8 |x log2 e| in the exponent, i.e. below 6e-6 relative wherever the
+// result is a normal number: 1 % of half an fp16 ulp.
+__device__ __forceinline__ float exp_f32_for16(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.44269502162933349609375f);
+}
+template <typename TOut>
+__device__ __forceinline__ float exp_for(float x) {
+  if constexpr (sizeof(TOut) == 2) {
+    return exp_f32_for16(x);
+  } else {
+    return exp_f32(x);
+  }
+}
+
 // Pins a value in a VGPR as an fp32 number. The compiler otherwise folds an fp32 multiply or
 // add into the following fp32->fp16 conversion (v_fma_mixlo_f16: one rounding instead of two),
 // and whether it does so depends on the surrounding code — which would make the same formula
