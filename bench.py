@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # Bytes per launch of the headline GEMM kernel between L2 and the memory side, measured with
 # rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the factors being what the same
 # counters read for tmb_copy_bytes moving 1 GiB: `--only copy`).
-GEMM_TRAFFIC_BYTES = 1.774e9
+GEMM_TRAFFIC_BYTES = 1.760e9
 
 
 def _parse():

@@ -3,19 +3,18 @@
 //
 // global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into LDS (lane l
 // of a wave lands at base + 16*l), so no staging registers and no ds_write instructions are
-// spent on the operands. K is walked in stages of 32; four stages form a ring in LDS and up to
-// three of them are in flight while one is multiplied. Each wave waits only for its own
-// loads of the stage needed next (s_waitcnt vmcnt(N) with N = the loads of the two younger
+// spent on the operands. K is walked in stages of BK (32 or 64); R stages form a ring in LDS
+// and up to R-1 of them are in flight while one is multiplied. Each wave waits only for its own
+// loads of the stage needed next (s_waitcnt vmcnt(N) with N = the loads of the younger
 // stages), then one s_barrier makes every wave's part of that stage visible.
 //
-// LDS stage layout: 64-byte lines (32 K-values) per matrix row, the four 16-byte chunks of a
-// line XOR-swizzled with (row>>2)&3: a ds_read_b128 is served sixteen lanes at a time from 64
+// LDS stage layout of a K-major operand: one line of BK*2 bytes per matrix row, its 16-byte
+// chunks XOR-swizzled (ring_swizzle): a ds_read_b128 is served sixteen lanes at a time from 64
 // banks (256 bytes), and the fragment fetch of 16 consecutive rows then touches 16 distinct
-// 16-byte bank groups (row%4 picks the line's quarter of the bank window, the swizzle the slot
-// inside it). The swizzle is applied on the global side: each lane of a load picks the source
-// chunk that belongs at its LDS slot.
+// 16-byte bank groups. The swizzle is applied on the global side: each lane of a load picks the
+// source chunk that belongs at its LDS slot.
 //
-// N-major B is staged as it lies in memory, [32 k][BN n], and its fragments are fetched with
+// N-major B is staged as it lies in memory, [BK k][BN n], and its fragments are fetched with
 // ds_read_b64_tr_b16: sixteen lanes read a 4(k) x 16(n) block as 8-byte row pieces and get it
 // back transposed (lane = n, four consecutive k), which is the MFMA operand layout, so no
 // shuffle or repacking is spent on the transpose. Its 16-byte chunks are XOR-swizzled with
