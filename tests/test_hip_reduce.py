@@ -148,6 +148,7 @@ def test_argmax_vocab_with_ties_is_bit_exact(dtype):
 
 
 @pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 64), (257, 1000), (5, 65537), (2, 1 << 21),
+                                   (256, 40001), (300, 70003),  # one wide workgroup per row
                                    (1, (1 << 23) + 3)])
 def test_argmax_shapes(shape):
     x = seeded(shape, seed=shape[1] % 991)

@@ -429,21 +429,22 @@ struct alignas(16) BestSlot {
   V val;
 };
 
-template <typename T>
-__global__ __launch_bounds__(kRedBlock) void argmax_chunk_kernel(int64_t* __restrict__ out,
-                                                                 void* __restrict__ ws,
-                                                                 const T* __restrict__ in,
-                                                                 int64_t rows, int64_t cols,
-                                                                 int splits, int64_t chunk) {
+template <typename T, int BLK>
+__global__ __launch_bounds__(BLK) void argmax_chunk_kernel(int64_t* __restrict__ out,
+                                                           void* __restrict__ ws,
+                                                           const T* __restrict__ in, int64_t rows,
+                                                           int64_t cols, int splits,
+                                                           int64_t chunk) {
   using V = typename ArgTraits<T>::val_t;
-  __shared__ BestSlot<V> slot[kRedWaves];
+  constexpr int WAVES = BLK / kWave;
+  __shared__ BestSlot<V> slot[WAVES];
   const int64_t item = blockIdx.x;
   const int64_t row = item / splits;
   const int split = static_cast<int>(item - row * splits);
   const int64_t c0 = static_cast<int64_t>(split) * chunk;
   int64_t n = cols - c0;
   if (n > chunk) n = chunk;
-  Best<V> b = argmax_range<T, kRedBlock>(in + row * cols + c0, n, threadIdx.x, c0);
+  Best<V> b = argmax_range<T, BLK>(in + row * cols + c0, n, threadIdx.x, c0);
   b = wave_best(b);
   const int wave = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) slot[wave] = BestSlot<V>{b.idx, b.val};
@@ -451,7 +452,7 @@ __global__ __launch_bounds__(kRedBlock) void argmax_chunk_kernel(int64_t* __rest
   if (threadIdx.x == 0) {
     Best<V> r{slot[0].val, slot[0].idx};
 #pragma unroll
-    for (int w = 1; w < kRedWaves; ++w) r = best_combine(r, Best<V>{slot[w].val, slot[w].idx});
+    for (int w = 1; w < WAVES; ++w) r = best_combine(r, Best<V>{slot[w].val, slot[w].idx});
     if (splits == 1) {
       out[row] = r.idx;
     } else {
@@ -489,12 +490,20 @@ static int launch_argmax(int64_t* out, const void* in_, int64_t rows, int64_t co
                          size_t ws_bytes, hipStream_t stream) {
   const T* in = static_cast<const T*>(in_);
   const SplitPlan plan = plan_splits(rows, cols);
+  // At least one row per CU and only a few chunks per row: one 1024-thread workgroup per row does
+  // the same work per thread in a single launch (the second stage alone costs 4-5 us).
+  if (plan.splits > 1 && plan.splits <= 4 && rows >= 256 && rows < (int64_t{1} << 31) &&
+      cols < (int64_t{1} << 30)) {
+    argmax_chunk_kernel<T, 1024><<<dim3(static_cast<unsigned>(rows)), dim3(1024), 0, stream>>>(
+        out, ws, in, rows, cols, 1, cols);
+    return check_launch();
+  }
   const int64_t items = rows * plan.splits;
   if (items >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
   if (plan.splits > 1) {
     if (ws == nullptr || ws_bytes < static_cast<size_t>(items) * 16) return TMB_ERR_WORKSPACE;
   }
-  argmax_chunk_kernel<T><<<dim3(static_cast<unsigned>(items)), dim3(kRedBlock), 0, stream>>>(
+  argmax_chunk_kernel<T, kRedBlock><<<dim3(static_cast<unsigned>(items)), dim3(kRedBlock), 0, stream>>>(
       out, ws, in, rows, cols, plan.splits, plan.chunk);
   int rc = check_launch();
   if (rc != 0 || plan.splits == 1) return rc;
