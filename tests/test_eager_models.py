@@ -1,0 +1,70 @@
+"""Whole models on the eager ``mojo`` device: the hot ops run on the HIP kernels, everything else
+a GPT-2 forward or a greedy decode loop touches runs on the holders (reference:
+mojo_device/mojo_device_aten_ops.py registers its ops one by one in the same way)."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mojo():
+    from torch_mojo_backend import register_mojo_devices
+    register_mojo_devices()
+    return torch.device("mojo")
+
+
+def test_demo_gpt2_forward_runs_eagerly_on_the_hip_kernels(mojo):
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend.mojo_device.mojo_device_aten_ops import EAGER_CALL_COUNTERS
+    model = build_gpt2_small(seed=0, n_layer=2)
+    idx = seeded_tokens(2, 32, seed=0)
+    with torch.no_grad():
+        want_logits, want_next = model(idx)
+    before = {k: v.call_count for k, v in EAGER_CALL_COUNTERS.items()}
+    with torch.no_grad():
+        logits, nxt = model.to(mojo)(idx.to(mojo))
+    assert logits.device.type == "mojo"
+    torch.testing.assert_close(logits.cpu(), want_logits, rtol=1e-4, atol=1e-4)
+    assert torch.equal(nxt.cpu(), want_next)
+    grew = {k for k, v in EAGER_CALL_COUNTERS.items() if v.call_count > before[k]}
+    # every hot op of the forward went through its fast_aten_* twin
+    # (eagerly, nn.Linear is aten::linear and F.softmax is aten::softmax.int; nothing decomposes)
+    for op in ("aten::linear", "aten::native_layer_norm", "aten::bmm", "aten::softmax.int",
+               "aten::gelu", "aten::argmax"):
+        assert op in grew, f"{op} did not run on the mojo device ({sorted(grew)})"
+
+
+def test_hf_gpt2_greedy_generate_matches_cpu(mojo):
+    transformers = pytest.importorskip("transformers")
+    torch.manual_seed(0)
+    model = transformers.GPT2LMHeadModel(transformers.GPT2Config(n_layer=2)).eval()
+    ids = torch.randint(0, 50257, (4, 8))
+    mask = torch.ones_like(ids)
+    kw = dict(max_new_tokens=6, min_new_tokens=6, do_sample=False, pad_token_id=50256)
+    with torch.no_grad():
+        want = model.generate(ids, attention_mask=mask, **kw)
+        got = model.to(mojo).generate(ids.to(mojo), attention_mask=mask.to(mojo), **kw)
+    assert got.device.type == "mojo"
+    assert torch.equal(got.cpu(), want)
+
+
+def test_views_share_memory_and_inplace_ops_return_their_input(mojo):
+    x = torch.arange(24, dtype=torch.float32).view(2, 3, 4).to(mojo)
+    v = x.transpose(0, 2)[1:3]
+    v.mul_(2.0)
+    want = torch.arange(24, dtype=torch.float32).view(2, 3, 4)
+    want.transpose(0, 2)[1:3].mul_(2.0)
+    assert torch.equal(x.cpu(), want)
+    y = x.add_(1.0)
+    assert y is x
+    parts = torch.split(x, 2, dim=2)
+    assert all(p.device.type == "mojo" for p in parts)
+    assert torch.equal(torch.cat(parts, dim=2).cpu(), want + 1.0)
+
+
+def test_an_op_without_a_registration_still_raises(mojo):
+    x = torch.rand(8).to(mojo)
+    with pytest.raises(NotImplementedError):
+        torch.erfinv(x)

@@ -120,7 +120,7 @@ def test_registry_entry_for_scaled_dot_product_attention():
     assert got.shape == (2, 4, 100, 64)
     want = cf.attention(as64(q), as64(k), as64(v), 0.125, True).transpose(0, 2, 1, 3)
     assert np.abs(as64(got) - want).max() <= 3e-2
-    # float32 and an explicit mask are not the kernel's: PyTorch's op answers
+    # float32 and an explicit mask are not the fused kernel's: GEMM + softmax + GEMM answers
     mask = torch.ones(100, 100, dtype=torch.bool, device="cuda").tril()
     via_mask = fn(q, k, v, attn_mask=mask)
     assert np.abs(as64(via_mask) - want).max() <= 3e-2
@@ -143,4 +143,76 @@ def test_eager_device_scaled_dot_product_attention():
     assert aten_fast.fast_aten_scaled_dot_product_attention(
         wrap(q), wrap(k), wrap(v), dropout_p=0.1) is aten_fast.NOT_HANDLED
     assert aten_fast.fast_aten_scaled_dot_product_attention(
-        wrap(q.float()), wrap(k.float()), wrap(v.float())) is aten_fast.NOT_HANDLED
+        wrap(q), wrap(k), wrap(v), enable_gqa=True) is aten_fast.NOT_HANDLED
+    # float32 goes through GEMM + softmax + GEMM
+    f32 = aten_fast.fast_aten_scaled_dot_product_attention(
+        wrap(q.float()), wrap(k.float()), wrap(v.float()), is_causal=True)
+    assert isinstance(f32, TorchMojoTensor) and f32._dtype == torch.float32
+    want32 = cf.attention(as64(q), as64(k), as64(v), 0.125, True).transpose(0, 2, 1, 3)
+    assert np.abs(as64(f32._holder) - want32).max() <= 1e-4
+
+
+# ---- composed attention: GEMM + softmax + GEMM for what the fused kernel does not take ----------
+def _sdpa64(q, k, v, scale, causal, mask):
+    """float64 closed form with an optional boolean / additive mask."""
+    s = np.einsum("...td,...sd->...ts", as64(q), as64(k)) * scale
+    t, n = s.shape[-2], s.shape[-1]
+    if causal:
+        s = np.where(np.tril(np.ones((t, n), dtype=bool)), s, -np.inf)
+    if mask is not None:
+        m = mask.numpy()
+        s = np.where(m, s, -np.inf) if m.dtype == np.bool_ else s + m.astype(np.float64)
+    s = s - s.max(axis=-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=-1, keepdims=True)
+    return np.einsum("...ts,...sd->...td", p, as64(v))
+
+
+@pytest.mark.parametrize("case", [
+    # (shape of q, keys, head_dim_v, dtype, causal, mask kind)
+    ((2, 3, 17, 32), 17, 32, torch.float32, True, None),
+    ((2, 3, 17, 32), 29, 48, torch.float32, False, "bool"),
+    ((1, 4, 40, 128), 40, 128, torch.bfloat16, True, None),
+    ((2, 12, 1, 64), 37, 64, torch.bfloat16, False, None),      # a decode step
+    ((2, 2, 9, 64), 21, 64, torch.float16, False, "float"),
+    ((3, 5, 80), 80, 80, torch.float32, False, None),           # no head dimension
+])
+def test_attention_composed_matches_closed_form(case):
+    qshape, keys, dv, dtype, causal, kind = case
+    q = seeded(qshape, seed=1, dtype=dtype)
+    k = seeded(qshape[:-2] + (keys, qshape[-1]), seed=2, dtype=dtype)
+    v = seeded(qshape[:-2] + (keys, dv), seed=3, dtype=dtype)
+    mask = None
+    if kind == "bool":
+        g = torch.Generator().manual_seed(5)
+        mask = torch.rand(qshape[0], 1, qshape[-2], keys, generator=g) > 0.3
+        mask[..., 0] = True  # every query keeps at least one key
+    elif kind == "float":
+        mask = seeded((qshape[-2], keys), seed=6, dtype=dtype)
+    scale = 1.0 / np.sqrt(qshape[-1])
+    got = _ops().attention_composed(q.cuda(), k.cuda(), v.cuda(), scale, causal,
+                                    None if mask is None else mask.cuda())
+    assert got.shape == qshape[:-1] + (dv,) and got.dtype == dtype
+    want = _sdpa64(q, k, v, scale, causal, mask)
+    tol = {torch.float32: 2e-5, torch.bfloat16: 4e-2, torch.float16: 5e-3}[dtype]
+    assert np.abs(as64(got) - want).max() <= tol
+    # and PyTorch's CPU op on the same inputs (fp32 only: its 16-bit CPU path rounds differently)
+    if dtype == torch.float32 and q.dim() == 4:
+        ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, is_causal=causal)
+        torch.testing.assert_close(got.cpu(), ref, rtol=1e-4, atol=1e-5)
+
+
+def test_sdpa_surfaces_use_the_composed_path_for_fp32_and_masks():
+    from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO, register_mojo_devices
+    register_mojo_devices()
+    q = seeded((2, 4, 12, 32), seed=1)
+    k = seeded((2, 4, 20, 32), seed=2)
+    v = seeded((2, 4, 20, 32), seed=3)
+    mask = torch.ones(12, 20, dtype=torch.bool).tril(8)
+    want = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+    fn = MAPPING_TORCH_ATEN_TO_MOJO[torch.ops.aten.scaled_dot_product_attention]
+    torch.testing.assert_close(fn(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).cpu(), want, rtol=1e-4, atol=1e-5)
+    got = torch.nn.functional.scaled_dot_product_attention(q.to("mojo"), k.to("mojo"), v.to("mojo"),
+                                                           attn_mask=mask.to("mojo"))
+    assert got.device.type == "mojo"
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-5)

@@ -267,13 +267,20 @@ def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout
                                       is_causal: bool = False, *, scale=None,
                                       enable_gqa: bool = False) -> torch.Tensor:
     """reference :3029-3087 (built there from matmul, softmax and matmul graph ops). The fused
-    HIP kernel takes the call when there is no explicit mask, no dropout, head_dim 64 and a
-    16-bit dtype; anything else is PyTorch-ROCm's own op."""
-    if attn_mask is None and dropout_p == 0.0 and not enable_gqa and query.dim() == 4 \
-            and hip_ops.attention_supported(query, key, value):
+    HIP kernel takes the call when there is no explicit mask, head_dim is 64 and the dtype has
+    16 bits; other head sizes, fp32 and explicit masks run as GEMM + softmax + GEMM on the same
+    kernels. Dropout and grouped-query attention are PyTorch-ROCm's own op."""
+    plain = dropout_p == 0.0 and not enable_gqa and query.dim() >= 2 \
+        and query.dtype in hip_ops.FLOAT_DTYPES and key.dtype == query.dtype \
+        and value.dtype == query.dtype and key.shape[:-2] == query.shape[:-2] \
+        and value.shape[:-2] == query.shape[:-2] and query.numel() > 0 and key.shape[-2] > 0 \
+        and not (attn_mask is not None and is_causal)
+    if plain:
         s = float(scale) if scale is not None else 1.0 / math.sqrt(query.shape[-1])
-        if s > 0.0:
+        if attn_mask is None and s > 0.0 and query.dim() == 4 \
+                and hip_ops.attention_supported(query, key, value):
             return hip_ops.attention(query, key, value, s, bool(is_causal)).transpose(1, 2)
+        return hip_ops.attention_composed(query, key, value, s, bool(is_causal), attn_mask)
     return aten.scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal,
                                              scale=scale, enable_gqa=enable_gqa)
 

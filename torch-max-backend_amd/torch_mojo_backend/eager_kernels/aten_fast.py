@@ -173,13 +173,26 @@ def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dr
     q, k, v = _t(query), _t(key), _t(value)
     if q is None or k is None or v is None or not _same_device(q, k, v):
         return NOT_HANDLED
-    if attn_mask is not None or dropout_p != 0.0 or enable_gqa or len(q._shape) != 4:
+    if dropout_p != 0.0 or enable_gqa or len(q._shape) < 2 or q._dtype not in _FLOAT_DTYPES \
+            or k._dtype != q._dtype or v._dtype != q._dtype:
         return NOT_HANDLED
+    if tuple(k._shape[:-2]) != tuple(q._shape[:-2]) or tuple(v._shape[:-2]) != tuple(q._shape[:-2]) \
+            or k._shape[-1] != q._shape[-1] or v._shape[-2] != k._shape[-2] or q._numel == 0 \
+            or k._shape[-2] == 0:
+        return NOT_HANDLED
+    mask = None
+    if attn_mask is not None:
+        mask = _t(attn_mask)
+        if mask is None or not _same_device(q, mask) or is_causal:
+            return NOT_HANDLED
     s = float(scale) if scale is not None else 1.0 / math.sqrt(q._shape[-1])
-    if not s > 0.0 or not hip_ops.attention_supported(q._holder, k._holder, v._holder):
-        return NOT_HANDLED
-    out = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal))
-    return _wrap(out.transpose(1, 2))  # [batch, heads, tokens, head_dim] view, as ATen returns it
+    if mask is None and s > 0.0 and len(q._shape) == 4 \
+            and hip_ops.attention_supported(q._holder, k._holder, v._holder):
+        out = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal))
+        return _wrap(out.transpose(1, 2))  # [batch, heads, tokens, head_dim] view, as ATen returns it
+    # other head sizes, fp32, explicit masks, decode shapes: GEMM + softmax + GEMM
+    return _wrap(hip_ops.attention_composed(q._holder, k._holder, v._holder, s, bool(is_causal),
+                                            None if mask is None else mask._holder))
 
 
 # ---------------------------------------------------------------------------

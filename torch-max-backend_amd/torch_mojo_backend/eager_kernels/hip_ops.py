@@ -64,7 +64,9 @@ def require_hip(*tensors: Optional[torch.Tensor]) -> torch.device:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The raw hipStream_t of PyTorch's current stream on the current device (the private
+    accessor costs a fraction of building a torch.cuda.Stream object per launch)."""
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 def code_of(dtype: torch.dtype) -> int:
@@ -247,6 +249,36 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, c
                                      int(bool(round_like_unfused)), code_of(q.dtype), _stream())
     _check("tmb_attention_fwd", rc)
     return out
+
+
+def attention_composed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                       causal: bool, attn_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``softmax(q kᵀ · scale + mask) v`` for [..., tokens, head_dim] operands of any head size and
+    dtype, built from the GEMM and softmax kernels the way the reference builds it from matmul,
+    softmax and matmul graph ops (aten_functions.py:3029-3087). ``attn_mask`` is boolean (True =
+    takes part) or additive, broadcastable to the scores; ``causal`` is the top-left aligned
+    lower triangle. Returns [..., tokens, head_dim_v]."""
+    require_hip(q, k, v, attn_mask)
+    if q.dim() < 2 or k.shape[:-2] != q.shape[:-2] or v.shape[:-2] != q.shape[:-2]:
+        raise ValueError(f"attention_composed: shapes {tuple(q.shape)}, {tuple(k.shape)}, "
+                         f"{tuple(v.shape)} do not match")
+    lead = tuple(q.shape[:-2])
+    t, s_len = q.shape[-2], k.shape[-2]
+    q3 = q.reshape(-1, t, q.shape[-1])
+    k3 = k.reshape(-1, s_len, k.shape[-1])
+    v3 = v.reshape(-1, s_len, v.shape[-1])
+    scores = gemm(q3, k3.transpose(1, 2))                       # [batch, t, s]
+    if attn_mask is None and scale > 0.0:
+        probs = softmax_scaled(scores, scale, t if causal else 0)
+    else:
+        scores = (scores * scale).view(*lead, t, s_len)
+        if attn_mask is not None and attn_mask.dtype == torch.bool:
+            scores = scores.masked_fill(~attn_mask, float("-inf"))
+        elif attn_mask is not None:
+            scores = scores + attn_mask.to(scores.dtype)
+        scores = scores.reshape(-1, t, s_len)
+        probs = softmax_scaled(scores, 1.0, t if causal else 0)
+    return gemm(probs, v3).view(*lead, t, v.shape[-1])
 
 
 def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optional[torch.Tensor],

@@ -205,4 +205,88 @@ _view_op("aten::slice.Tensor", lambda h, dim=0, start=None, end=None, step=1:
          h[(slice(None),) * (dim % max(h.dim(), 1)) + (slice(start, end, step),)])
 _view_op("aten::alias", lambda h: h.alias() if hasattr(h, "alias") else h.view(h.shape))
 _view_op("aten::detach", lambda h: h.detach())
-_view_op("aten::clone", lambda h, memory_format=None: h.clone())
+_view_op("aten::clone", lambda h, memory_format=None:
+         h.clone(memory_format=memory_format if memory_format is not None else torch.preserve_format))
+
+
+# ---------------------------------------------------------------------------
+# Cold ops: everything else a GPT-2 forward or a greedy `generate` loop touches (elementwise
+# arithmetic, comparisons, indexing, concatenation, factories). The reference gives each of them
+# a Mojo kernel of its own (e.g. `Gather0` aten_fast.py:5336-5371, `AddF32Bf16Spec` :657-687);
+# here they run as the PyTorch-ROCm kernel of the same op on the holders, exactly as the graph
+# surface registers its non-hot ops. An op that is not listed still raises NotImplementedError.
+# ---------------------------------------------------------------------------
+def _resolve_overload(op_name: str):
+    qual, _, overload = op_name.partition(".")
+    namespace, _, name = qual.partition("::")
+    packet = getattr(getattr(torch.ops, namespace), name)
+    return getattr(packet, overload or "default")
+
+
+def holder_impl(op_name: str) -> Callable:
+    """The op on the HIP holders of its mojo arguments; results are wrapped (an output that is
+    one of the inputs' holders — in-place and out= forms — comes back as that input)."""
+    op = None
+
+    def impl(*args, **kwargs):
+        nonlocal op
+        if op is None:
+            op = _resolve_overload(op_name)
+        owners = {}
+
+        def unwrap(x):
+            if isinstance(x, TorchMojoTensor):
+                owners[id(x._holder)] = x
+                return x._holder
+            if isinstance(x, (list, tuple)):
+                return type(x)(unwrap(y) for y in x)
+            if isinstance(x, torch.device) and x.type == "mojo":
+                return hip_device_of(x)
+            return x
+
+        def wrap(y):
+            if isinstance(y, torch.Tensor):
+                owner = owners.get(id(y))
+                return owner if owner is not None else TorchMojoTensor._wrap(y)
+            if isinstance(y, (list, tuple)):
+                return type(y)(wrap(z) for z in y)
+            return y
+
+        if kwargs:
+            return wrap(op(*[unwrap(a) for a in args], **{k: unwrap(v) for k, v in kwargs.items()}))
+        return wrap(op(*[unwrap(a) for a in args]))
+
+    return impl
+
+
+_HOLDER_OPS = (
+    # elementwise arithmetic and activations
+    "aten::add.Tensor", "aten::add.Scalar", "aten::add_.Tensor", "aten::sub.Tensor",
+    "aten::sub.Scalar", "aten::rsub.Scalar", "aten::mul.Tensor", "aten::mul.Scalar",
+    "aten::mul_.Tensor", "aten::div.Tensor", "aten::div.Scalar", "aten::neg", "aten::pow.Tensor_Scalar",
+    "aten::tanh", "aten::exp", "aten::sqrt", "aten::rsqrt", "aten::sigmoid", "aten::relu",
+    "aten::where.self", "aten::masked_fill.Scalar", "aten::masked_fill_.Scalar",
+    "aten::masked_fill.Tensor", "aten::clamp", "aten::clamp_min",
+    # comparisons and boolean logic
+    "aten::eq.Scalar", "aten::eq.Tensor", "aten::ne.Scalar", "aten::ne.Tensor", "aten::lt.Scalar",
+    "aten::lt.Tensor", "aten::le.Scalar", "aten::le.Tensor", "aten::gt.Scalar", "aten::gt.Tensor",
+    "aten::ge.Scalar", "aten::ge.Tensor", "aten::bitwise_and.Tensor", "aten::bitwise_or.Tensor",
+    "aten::bitwise_not", "aten::logical_not", "aten::any", "aten::any.dim", "aten::all",
+    "aten::all.dim", "aten::isin.Tensor_Tensor", "aten::isin.Tensor_Scalar",
+    # reductions that are not hot, scans, selection
+    "aten::max", "aten::max.dim", "aten::min", "aten::cumsum", "aten::topk", "aten::sort",
+    "aten::multinomial",
+    # indexing, gathering, concatenation
+    "aten::embedding", "aten::index_select", "aten::gather", "aten::index.Tensor",
+    "aten::index_put_", "aten::cat", "aten::stack", "aten::split.Tensor",
+    "aten::split_with_sizes", "aten::unbind.int", "aten::squeeze", "aten::flatten.using_ints",
+    "aten::tril", "aten::triu", "aten::repeat", "aten::roll",
+    # fills, copies and factories
+    "aten::fill_.Scalar", "aten::fill_.Tensor", "aten::zero_", "aten::copy_", "aten::full",
+    "aten::full_like", "aten::zeros", "aten::zeros_like", "aten::ones", "aten::ones_like",
+    "aten::new_ones", "aten::new_zeros", "aten::new_full", "aten::new_empty",
+    "aten::empty_like", "aten::arange", "aten::arange.start", "aten::arange.start_step",
+    "aten::scalar_tensor", "aten::lift_fresh", "aten::contiguous",
+)
+for _name in _HOLDER_OPS:
+    register_aten_op(_name)(holder_impl(_name))

@@ -22,6 +22,11 @@ def register_mojo_devices() -> None:
     # Tied parameters (GPT-2's wte / lm_head) must stay one Parameter through .to("mojo").
     torch.__future__.set_swap_module_params_on_conversion(True)
     _setup_privateuseone_for_python_backend("mojo", backend_module=torch_mojo_device_module)
+    from .mojo_device_aten_ops import _resolve_overload
+    from .torch_mojo_tensor import DIRECT_IMPLS
+
     for op_name, func in _aten_ops_registry:
         torch.library.impl(op_name, "privateuseone")(func)
+        # "aten::mean" names the default overload, as torch.library resolves it
+        DIRECT_IMPLS[_resolve_overload(op_name)] = func
     _registered = True
