@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot-op kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|gpt2|copy|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|gpt2|generate|copy|all]
 
 Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
@@ -48,7 +48,7 @@ def _parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "gpt2", "copy"])
+    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "gpt2", "generate", "copy"])
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return p.parse_args()
 
@@ -402,6 +402,46 @@ def main() -> int:
                                f"(the workload's CPU configuration), {cpu_threads} threads")
         sweep[f"gpt2_small_fwd_bf16_B{B}_T{T}"] = row
         del model, compiled
+
+    # ------------------------------------------------------------------ eager decode loop
+    # The reference's own eager benchmark (bench_gpt2_batch.py / current_bench/: HF GPT-2
+    # `generate`, greedy, batch 512, prompt 8, 200 new tokens, bf16), with random-init weights
+    # of the same architecture (no checkpoint offline), on the `mojo` device. Host-bound: about
+    # 480 aten calls per decoded token; PyTorch-ROCm's own eager run is timed beside it.
+    if want in ("all", "generate"):
+        try:
+            from transformers import GPT2Config, GPT2LMHeadModel
+        except Exception as exc:  # noqa: BLE001
+            sweep["gpt2_hf_generate_bf16_B512_eager"] = {"skipped": f"transformers not importable: {exc}"}
+        else:
+            from torch_mojo_backend import register_mojo_devices
+
+            register_mojo_devices()
+            torch.manual_seed(0)
+            B, P, NEW = 512, 8, 200
+            hf = GPT2LMHeadModel(GPT2Config()).eval().to(torch.bfloat16)
+            ids = torch.randint(0, 50257, (B, P))
+            mask = torch.ones_like(ids)
+
+            def gen_rate(device):
+                mdl, i, a = hf.to(device), ids.to(device), mask.to(device)
+                kw = dict(do_sample=False, pad_token_id=50256, attention_mask=a)
+                with torch.no_grad():
+                    mdl.generate(i, max_new_tokens=8, min_new_tokens=8, **kw)
+                    sync()
+                    t0 = time.perf_counter()
+                    mdl.generate(i, max_new_tokens=NEW, min_new_tokens=NEW, **kw)
+                    sync()
+                return B * NEW / (time.perf_counter() - t0)
+
+            rocm = gen_rate(dev)
+            ours = gen_rate("mojo")
+            sweep["gpt2_hf_generate_bf16_B512_eager"] = {
+                "tokens/s": round(ours, 1), "ms_per_decode_step": round(B / ours * 1e3, 3),
+                "pytorch_rocm_eager_tokens/s": round(rocm, 1), "batch": B, "prompt": P,
+                "new_tokens": NEW, "dtype": "bf16",
+                "note": "HF GPT2LMHeadModel.generate on the eager mojo device, random-init weights"}
+            del hf
 
     line = {
         "metric": "GEMM TFLOP/s (bf16 addmm M=N=K=8192, fp32 accumulate)",
