@@ -292,3 +292,36 @@ def test_residual_with_gelu_batches_and_fallbacks():
     assert torch.equal(_ops().gemm(a32, b32, residual=r32), _ops().gemm(a32, b32) + r32)
     with pytest.raises(ValueError):
         _ops().gemm(a2, b2, residual=r2[:, :100])
+
+
+# ---- transposed A (the weight-gradient product dy^T x) -------------------------------------------
+# (m, n, k): A is the .t() view of a [k, m] matrix, B is [k, n]. The MFMA ring takes m, n multiples
+# of 8 with k a multiple of 32 and >= 256 (both tile sizes are covered); the rest is the SIMT path.
+TRANS_A = [(768, 768, 4096), (256, 264, 512), (264, 136, 320), (3072, 768, 2048), (520, 776, 256),
+           (100, 72, 200)]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", TRANS_A)
+def test_mm_transposed_a(mnk, dtype):
+    m, n, k = mnk
+    a_km = seeded((k, m), seed=1, dtype=dtype)
+    b = seeded((k, n), seed=2, dtype=dtype)
+    got = _ops().gemm(_dev(a_km).t(), _dev(b))
+    assert got.dtype == dtype and tuple(got.shape) == (m, n)
+    want = as64(a_km).T @ as64(b)
+    assert rel_frobenius(got, want) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    # every element, not just the norm: fp32 accumulation + one rounding to the storage type
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert np.abs(as64(got) - want).max() <= ulp * np.abs(want).max() + 1e-3
+
+
+def test_mm_transposed_a_batched_and_strided():
+    # a pitch wider than m, batches, and the result of the same product through the SIMT path
+    k, m, n = 512, 256, 320
+    a_store = seeded((3, k, m + 24), seed=3, dtype=torch.bfloat16)
+    b = seeded((3, k, n), seed=4, dtype=torch.bfloat16)
+    a_view = _dev(a_store)[:, :, :m].transpose(1, 2)
+    got = _ops().gemm(a_view, _dev(b))
+    want = np.einsum("bkm,bkn->bmn", as64(a_store)[:, :, :m], as64(b))
+    assert rel_frobenius(got, want) <= 1e-2

@@ -148,6 +148,27 @@ static int launch_simt(const GemmArgs& g, int64_t batch, int trans_a, int trans_
   return check_launch();
 }
 
+// A stored [K, M] with B stored [K, N] (both "k-outer": the weight-gradient product dy^T x):
+// the ring kernel stages A the way it stages N-major B. Needs whole 16-byte chunks along m and n
+// and enough K for the ring.
+template <typename T>
+static int mfma_transposed_a(const GemmArgs& g, int64_t batch, hipStream_t stream) {
+  const int64_t t256 = ((g.m + 255) / 256) * ((g.n + 255) / 256) * batch;
+  if (g.k % 64 == 0 && t256 >= 192)
+    return launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, true>(g, batch, stream);
+  return launch_ring<T, 128, 128, 32, 2, 2, 4, false, TMB_EPI_NONE, true>(g, batch, stream);
+}
+
+static bool mfma_transposed_a_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b,
+                                       int epilogue) {
+  if (!trans_a || trans_b || epilogue != TMB_EPI_NONE) return false;
+  if (g.k % 32 != 0 || g.k < 256 || g.m % 8 != 0 || g.n % 8 != 0 || g.n <= 64) return false;
+  if (g.lda % 8 != 0 || g.ldb % 8 != 0 || !aligned16(g.a) || !aligned16(g.b)) return false;
+  if (batch > 1 && (g.stride_a % 8 != 0 || g.stride_b % 8 != 0)) return false;
+  const int64_t a_span = g.k * g.lda * 2, b_span = g.k * g.ldb * 2;
+  return a_span < (int64_t{1} << 32) && b_span < (int64_t{1} << 32);
+}
+
 static bool mfma_eligible(const GemmArgs& g, int64_t batch, int trans_a, int trans_b) {
   if (trans_a) return false;
   if (g.k % 8 != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return false;
@@ -165,6 +186,8 @@ template <typename T, int EPI>
 static int gemm_typed(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, bool half,
                       hipStream_t stream) {
   if constexpr (!__is_same(T, float)) {
+    if (half && mfma_transposed_a_eligible(g, batch, trans_a, trans_b, EPI))
+      return mfma_transposed_a<T>(g, batch, stream);
     if (half && mfma_eligible(g, batch, trans_a, trans_b)) {
       return trans_b ? mfma_pick_tile<T, true, EPI>(g, batch, stream)
                      : mfma_pick_tile<T, false, EPI>(g, batch, stream);

@@ -76,7 +76,10 @@ constexpr int ring_waves_per_simd(int bm, int bn, int bk, int waves, int stages)
 template <int BM, int BN, int BK, int WAVES, int R>
 constexpr bool kRingPersistent = ring_waves_per_simd(BM, BN, BK, WAVES, R) <= 2;
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
+// A_MMAJOR: A is stored [K, M] (the transposed view of a [K, M] matrix: the weight-gradient
+// product dy^T x); it is then staged and read exactly like N-major B.
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
+          bool A_MMAJOR = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
                              ring_waves_per_simd(BM, BN, BK, WAVES_M* WAVES_N, R))
 void gemm_ring_kernel(GemmArgs g) {
@@ -117,11 +120,21 @@ void gemm_ring_kernel(GemmArgs g) {
   auto plan_tile_loads = [&]() {
 #pragma unroll
   for (int j = 0; j < A_GROUPS; ++j) {
-    const int row = (wave * A_GROUPS + j) * RPG + r_in;
-    const int chunk = slot ^ ring_swizzle<LINE>(row);
-    int64_t grow = m0 + row;
-    grow = grow < M ? grow : M - 1;
-    a_off[j] = static_cast<uint32_t>((grow * g.lda + chunk * 8) * 2);
+    if constexpr (!A_MMAJOR) {
+      const int row = (wave * A_GROUPS + j) * RPG + r_in;
+      const int chunk = slot ^ ring_swizzle<LINE>(row);
+      int64_t grow = m0 + row;
+      grow = grow < M ? grow : M - 1;
+      a_off[j] = static_cast<uint32_t>((grow * g.lda + chunk * 8) * 2);
+    } else {
+      // stage bytes [group*1024 + 16*lane] = k-row (BM*2 bytes each), swizzled 16-byte slot
+      const int at = (wave * A_GROUPS + j) * 1024 + lane * 16;
+      const int krow = at / (BM * 2);
+      const int chunk = ((at % (BM * 2)) >> 4) ^ ((krow & 3) << 2);
+      int64_t col = m0 + chunk * 8;
+      col = col < M ? col : m0;  // rows past the edge: any valid address, never stored
+      a_off[j] = static_cast<uint32_t>((krow * g.lda + col) * 2);
+    }
   }
 #pragma unroll
   for (int j = 0; j < B_GROUPS; ++j) {
@@ -143,6 +156,7 @@ void gemm_ring_kernel(GemmArgs g) {
   }
   };
   const int64_t b_kstep = B_KMAJOR ? 2 : g.ldb * 2;  // bytes per unit of k in B
+  const int64_t a_kstep = A_MMAJOR ? g.lda * 2 : 2;
 
   // The loads are written as inline assembly: M0 carries the LDS destination of the wave's
   // 1 KiB, the SGPR pair the tile's base at this k, the VGPR the lane's byte offset. Issued
@@ -162,7 +176,7 @@ void gemm_ring_kernel(GemmArgs g) {
                  : "memory");
   };
   auto fetch_stage = [&](uint32_t stage_off, int64_t k0) {
-    const unsigned char* ak = a_base + k0 * 2;
+    const unsigned char* ak = a_base + k0 * a_kstep;
     const unsigned char* bk = b_base + k0 * b_kstep;
 #pragma unroll
     for (int j = 0; j < A_GROUPS; ++j) dma16(a_m0 + stage_off + j * 1024, a_off[j], ak);
@@ -197,14 +211,34 @@ void gemm_ring_kernel(GemmArgs g) {
       bt_lane[j] = A_BYTES + krow * (BN * 2) + (((ncol >> 3) ^ (q << 2)) << 4) + (ncol & 7) * 2;
     }
   }
+  int at_lane[TM];
+  if constexpr (A_MMAJOR) {
+    const int j16 = lane & 15, q = j16 >> 2, msub = (lane >> 4) & 1;
+    const int krow = frag_half * 8 + q;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int mcol = wm * WM + i * 32 + msub * 16 + (j16 & 3) * 4;
+      at_lane[i] = krow * (BM * 2) + (((mcol >> 3) ^ (q << 2)) << 4) + (mcol & 7) * 2;
+    }
+  }
   typedef __attribute__((address_space(3))) u32x4_t lds_u32x4_t;
   u32x4_t af[2][TM], bf[2][TN];
   // ks is a compile-time constant at every call site (the k-step loop is unrolled).
   auto load_frags = [&](uint32_t stage_off, int ks, int s) {
     lds_u8* stage = (lds_u8*)ring + stage_off;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-      af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (32 * LINE));
+    for (int i = 0; i < TM; ++i) {
+      if constexpr (!A_MMAJOR) {
+        af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (32 * LINE));
+      } else {
+        lds_u8* src = stage + at_lane[i] + ks * 16 * (BM * 2);
+        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
+        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src + 4 * (BM * 2)));
+        typedef short i16x8_t __attribute__((ext_vector_type(8)));
+        const i16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        af[s][i] = __builtin_bit_cast(u32x4_t, both);
+      }
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if constexpr (B_KMAJOR) {
@@ -353,7 +387,8 @@ static int compute_units() {
   return cus;
 }
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI>
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
+          bool A_MMAJOR = false>
 static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
@@ -371,7 +406,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   const int64_t grid_x = (!kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R> || tiles < resident)
                              ? tiles
                              : resident;
-  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI>
+  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR>
       <<<dim3(static_cast<unsigned>(grid_x), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();
