@@ -157,6 +157,35 @@ int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v, in
 int tmb_gelu(void* out, const void* in, int64_t numel, int dtype, int approximate_tanh,
              void* stream);
 
+/* GELU backward over `numel` contiguous elements: grad_in = grad_out * gelu'(in), fp32 inside,
+ * one cast; all three tensors have type `dtype`. Replaces `GeluBackwardF32` / `GeluBackwardBF16`
+ * (eager_kernels/activation_backward_ops.mojo:50-73 for the two derivatives, aten_fast.py:1413-1447
+ * for the call) and `custom_mojo_ops.gelu_backward` (aten_functions.py:2070-2102). */
+int tmb_gelu_backward(void* grad_in, const void* grad_out, const void* in, int64_t numel,
+                      int dtype, int approximate_tanh, void* stream);
+
+/* Backward of a row softmax (log_mode 0: grad_in = out * (grad_out - sum(grad_out * out))) or
+ * log-softmax (log_mode 1: grad_in = grad_out - exp(out) * sum(grad_out)) from the saved output;
+ * contiguous [rows, cols], one dtype for the three tensors. Replaces the composed
+ * sum -> exp -> addcmul of aten_functions.py:788-833 and the fused kernel behind
+ * `fast_aten__log_softmax_backward_data` (aten_fast.py:3237-3330). */
+int tmb_softmax_backward_rows(void* grad_in, const void* grad_out, const void* out, int64_t rows,
+                              int64_t cols, int dtype, int log_mode, void* stream);
+
+/* Layer-norm backward over contiguous [rows, cols] from the saved fp32 statistics:
+ *   grad_in    = rstd * (g dy - mean_row(g dy) - xhat * mean_row(g dy xhat)),  xhat = (x - mean) rstd
+ *   grad_gamma = sum over rows of dy * xhat,   grad_beta = sum over rows of dy
+ * Any of the three outputs may be NULL (ATen's output_mask); `gamma` may be NULL (no affine).
+ * The parameter gradients are summed slab by slab through `workspace`
+ * (tmb_layer_norm_backward_workspace_bytes) in an order that depends on the shape only.
+ * Replaces `LayerNormBackwardF32(grad_input, grad_weight, grad_bias, grad, x, mean, rstd, gamma,
+ * rows, cols, mask_bits, ctx)` (aten_fast.py:2797-2913). */
+size_t tmb_layer_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_beta,
+                                 const void* grad_out, const void* in, const float* mean,
+                                 const float* rstd, const void* gamma, int64_t rows, int64_t cols,
+                                 int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Plain device copy kernel (16-byte vectors, grid-stride) — the bandwidth yardstick the
  * benchmark and the counter calibration use. No reference counterpart. */
 int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* stream);

@@ -76,6 +76,11 @@ def lib() -> ctypes.CDLL:
         L.orc_reduce.argtypes = [vp, vp, i64, i64, ci, ci]
         L.orc_argmax.argtypes = [vp, vp, i64, i64, ci]
         L.orc_gelu.argtypes = [vp, vp, i64, ci, ci]
+        L.orc_gelu_backward.argtypes = [vp, vp, vp, i64, ci, ci]
+        L.orc_softmax_backward.argtypes = [vp, vp, vp, i64, i64, ci, ci]
+        L.orc_layer_norm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, vp]
+        for f in (L.orc_gelu_backward, L.orc_softmax_backward, L.orc_layer_norm_backward):
+            f.restype = ci
         L.orc_convert_to_f32.argtypes = [vp, vp, i64, ci]
         L.orc_convert_from_f32.argtypes = [vp, vp, i64, ci]
         for f in (L.orc_gemm, L.orc_softmax, L.orc_layer_norm, L.orc_reduce, L.orc_argmax,
@@ -233,6 +238,46 @@ def gelu(x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
         _check(lib().orc_gelu(out.data_ptr(), x.data_ptr(), x.numel(), _code(x.dtype),
                               int(approximate == "tanh")), "gelu")
     return out
+
+
+def gelu_backward(grad: torch.Tensor, x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
+    grad, x = _cpu(grad), _cpu(x)
+    out = torch.empty_like(x)
+    if x.numel():
+        _check(lib().orc_gelu_backward(out.data_ptr(), grad.data_ptr(), x.data_ptr(), x.numel(),
+                                       _code(x.dtype), int(approximate == "tanh")), "gelu_backward")
+    return out
+
+
+def softmax_backward_rows(grad: torch.Tensor, out: torch.Tensor, log: bool) -> torch.Tensor:
+    grad, out = _cpu(grad), _cpu(out)
+    assert out.dim() == 2 and grad.shape == out.shape
+    res = torch.empty_like(out)
+    if out.numel():
+        _check(lib().orc_softmax_backward(res.data_ptr(), grad.data_ptr(), out.data_ptr(),
+                                          out.shape[0], out.shape[1], _code(out.dtype), int(log)),
+               "softmax_backward")
+    return res
+
+
+def layer_norm_backward_rows(grad: torch.Tensor, x: torch.Tensor, mean: torch.Tensor,
+                             rstd: torch.Tensor, gamma: Optional[torch.Tensor]):
+    """(dx, dgamma, dbeta) for [rows, cols] inputs and float32 per-row statistics."""
+    grad, x = _cpu(grad), _cpu(x)
+    assert x.dim() == 2 and grad.shape == x.shape
+    rows, cols = x.shape
+    mean = _cpu(mean.reshape(-1).float())
+    rstd = _cpu(rstd.reshape(-1).float())
+    g = None if gamma is None else _cpu(gamma.reshape(-1))
+    dx = torch.empty_like(x)
+    dg = torch.empty(cols, dtype=x.dtype)
+    db = torch.empty(cols, dtype=x.dtype)
+    scratch = torch.empty(2 * cols, dtype=torch.float32)
+    _check(lib().orc_layer_norm_backward(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), grad.data_ptr(),
+                                         x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), _ptr(g),
+                                         rows, cols, _code(x.dtype), scratch.data_ptr()),
+           "layer_norm_backward")
+    return dx, dg, db
 
 
 # ---------------------------------------------------------------------------

@@ -23,6 +23,11 @@
  *                   is what ATen does and what the reference's tests compare with; the
  *                   reference's scan only keeps a NaN that sits at index 0.
  *   orc_gelu        activation_forward_kernels.mojo:22-56 (fp32 inside, one cast)
+ *   orc_gelu_backward       activation_backward_ops.mojo:50-73 (`_exact_grad`, `_tanh_grad`)
+ *   orc_softmax_backward    ../aten_functions.py:788-833 (grad - exp(out) * sum(grad)) and its
+ *                           softmax twin out * (grad - sum(grad * out))
+ *   orc_layer_norm_backward aten_fast.py:2797-2913 (LayerNormBackwardF32: grad_input from the
+ *                           saved mean / rstd, grad_weight = sum dy*xhat, grad_bias = sum dy)
  *
  * Pinning: tests/test_oracle_pins.py checks every function against float64 closed forms,
  * brute-force Python loops on tiny inputs, mathematical invariants and PyTorch CPU eager (the
@@ -331,6 +336,81 @@ int orc_gelu(void* out, const void* in, int64_t numel, int dtype, int approximat
   for (int64_t i = 0; i < numel; ++i) {
     const float x = load_f(in, i, dtype);
     store_f(out, i, dtype, approximate_tanh ? gelu_tanh(x) : gelu_erf(x));
+  }
+  return 0;
+}
+
+int orc_gelu_backward(void* out, const void* grad, const void* in, int64_t numel, int dtype,
+                      int approximate_tanh) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < numel; ++i) {
+    const float x = load_f(in, i, dtype), g = load_f(grad, i, dtype);
+    float d;
+    if (approximate_tanh) {
+      const float beta = 0.7978845608028654f, kappa = 0.044715f;
+      const float x2 = x * x;
+      const float t = tanhf(beta * (x + kappa * (x2 * x)));
+      d = 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * beta * (1.0f + 3.0f * kappa * x2);
+    } else {
+      const float cdf = 0.5f * (1.0f + erff(x * 0.7071067811865476f));
+      const float pdf = 0.3989422804014327f * expf(-0.5f * (x * x));
+      d = cdf + x * pdf;
+    }
+    store_f(out, i, dtype, g * d);
+  }
+  return 0;
+}
+
+int orc_softmax_backward(void* gin, const void* gout, const void* y, int64_t rows, int64_t cols,
+                         int dtype, int log_mode) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * cols;
+    float s = 0.0f;
+    for (int64_t j = 0; j < cols; ++j) {
+      const float g = load_f(gout, base + j, dtype);
+      s += log_mode ? g : g * load_f(y, base + j, dtype);
+    }
+    for (int64_t j = 0; j < cols; ++j) {
+      const float g = load_f(gout, base + j, dtype), o = load_f(y, base + j, dtype);
+      store_f(gin, base + j, dtype, log_mode ? g - expf(o) * s : o * (g - s));
+    }
+  }
+  return 0;
+}
+
+/* dgamma / dbeta are accumulated row after row in fp32 (any of the outputs may be NULL). */
+int orc_layer_norm_backward(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x,
+                            const float* mean, const float* rstd, const void* gamma,
+                            int64_t rows, int64_t cols, int dtype, float* scratch) {
+  float* sg = scratch;          /* [cols] */
+  float* sb = scratch + cols;   /* [cols] */
+  for (int64_t j = 0; j < 2 * cols; ++j) scratch[j] = 0.0f;
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * cols;
+    const float mu = mean[r], rs = rstd[r];
+    float s1 = 0.0f, s2 = 0.0f;
+    for (int64_t j = 0; j < cols; ++j) {
+      const float d = load_f(dy, base + j, dtype);
+      const float gd = d * (gamma ? load_f(gamma, j, dtype) : 1.0f);
+      const float xh = (load_f(x, base + j, dtype) - mu) * rs;
+      s1 += gd;
+      s2 += gd * xh;
+      sg[j] += d * xh;
+      sb[j] += d;
+    }
+    if (dx) {
+      const float m1 = s1 / (float)cols, m2 = s2 / (float)cols;
+      for (int64_t j = 0; j < cols; ++j) {
+        const float gd = load_f(dy, base + j, dtype) * (gamma ? load_f(gamma, j, dtype) : 1.0f);
+        const float xh = (load_f(x, base + j, dtype) - mu) * rs;
+        store_f(dx, base + j, dtype, rs * (gd - m1 - xh * m2));
+      }
+    }
+  }
+  for (int64_t j = 0; j < cols; ++j) {
+    if (dgamma) store_f(dgamma, j, dtype, sg[j]);
+    if (dbeta) store_f(dbeta, j, dtype, sb[j]);
   }
   return 0;
 }

@@ -1,0 +1,173 @@
+"""GPU parity of the backward twins (gelu, softmax / log-softmax, layer norm, linear) against the
+C oracle, float64 autograd and the invariants the formulas fix."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import as64, seeded
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = [torch.float32, torch.bfloat16, torch.float16]
+TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2, torch.float16: 3e-3}
+
+
+def _ops():
+    from torch_mojo_backend.eager_kernels import hip_ops
+    return hip_ops
+
+
+def _autograd64(fn, *inputs):
+    """Gradients of sum(fn(*inputs) * g) in float64 on the CPU (inputs given in storage precision)."""
+    xs = [x.double().requires_grad_(True) for x in inputs[:-1]]
+    g = inputs[-1].double()
+    (fn(*xs) * g).sum().backward()
+    return [x.grad.numpy() for x in xs]
+
+
+# ---- gelu ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("approximate", ["none", "tanh"])
+@pytest.mark.parametrize("numel", [1, 7, 4096, 100003])
+def test_gelu_backward(dtype, approximate, numel):
+    x = seeded((numel,), seed=1, dtype=dtype) * 3
+    g = seeded((numel,), seed=2, dtype=dtype)
+    got = _ops().gelu_backward(g.cuda(), x.cuda(), approximate)
+    assert got.dtype == dtype and got.shape == x.shape
+    (want,) = _autograd64(lambda t: torch.nn.functional.gelu(t, approximate=approximate), x, g)
+    scale = np.abs(as64(g)).max() + 1.0
+    assert np.abs(as64(got) - want).max() <= TOL[dtype] * scale
+    ref = oracle.gelu_backward(g, x, approximate)
+    assert np.abs(as64(got) - as64(ref)).max() <= TOL[dtype] * scale
+
+
+def test_gelu_backward_limits():
+    x = torch.tensor([0.0, 30.0, -30.0, 1e4, -1e4], dtype=torch.float32)
+    g = torch.full_like(x, 2.0)
+    for mode in ("none", "tanh"):
+        got = _ops().gelu_backward(g.cuda(), x.cuda(), mode).cpu()
+        assert torch.allclose(got, torch.tensor([1.0, 2.0, 0.0, 2.0, 0.0]), atol=1e-6), (mode, got)
+
+
+# ---- softmax / log-softmax ----------------------------------------------------------------------
+SOFTMAX_SHAPES = [(1, 1), (3, 5), (33, 257), (64, 1024), (17, 4096), (5, 8192), (4, 50257), (2, 70000)]
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_backward_rows(shape, dtype, log):
+    x = seeded(shape, seed=3, dtype=torch.float32) * 2
+    fwd = (torch.log_softmax if log else torch.softmax)(x, -1).to(dtype)
+    g = seeded(shape, seed=4, dtype=dtype)
+    got = _ops().softmax_backward(g.cuda(), fwd.cuda(), -1, log)
+    assert got.dtype == dtype and got.shape == fwd.shape
+    y64, g64 = as64(fwd), as64(g)
+    if log:
+        want = g64 - np.exp(y64) * g64.sum(-1, keepdims=True)
+    else:
+        want = y64 * (g64 - (g64 * y64).sum(-1, keepdims=True))
+    # the row sum carries the fp32 error of `cols` terms of size |g| <= ~4
+    bound = TOL[dtype] * (np.abs(want).max() + 1.0) + shape[1] * 2.0 ** -24 * 8.0 * (np.abs(np.exp(y64)).max() if log else 1.0)
+    assert np.abs(as64(got) - want).max() <= bound
+    ref = oracle.softmax_backward_rows(g, fwd, log)
+    assert np.abs(as64(got) - as64(ref)).max() <= 2 * bound
+
+
+def test_softmax_backward_invariants_and_dims():
+    # a constant upstream gradient cancels (softmax) / the row of gradients sums to zero (log)
+    x = seeded((6, 300), seed=5)
+    y = torch.softmax(x, -1)
+    got = _ops().softmax_backward(torch.full_like(y, 3.0).cuda(), y.cuda(), -1, False).cpu()
+    assert got.abs().max().item() <= 1e-6
+    ly = torch.log_softmax(x, -1)
+    g = seeded((6, 300), seed=6)
+    got = _ops().softmax_backward(g.cuda(), ly.cuda(), -1, True).cpu()
+    assert got.sum(-1).abs().max().item() <= 1e-4
+    # other dims go through a transposed copy
+    x3 = seeded((4, 9, 11), seed=7)
+    g3 = seeded((4, 9, 11), seed=8)
+    for dim in (0, 1, -1):
+        xr = x3.clone().requires_grad_(True)
+        out = torch.softmax(xr, dim)
+        out.backward(g3)
+        got = _ops().softmax_backward(g3.cuda(), out.detach().cuda(), dim, False).cpu()
+        torch.testing.assert_close(got, xr.grad, rtol=1e-5, atol=1e-6)
+
+
+# ---- layer norm ---------------------------------------------------------------------------------
+LN_SHAPES = [(1, 8), (5, 65), (33, 768), (64, 1000), (9, 4096), (300, 768), (7, 12288), (3, 50257)]
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", LN_SHAPES)
+@pytest.mark.parametrize("affine", [True, False])
+def test_layer_norm_backward(shape, dtype, affine):
+    rows, cols = shape
+    x = seeded(shape, seed=9, dtype=dtype)
+    g = seeded(shape, seed=10, dtype=dtype)
+    w = (1 + 0.1 * seeded((cols,), seed=11)).to(dtype) if affine else None
+    out, mean, rstd = _ops().layer_norm(x.cuda(), [cols], None if w is None else w.cuda(), None, 1e-5)
+    dx, dw, db = _ops().layer_norm_backward(g.cuda(), x.cuda(), [cols], mean, rstd,
+                                            None if w is None else w.cuda(), [True, affine, True])
+    assert dx.dtype == dtype and dx.shape == x.shape and db.shape == (cols,)
+    x64 = x.double().requires_grad_(True)
+    w64 = None if w is None else w.double().requires_grad_(True)
+    b64 = torch.zeros(cols, dtype=torch.float64, requires_grad=True)
+    (torch.nn.functional.layer_norm(x64, [cols], w64, b64, 1e-5) * g.double()).sum().backward()
+    scale = np.abs(x64.grad.numpy()).max() + 1.0
+    assert np.abs(as64(dx) - x64.grad.numpy()).max() <= TOL[dtype] * scale * 4
+    col_tol = TOL[dtype] * (np.abs(b64.grad.numpy()).max() + 1.0) + rows * 2.0 ** -22
+    assert np.abs(as64(db) - b64.grad.numpy()).max() <= col_tol * 4
+    if affine:
+        assert np.abs(as64(dw) - w64.grad.numpy()).max() <= \
+            (TOL[dtype] * (np.abs(w64.grad.numpy()).max() + 1.0) + rows * 2.0 ** -22) * 4
+    rdx, rdw, rdb = oracle.layer_norm_backward_rows(g, x, mean.cpu(), rstd.cpu(), w)
+    assert np.abs(as64(dx) - as64(rdx)).max() <= TOL[dtype] * scale * 4
+    assert np.abs(as64(db) - as64(rdb)).max() <= col_tol * 4
+
+
+def test_layer_norm_backward_invariants_and_masks():
+    x = seeded((40, 512), seed=12)
+    g = seeded((40, 512), seed=13)
+    w = 1 + 0.1 * seeded((512,), seed=14)
+    _, mean, rstd = _ops().layer_norm(x.cuda(), [512], w.cuda(), None, 1e-5)
+    dx, dw, db = _ops().layer_norm_backward(g.cuda(), x.cuda(), [512], mean, rstd, w.cuda(),
+                                            [True, False, False])
+    assert dw is None and db is None
+    dx = dx.cpu()
+    xhat = (x - x.mean(-1, keepdim=True)) * rstd.cpu().view(-1, 1)
+    # grad_input is orthogonal to the constant vector and to xhat
+    assert dx.sum(-1).abs().max().item() <= 2e-4
+    assert (dx * xhat).sum(-1).abs().max().item() <= 2e-3
+    only_params = _ops().layer_norm_backward(g.cuda(), x.cuda(), [512], mean, rstd, w.cuda(),
+                                             [False, True, True])
+    assert only_params[0] is None
+    torch.testing.assert_close(only_params[2].cpu(), g.sum(0), rtol=1e-5, atol=1e-4)
+    # same call twice: bit-identical parameter gradients (fixed summation order)
+    again = _ops().layer_norm_backward(g.cuda(), x.cuda(), [512], mean, rstd, w.cuda(),
+                                       [False, True, True])
+    assert torch.equal(only_params[1], again[1]) and torch.equal(only_params[2], again[2])
+
+
+# ---- linear -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [((4, 33, 64), 48), ((512, 768), 2304), ((8, 128, 768), 768)])
+def test_linear_backward(shape, dtype):
+    xshape, out_f = shape
+    in_f = xshape[-1]
+    x = seeded(xshape, seed=15, dtype=dtype)
+    w = (seeded((out_f, in_f), seed=16) * 0.05).to(dtype)
+    g = seeded(xshape[:-1] + (out_f,), seed=17, dtype=dtype)
+    dx, dw, db = _ops().linear_backward(x.cuda(), g.cuda(), w.cuda(), [True, True, True])
+    x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    b64 = torch.zeros(out_f, dtype=torch.float64, requires_grad=True)
+    (torch.nn.functional.linear(x64, w64, b64) * g.double()).sum().backward()
+    rel = 1e-5 if dtype == torch.float32 else 1e-2
+    for got, want in ((dx, x64.grad), (dw, w64.grad), (db, b64.grad)):
+        want = want.numpy()
+        assert np.linalg.norm(as64(got) - want) <= rel * np.linalg.norm(want) + 1e-6
+    none_x = _ops().linear_backward(x.cuda(), g.cuda(), w.cuda(), [False, True, False])
+    assert none_x[0] is None and none_x[1] is not None and none_x[2].abs().sum().item() == 0

@@ -1,0 +1,527 @@
+// Backward twins of the hot ops for gfx950: GELU, softmax / log-softmax and layer norm.
+//
+// All of them are bound by HBM traffic and use the forward kernels' layout: a row lives in the
+// registers of WPR cooperating waves (VPL 16-byte vectors per lane and input stream), loads are
+// non-temporal (every element is read once), reductions are DPP inside a wave and a fixed-order
+// LDS combine across the waves of a row, arithmetic is fp32 with one cast on store.
+//
+// Formulas follow the reference:
+//   gelu_backward          eager_kernels/activation_backward_ops.mojo:50-73
+//   log_softmax backward   aten_functions.py:788-833  (grad - exp(out) * sum(grad))
+//   softmax backward       out * (grad - sum(grad * out))
+//   layer norm backward    eager_kernels/aten_fast.py:2797-2913 (LayerNormBackwardF32):
+//                          dx = rstd * (g dy - mean(g dy) - xhat mean(g dy xhat)),
+//                          dgamma = sum_rows dy xhat, dbeta = sum_rows dy
+#include <type_traits>
+
+#include "tmb_common.h"
+
+namespace tmb {
+
+// ---------------------------------------------------------------------------
+// GELU backward
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_grad_erf(float x, float g) {
+#pragma clang fp contract(off)
+  const float cdf = 0.5f * (1.0f + erff(x * 0.7071067811865476f));
+  const float pdf = 0.3989422804014327f * exp_f32(-0.5f * (x * x));
+  return g * (cdf + x * pdf);
+}
+__device__ __forceinline__ float gelu_grad_tanh(float x, float g) {
+#pragma clang fp contract(off)
+  constexpr float kBeta = 0.7978845608028654f, kKappa = 0.044715f;
+  const float x2 = x * x;
+  const float inner = kBeta * (x + kKappa * (x2 * x));
+  // tanh(u) = 1 - 2 / (1 + e^(2u)); e^(2u) overflows to +inf (t = 1) and underflows to 0 (t = -1)
+  const float e = __builtin_amdgcn_exp2f(inner * 2.8853900817779268f);
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
+  const float d = 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * kBeta * (1.0f + 3.0f * kKappa * x2);
+  return g * d;
+}
+
+template <typename T, bool TANH>
+__global__ __launch_bounds__(256) void gelu_backward_kernel(T* __restrict__ out,
+                                                            const T* __restrict__ grad,
+                                                            const T* __restrict__ in,
+                                                            int64_t numel, int64_t nvec) {
+  constexpr int EPV = Vec16<T>::N;
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid < nvec) {
+    const Vec16<T> xv = load_vec16_stream(in + tid * EPV);
+    const Vec16<T> gv = load_vec16_stream(grad + tid * EPV);
+    float y[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      const float x = to_f32(xv.v[e]), g = to_f32(gv.v[e]);
+      y[e] = TANH ? gelu_grad_tanh(x, g) : gelu_grad_erf(x, g);
+    }
+    store_converted<T, EPV>(out + tid * EPV, y);
+  }
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = nvec * EPV + tid; i < numel; i += stride) {
+    const float x = to_f32(in[i]), g = to_f32(grad[i]);
+    out[i] = from_f32<T>(TANH ? gelu_grad_tanh(x, g) : gelu_grad_erf(x, g));
+  }
+}
+
+template <typename T>
+static int launch_gelu_backward(void* out_, const void* grad_, const void* in_, int64_t numel,
+                                int tanh_mode, hipStream_t s) {
+  T* out = static_cast<T*>(out_);
+  const T* grad = static_cast<const T*>(grad_);
+  const T* in = static_cast<const T*>(in_);
+  constexpr int EPV = Vec16<T>::N;
+  const int64_t nvec = (aligned16(in) && aligned16(out) && aligned16(grad)) ? numel / EPV : 0;
+  const int64_t work = nvec > 0 ? nvec : numel;
+  int64_t blocks = (work + 255) / 256;
+  if (blocks > (int64_t{1} << 30)) blocks = int64_t{1} << 30;
+  if (blocks < 1) blocks = 1;
+  if (tanh_mode)
+    gelu_backward_kernel<T, true><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(out, grad, in, numel, nvec);
+  else
+    gelu_backward_kernel<T, false><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(out, grad, in, numel, nvec);
+  return check_launch();
+}
+
+// ---------------------------------------------------------------------------
+// softmax / log-softmax backward (from the saved output)
+// ---------------------------------------------------------------------------
+template <typename T, int WPR, int VPL, bool LOG, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void softmax_backward_regs_kernel(T* __restrict__ gin,
+                                                                      const T* __restrict__ gout,
+                                                                      const T* __restrict__ y,
+                                                                      int64_t rows, int cols) {
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int WAVES = BLOCK / kWave;
+  constexpr int GROUPS = WAVES / WPR;
+  __shared__ float slot[WAVES];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int group = wave / WPR, wave_in_row = wave - group * WPR;
+  const int nvec = cols / EPV;
+  int64_t row = static_cast<int64_t>(blockIdx.x) * GROUPS + group;
+  const bool live = row < rows;
+  if (!live) row = rows - 1;  // keep lock-step for the barriers; nothing is stored
+  const T* gsrc = gout + row * static_cast<int64_t>(cols);
+  const T* ysrc = y + row * static_cast<int64_t>(cols);
+
+  float g[VPL][EPV], o[VPL][EPV];
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WPR + wave_in_row) * kWave + lane;
+    const bool ok = vi < nvec;
+    const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
+    const Vec16<T> gv = load_vec16_stream(gsrc + at);
+    const Vec16<T> yv = load_vec16_stream(ysrc + at);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      g[v][e] = ok ? to_f32(gv.v[e]) : 0.0f;
+      o[v][e] = ok ? to_f32(yv.v[e]) : (LOG ? -__builtin_inff() : 0.0f);
+    }
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) s += LOG ? g[v][e] : g[v][e] * o[v][e];
+  s = wave_sum(s);
+  s = group_reduce(s, slot, wave, group * WPR, WPR, SumOp{});
+  if (!live) return;
+  T* dst = gin + row * static_cast<int64_t>(cols);
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WPR + wave_in_row) * kWave + lane;
+    float r[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e)
+      r[e] = LOG ? g[v][e] - exp_for<T>(o[v][e]) * s : o[v][e] * (g[v][e] - s);
+    if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r);
+  }
+}
+
+// Any width / alignment: one workgroup per row, the row is read twice (the second time from L2).
+template <typename T, bool LOG>
+__global__ __launch_bounds__(256) void softmax_backward_generic_kernel(T* __restrict__ gin,
+                                                                       const T* __restrict__ gout,
+                                                                       const T* __restrict__ y,
+                                                                       int64_t rows, int64_t cols) {
+  __shared__ float slot[4];
+  const int wave = threadIdx.x >> 6;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const T* gsrc = gout + row * cols;
+    const T* ysrc = y + row * cols;
+    float s = 0.0f;
+    for (int64_t j = threadIdx.x; j < cols; j += 256)
+      s += LOG ? to_f32(gsrc[j]) : to_f32(gsrc[j]) * to_f32(ysrc[j]);
+    s = wave_sum(s);
+    s = group_reduce(s, slot, wave, 0, 4, SumOp{});
+    for (int64_t j = threadIdx.x; j < cols; j += 256) {
+      const float g = to_f32(gsrc[j]), o = to_f32(ysrc[j]);
+      gin[row * cols + j] = from_f32<T>(LOG ? g - exp_for<T>(o) * s : o * (g - s));
+    }
+  }
+}
+
+template <typename T, bool LOG>
+static int softmax_backward_dispatch(void* gin_, const void* gout_, const void* y_, int64_t rows,
+                                     int64_t cols, hipStream_t stream) {
+  T* gin = static_cast<T*>(gin_);
+  const T* gout = static_cast<const T*>(gout_);
+  const T* y = static_cast<const T*>(y_);
+  constexpr int EPV = Vec16<T>::N;
+  const bool vec_ok = cols % EPV == 0 && aligned16(gin) && aligned16(gout) && aligned16(y) &&
+                      rows < (int64_t{1} << 31);
+  const int64_t nvec = cols / EPV;
+#define TMB_SB(WPR, VPL, BLOCK)                                                                   \
+  {                                                                                               \
+    constexpr int RPB = (BLOCK / kWave) / WPR;                                                    \
+    const int64_t blocks = (rows + RPB - 1) / RPB;                                                \
+    softmax_backward_regs_kernel<T, WPR, VPL, LOG, BLOCK>                                         \
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(gin, gout, y, rows,     \
+                                                                         static_cast<int>(cols)); \
+    return check_launch();                                                                        \
+  }
+  if (vec_ok && nvec <= 16 * 64 * 4) {
+    // same geometry rule as the forward kernel: light waves, up to 16 per row
+    if (nvec <= 64) TMB_SB(1, 1, 256)
+    if (nvec <= 128) TMB_SB(2, 1, 256)
+    if (nvec <= 256) TMB_SB(2, 2, 256)
+    if (nvec <= 512) TMB_SB(4, 2, 256)
+    if (nvec <= 1024) TMB_SB(8, 2, 512)
+    if (nvec <= 2048) TMB_SB(16, 2, 1024)
+    TMB_SB(16, 4, 1024)
+  }
+#undef TMB_SB
+  const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
+  softmax_backward_generic_kernel<T, LOG>
+      <<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(gin, gout, y, rows, cols);
+  return check_launch();
+}
+
+// ---------------------------------------------------------------------------
+// layer norm backward: grad_input
+// ---------------------------------------------------------------------------
+template <typename T, int WPR, int VPL, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
+    T* __restrict__ dx, const T* __restrict__ dy, const T* __restrict__ x,
+    const float* __restrict__ mean, const float* __restrict__ rstd, const T* __restrict__ gamma,
+    int64_t rows, int cols) {
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int WAVES = BLOCK / kWave;
+  constexpr int GROUPS = WAVES / WPR;
+  __shared__ float slot[WAVES];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int group = wave / WPR, wave_in_row = wave - group * WPR;
+  const int nvec = cols / EPV;
+  const float n = static_cast<float>(cols);
+  int64_t row = static_cast<int64_t>(blockIdx.x) * GROUPS + group;
+  const bool live = row < rows;
+  if (!live) row = rows - 1;
+  const T* dsrc = dy + row * static_cast<int64_t>(cols);
+  const T* xsrc = x + row * static_cast<int64_t>(cols);
+  const float mu = mean[row], rs = rstd[row];
+
+  float gd[VPL][EPV], xh[VPL][EPV];  // gamma*dy and xhat
+  float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WPR + wave_in_row) * kWave + lane;
+    const bool ok = vi < nvec;
+    const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
+    const Vec16<T> dv = load_vec16_stream(dsrc + at);
+    const Vec16<T> xv = load_vec16_stream(xsrc + at);
+    Vec16<T> gv;
+    if (gamma != nullptr) gv = load_vec16(gamma + at);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      const float d = to_f32(dv.v[e]) * (gamma != nullptr ? to_f32(gv.v[e]) : 1.0f);
+      gd[v][e] = ok ? d : 0.0f;
+      xh[v][e] = ok ? (to_f32(xv.v[e]) - mu) * rs : 0.0f;
+      s1 += gd[v][e];
+      s2 += gd[v][e] * xh[v][e];
+    }
+  }
+  s1 = wave_sum(s1);
+  s1 = group_reduce(s1, slot, wave, group * WPR, WPR, SumOp{});
+  s2 = wave_sum(s2);
+  s2 = group_reduce(s2, slot, wave, group * WPR, WPR, SumOp{});
+  if (!live) return;
+  const float m1 = s1 / n, m2 = s2 / n;
+  T* dst = dx + row * static_cast<int64_t>(cols);
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WPR + wave_in_row) * kWave + lane;
+    float r[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) r[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
+    if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_backward_dx_generic_kernel(
+    T* __restrict__ dx, const T* __restrict__ dy, const T* __restrict__ x,
+    const float* __restrict__ mean, const float* __restrict__ rstd, const T* __restrict__ gamma,
+    int64_t rows, int64_t cols) {
+  __shared__ float slot[4];
+  const int wave = threadIdx.x >> 6;
+  const float n = static_cast<float>(cols);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const T* dsrc = dy + row * cols;
+    const T* xsrc = x + row * cols;
+    const float mu = mean[row], rs = rstd[row];
+    float s1 = 0.0f, s2 = 0.0f;
+    for (int64_t j = threadIdx.x; j < cols; j += 256) {
+      const float d = to_f32(dsrc[j]) * (gamma != nullptr ? to_f32(gamma[j]) : 1.0f);
+      s1 += d;
+      s2 += d * ((to_f32(xsrc[j]) - mu) * rs);
+    }
+    s1 = wave_sum(s1);
+    s1 = group_reduce(s1, slot, wave, 0, 4, SumOp{});
+    s2 = wave_sum(s2);
+    s2 = group_reduce(s2, slot, wave, 0, 4, SumOp{});
+    const float m1 = s1 / n, m2 = s2 / n;
+    for (int64_t j = threadIdx.x; j < cols; j += 256) {
+      const float d = to_f32(dsrc[j]) * (gamma != nullptr ? to_f32(gamma[j]) : 1.0f);
+      const float xh = (to_f32(xsrc[j]) - mu) * rs;
+      dx[row * cols + j] = from_f32<T>(rs * (d - m1 - xh * m2));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// layer norm backward: grad_weight / grad_bias (sums over the rows, per column)
+// A workgroup owns 64 column vectors (VEC: 16 bytes each, otherwise single elements) and a slab
+// of rows; its four waves take every fourth row of the slab, so each wave-wide load covers 1 KiB
+// of one row. Partials go to an fp32 workspace [slabs][2][cols]; a second kernel adds the slabs
+// in order. No atomics: the result depends on the shape only.
+// ---------------------------------------------------------------------------
+constexpr int kParamWaves = 4;
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kParamWaves* kWave) void layer_norm_param_partial_kernel(
+    float* __restrict__ partial, const T* __restrict__ dy, const T* __restrict__ x,
+    const float* __restrict__ mean, const float* __restrict__ rstd, int64_t rows, int64_t cols,
+    int64_t rows_per_slab) {
+  constexpr int EPV = VEC ? Vec16<T>::N : 1;
+  __shared__ float lds[kParamWaves][2][kWave * EPV];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t unit = static_cast<int64_t>(blockIdx.x) * kWave + lane;  // vector / element index
+  const int64_t col0 = unit * EPV;
+  const bool ok = col0 < cols;
+  const int64_t slab = blockIdx.y;
+  const int64_t r_begin = slab * rows_per_slab;
+  const int64_t r_end = r_begin + rows_per_slab < rows ? r_begin + rows_per_slab : rows;
+  float dg[EPV], db[EPV];
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) dg[e] = db[e] = 0.0f;
+  for (int64_t row = r_begin + wave; row < r_end; row += kParamWaves) {
+    const float mu = mean[row], rs = rstd[row];
+    if (ok) {
+      if constexpr (VEC) {
+        const Vec16<T> dv = load_vec16_stream(dy + row * cols + col0);
+        const Vec16<T> xv = load_vec16_stream(x + row * cols + col0);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          const float d = to_f32(dv.v[e]);
+          dg[e] += d * ((to_f32(xv.v[e]) - mu) * rs);
+          db[e] += d;
+        }
+      } else {
+        const float d = to_f32(dy[row * cols + col0]);
+        dg[0] += d * ((to_f32(x[row * cols + col0]) - mu) * rs);
+        db[0] += d;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) {
+    lds[wave][0][lane * EPV + e] = dg[e];
+    lds[wave][1][lane * EPV + e] = db[e];
+  }
+  __syncthreads();
+  // fixed order over the waves; thread t finishes element t (and t + 256, ...) of the tile
+  for (int i = threadIdx.x; i < kWave * EPV; i += kParamWaves * kWave) {
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * kWave * EPV + i;
+    if (col < cols) {
+      float sg = lds[0][0][i], sb = lds[0][1][i];
+#pragma unroll
+      for (int w = 1; w < kParamWaves; ++w) {
+        sg += lds[w][0][i];
+        sb += lds[w][1][i];
+      }
+      partial[(slab * 2 + 0) * cols + col] = sg;
+      partial[(slab * 2 + 1) * cols + col] = sb;
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_param_final_kernel(
+    T* __restrict__ dgamma, T* __restrict__ dbeta, const float* __restrict__ partial, int64_t cols,
+    int64_t slabs) {
+  const int64_t col = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (col >= cols) return;
+  float sg = 0.0f, sb = 0.0f;
+  for (int64_t s = 0; s < slabs; ++s) {
+    sg += partial[(s * 2 + 0) * cols + col];
+    sb += partial[(s * 2 + 1) * cols + col];
+  }
+  if (dgamma != nullptr) dgamma[col] = from_f32<T>(sg);
+  if (dbeta != nullptr) dbeta[col] = from_f32<T>(sb);
+}
+
+// Slabs of rows for the parameter gradients: enough workgroups to fill the GPU, each with at
+// least 16 rows (pure function of the shape: the workspace size and the summation order follow).
+static int64_t param_slabs(int64_t rows, int64_t cols, int epv) {
+  const int64_t col_tiles = (cols + 64 * epv - 1) / (64 * epv);
+  int64_t slabs = (2048 + col_tiles - 1) / col_tiles;
+  const int64_t by_rows = (rows + 15) / 16;
+  if (slabs > by_rows) slabs = by_rows;
+  if (slabs < 1) slabs = 1;
+  if (slabs > 65535) slabs = 65535;
+  return slabs;
+}
+
+template <typename T>
+static bool param_vec_ok(const void* dy, const void* x, int64_t cols) {
+  return cols % Vec16<T>::N == 0 && aligned16(dy) && aligned16(x);
+}
+
+template <typename T>
+static int layer_norm_backward_dispatch(void* dx_, void* dgamma_, void* dbeta_, const void* dy_,
+                                        const void* x_, const float* mean, const float* rstd,
+                                        const void* gamma_, int64_t rows, int64_t cols,
+                                        void* workspace, size_t workspace_bytes,
+                                        hipStream_t stream) {
+  T* dx = static_cast<T*>(dx_);
+  const T* dy = static_cast<const T*>(dy_);
+  const T* x = static_cast<const T*>(x_);
+  const T* gamma = static_cast<const T*>(gamma_);
+  constexpr int EPV = Vec16<T>::N;
+  int rc = 0;
+  if (dx != nullptr) {
+    const bool vec_ok = cols % EPV == 0 && aligned16(dx) && aligned16(dy) && aligned16(x) &&
+                        (gamma == nullptr || aligned16(gamma)) && rows < (int64_t{1} << 31);
+    const int64_t nvec = cols / EPV;
+    bool done = false;
+#define TMB_LB(WPR, VPL, BLOCK)                                                                  \
+  {                                                                                              \
+    constexpr int RPB = (BLOCK / kWave) / WPR;                                                   \
+    const int64_t blocks = (rows + RPB - 1) / RPB;                                               \
+    layer_norm_backward_dx_kernel<T, WPR, VPL, BLOCK>                                            \
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, stream>>>(                       \
+            dx, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols));                         \
+    done = true;                                                                                 \
+  }
+    if (vec_ok && nvec <= 16 * 64 * 4) {
+      if (nvec <= 64) TMB_LB(1, 1, 256)
+      else if (nvec <= 128) TMB_LB(2, 1, 256)
+      else if (nvec <= 256) TMB_LB(2, 2, 256)
+      else if (nvec <= 512) TMB_LB(4, 2, 256)
+      else if (nvec <= 1024) TMB_LB(8, 2, 512)
+      else if (nvec <= 2048) TMB_LB(16, 2, 1024)
+      else TMB_LB(16, 4, 1024)
+    }
+#undef TMB_LB
+    if (!done) {
+      const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
+      layer_norm_backward_dx_generic_kernel<T>
+          <<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(dx, dy, x, mean, rstd,
+                                                                         gamma, rows, cols);
+    }
+    rc = check_launch();
+    if (rc != 0) return rc;
+  }
+  if (dgamma_ == nullptr && dbeta_ == nullptr) return rc;
+  const bool vec = param_vec_ok<T>(dy, x, cols);
+  const int epv = vec ? EPV : 1;
+  const int64_t slabs = param_slabs(rows, cols, epv);
+  if (workspace == nullptr || workspace_bytes < static_cast<size_t>(slabs) * 2 * cols * 4)
+    return TMB_ERR_WORKSPACE;
+  const int64_t rows_per_slab = (rows + slabs - 1) / slabs;
+  const int64_t col_tiles = (cols + 64 * epv - 1) / (64 * epv);
+  if (col_tiles >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  float* partial = static_cast<float*>(workspace);
+  const dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(slabs));
+  if (vec)
+    layer_norm_param_partial_kernel<T, true><<<grid, dim3(kParamWaves * kWave), 0, stream>>>(
+        partial, dy, x, mean, rstd, rows, cols, rows_per_slab);
+  else
+    layer_norm_param_partial_kernel<T, false><<<grid, dim3(kParamWaves * kWave), 0, stream>>>(
+        partial, dy, x, mean, rstd, rows, cols, rows_per_slab);
+  rc = check_launch();
+  if (rc != 0) return rc;
+  layer_norm_param_final_kernel<T><<<dim3(static_cast<unsigned>((cols + 255) / 256)), dim3(256), 0, stream>>>(
+      static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, slabs);
+  return check_launch();
+}
+
+}  // namespace tmb
+
+extern "C" int tmb_gelu_backward(void* grad_in, const void* grad_out, const void* in, int64_t numel,
+                                 int dtype, int approximate_tanh, void* stream) {
+  if (numel < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (numel == 0) return TMB_OK;
+  if (grad_in == nullptr || grad_out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case TMB_F32: return tmb::launch_gelu_backward<float>(grad_in, grad_out, in, numel, approximate_tanh, s);
+    case TMB_F16: return tmb::launch_gelu_backward<tmb::f16_t>(grad_in, grad_out, in, numel, approximate_tanh, s);
+    case TMB_BF16: return tmb::launch_gelu_backward<tmb::bf16_t>(grad_in, grad_out, in, numel, approximate_tanh, s);
+    default: return TMB_ERR_UNSUPPORTED;
+  }
+}
+
+extern "C" int tmb_softmax_backward_rows(void* grad_in, const void* grad_out, const void* out,
+                                         int64_t rows, int64_t cols, int dtype, int log_mode,
+                                         void* stream) {
+  if (rows < 0 || cols < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || cols == 0) return TMB_OK;
+  if (grad_in == nullptr || grad_out == nullptr || out == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  using namespace tmb;
+  switch (dtype) {
+    case TMB_F32:
+      return log_mode ? softmax_backward_dispatch<float, true>(grad_in, grad_out, out, rows, cols, s)
+                      : softmax_backward_dispatch<float, false>(grad_in, grad_out, out, rows, cols, s);
+    case TMB_F16:
+      return log_mode ? softmax_backward_dispatch<f16_t, true>(grad_in, grad_out, out, rows, cols, s)
+                      : softmax_backward_dispatch<f16_t, false>(grad_in, grad_out, out, rows, cols, s);
+    case TMB_BF16:
+      return log_mode ? softmax_backward_dispatch<bf16_t, true>(grad_in, grad_out, out, rows, cols, s)
+                      : softmax_backward_dispatch<bf16_t, false>(grad_in, grad_out, out, rows, cols, s);
+    default: return TMB_ERR_UNSUPPORTED;
+  }
+}
+
+extern "C" size_t tmb_layer_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
+  if (rows <= 0 || cols <= 0) return 0;
+  // sized for the scalar geometry when the vector one does not apply: take the larger of both
+  const int epv = dtype == TMB_F32 ? 4 : 8;
+  const int64_t a = tmb::param_slabs(rows, cols, epv), b = tmb::param_slabs(rows, cols, 1);
+  return static_cast<size_t>(a > b ? a : b) * 2 * static_cast<size_t>(cols) * 4;
+}
+
+extern "C" int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_beta,
+                                            const void* grad_out, const void* in,
+                                            const float* mean, const float* rstd,
+                                            const void* gamma, int64_t rows, int64_t cols,
+                                            int dtype, void* workspace, size_t workspace_bytes,
+                                            void* stream) {
+  if (rows < 0 || cols <= 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0) return TMB_OK;  // the caller zero-fills the parameter gradients of an empty batch
+  if (grad_out == nullptr || in == nullptr || mean == nullptr || rstd == nullptr)
+    return TMB_ERR_INVALID_ARGUMENT;
+  if (grad_in == nullptr && grad_gamma == nullptr && grad_beta == nullptr) return TMB_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  using namespace tmb;
+  switch (dtype) {
+    case TMB_F32:
+      return layer_norm_backward_dispatch<float>(grad_in, grad_gamma, grad_beta, grad_out, in, mean, rstd, gamma, rows, cols, workspace, workspace_bytes, s);
+    case TMB_F16:
+      return layer_norm_backward_dispatch<f16_t>(grad_in, grad_gamma, grad_beta, grad_out, in, mean, rstd, gamma, rows, cols, workspace, workspace_bytes, s);
+    case TMB_BF16:
+      return layer_norm_backward_dispatch<bf16_t>(grad_in, grad_gamma, grad_beta, grad_out, in, mean, rstd, gamma, rows, cols, workspace, workspace_bytes, s);
+    default: return TMB_ERR_UNSUPPORTED;
+  }
+}

@@ -5,7 +5,7 @@ here="$(cd "$(dirname "$0")" && pwd)"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops"
 objs=""
-for f in softmax layer_norm reduce gemm attention misc; do
+for f in softmax layer_norm reduce gemm attention backward misc; do
   "$HIPCC" $FLAGS "$@" -c "$here/$f.hip" -o "$here/$f.o" &
   objs="$objs $here/$f.o"
 done

@@ -38,6 +38,10 @@ SIGNATURES = {
     "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
                                 _flt, _ci, _ci, _ci, _vp]),
     "tmb_gelu": (_ci, [_vp, _vp, _i64, _ci, _ci, _vp]),
+    "tmb_gelu_backward": (_ci, [_vp, _vp, _vp, _i64, _ci, _ci, _vp]),
+    "tmb_softmax_backward_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _ci, _ci, _vp]),
+    "tmb_layer_norm_backward_workspace_bytes": (_sz, [_i64, _i64, _ci]),
+    "tmb_layer_norm_backward_rows": (_ci, [_vp] * 8 + [_i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
 }
 

@@ -393,6 +393,122 @@ def gelu(x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
     return out
 
 
+# ---------------------------------------------------------------------------
+# Backward twins
+# ---------------------------------------------------------------------------
+def gelu_backward(grad: torch.Tensor, x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
+    """``grad * gelu'(x)`` (reference: activation_backward_ops.mojo:50-73)."""
+    require_hip(grad, x)
+    if approximate not in ("none", "tanh"):
+        raise ValueError(f"gelu_backward: approximate must be 'none' or 'tanh', got {approximate!r}")
+    if x.dtype not in FLOAT_DTYPES or grad.dtype != x.dtype or grad.shape != x.shape:
+        raise TypeError(f"gelu_backward: {tuple(grad.shape)} {grad.dtype} vs {tuple(x.shape)} {x.dtype}")
+    gc = grad if grad.is_contiguous() else grad.contiguous()
+    xc = x if x.is_contiguous() else x.contiguous()
+    out = torch.empty_like(xc)
+    if out.numel():
+        _check("tmb_gelu_backward", _ek.lib().tmb_gelu_backward(
+            out.data_ptr(), gc.data_ptr(), xc.data_ptr(), out.numel(), code_of(x.dtype),
+            int(approximate == "tanh"), _stream()))
+    return out
+
+
+def softmax_backward(grad: torch.Tensor, out: torch.Tensor, dim: int, log: bool) -> torch.Tensor:
+    """Gradient of softmax (``log`` False) or log-softmax (True) along ``dim`` from the saved
+    output (reference: aten_functions.py:788-833)."""
+    require_hip(grad, out)
+    if out.dtype not in FLOAT_DTYPES or grad.dtype != out.dtype or grad.shape != out.shape:
+        raise TypeError(f"softmax_backward: {tuple(grad.shape)} {grad.dtype} vs "
+                        f"{tuple(out.shape)} {out.dtype}")
+    if out.dim() == 0:
+        return torch.zeros_like(out) if not log else grad - torch.exp(out) * grad
+    dim %= out.dim()
+    last = out.dim() - 1
+    g = grad if dim == last else grad.transpose(dim, last)
+    o = out if dim == last else out.transpose(dim, last)
+    gc, oc = g.contiguous(), o.contiguous()
+    res = torch.empty_like(oc)
+    cols = oc.shape[-1]
+    if res.numel():
+        _check("tmb_softmax_backward_rows", _ek.lib().tmb_softmax_backward_rows(
+            res.data_ptr(), gc.data_ptr(), oc.data_ptr(), oc.numel() // cols, cols,
+            code_of(out.dtype), int(bool(log)), _stream()))
+    return res if dim == last else res.transpose(dim, last).contiguous()
+
+
+def layer_norm_backward(grad: torch.Tensor, x: torch.Tensor, normalized_shape: Sequence[int],
+                        mean: torch.Tensor, rstd: torch.Tensor, weight: Optional[torch.Tensor],
+                        output_mask: Sequence[bool]):
+    """(grad_input, grad_weight, grad_bias), each None where ``output_mask`` says so
+    (reference: aten_fast.py:2797-2913). ``mean`` / ``rstd`` are the float32 statistics the
+    forward returned."""
+    require_hip(grad, x, mean, rstd, weight)
+    normalized_shape = tuple(normalized_shape)
+    k = len(normalized_shape)
+    if x.dtype not in FLOAT_DTYPES or grad.dtype != x.dtype or grad.shape != x.shape or k < 1 \
+            or tuple(x.shape[x.dim() - k:]) != normalized_shape:
+        raise ValueError(f"layer_norm_backward: grad {tuple(grad.shape)} {grad.dtype}, input "
+                         f"{tuple(x.shape)} {x.dtype}, normalized_shape {normalized_shape}")
+    cols = math.prod(normalized_shape)
+    rows = x.numel() // cols if cols else 0
+    if mean.dtype != torch.float32 or rstd.dtype != torch.float32 or mean.numel() != rows \
+            or rstd.numel() != rows:
+        raise ValueError("layer_norm_backward: mean / rstd must be float32 with one value per row")
+    if weight is not None and (weight.dtype != x.dtype or tuple(weight.shape) != normalized_shape):
+        raise ValueError(f"layer_norm_backward: weight must be {normalized_shape} {x.dtype}")
+    want_x, want_w, want_b = (bool(m) for m in output_mask)
+    gc, xc = grad.contiguous(), x.contiguous()
+    dx = torch.empty_like(xc) if want_x else None
+    dw = torch.empty(normalized_shape, dtype=x.dtype, device=x.device) if want_w else None
+    db = torch.empty(normalized_shape, dtype=x.dtype, device=x.device) if want_b else None
+    if rows == 0 or cols == 0:
+        for t in (dw, db):
+            if t is not None:
+                t.zero_()
+        return dx, dw, db
+    code = code_of(x.dtype)
+    ws, ws_bytes = None, 0
+    if want_w or want_b:
+        ws_bytes = _ek.lib().tmb_layer_norm_backward_workspace_bytes(rows, cols, code)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    wc = None if weight is None else weight.contiguous()
+    _check("tmb_layer_norm_backward_rows", _ek.lib().tmb_layer_norm_backward_rows(
+        None if dx is None else dx.data_ptr(), None if dw is None else dw.data_ptr(),
+        None if db is None else db.data_ptr(), gc.data_ptr(), xc.data_ptr(),
+        mean.contiguous().data_ptr(), rstd.contiguous().data_ptr(),
+        None if wc is None else wc.data_ptr(), rows, cols, code,
+        None if ws is None else ws.data_ptr(), ws_bytes, _stream()))
+    return dx, dw, db
+
+
+def linear_backward(x: torch.Tensor, grad: torch.Tensor, weight: torch.Tensor,
+                    output_mask: Sequence[bool]):
+    """(grad_input, grad_weight, grad_bias) of ``x @ weight.T + bias`` (reference:
+    aten_functions.py:2323-2375): grad_input = dy W, grad_weight = dyᵀ x (the transposed-A GEMM),
+    grad_bias = column sums of dy. The two parameter outputs are both defined whenever either is
+    asked for, as in the reference."""
+    require_hip(x, grad, weight)
+    if weight.dim() != 2 or x.dim() < 1 or x.shape[-1] != weight.shape[1] \
+            or grad.shape[-1] != weight.shape[0] or grad.shape[:-1] != x.shape[:-1]:
+        raise ValueError(f"linear_backward: input {tuple(x.shape)}, grad {tuple(grad.shape)}, "
+                         f"weight {tuple(weight.shape)}")
+    want_x, want_w, want_b = (bool(m) for m in output_mask)
+    out_f, in_f = weight.shape
+    rows = x.numel() // in_f if in_f else 0
+    x2 = x.reshape(rows, in_f)
+    g2 = grad.reshape(rows, out_f)
+    dx = dw = db = None
+    if want_x:
+        dx = (torch.zeros_like(x) if out_f == 0 else gemm(g2, weight).view(x.shape))
+    if want_w or want_b:
+        dw = (torch.zeros_like(weight) if rows == 0 else gemm(g2.t(), x2))
+        if want_b and rows > 0:
+            db = reduce(g2, [0], False, _ek.SUM)
+        else:
+            db = torch.zeros(out_f, dtype=grad.dtype, device=grad.device)
+    return dx, dw, db
+
+
 def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     """Plain device copy through the library's yardstick kernel (benchmarks only)."""
     require_hip(dst, src)
