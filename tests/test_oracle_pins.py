@@ -437,3 +437,75 @@ def test_attention_oracle_special_cases():
     v3 = seeded((1, 1, 4, 8), seed=6)
     got3 = oracle.attention(seeded((1, 1, 2, 8), seed=7), k3, v3, 1.0, False)
     np.testing.assert_allclose(as64(got3)[0, :, 0], np.broadcast_to(as64(v3)[0, 0].mean(0), (2, 8)), rtol=1e-6)
+
+
+# ---------------------------------------------------------------- backward twins
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("approximate", ["none", "tanh"])
+def test_gelu_backward_oracle_vs_autograd_and_limits(dtype, approximate):
+    x = (seeded((9, 77), seed=1) * 3).to(dtype)
+    g = seeded((9, 77), seed=2).to(dtype)
+    got = oracle.gelu_backward(g, x, approximate)
+    x64 = x.double().requires_grad_(True)
+    (torch.nn.functional.gelu(x64, approximate=approximate) * g.double()).sum().backward()
+    tol = {torch.float32: 1e-6, torch.bfloat16: 2e-2, torch.float16: 3e-3}[dtype]
+    assert (got.double() - x64.grad).abs().max().item() <= tol * 5
+    # gelu'(0) = 1/2, gelu'(+large) = 1, gelu'(-large) = 0
+    pts = torch.tensor([0.0, 40.0, -40.0], dtype=dtype)
+    lim = oracle.gelu_backward(torch.full_like(pts, 2.0), pts, approximate).float()
+    assert torch.allclose(lim, torch.tensor([1.0, 2.0, 0.0]), atol=1e-6)
+
+
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_backward_oracle_vs_autograd_and_invariants(log):
+    x = seeded((7, 130), seed=3)
+    g = seeded((7, 130), seed=4)
+    xr = x.double().requires_grad_(True)
+    out = (torch.log_softmax if log else torch.softmax)(xr, -1)
+    (out * g.double()).sum().backward()
+    got = oracle.softmax_backward_rows(g, out.detach().float(), log)
+    assert (got.double() - xr.grad).abs().max().item() <= 5e-6
+    # brute force on a tiny row from the Jacobian d out_i / d x_j
+    y = torch.softmax(torch.tensor([[0.3, -1.2, 2.0]]), -1)
+    gg = torch.tensor([[1.0, -2.0, 0.5]])
+    if log:
+        jac = torch.eye(3) - y.expand(3, 3)            # d log y_i / d x_j = delta_ij - y_j
+        saved = y.log()
+    else:
+        jac = torch.diag(y[0]) - y.t() @ y             # d y_i / d x_j = y_i (delta_ij - y_j)
+        saved = y
+    want = gg @ jac
+    torch.testing.assert_close(oracle.softmax_backward_rows(gg, saved, log), want, rtol=1e-5, atol=1e-6)
+    # a gradient that is constant along the row: zero for softmax; rows sum to zero for log-softmax
+    const = oracle.softmax_backward_rows(torch.full((7, 130), 2.5), out.detach().float(), log)
+    if log:
+        assert const.sum(-1).abs().max().item() <= 1e-4
+    else:
+        assert const.abs().max().item() <= 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layer_norm_backward_oracle_vs_autograd_and_invariants(dtype, affine):
+    rows, cols = 11, 96
+    x = seeded((rows, cols), seed=5).to(dtype)
+    g = seeded((rows, cols), seed=6).to(dtype)
+    w = (1 + 0.1 * seeded((cols,), seed=7)).to(dtype) if affine else None
+    _, mean, rstd = oracle.layer_norm_rows(x, w, None, 1e-5)
+    dx, dw, db = oracle.layer_norm_backward_rows(g, x, mean, rstd, w)
+    x64 = x.double().requires_grad_(True)
+    w64 = None if w is None else w.double().requires_grad_(True)
+    b64 = torch.zeros(cols, dtype=torch.float64, requires_grad=True)
+    (torch.nn.functional.layer_norm(x64, [cols], w64, b64, 1e-5) * g.double()).sum().backward()
+    tol = {torch.float32: 2e-5, torch.bfloat16: 4e-2}[dtype]
+    assert (dx.double() - x64.grad).abs().max().item() <= tol * 4
+    assert (db.double() - b64.grad).abs().max().item() <= tol * 8
+    if affine:
+        assert (dw.double() - w64.grad).abs().max().item() <= tol * 8
+    if dtype == torch.float32:
+        # grad_input is orthogonal to the constant vector and to xhat (the two directions the
+        # normalisation removes); grad_bias is the column sum of the upstream gradient
+        xhat = (x - mean.view(-1, 1)) * rstd.view(-1, 1)
+        assert dx.sum(-1).abs().max().item() <= 1e-4
+        assert (dx * xhat).sum(-1).abs().max().item() <= 1e-3
+        torch.testing.assert_close(db, g.sum(0), rtol=1e-5, atol=1e-5)

@@ -285,6 +285,77 @@ def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout
                                              scale=scale, enable_gqa=enable_gqa)
 
 
+# ---------------------------------------------------------------------------
+# Backward twins of the hot ops (reference :788-833, :2070-2102, :2323-2375; the layer-norm
+# backward is eager-only there, eager_kernels/aten_fast.py:2797-2913)
+# ---------------------------------------------------------------------------
+@map_to(aten.gelu_backward)
+def aten_gelu_backward(grad_output: torch.Tensor, input: torch.Tensor, *,
+                       approximate: str = "none") -> torch.Tensor:
+    if approximate not in ("none", "tanh"):
+        raise ValueError(f"Invalid approximate argument '{approximate}'. Supported values are "
+                         "'none' and 'tanh'.")
+    return hip_ops.gelu_backward(grad_output, input, approximate)
+
+
+def _softmax_backward(grad_output, output, dim, input_dtype, log):
+    if grad_output.dtype != output.dtype:
+        raise ValueError("grad_output and output must have the same dtype")
+    if tuple(grad_output.shape) != tuple(output.shape):
+        raise ValueError("grad_output and output must have the same shape")
+    if grad_output.dtype != input_dtype and not (
+            grad_output.dtype == torch.float32 and input_dtype == torch.float16):
+        raise ValueError("input and grad dtypes must match, or input must be float16 and grad "
+                         "must be float32")
+    rank = grad_output.dim()
+    if rank and not -rank <= dim < rank:
+        raise ValueError("dim must refer to an input dimension")
+    if rank == 0 and dim not in (-1, 0):
+        raise ValueError("dim must be -1 or 0 for a scalar input")
+    result = hip_ops.softmax_backward(grad_output, output, dim, log)
+    return result if result.dtype == input_dtype else result.to(input_dtype)
+
+
+@map_to(aten._log_softmax_backward_data)
+def aten__log_softmax_backward_data(grad_output: torch.Tensor, output: torch.Tensor, dim: int,
+                                    input_dtype: torch.dtype) -> torch.Tensor:
+    """reference :788-833: grad - exp(output) * sum(grad, dim)."""
+    return _softmax_backward(grad_output, output, dim, input_dtype, True)
+
+
+@map_to(aten._softmax_backward_data)
+def aten__softmax_backward_data(grad_output: torch.Tensor, output: torch.Tensor, dim: int,
+                                input_dtype: torch.dtype) -> torch.Tensor:
+    """output * (grad - sum(grad * output, dim)): the same row kernel in its softmax form."""
+    return _softmax_backward(grad_output, output, dim, input_dtype, False)
+
+
+@map_to(aten.native_layer_norm_backward)
+def aten_native_layer_norm_backward(grad_out, input, normalized_shape, mean, rstd, weight, bias,
+                                    output_mask):
+    """(grad_input, grad_weight, grad_bias) from the saved statistics (eager twin:
+    aten_fast.py:2797-2913)."""
+    mask = [bool(m) for m in output_mask]
+    if len(mask) != 3:
+        raise ValueError("native_layer_norm_backward output_mask must contain three booleans")
+    if (mask[1] and weight is None) or (mask[2] and bias is None):
+        raise ValueError("native_layer_norm_backward: a parameter gradient was requested for a "
+                         "parameter that is None")
+    return hip_ops.layer_norm_backward(grad_out, input, normalized_shape, mean.float(),
+                                       rstd.float(), weight, mask)
+
+
+@map_to(aten.linear_backward)
+def aten_linear_backward(self, grad_output, weight, output_mask):
+    """reference :2323-2375."""
+    mask = tuple(output_mask)
+    if len(mask) != 3 or any(not isinstance(m, bool) for m in mask):
+        raise ValueError("linear_backward output_mask must contain three booleans")
+    if self.dim() < 1 or weight.dim() != 2:
+        raise ValueError("linear_backward expects rank >= 1 input and rank 2 weight")
+    return hip_ops.linear_backward(self, grad_output, weight, mask)
+
+
 HOT_OPS = (aten.mm, aten.bmm, aten.addmm, aten.linear, aten._softmax, aten.softmax,
            aten._log_softmax, aten.native_layer_norm, aten.sum, aten.mean, aten.amax,
            aten.argmax, aten.gelu)
@@ -296,12 +367,12 @@ _PASSTHROUGH = """
 floordiv _local_scalar_dense all _adaptive_avg_pool2d _adaptive_avg_pool2d_backward
 _native_batch_norm_legit_no_training _scaled_dot_product_attention_math
 _scaled_dot_product_efficient_attention _scaled_dot_product_flash_attention
-_log_softmax_backward_data.default _to_copy abs acos add addcdiv addcmul alias amin any arange
+_to_copy abs acos add addcdiv addcmul alias amin any arange
 argmin asinh atanh avg_pool2d bitwise_and.Scalar bitwise_and.Tensor bitwise_not bitwise_or.Scalar
 bitwise_or.Tensor bitwise_xor.Scalar bitwise_xor.Tensor cat ceil clamp clone constant_pad_nd
 convolution copy cos cosh cumsum detach div embedding empty.memory_format empty_strided empty_like
-empty_permuted eq erf exp expand fill fill_ floor full full_like ge gelu_backward gt index isin
-isnan le linear_backward.default lift_fresh_copy log log1p logical_and logical_not logical_xor lt
+empty_permuted eq erf exp expand fill fill_ floor full full_like ge gt index isin
+isnan le lift_fresh_copy log log1p logical_and logical_not logical_xor lt
 max max_pool2d_with_indices maximum mean.out min minimum mul native_batch_norm native_group_norm
 normal_ ne neg nonzero ones_like permute pow reciprocal relu remainder repeat relu_ rsqrt
 scalar_tensor scaled_dot_product_attention scatter.src scatter.value select select_scatter sigmoid
@@ -314,6 +385,15 @@ _foreach_pow.List _foreach_pow.ScalarAndTensor _foreach_div.Scalar _foreach_div.
 _foreach_div.Tensor _foreach_div.List _foreach_reciprocal _foreach_sqrt _foreach_addcdiv.Scalar
 _foreach_addcdiv.ScalarList _foreach_addcmul.Scalar _foreach_addcmul.ScalarList masked_fill
 transpose sym_size sym_numel sym_stride sym_storage_offset
+""".split()
+
+# Cold ops that only a backward graph contains (loss, embedding and indexing gradients): beyond
+# what the reference's graph surface maps, so that a compiled training step runs end to end.
+_PASSTHROUGH += """
+index_put index_put_ gather scatter_add nll_loss_forward nll_loss_backward nll_loss2d_forward
+embedding_dense_backward tanh_backward sigmoid_backward threshold_backward new_zeros new_empty
+new_empty_strided zeros_like zeros ones sum_to_size expand_as squeeze_ unsqueeze_ mse_loss
+mse_loss_backward _softmax_backward_data.out log sqrt_ rsub addcmul_ addcdiv_ lerp
 """.split()
 
 

@@ -345,6 +345,97 @@ def fast_aten_gelu(input, approximate="none"):
 
 
 # ---------------------------------------------------------------------------
+# Backward twins (reference :1413-1447, :2797-2913, :3237-3330, :4939-5031)
+# ---------------------------------------------------------------------------
+def fast_aten_gelu_backward(grad_output, self, *, approximate="none"):
+    grad, a = _t(grad_output), _t(self)
+    if approximate not in ("none", "tanh") or grad is None or a is None \
+            or not _same_device(grad, a) or grad._dtype != a._dtype \
+            or a._dtype not in _FLOAT_DTYPES or tuple(grad._shape) != tuple(a._shape):
+        return NOT_HANDLED
+    return _wrap(hip_ops.gelu_backward(grad._holder, a._holder, approximate))
+
+
+def _softmax_backward_data(grad_output, output, dim, input_dtype, log):
+    grad, saved = _t(grad_output), _t(output)
+    if grad is None or saved is None or tuple(grad._shape) != tuple(saved._shape) \
+            or grad._dtype != saved._dtype or not _same_device(grad, saved) \
+            or grad._dtype not in _FLOAT_DTYPES or input_dtype not in _FLOAT_DTYPES \
+            or not isinstance(dim, int) or isinstance(dim, bool):
+        return NOT_HANDLED
+    if grad._dtype != input_dtype and not (grad._dtype == torch.float32
+                                           and input_dtype == torch.float16):
+        return NOT_HANDLED
+    rank = len(grad._shape)
+    if rank == 0:
+        if dim not in (-1, 0):
+            return NOT_HANDLED
+    elif not -rank <= dim < rank:
+        return NOT_HANDLED
+    result = hip_ops.softmax_backward(grad._holder, saved._holder, dim, log)
+    return _wrap(result if result.dtype == input_dtype else result.to(input_dtype))
+
+
+def fast_aten__log_softmax_backward_data(grad_output, output, dim, input_dtype):
+    return _softmax_backward_data(grad_output, output, dim, input_dtype, True)
+
+
+def fast_aten__softmax_backward_data(grad_output, output, dim, input_dtype):
+    return _softmax_backward_data(grad_output, output, dim, input_dtype, False)
+
+
+def fast_aten_native_layer_norm_backward(grad_out, input, normalized_shape, mean, rstd, weight,
+                                         bias, output_mask):
+    """Everything is validated from metadata before anything is materialised or allocated
+    (reference :2797-2813)."""
+    grad, a, saved_mean, saved_rstd = _t(grad_out), _t(input), _t(mean), _t(rstd)
+    gamma = _t(weight) if weight is not None else None
+    beta = _t(bias) if bias is not None else None
+    normalized_shape = tuple(int(s) for s in normalized_shape)
+    mask = tuple(output_mask)
+    k = len(normalized_shape)
+    if len(mask) != 3 or any(not isinstance(m, bool) for m in mask) or grad is None or a is None \
+            or saved_mean is None or saved_rstd is None or a._dtype not in _FLOAT_DTYPES \
+            or grad._dtype != a._dtype or saved_mean._dtype != torch.float32 \
+            or saved_rstd._dtype != torch.float32 \
+            or not _same_device(grad, a, saved_mean, saved_rstd, gamma, beta) \
+            or tuple(grad._shape) != tuple(a._shape) or k < 1 or len(a._shape) < k \
+            or tuple(a._shape[-k:]) != normalized_shape:
+        return NOT_HANDLED
+    cols = math.prod(normalized_shape)
+    if cols <= 0:
+        return NOT_HANDLED
+    rows = a._numel // cols
+    if saved_mean._numel != rows or saved_rstd._numel != rows:
+        return NOT_HANDLED
+    for given, t in ((weight, gamma), (bias, beta)):
+        if given is not None and (t is None or t._dtype != a._dtype
+                                  or tuple(t._shape) != normalized_shape):
+            return NOT_HANDLED
+    if (mask[1] and gamma is None) or (mask[2] and beta is None):
+        return NOT_HANDLED
+    if not any(mask):
+        return None, None, None
+    dx, dw, db = hip_ops.layer_norm_backward(
+        grad._holder, a._holder, normalized_shape, saved_mean._holder, saved_rstd._holder,
+        None if gamma is None else gamma._holder, mask)
+    return tuple(None if t is None else _wrap(t) for t in (dx, dw, db))
+
+
+def fast_aten_linear_backward(self, grad_output, weight, output_mask):
+    a, grad, w = _t(self), _t(grad_output), _t(weight)
+    mask = tuple(output_mask)
+    if len(mask) != 3 or any(not isinstance(m, bool) for m in mask) or a is None or grad is None \
+            or w is None or not _same_device(a, grad, w) or a._dtype not in _FLOAT_DTYPES \
+            or grad._dtype != a._dtype or w._dtype != a._dtype or len(w._shape) != 2 \
+            or len(a._shape) < 1 or a._shape[-1] != w._shape[1] or grad._shape[-1] != w._shape[0] \
+            or tuple(grad._shape[:-1]) != tuple(a._shape[:-1]):
+        return NOT_HANDLED
+    dx, dw, db = hip_ops.linear_backward(a._holder, grad._holder, w._holder, mask)
+    return tuple(None if t is None else _wrap(t) for t in (dx, dw, db))
+
+
+# ---------------------------------------------------------------------------
 # Call counting under TORCH_MOJO_BACKEND_TESTING=1 (reference :5499-5522)
 # ---------------------------------------------------------------------------
 def _instrument_call_counts():

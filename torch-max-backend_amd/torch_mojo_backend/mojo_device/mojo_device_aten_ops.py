@@ -127,6 +127,12 @@ _register_fast("aten::native_layer_norm", "fast_aten_native_layer_norm")
 _register_fast("aten::scaled_dot_product_attention", "fast_aten_scaled_dot_product_attention")
 _register_fast("aten::softmax.int", "fast_aten_softmax")
 _register_fast("aten::sum.dim_IntList", "fast_aten_sum")
+# backward twins (reference :930-1000 registers the same op names)
+_register_fast("aten::gelu_backward", "fast_aten_gelu_backward")
+_register_fast("aten::_log_softmax_backward_data", "fast_aten__log_softmax_backward_data")
+_register_fast("aten::_softmax_backward_data", "fast_aten__softmax_backward_data")
+_register_fast("aten::native_layer_norm_backward", "fast_aten_native_layer_norm_backward")
+_register_fast("aten::linear_backward", "fast_aten_linear_backward")
 
 
 @register_aten_op("aten::sum")
@@ -287,6 +293,13 @@ _HOLDER_OPS = (
     "aten::new_ones", "aten::new_zeros", "aten::new_full", "aten::new_empty",
     "aten::empty_like", "aten::arange", "aten::arange.start", "aten::arange.start_step",
     "aten::scalar_tensor", "aten::lift_fresh", "aten::contiguous",
+    # what a training step adds: losses, their gradients, embedding and elementwise backward ops,
+    # the optimizer's in-place arithmetic
+    "aten::nll_loss_forward", "aten::nll_loss_backward", "aten::embedding_dense_backward",
+    "aten::tanh_backward", "aten::sigmoid_backward", "aten::threshold_backward",
+    "aten::mse_loss", "aten::mse_loss_backward", "aten::sub_.Tensor", "aten::div_.Tensor",
+    "aten::mul_.Scalar", "aten::add_.Scalar", "aten::addcmul_", "aten::addcdiv_", "aten::sqrt_",
+    "aten::lerp_.Scalar", "aten::log", "aten::sum_to_size",
 )
 for _name in _HOLDER_OPS:
     register_aten_op(_name)(holder_impl(_name))
