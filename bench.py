@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot-op kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|gpt2|generate|copy|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|backward|gpt2|generate|copy|all]
 
 Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
@@ -48,7 +48,7 @@ def _parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "gpt2", "generate", "copy"])
+    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "backward", "gpt2", "generate", "copy"])
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return p.parse_args()
 
@@ -358,6 +358,66 @@ def main() -> int:
                 rows * cols * 4 + rows * 8, steps=100, cpu_fn=cpu_argmax)
         assert torch.equal(out_idx, torch.argmax(bufs[(99 + 8) % len(bufs)], dim=1))
         del bufs
+
+    # ------------------------------------------------------------------ backward twins
+    # Shapes of the GPT-2 training step at B=32, T=1024 (bf16) and the forward sweep's row shapes.
+    # Algorithmic bytes: every input read once, every output written once (the layer-norm
+    # backward reads dy and x a second time for the parameter gradients: counted once here).
+    if want in ("all", "backward"):
+        for dtype, dn in ((torch.bfloat16, "bf16"), (torch.float32, "fp32")):
+            es = torch.finfo(dtype).bits // 8
+            code = hip_ops.code_of(dtype)
+            # gelu_backward over the MLP activation [32768, 3072]
+            numel = 32768 * 3072
+            nb = numel * es
+            xs = rotating(lambda i: gen((numel,), 40 + i, dtype), 2 * nb)
+            gs = [gen((numel,), 60 + i, dtype) for i in range(len(xs))]
+            outs = [torch.empty_like(x_) for x_ in xs]
+            hbm_row(f"gelu_backward_tanh_{dn}_32768x3072", len(xs),
+                    lambda i: lib.tmb_gelu_backward(outs[i].data_ptr(), gs[i].data_ptr(), xs[i].data_ptr(),
+                                                    numel, code, 1, stream), 3 * nb)
+            del xs, gs, outs
+            # softmax backward over attention probabilities [98304, 1024]
+            rows, cols = 98304, 1024
+            nb = rows * cols * es
+            ys = rotating(lambda i: torch.softmax(gen((rows, cols), 70 + i, torch.float32), -1).to(dtype), 2 * nb)
+            gs = [gen((rows, cols), 80 + i, dtype) for i in range(len(ys))]
+            outs = [torch.empty_like(y_) for y_ in ys]
+            hbm_row(f"softmax_backward_{dn}_{rows}x{cols}", len(ys),
+                    lambda i: lib.tmb_softmax_backward_rows(outs[i].data_ptr(), gs[i].data_ptr(),
+                                                            ys[i].data_ptr(), rows, cols, code, 0, stream),
+                    3 * nb)
+            del ys, gs, outs
+            # layer norm backward (all three outputs)
+            for (rows, cols) in ((32768, 768), (16384, 4096)):
+                nb = rows * cols * es
+                xs = rotating(lambda i: gen((rows, cols), 90 + i, dtype), 2 * nb)
+                gs = [gen((rows, cols), 100 + i, dtype) for i in range(len(xs))]
+                dxs = [torch.empty_like(x_) for x_ in xs]
+                gamma = gen((cols,), 1, dtype, scale=0.1, shift=1.0)
+                dgm, dbt = torch.empty_like(gamma), torch.empty_like(gamma)
+                stats = [hip_ops.layer_norm(x_, [cols], gamma, None, 1e-5)[1:] for x_ in xs]
+                ws_b = lib.tmb_layer_norm_backward_workspace_bytes(rows, cols, code)
+                wsp = torch.empty(max(ws_b, 16), dtype=torch.uint8, device=dev)
+                hbm_row(f"layer_norm_backward_{dn}_{rows}x{cols}", len(xs),
+                        lambda i: lib.tmb_layer_norm_backward_rows(
+                            dxs[i].data_ptr(), dgm.data_ptr(), dbt.data_ptr(), gs[i].data_ptr(),
+                            xs[i].data_ptr(), stats[i][0].data_ptr(), stats[i][1].data_ptr(),
+                            gamma.data_ptr(), rows, cols, code, wsp.data_ptr(), ws_b, stream),
+                        3 * nb + 3 * cols * es + 2 * rows * 4)
+                del xs, gs, dxs, stats
+        # the two GEMMs of linear_backward for the MLP up-projection: dgrad (NN) and wgrad (TN)
+        rows_, in_f, out_f = 32768, 768, 3072
+        dy = gen((rows_, out_f), 110, torch.bfloat16)
+        xin = gen((rows_, in_f), 111, torch.bfloat16)
+        wt = gen((out_f, in_f), 112, torch.bfloat16)
+        for name, fn, fl in (
+                ("linear_backward_dgrad_bf16_32768x768x3072", lambda: hip_ops.gemm(dy, wt), 2.0 * rows_ * in_f * out_f),
+                ("linear_backward_wgrad_bf16_3072x768x32768", lambda: hip_ops.gemm(dy.t(), xin), 2.0 * rows_ * in_f * out_f)):
+            _, ms = timed(fn, 30, 8)
+            sweep[name] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(fl / ms / 1e9, 2),
+                           "frac_mfma": round(fl / ms / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4)}
+        del dy, xin, wt
 
     # ------------------------------------------------------------------ GPT-2 forward
     if want in ("all", "gpt2"):

@@ -314,22 +314,43 @@ __global__ __launch_bounds__(kParamWaves* kWave) void layer_norm_param_partial_k
   float dg[EPV], db[EPV];
 #pragma unroll
   for (int e = 0; e < EPV; ++e) dg[e] = db[e] = 0.0f;
-  for (int64_t row = r_begin + wave; row < r_end; row += kParamWaves) {
-    const float mu = mean[row], rs = rstd[row];
-    if (ok) {
-      if constexpr (VEC) {
-        const Vec16<T> dv = load_vec16_stream(dy + row * cols + col0);
-        const Vec16<T> xv = load_vec16_stream(x + row * cols + col0);
+  // four rows of the wave's share in flight at a time (eight independent 16-byte loads per lane)
+  constexpr int kUnroll = 4;
+  for (int64_t row0 = r_begin + wave; row0 < r_end; row0 += kParamWaves * kUnroll) {
+    if constexpr (VEC) {
+      Vec16<T> dv[kUnroll], xv[kUnroll];
+      float mu[kUnroll], rs[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        int64_t row = row0 + u * kParamWaves;
+        const bool in = row < r_end && ok;
+        if (row >= r_end) row = r_end - 1;  // a valid address; the values are not used
+        mu[u] = mean[row];
+        rs[u] = in ? rstd[row] : 0.0f;
+        dv[u] = load_vec16_stream(dy + row * cols + (ok ? col0 : 0));
+        xv[u] = load_vec16_stream(x + row * cols + (ok ? col0 : 0));
+        if (!in) {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) dv[u].v[e] = from_f32<T>(0.0f);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
-          const float d = to_f32(dv.v[e]);
-          dg[e] += d * ((to_f32(xv.v[e]) - mu) * rs);
+          const float d = to_f32(dv[u].v[e]);
+          dg[e] += d * ((to_f32(xv[u].v[e]) - mu[u]) * rs[u]);
           db[e] += d;
         }
-      } else {
-        const float d = to_f32(dy[row * cols + col0]);
-        dg[0] += d * ((to_f32(x[row * cols + col0]) - mu) * rs);
-        db[0] += d;
+    } else {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t row = row0 + u * kParamWaves;
+        if (row < r_end && ok) {
+          const float d = to_f32(dy[row * cols + col0]);
+          dg[0] += d * ((to_f32(x[row * cols + col0]) - mean[row]) * rstd[row]);
+          db[0] += d;
+        }
       }
     }
   }
@@ -355,27 +376,42 @@ __global__ __launch_bounds__(kParamWaves* kWave) void layer_norm_param_partial_k
   }
 }
 
+// 32 columns per workgroup; the 32 threads that share a column take every 32nd slab and their
+// sums are added in thread order (fixed), so the result depends on the shape only.
 template <typename T>
-__global__ __launch_bounds__(256) void layer_norm_param_final_kernel(
+__global__ __launch_bounds__(1024) void layer_norm_param_final_kernel(
     T* __restrict__ dgamma, T* __restrict__ dbeta, const float* __restrict__ partial, int64_t cols,
     int64_t slabs) {
-  const int64_t col = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (col >= cols) return;
+  __shared__ float lds[2][32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t col = static_cast<int64_t>(blockIdx.x) * 32 + tx;
   float sg = 0.0f, sb = 0.0f;
-  for (int64_t s = 0; s < slabs; ++s) {
-    sg += partial[(s * 2 + 0) * cols + col];
-    sb += partial[(s * 2 + 1) * cols + col];
+  if (col < cols) {
+    for (int64_t s = ty; s < slabs; s += 32) {
+      sg += partial[(s * 2 + 0) * cols + col];
+      sb += partial[(s * 2 + 1) * cols + col];
+    }
   }
-  if (dgamma != nullptr) dgamma[col] = from_f32<T>(sg);
-  if (dbeta != nullptr) dbeta[col] = from_f32<T>(sb);
+  lds[0][ty][tx] = sg;
+  lds[1][ty][tx] = sb;
+  __syncthreads();
+  if (ty == 0 && col < cols) {
+    float tg = lds[0][0][tx], tb = lds[1][0][tx];
+    for (int i = 1; i < 32; ++i) {
+      tg += lds[0][i][tx];
+      tb += lds[1][i][tx];
+    }
+    if (dgamma != nullptr) dgamma[col] = from_f32<T>(tg);
+    if (dbeta != nullptr) dbeta[col] = from_f32<T>(tb);
+  }
 }
 
 // Slabs of rows for the parameter gradients: enough workgroups to fill the GPU, each with at
-// least 16 rows (pure function of the shape: the workspace size and the summation order follow).
+// least 64 rows (pure function of the shape: the workspace size and the summation order follow).
 static int64_t param_slabs(int64_t rows, int64_t cols, int epv) {
   const int64_t col_tiles = (cols + 64 * epv - 1) / (64 * epv);
-  int64_t slabs = (2048 + col_tiles - 1) / col_tiles;
-  const int64_t by_rows = (rows + 15) / 16;
+  int64_t slabs = (1024 + col_tiles - 1) / col_tiles;
+  const int64_t by_rows = (rows + 63) / 64;
   if (slabs > by_rows) slabs = by_rows;
   if (slabs < 1) slabs = 1;
   if (slabs > 65535) slabs = 65535;
@@ -451,7 +487,7 @@ static int layer_norm_backward_dispatch(void* dx_, void* dgamma_, void* dbeta_, 
         partial, dy, x, mean, rstd, rows, cols, rows_per_slab);
   rc = check_launch();
   if (rc != 0) return rc;
-  layer_norm_param_final_kernel<T><<<dim3(static_cast<unsigned>((cols + 255) / 256)), dim3(256), 0, stream>>>(
+  layer_norm_param_final_kernel<T><<<dim3(static_cast<unsigned>((cols + 31) / 32)), dim3(1024), 0, stream>>>(
       static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, slabs);
   return check_launch();
 }
