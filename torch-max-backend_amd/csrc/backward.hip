@@ -257,6 +257,121 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
   }
 }
 
+// grad_input and the parameter-gradient partials in one pass: a group of WPR waves walks `walk`
+// consecutive rows; every lane keeps the column sums of dy*xhat and dy for the columns it owns
+// in registers and writes them once, as one fp32 partial row per group, at the end. dy and x are
+// read exactly once.
+template <typename T, int WPR, int VPL, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
+    T* __restrict__ dx, float* __restrict__ partial, const T* __restrict__ dy,
+    const T* __restrict__ x, const float* __restrict__ mean, const float* __restrict__ rstd,
+    const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk) {
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int WAVES = BLOCK / kWave;
+  constexpr int GROUPS = WAVES / WPR;
+  __shared__ float slot[WAVES];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int group = wave / WPR, wave_in_row = wave - group * WPR;
+  const int nvec = cols / EPV;
+  const float n = static_cast<float>(cols);
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * GROUPS + group;
+  const int64_t first = gid * walk;
+
+  Vec16<T> gv[VPL];
+  if (gamma != nullptr) {
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const int vi = (v * WPR + wave_in_row) * kWave + lane;
+      gv[v] = load_vec16(gamma + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV);
+    }
+  }
+  float dg[VPL][EPV], db[VPL][EPV];
+#pragma unroll
+  for (int v = 0; v < VPL; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) dg[v][e] = db[v][e] = 0.0f;
+
+  // every group of the workgroup runs `walk` iterations (the reductions contain barriers); rows
+  // past the end re-read the last row and contribute nothing
+  for (int64_t i = 0; i < walk; ++i) {
+    int64_t row = first + i;
+    const bool live = row < rows;
+    if (!live) row = rows - 1;
+    const T* dsrc = dy + row * static_cast<int64_t>(cols);
+    const T* xsrc = x + row * static_cast<int64_t>(cols);
+    const float mu = mean[row], rs = rstd[row];
+    float gd[VPL][EPV], xh[VPL][EPV];
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const int vi = (v * WPR + wave_in_row) * kWave + lane;
+      const bool ok = vi < nvec && live;
+      const int64_t at = static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
+      const Vec16<T> dv = load_vec16_stream(dsrc + at);
+      const Vec16<T> xv = load_vec16_stream(xsrc + at);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float d = ok ? to_f32(dv.v[e]) : 0.0f;
+        const float h = ok ? (to_f32(xv.v[e]) - mu) * rs : 0.0f;
+        gd[v][e] = d * (gamma != nullptr ? to_f32(gv[v].v[e]) : 1.0f);
+        xh[v][e] = h;
+        s1 += gd[v][e];
+        s2 += gd[v][e] * h;
+        dg[v][e] += d * h;
+        db[v][e] += d;
+      }
+    }
+    s1 = wave_sum(s1);
+    s1 = group_reduce(s1, slot, wave, group * WPR, WPR, SumOp{});
+    s2 = wave_sum(s2);
+    s2 = group_reduce(s2, slot, wave, group * WPR, WPR, SumOp{});
+    if (live) {
+      const float m1 = s1 / n, m2 = s2 / n;
+      T* dst = dx + row * static_cast<int64_t>(cols);
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) {
+        const int vi = (v * WPR + wave_in_row) * kWave + lane;
+        float r[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) r[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
+        if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r);
+      }
+    }
+  }
+  float* pg = partial + (gid * 2 + 0) * static_cast<int64_t>(cols);
+  float* pb = partial + (gid * 2 + 1) * static_cast<int64_t>(cols);
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WPR + wave_in_row) * kWave + lane;
+    if (vi < nvec) {
+      store_converted<float, EPV>(pg + static_cast<int64_t>(vi) * EPV, dg[v]);
+      store_converted<float, EPV>(pb + static_cast<int64_t>(vi) * EPV, db[v]);
+    }
+  }
+}
+
+// Geometry of the fused kernel (a pure function of the shape: the workspace size and the order
+// of the final summation follow from it): waves per row as in the forward kernels, about 2048
+// waves in flight (measured best of 1024 .. 16384), 8 to 64 rows per group, partial rows for
+// whole workgroups.
+struct FusedPlan {
+  int wpr, groups_per_block;
+  int64_t walk, groups, padded_groups;
+};
+static FusedPlan fused_plan(int64_t rows, int64_t nvec) {
+  FusedPlan p;
+  p.wpr = nvec <= 64 ? 1 : nvec <= 256 ? 2 : nvec <= 512 ? 4 : nvec <= 1024 ? 8 : 16;
+  const int block = nvec <= 512 ? 256 : nvec <= 1024 ? 512 : 1024;
+  p.groups_per_block = block / kWave / p.wpr;
+  const int64_t target = 2048 / p.wpr;
+  p.walk = (rows + target - 1) / target;
+  if (p.walk < 8) p.walk = 8;
+  if (p.walk > 64) p.walk = 64;
+  p.groups = (rows + p.walk - 1) / p.walk;
+  p.padded_groups = (p.groups + p.groups_per_block - 1) / p.groups_per_block * p.groups_per_block;
+  return p;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void layer_norm_backward_dx_generic_kernel(
     T* __restrict__ dx, const T* __restrict__ dy, const T* __restrict__ x,
@@ -435,6 +550,34 @@ static int layer_norm_backward_dispatch(void* dx_, void* dgamma_, void* dbeta_, 
   const T* gamma = static_cast<const T*>(gamma_);
   constexpr int EPV = Vec16<T>::N;
   int rc = 0;
+  // (rows of up to 128 vectors measured 5-10 % faster through the two separate passes below)
+  if (dx != nullptr && (dgamma_ != nullptr || dbeta_ != nullptr) && cols % EPV == 0 &&
+      cols / EPV > 128 && cols / EPV <= 16 * 64 * 2 && aligned16(dx) && aligned16(dy) && aligned16(x) &&
+      (gamma == nullptr || aligned16(gamma)) && rows < (int64_t{1} << 31)) {
+    const int64_t nvec = cols / EPV;
+    const FusedPlan plan = fused_plan(rows, nvec);
+    if (workspace == nullptr ||
+        workspace_bytes < static_cast<size_t>(plan.padded_groups) * 2 * cols * 4)
+      return TMB_ERR_WORKSPACE;
+    float* partial = static_cast<float*>(workspace);
+    const dim3 grid(static_cast<unsigned>(plan.padded_groups / plan.groups_per_block));
+#define TMB_LF(WPR, VPL, BLOCK)                                                               \
+  layer_norm_backward_fused_kernel<T, WPR, VPL, BLOCK><<<grid, dim3(BLOCK), 0, stream>>>(     \
+      dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), plan.walk);
+    // (groups past the last row write partial rows of zeros, which the final stage adds)
+    if (nvec <= 64) TMB_LF(1, 1, 256)
+    else if (nvec <= 128) TMB_LF(2, 1, 256)
+    else if (nvec <= 256) TMB_LF(2, 2, 256)
+    else if (nvec <= 512) TMB_LF(4, 2, 256)
+    else if (nvec <= 1024) TMB_LF(8, 2, 512)
+    else TMB_LF(16, 2, 1024)
+#undef TMB_LF
+    rc = check_launch();
+    if (rc != 0) return rc;
+    layer_norm_param_final_kernel<T><<<dim3(static_cast<unsigned>((cols + 31) / 32)), dim3(1024), 0, stream>>>(
+        static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, plan.padded_groups);
+    return check_launch();
+  }
   if (dx != nullptr) {
     const bool vec_ok = cols % EPV == 0 && aligned16(dx) && aligned16(dy) && aligned16(x) &&
                         (gamma == nullptr || aligned16(gamma)) && rows < (int64_t{1} << 31);
@@ -534,8 +677,14 @@ extern "C" size_t tmb_layer_norm_backward_workspace_bytes(int64_t rows, int64_t 
   if (rows <= 0 || cols <= 0) return 0;
   // sized for the scalar geometry when the vector one does not apply: take the larger of both
   const int epv = dtype == TMB_F32 ? 4 : 8;
-  const int64_t a = tmb::param_slabs(rows, cols, epv), b = tmb::param_slabs(rows, cols, 1);
-  return static_cast<size_t>(a > b ? a : b) * 2 * static_cast<size_t>(cols) * 4;
+  int64_t most = tmb::param_slabs(rows, cols, epv);
+  const int64_t scalar = tmb::param_slabs(rows, cols, 1);
+  if (scalar > most) most = scalar;
+  if (cols % epv == 0) {
+    const int64_t fused = tmb::fused_plan(rows, cols / epv).padded_groups;
+    if (fused > most) most = fused;
+  }
+  return static_cast<size_t>(most) * 2 * static_cast<size_t>(cols) * 4;
 }
 
 extern "C" int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_beta,
