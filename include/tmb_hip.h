@@ -117,6 +117,21 @@ int tmb_gemm(void* c, const void* a, const void* b, const void* bias, int64_t ba
              int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
              int epilogue, void* stream);
 
+/* tmb_gemm with a caller-provided workspace. Products with few output tiles and a long K (the
+ * weight gradient dy^T x, narrow projections) then run split along K: fp32 partials
+ * [splits][m][n] in the workspace, added in split order by a second kernel that applies bias,
+ * epilogue and the one cast (still fp32 accumulation and one rounding; the result depends on the
+ * shape only). tmb_gemm_workspace_bytes is 0 when the shape would not be split; with a NULL or
+ * too small workspace the call behaves exactly like tmb_gemm.
+ * The reference's GPU GEMM takes its split-K scratch from the MAX runtime
+ * (eager_kernels/matmul_ops.mojo:1040-1049, `multistage_gemm_kernel`); here the caller owns it,
+ * as with every other buffer. */
+size_t tmb_gemm_workspace_bytes(int64_t batch, int64_t m, int64_t n, int64_t k, int dtype);
+int tmb_gemm_ws(void* c, const void* a, const void* b, const void* bias, int64_t batch, int64_t m,
+                int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+                int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
+                int epilogue, void* workspace, size_t workspace_bytes, void* stream);
+
 /* tmb_gemm followed by an elementwise add of `residual` [batch][m, n] (row pitch `ldr`, batch
  * stride `stride_r`) in the same launch: c = T(float(T(epilogue(a b + bias))) + float(residual)),
  * rounded twice exactly as a GEMM kernel followed by an add kernel would (the residual

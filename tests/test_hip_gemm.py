@@ -325,3 +325,55 @@ def test_mm_transposed_a_batched_and_strided():
     got = _ops().gemm(a_view, _dev(b))
     want = np.einsum("bkm,bkn->bmn", as64(a_store)[:, :, :m], as64(b))
     assert rel_frobenius(got, want) <= 1e-2
+
+
+# ---- split-K (few output tiles, long K) ----------------------------------------------------------
+SPLITK = [  # (m, n, k, trans_a, trans_b)
+    (1024, 768, 3072, False, False), (1024, 768, 3072, False, True), (128, 768, 4096, False, True),
+    (3072, 768, 8192, True, False), (768, 768, 32768, True, False), (264, 136, 2048, False, False),
+    (100, 72, 2304, False, True),
+]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("case", SPLITK)
+def test_split_k_matches_float64_and_the_unsplit_kernel(case, dtype):
+    m, n, k, ta, tb = case
+    a = seeded((k, m) if ta else (m, k), seed=21, dtype=dtype) * 0.25
+    b = seeded((n, k) if tb else (k, n), seed=22, dtype=dtype) * 0.25
+    bias = None if ta else seeded((n,), seed=23, dtype=dtype)
+    av = _dev(a).t() if ta else _dev(a)
+    bv = _dev(b).t() if tb else _dev(b)
+    assert _ek().lib().tmb_gemm_workspace_bytes(1, m, n, k, _ops().code_of(dtype)) > 0
+    got = _ops().gemm(av, bv, None if bias is None else _dev(bias))
+    a64 = as64(a).T if ta else as64(a)
+    b64 = as64(b).T if tb else as64(b)
+    want = a64 @ b64 + (0 if bias is None else as64(bias))
+    assert rel_frobenius(got, want) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert np.abs(as64(got) - want).max() <= ulp * np.abs(want).max() + 1e-3
+    # one rounding: at most one storage ulp away from the kernel that does not split
+    lib, ek = _ek().lib(), _ek()
+    plain = torch.empty_like(got)
+    ac, bc = av.contiguous() if ta else av, bv
+    rc = lib.tmb_gemm(plain.data_ptr(), av.data_ptr(), bv.data_ptr(),
+                      None if bias is None else _dev(bias).data_ptr(), 1, m, n, k,
+                      a.shape[1], b.shape[1], n, 0, 0, m * n, int(ta), int(tb),
+                      _ops().code_of(dtype), ek.EPI_NONE, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    del ac, bc
+    assert np.abs(as64(got) - as64(plain)).max() <= 2 * ulp * np.abs(want).max() + 1e-3
+
+
+def test_split_k_is_reproducible_and_needs_scratch_only_when_it_pays():
+    lib = _ek().lib()
+    code = _ops().code_of(torch.bfloat16)
+    assert lib.tmb_gemm_workspace_bytes(1, 8192, 8192, 8192, code) == 0      # plenty of tiles
+    assert lib.tmb_gemm_workspace_bytes(1, 1024, 768, 768, code) == 0        # short K
+    assert lib.tmb_gemm_workspace_bytes(4, 1024, 768, 4096, code) == 0       # batched
+    assert lib.tmb_gemm_workspace_bytes(1, 1024, 768, 4096, _ops().code_of(torch.float32)) == 0
+    a = _dev(seeded((512, 4096), seed=31, dtype=torch.bfloat16))
+    b = _dev(seeded((4096, 384), seed=32, dtype=torch.bfloat16))
+    first = _ops().gemm(a, b)
+    for _ in range(3):
+        assert torch.equal(first, _ops().gemm(a, b))

@@ -182,10 +182,70 @@ static bool mfma_eligible(const GemmArgs& g, int64_t batch, int trans_a, int tra
   return true;
 }
 
+// Split-K: products with few output tiles and a long K (weight gradients, narrow projections)
+// leave most CUs idle. K is cut into `splits` equal chunks that run as the batch dimension of one
+// launch of the 128x128 ring kernel and store fp32 partials [splits][M][N] into a workspace; a
+// second kernel adds them in split order and applies bias, epilogue and the one cast, so the
+// result is still "fp32 accumulation, one rounding" and depends on the shape only.
+struct SplitKPlan {
+  int splits;       // 0: not used
+  int64_t k_chunk;
+};
+static SplitKPlan splitk_plan(int64_t batch, int64_t m, int64_t n, int64_t k) {
+  SplitKPlan p{0, 0};
+  if (batch != 1 || k < 2048 || k % 32 != 0 || n <= 64 || m < 1) return p;
+  const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128);
+  if (tiles >= 256) return p;  // at least one tile per CU: no split
+  int64_t splits = 512 / tiles;
+  if (splits > 16) splits = 16;
+  if (splits > k / 512) splits = k / 512;
+  while (splits >= 2 && k % (splits * 32) != 0) --splits;
+  if (splits < 2) return p;
+  p.splits = static_cast<int>(splits);
+  p.k_chunk = k / splits;
+  return p;
+}
+
+template <typename T, int EPI>
+static int launch_splitk(const GemmArgs& g, const SplitKPlan& plan, int trans_a, int trans_b,
+                         float* workspace, hipStream_t stream) {
+  GemmArgs part = g;
+  part.c = workspace;
+  part.bias = nullptr;
+  part.residual = nullptr;
+  part.k = plan.k_chunk;
+  part.ldc = g.n;
+  part.stride_c = g.m * g.n;
+  part.stride_a = trans_a ? plan.k_chunk * g.lda : plan.k_chunk;
+  part.stride_b = trans_b ? plan.k_chunk : plan.k_chunk * g.ldb;
+  int rc;
+  if (trans_a)
+    rc = launch_ring<T, 128, 128, 32, 2, 2, 4, false, TMB_EPI_NONE, true, true>(part, plan.splits, stream);
+  else if (trans_b)
+    rc = launch_ring<T, 128, 128, 32, 2, 2, 4, true, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+  else
+    rc = launch_ring<T, 128, 128, 32, 2, 2, 4, false, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+  if (rc != 0) return rc;
+  const int64_t total = g.m * g.n;
+  splitk_reduce_kernel<T, EPI><<<dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream>>>(
+      static_cast<T*>(g.c), workspace, static_cast<const T*>(g.bias), g.m, g.n, g.ldc, plan.splits);
+  return check_launch();
+}
+
 template <typename T, int EPI>
 static int gemm_typed(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, bool half,
-                      hipStream_t stream) {
+                      hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0) {
   if constexpr (!__is_same(T, float)) {
+    if (half && workspace != nullptr && g.residual == nullptr) {
+      const SplitKPlan plan = splitk_plan(batch, g.m, g.n, g.k);
+      const bool operands_ok =
+          trans_a ? mfma_transposed_a_eligible(g, batch, trans_a, trans_b, TMB_EPI_NONE)
+                  : (mfma_eligible(g, batch, trans_a, trans_b) && (trans_b || g.n % 8 == 0));
+      if (plan.splits > 0 && operands_ok && g.m * g.n < (int64_t{1} << 31) &&
+          workspace_bytes >= static_cast<size_t>(plan.splits) * g.m * g.n * 4)
+        return launch_splitk<T, EPI>(g, plan, trans_a, trans_b, static_cast<float*>(workspace),
+                                     stream);
+    }
     if (half && mfma_transposed_a_eligible(g, batch, trans_a, trans_b, EPI))
       return mfma_transposed_a<T>(g, batch, stream);
     if (half && mfma_eligible(g, batch, trans_a, trans_b)) {
@@ -198,11 +258,11 @@ static int gemm_typed(const GemmArgs& g, int64_t batch, int trans_a, int trans_b
 
 template <typename T>
 static int gemm_epi(const GemmArgs& g, int64_t batch, int ta, int tb, int epilogue,
-                    hipStream_t stream) {
+                    hipStream_t stream, void* ws, size_t ws_bytes) {
   switch (epilogue) {
-    case TMB_EPI_NONE: return gemm_typed<T, TMB_EPI_NONE>(g, batch, ta, tb, true, stream);
-    case TMB_EPI_GELU_TANH: return gemm_typed<T, TMB_EPI_GELU_TANH>(g, batch, ta, tb, true, stream);
-    case TMB_EPI_GELU_ERF: return gemm_typed<T, TMB_EPI_GELU_ERF>(g, batch, ta, tb, true, stream);
+    case TMB_EPI_NONE: return gemm_typed<T, TMB_EPI_NONE>(g, batch, ta, tb, true, stream, ws, ws_bytes);
+    case TMB_EPI_GELU_TANH: return gemm_typed<T, TMB_EPI_GELU_TANH>(g, batch, ta, tb, true, stream, ws, ws_bytes);
+    case TMB_EPI_GELU_ERF: return gemm_typed<T, TMB_EPI_GELU_ERF>(g, batch, ta, tb, true, stream, ws, ws_bytes);
     default: return TMB_ERR_INVALID_ARGUMENT;
   }
 }
@@ -227,7 +287,8 @@ static int gemm_entry(void* c, const void* a, const void* b, const void* bias,
                       const void* residual, int64_t batch, int64_t m, int64_t n, int64_t k,
                       int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr, int64_t stride_a,
                       int64_t stride_b, int64_t stride_c, int64_t stride_r, int trans_a,
-                      int trans_b, int dtype, int epilogue, void* stream) {
+                      int trans_b, int dtype, int epilogue, void* stream,
+                      void* workspace = nullptr, size_t workspace_bytes = 0) {
   using namespace tmb;
   if (batch < 0 || m < 0 || n < 0 || k < 0) return TMB_ERR_INVALID_ARGUMENT;
   if (epilogue < TMB_EPI_NONE || epilogue > TMB_EPI_GELU_ERF) return TMB_ERR_INVALID_ARGUMENT;
@@ -263,9 +324,9 @@ static int gemm_entry(void* c, const void* a, const void* b, const void* bias,
     return check_launch();
   }
   switch (dtype) {
-    case TMB_F32: return gemm_epi<float>(g, batch, trans_a, trans_b, epilogue, s);
-    case TMB_F16: return gemm_epi<f16_t>(g, batch, trans_a, trans_b, epilogue, s);
-    default: return gemm_epi<bf16_t>(g, batch, trans_a, trans_b, epilogue, s);
+    case TMB_F32: return gemm_epi<float>(g, batch, trans_a, trans_b, epilogue, s, workspace, workspace_bytes);
+    case TMB_F16: return gemm_epi<f16_t>(g, batch, trans_a, trans_b, epilogue, s, workspace, workspace_bytes);
+    default: return gemm_epi<bf16_t>(g, batch, trans_a, trans_b, epilogue, s, workspace, workspace_bytes);
   }
 }
 
@@ -275,6 +336,24 @@ extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias,
                         int trans_b, int dtype, int epilogue, void* stream) {
   return gemm_entry(c, a, b, bias, nullptr, batch, m, n, k, lda, ldb, ldc, 0, stride_a, stride_b,
                     stride_c, 0, trans_a, trans_b, dtype, epilogue, stream);
+}
+
+extern "C" size_t tmb_gemm_workspace_bytes(int64_t batch, int64_t m, int64_t n, int64_t k,
+                                           int dtype) {
+  if (dtype != TMB_F16 && dtype != TMB_BF16) return 0;
+  const tmb::SplitKPlan plan = tmb::splitk_plan(batch, m, n, k);
+  if (plan.splits == 0 || m * n >= (int64_t{1} << 31)) return 0;
+  return static_cast<size_t>(plan.splits) * static_cast<size_t>(m) * static_cast<size_t>(n) * 4;
+}
+
+extern "C" int tmb_gemm_ws(void* c, const void* a, const void* b, const void* bias, int64_t batch,
+                           int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
+                           int64_t stride_a, int64_t stride_b, int64_t stride_c, int trans_a,
+                           int trans_b, int dtype, int epilogue, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  return gemm_entry(c, a, b, bias, nullptr, batch, m, n, k, lda, ldb, ldc, 0, stride_a, stride_b,
+                    stride_c, 0, trans_a, trans_b, dtype, epilogue, stream, workspace,
+                    workspace_bytes);
 }
 
 extern "C" int tmb_gemm_residual(void* c, const void* a, const void* b, const void* bias,

@@ -294,6 +294,55 @@ __device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byt
   }
 }
 
+// Split-K partials: the wave tile's fp32 accumulators go to P [M, N] (pitch ldp, in floats) as
+// they are; a lane holds four consecutive columns of one row per 8-column group, so lanes l and
+// l+32 together write 32 contiguous bytes of a row. The partials are summed by
+// splitk_reduce_kernel, which also applies bias, epilogue and the one cast.
+typedef float f32x4_unaligned_t __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int TM, int TN>
+__device__ __forceinline__ void store_wave_tile_f32(f32x16_t (&acc)[TM][TN], float* __restrict__ P,
+                                                    int64_t ldp, int64_t row0, int64_t col0,
+                                                    int64_t M, int64_t N, int lane) {
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t row = row0 + i * 32 + (lane & 31);
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = col0 + j * 32 + 8 * q + 4 * (lane >> 5);
+        float* dst = P + row * ldp + col;
+        if (col + 4 <= N) {
+          f32x4_unaligned_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                 acc[i][j][4 * q + 3]};
+          *reinterpret_cast<f32x4_unaligned_t*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (col + e < N) dst[e] = acc[i][j][4 * q + e];
+        }
+      }
+  }
+}
+
+// c[m, n] = epilogue(sum over the splits (in order) of partial[s][m][n] + bias[n]), one cast.
+template <typename T, int EPI>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(T* __restrict__ c,
+                                                            const float* __restrict__ partial,
+                                                            const T* __restrict__ bias, int64_t m,
+                                                            int64_t n, int64_t ldc, int splits) {
+  const int64_t total = m * n;
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  float sum = partial[i];
+  for (int s = 1; s < splits; ++s) sum += partial[s * total + i];
+  const int64_t row = i / n, col = i - row * n;
+  if (bias != nullptr) sum += to_f32(bias[col]);
+  c[row * ldc + col] = finish<T, EPI>(sum);
+}
+
 // B_KMAJOR: B is stored [N, K] (ldb = pitch of an N-row); otherwise [K, N].
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmArgs g) {

@@ -78,8 +78,10 @@ constexpr bool kRingPersistent = ring_waves_per_simd(BM, BN, BK, WAVES, R) <= 2;
 
 // A_MMAJOR: A is stored [K, M] (the transposed view of a [K, M] matrix: the weight-gradient
 // product dy^T x); it is then staged and read exactly like N-major B.
+// OUT_F32: a split-K launch: the batch index is the split, the accumulators are stored as fp32
+// partials (no bias, no epilogue, no cast).
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
-          bool A_MMAJOR = false>
+          bool A_MMAJOR = false, bool OUT_F32 = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
                              ring_waves_per_simd(BM, BN, BK, WAVES_M* WAVES_N, R))
 void gemm_ring_kernel(GemmArgs g) {
@@ -349,6 +351,11 @@ void gemm_ring_kernel(GemmArgs g) {
   });
   mfma_step((KSTEPS - 1) & 1);
 
+  if constexpr (OUT_F32) {
+    float* P = static_cast<float*>(g.c) + batch * g.stride_c;
+    store_wave_tile_f32<TM, TN>(acc, P, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, lane);
+    return;
+  }
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
   __syncthreads();  // every wave is done with the ring: reuse it for the output
   static_assert(NW * BandLayout<WN>::BYTES <= R * STAGE_BYTES, "band staging");
@@ -388,7 +395,7 @@ static int compute_units() {
 }
 
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
-          bool A_MMAJOR = false>
+          bool A_MMAJOR = false, bool OUT_F32 = false>
 static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
@@ -406,7 +413,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   const int64_t grid_x = (!kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R> || tiles < resident)
                              ? tiles
                              : resident;
-  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR>
+  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR, OUT_F32>
       <<<dim3(static_cast<unsigned>(grid_x), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();

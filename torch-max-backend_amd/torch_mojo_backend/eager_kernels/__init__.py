@@ -34,6 +34,8 @@ SIGNATURES = {
     "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
     "tmb_argmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_gemm": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp]),
+    "tmb_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _ci]),
+    "tmb_gemm_ws": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp, _sz, _vp]),
     "tmb_gemm_residual": (_ci, [_vp, _vp, _vp, _vp, _vp] + [_i64] * 12 + [_ci] * 4 + [_vp]),
     "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
                                 _flt, _ci, _ci, _ci, _vp]),

@@ -132,6 +132,11 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
     if out.numel() == 0:
         return out
     lib = _ek.lib()
+    # few output tiles and a long K: the library splits K when it is handed scratch memory
+    ws_bytes = lib.tmb_gemm_workspace_bytes(batch, m, n, k, code_of(a.dtype))
+    if residual is not None and ws_bytes:
+        # the split kernels have no residual step; the separate add has the same bits
+        return gemm(a, b, bias, epilogue) + residual
     if residual is not None:
         res = residual if residual.stride(-1) == 1 and residual.stride(-2) >= n else residual.contiguous()
         rc = lib.tmb_gemm_residual(
@@ -143,6 +148,14 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
         if rc == _ek.ERR_UNSUPPORTED:
             return gemm(a, b, bias, epilogue) + residual
         _check("tmb_gemm_residual", rc)
+        return out
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+        rc = lib.tmb_gemm_ws(
+            out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
+            batch, m, n, k, la[1], lb[1], n, 0, 0, m * n, la[0], lb[0], code_of(a.dtype), epilogue,
+            ws.data_ptr(), ws_bytes, _stream())
+        _check("tmb_gemm_ws", rc)
         return out
     rc = lib.tmb_gemm(
         out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
