@@ -422,7 +422,6 @@ def main() -> int:
     # ------------------------------------------------------------------ GPT-2 forward
     if want in ("all", "gpt2"):
         from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
-        from torch_mojo_backend import aten_functions as af
         from torch_mojo_backend import mojo_backend
         from torch_mojo_backend.torch_compile_backend import compiler
 

@@ -57,6 +57,23 @@ def test_host_side_argument_validation_needs_no_gpu():
     assert L.tmb_gemm(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 9, None) == -1
     assert L.tmb_gemm(None, None, None, None, 0, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 0, None) == 0
     assert L.tmb_gelu(None, None, -5, ek.F32, 1, None) == -1
+    # the entry points added later obey the same rules
+    assert L.tmb_softmax_rows_scaled(None, None, 2, 2, ek.F32, 1.0, 0, 0, None) == -1
+    strides = (ctypes.c_int64 * 3)(64, 64, 64)
+    assert L.tmb_attention_fwd(None, None, None, None, 1, 1, 4, 4, 64, strides, strides, strides,
+                               strides, 0.125, 0, 0, ek.BF16, None) == -1
+    assert L.tmb_gemm_residual(None, None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, 0,
+                               ek.BF16, 0, None) == -1
+    assert L.tmb_gemm_ws(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 0, None, 0,
+                         None) == -1
+    assert L.tmb_gelu_backward(None, None, None, 8, ek.F32, 0, None) == -1
+    assert L.tmb_gelu_backward(None, None, None, 0, ek.F32, 0, None) == 0
+    assert L.tmb_softmax_backward_rows(None, None, None, 2, 2, ek.F32, 0, None) == -1
+    assert L.tmb_softmax_backward_rows(None, None, None, -2, 2, ek.F32, 0, None) == -1
+    assert L.tmb_layer_norm_backward_rows(None, None, None, None, None, None, None, None, 2, 2,
+                                          ek.F32, None, 0, None) == -1
+    assert L.tmb_layer_norm_backward_rows(None, None, None, None, None, None, None, None, 2, 0,
+                                          ek.F32, None, 0, None) == -1
 
 
 def test_workspace_plan_is_a_pure_function_of_the_shape():
@@ -69,6 +86,16 @@ def test_workspace_plan_is_a_pure_function_of_the_shape():
     assert full == L.tmb_reduce_workspace_bytes(1, 65536 * 4096, ek.BF16)
     assert L.tmb_reduce_workspace_bytes(512, 50257, ek.F32) == 512 * 3 * 16
     assert L.tmb_reduce_workspace_bytes(0, 10, ek.F32) == 0
+    # split-K scratch: only for half-precision products with fewer tiles than CUs and a long K
+    assert L.tmb_gemm_workspace_bytes(1, 8192, 8192, 8192, ek.BF16) == 0
+    assert L.tmb_gemm_workspace_bytes(1, 1024, 768, 3072, ek.F32) == 0
+    assert L.tmb_gemm_workspace_bytes(1, 1024, 768, 3072, ek.BF16) == 6 * 1024 * 768 * 4
+    assert L.tmb_gemm_workspace_bytes(2, 1024, 768, 3072, ek.BF16) == 0
+    # layer-norm backward partials: a whole number of fp32 row pairs, same for both 16-bit types
+    ln = L.tmb_layer_norm_backward_workspace_bytes(32768, 768, ek.BF16)
+    assert ln > 0 and ln % (2 * 768 * 4) == 0
+    assert ln == L.tmb_layer_norm_backward_workspace_bytes(32768, 768, ek.F16)
+    assert L.tmb_layer_norm_backward_workspace_bytes(0, 768, ek.F32) == 0
 
 
 def test_product_refuses_cpu_tensors_and_never_falls_back():
