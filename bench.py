@@ -241,6 +241,25 @@ def main() -> int:
             "frac_mfma": round(useful / ms / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4),
             "GB/s": round(algo_bytes / ms / 1e6, 1), "flops": useful, "bytes": algo_bytes,
             "note": "useful FLOPs (masked half not counted); scores never reach memory"}
+        # a decode step of the eager generation benchmark (batch 512, 12 heads, 1 query, 208 keys):
+        # K and V are read once; rotated over several caches so no cache level holds them
+        Bd, Sd = 512, 208
+        qd = gen((Bd, Hq, 1, 64), 32, torch.bfloat16)
+        caches = rotating(lambda i: gen((2, Bd, Hq, Sd, 64), 33 + i, torch.bfloat16), 2 * Bd * Hq * Sd * 64 * 2)
+        state = {"i": 0}
+
+        def decode_step():
+            kv = caches[state["i"] % len(caches)]
+            state["i"] += 1
+            hip_ops.attention_decode(qd, kv[0], kv[1], 0.125, False, None)
+
+        _, ms = timed(decode_step, 60, 10)
+        dec_bytes = 2 * Bd * Hq * Sd * 64 * 2 + 2 * Bd * Hq * 64 * 2
+        sweep["attention_decode_bf16_512x12x1x208x64"] = {
+            "us": round(ms * 1e3, 2), "GB/s": round(dec_bytes / ms / 1e6, 1),
+            "frac_hbm": round(dec_bytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": dec_bytes,
+            "note": "one wave per query row, K and V read once (includes the Python wrapper)"}
+        del caches
         # the softmax of the same attention when it runs on its own: [B*H*T, T] scores in,
         # probabilities out; the masked half of every row is not read
         rows, cols = Bq * Hq * Tq, Tq

@@ -166,6 +166,22 @@ int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v, in
                       const int64_t* v_strides, const int64_t* out_strides, float scale,
                       int causal, int round_like_unfused, int dtype, void* stream);
 
+/* Attention for a few queries per (batch, head) — the decode step of a generation loop — as one
+ * memory-bound launch (K and V are read once, nothing goes through MFMA): out = softmax(scale *
+ * q k^T [+ mask]) v with an online softmax in fp32. Strides are in elements as in
+ * tmb_attention_fwd; head_dim 64 or 128, fp16 / bf16. `mask` is NULL or a boolean (1 byte, nonzero
+ * = the key takes part) tensor addressed as mask[b*ms[0] + h*ms[1] + t*ms[2] + s*ms[3]] (stride 0
+ * where it broadcasts); `causal` keeps key s for query t if s <= t. A query without any key
+ * yields NaN, as in ATen. Returns TMB_ERR_UNSUPPORTED for layouts it does not take (the caller
+ * then composes GEMM + softmax + GEMM).
+ * Replaces `fast_aten_scaled_dot_product_attention` (aten_fast.py:5177-5285) on decode shapes. */
+int tmb_attention_decode(void* out, const void* q, const void* k, const void* v, const void* mask,
+                         int64_t batch, int64_t heads, int64_t q_len, int64_t kv_len,
+                         int64_t head_dim, const int64_t* q_strides, const int64_t* k_strides,
+                         const int64_t* v_strides, const int64_t* out_strides,
+                         const int64_t* mask_strides, float scale, int causal, int dtype,
+                         void* stream);
+
 /* Elementwise GELU over `numel` contiguous elements, fp32 inside, one cast.
  * `approximate_tanh` != 0 selects the tanh form. Replaces activation_forward_kernels.mojo:22-56
  * (used when the GELU cannot be fused into the producing GEMM's epilogue). */

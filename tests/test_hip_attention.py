@@ -216,3 +216,70 @@ def test_sdpa_surfaces_use_the_composed_path_for_fp32_and_masks():
                                                            attn_mask=mask.to("mojo"))
     assert got.device.type == "mojo"
     torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-5)
+
+
+# ---- decode kernel: a few queries per head, K and V read once ------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", [
+    # (batch, heads, queries, keys, head_dim, causal, mask)
+    (2, 3, 1, 1, 64, False, False), (4, 12, 1, 37, 64, False, True), (2, 2, 1, 208, 64, False, False),
+    (1, 2, 5, 64, 64, True, False), (2, 4, 16, 100, 64, False, True), (3, 2, 1, 333, 128, False, True),
+    (1, 3, 7, 7, 128, True, False), (2, 2, 2, 1000, 64, False, False),
+])
+def test_attention_decode_matches_closed_form(case, dtype):
+    b, h, t, s, d, causal, with_mask = case
+    q = seeded((b, h, t, d), seed=1, dtype=dtype)
+    k = seeded((b, h, s, d), seed=2, dtype=dtype)
+    v = seeded((b, h, s, d), seed=3, dtype=dtype)
+    mask = None
+    if with_mask:
+        mask = torch.rand(b, 1, t, s, generator=torch.Generator().manual_seed(9)) > 0.3
+        mask[..., 0] = True
+    scale = 1.0 / np.sqrt(d)
+    assert _ops().attention_decode_supported(q.cuda(), k.cuda(), v.cuda(), None if mask is None else mask.cuda())
+    got = _ops().attention_decode(q.cuda(), k.cuda(), v.cuda(), scale, causal,
+                                  None if mask is None else mask.cuda())
+    assert got.shape == (b, h, t, d) and got.dtype == dtype and got.is_contiguous()
+    want = _sdpa64(q, k, v, scale, causal, mask)
+    tol = {torch.bfloat16: 2e-2, torch.float16: 3e-3}[dtype]
+    assert np.abs(as64(got) - want).max() <= tol
+
+
+def test_attention_decode_strided_views_masked_rows_and_rejections():
+    ops = _ops()
+    # q/k/v as the thirds of a packed projection (strided heads), keys as a slice of a longer cache
+    b, h, t, s, d = 2, 4, 1, 50, 64
+    qkv = seeded((b, t, 3 * h * d), seed=4, dtype=torch.bfloat16).cuda()
+    q = qkv[..., :h * d].view(b, t, h, d).transpose(1, 2)
+    cache = seeded((2, b, h, 128, d), seed=5, dtype=torch.bfloat16).cuda()
+    k, v = cache[0, :, :, :s], cache[1, :, :, :s]
+    got = ops.attention_decode(q, k, v, 0.125, False, None)
+    want = _sdpa64(q.cpu(), k.cpu(), v.cpu(), 0.125, False, None)
+    assert np.abs(as64(got) - want).max() <= 2e-2
+    # a query whose keys are all masked out yields NaN, like ATen
+    mask = torch.ones(b, 1, t, s, dtype=torch.bool)
+    mask[1] = False
+    out = ops.attention_decode(q, k, v, 0.125, False, mask.cuda()).float().cpu()
+    assert torch.isnan(out[1]).all() and not torch.isnan(out[0]).any()
+    # what it does not take
+    assert not ops.attention_decode_supported(q.float(), k.float(), v.float(), None)
+    assert not ops.attention_decode_supported(q, k, v, torch.zeros(t, s, device="cuda"))  # additive
+    big_q = seeded((b, h, 17, d), seed=6, dtype=torch.bfloat16).cuda()
+    assert not ops.attention_decode_supported(big_q, k, v, None)
+
+
+def test_sdpa_surfaces_route_decode_shapes_to_the_decode_kernel(monkeypatch):
+    from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO
+    from torch_mojo_backend.eager_kernels import hip_ops
+    calls = []
+    real = hip_ops.attention_decode
+    monkeypatch.setattr(hip_ops, "attention_decode", lambda *a, **kw: calls.append(1) or real(*a, **kw))
+    q = seeded((2, 4, 1, 64), seed=1, dtype=torch.bfloat16).cuda()
+    k = seeded((2, 4, 30, 64), seed=2, dtype=torch.bfloat16).cuda()
+    v = seeded((2, 4, 30, 64), seed=3, dtype=torch.bfloat16).cuda()
+    mask = torch.ones(2, 1, 1, 30, dtype=torch.bool, device="cuda")
+    fn = MAPPING_TORCH_ATEN_TO_MOJO[torch.ops.aten.scaled_dot_product_attention]
+    got = fn(q, k, v, mask)
+    assert calls and got.shape == (2, 4, 1, 64)
+    want = _sdpa64(q.cpu(), k.cpu(), v.cpu(), 0.125, False, mask.cpu())
+    assert np.abs(as64(got) - want).max() <= 2e-2

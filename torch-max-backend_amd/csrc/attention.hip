@@ -292,6 +292,108 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #endif
 }
 
+// ---------------------------------------------------------------------------
+// Few queries per (batch, head): the decode step of a generation loop. One wave per query row;
+// the work is reading K and V once, so there is no MFMA: D/8 lanes share a key (16 bytes of the
+// row each), a wave covers 64/(D/8) keys per step with whole-row loads, every key group keeps its
+// own running maximum, sum and output chunk (online softmax), and the groups are merged at the
+// end. An optional boolean mask (broadcastable, True = takes part) and the top-left aligned
+// causal rule are applied to the scores; a row without any key comes out as NaN, as in ATen.
+// ---------------------------------------------------------------------------
+struct AttnDecodeArgs {
+  void* out;
+  const void* q;
+  const void* k;
+  const void* v;
+  const unsigned char* mask;      // may be null
+  int64_t q_sb, q_sh, q_st;
+  int64_t k_sb, k_sh, k_st;
+  int64_t v_sb, v_sh, v_st;
+  int64_t o_sb, o_sh, o_st;
+  int64_t m_sb, m_sh, m_st, m_ss;  // mask element strides (0 where it broadcasts)
+  int64_t rows;                    // batch * heads * q_len
+  int heads, q_len, kv_len;
+  float scale;
+  int causal;
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attention_decode_kernel(AttnDecodeArgs a) {
+  constexpr int LPK = D / 8;        // lanes per key
+  constexpr int KPI = kWave / LPK;  // keys per step of a wave
+  const int lane = threadIdx.x & 63;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;  // whole waves leave; no barriers below
+  const int t = static_cast<int>(row % a.q_len);
+  const int64_t bh = row / a.q_len;
+  const int h = static_cast<int>(bh % a.heads);
+  const int64_t b = bh / a.heads;
+  const int sub = lane % LPK, kg = lane / LPK;
+
+  const T* qrow = static_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh + t * a.q_st + sub * 8;
+  const T* kbase = static_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh + sub * 8;
+  const T* vbase = static_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh + sub * 8;
+  const unsigned char* mrow =
+      a.mask == nullptr ? nullptr : a.mask + b * a.m_sb + h * a.m_sh + t * a.m_st;
+
+  const float c = a.scale * 1.44269504088896340736f;  // scores in the log2 domain
+  float qf[8];
+  {
+    const Vec16<T> qv = load_vec16(qrow);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[e] = to_f32(qv.v[e]) * c;
+  }
+  const float neg_inf = -__builtin_inff();
+  float m = neg_inf, l = 0.0f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+
+  const int last = a.causal ? (t < a.kv_len - 1 ? t : a.kv_len - 1) : a.kv_len - 1;
+  for (int s0 = 0; s0 <= last; s0 += KPI) {
+    const int s = s0 + kg;
+    bool valid = s <= last;
+    if (valid && mrow != nullptr) valid = mrow[s * a.m_ss] != 0;
+    const int sr = s <= last ? s : last;  // a readable row for lanes without a key
+    const Vec16<T> kv = load_vec16_stream(kbase + static_cast<int64_t>(sr) * a.k_st);
+    const Vec16<T> vv = load_vec16_stream(vbase + static_cast<int64_t>(sr) * a.v_st);
+    float x = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x = __builtin_fmaf(qf[e], to_f32(kv.v[e]), x);
+#pragma unroll
+    for (int w = 1; w < LPK; w <<= 1) x += __shfl_xor(x, w, kWave);
+    if (valid) {
+      const float m_new = fmaxf(m, x);
+      const float corr = __builtin_amdgcn_exp2f(m - m_new);  // 0 on the first key (m = -inf)
+      const float p = __builtin_amdgcn_exp2f(x - m_new);
+      l = l * corr + p;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * corr + p * to_f32(vv.v[e]);
+      m = m_new;
+    }
+  }
+  // merge the key groups (lanes with equal `sub`)
+  float big = m;
+#pragma unroll
+  for (int w = LPK; w < kWave; w <<= 1) big = fmaxf(big, __shfl_xor(big, w, kWave));
+  const float wgt = m == neg_inf ? 0.0f : __builtin_amdgcn_exp2f(m - big);
+  l *= wgt;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] *= wgt;
+#pragma unroll
+  for (int w = LPK; w < kWave; w <<= 1) {
+    l += __shfl_xor(l, w, kWave);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], w, kWave);
+  }
+  if (kg == 0) {
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = acc[e] / l;  // 0/0 = NaN for a row without keys
+    T* dst = static_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + t * a.o_st + sub * 8;
+    store_converted<T, 8>(dst, r);
+  }
+}
+
 }  // namespace tmb
 
 extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v,
@@ -341,5 +443,55 @@ extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const 
   } else {
     attention_fwd_kernel<f16_t><<<grid, dim3(256), 0, s>>>(a);
   }
+  return check_launch();
+}
+
+extern "C" int tmb_attention_decode(void* out, const void* q, const void* k, const void* v,
+                                    const void* mask, int64_t batch, int64_t heads, int64_t q_len,
+                                    int64_t kv_len, int64_t head_dim, const int64_t* q_strides,
+                                    const int64_t* k_strides, const int64_t* v_strides,
+                                    const int64_t* out_strides, const int64_t* mask_strides,
+                                    float scale, int causal, int dtype, void* stream) {
+  using namespace tmb;
+  if (batch < 0 || heads < 0 || q_len < 0 || kv_len < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (dtype != TMB_F16 && dtype != TMB_BF16) return TMB_ERR_UNSUPPORTED;
+  if (head_dim != 64 && head_dim != 128) return TMB_ERR_UNSUPPORTED;
+  if (!(scale == scale)) return TMB_ERR_INVALID_ARGUMENT;
+  if (batch == 0 || heads == 0 || q_len == 0) return TMB_OK;
+  if (kv_len == 0) return TMB_ERR_UNSUPPORTED;
+  if (!out || !q || !k || !v || !q_strides || !k_strides || !v_strides || !out_strides ||
+      (mask != nullptr && !mask_strides))
+    return TMB_ERR_INVALID_ARGUMENT;
+  if (heads >= (int64_t{1} << 31) || q_len >= (int64_t{1} << 31) || kv_len >= (int64_t{1} << 31) ||
+      batch * heads * q_len >= (int64_t{1} << 33))
+    return TMB_ERR_UNSUPPORTED;
+  auto aligned = [](const void* p, const int64_t* s) {
+    return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && s[0] % 8 == 0 && s[1] % 8 == 0 &&
+           s[2] % 8 == 0 && s[0] >= 0 && s[1] >= 0 && s[2] >= 0;
+  };
+  if (!aligned(q, q_strides) || !aligned(k, k_strides) || !aligned(v, v_strides) ||
+      !aligned(out, out_strides))
+    return TMB_ERR_UNSUPPORTED;
+  if (mask != nullptr)
+    for (int i = 0; i < 4; ++i)
+      if (mask_strides[i] < 0) return TMB_ERR_UNSUPPORTED;
+  AttnDecodeArgs a{out, q, k, v, static_cast<const unsigned char*>(mask),
+                   q_strides[0], q_strides[1], q_strides[2],
+                   k_strides[0], k_strides[1], k_strides[2],
+                   v_strides[0], v_strides[1], v_strides[2],
+                   out_strides[0], out_strides[1], out_strides[2],
+                   mask ? mask_strides[0] : 0, mask ? mask_strides[1] : 0,
+                   mask ? mask_strides[2] : 0, mask ? mask_strides[3] : 0,
+                   batch * heads * q_len, static_cast<int>(heads), static_cast<int>(q_len),
+                   static_cast<int>(kv_len), scale, causal ? 1 : 0};
+  const dim3 grid(static_cast<unsigned>((a.rows + 3) / 4));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define TMB_AD(T, D) attention_decode_kernel<T, D><<<grid, dim3(256), 0, s>>>(a)
+  if (dtype == TMB_BF16) {
+    if (head_dim == 64) TMB_AD(bf16_t, 64); else TMB_AD(bf16_t, 128);
+  } else {
+    if (head_dim == 64) TMB_AD(f16_t, 64); else TMB_AD(f16_t, 128);
+  }
+#undef TMB_AD
   return check_launch();
 }

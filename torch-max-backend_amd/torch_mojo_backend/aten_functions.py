@@ -268,8 +268,8 @@ def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout
                                       enable_gqa: bool = False) -> torch.Tensor:
     """reference :3029-3087 (built there from matmul, softmax and matmul graph ops). The fused
     HIP kernel takes the call when there is no explicit mask, head_dim is 64 and the dtype has
-    16 bits; other head sizes, fp32 and explicit masks run as GEMM + softmax + GEMM on the same
-    kernels. Dropout and grouped-query attention are PyTorch-ROCm's own op."""
+    16 bits; up to 16 queries per head (decode) run in the decode kernel; other head sizes, fp32
+    and additive masks run as GEMM + softmax + GEMM on the same kernels. Dropout and grouped-query attention are PyTorch-ROCm's own op."""
     plain = dropout_p == 0.0 and not enable_gqa and query.dim() >= 2 \
         and query.dtype in hip_ops.FLOAT_DTYPES and key.dtype == query.dtype \
         and value.dtype == query.dtype and key.shape[:-2] == query.shape[:-2] \
@@ -280,6 +280,9 @@ def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout
         if attn_mask is None and s > 0.0 and query.dim() == 4 \
                 and hip_ops.attention_supported(query, key, value):
             return hip_ops.attention(query, key, value, s, bool(is_causal)).transpose(1, 2)
+        if query.dim() == 4 and query.shape[2] <= hip_ops.DECODE_MAX_QUERIES \
+                and hip_ops.attention_decode_supported(query, key, value, attn_mask):
+            return hip_ops.attention_decode(query, key, value, s, bool(is_causal), attn_mask)
         return hip_ops.attention_composed(query, key, value, s, bool(is_causal), attn_mask)
     return aten.scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal,
                                              scale=scale, enable_gqa=enable_gqa)

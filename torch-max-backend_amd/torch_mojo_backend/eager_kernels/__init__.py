@@ -39,6 +39,7 @@ SIGNATURES = {
     "tmb_gemm_residual": (_ci, [_vp, _vp, _vp, _vp, _vp] + [_i64] * 12 + [_ci] * 4 + [_vp]),
     "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
                                 _flt, _ci, _ci, _ci, _vp]),
+    "tmb_attention_decode": (_ci, [_vp] * 5 + [_i64] * 5 + [_vp] * 5 + [_flt, _ci, _ci, _vp]),
     "tmb_gelu": (_ci, [_vp, _vp, _i64, _ci, _ci, _vp]),
     "tmb_gelu_backward": (_ci, [_vp, _vp, _vp, _i64, _ci, _ci, _vp]),
     "tmb_softmax_backward_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _ci, _ci, _vp]),

@@ -264,6 +264,60 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, c
     return out
 
 
+# Queries per (batch, head) up to which the decode kernel (one wave per query row, K and V read
+# once per query) is used instead of the GEMM-based paths.
+DECODE_MAX_QUERIES = 16
+
+
+def attention_decode_supported(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                               attn_mask: Optional[torch.Tensor]) -> bool:
+    """True when `attention_decode` takes these [batch, heads, tokens, head_dim] tensors."""
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or not (q.is_cuda and k.is_cuda and v.is_cuda):
+        return False
+    if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        return False
+    b, h, t, d = q.shape
+    if d not in (64, 128) or t == 0 or t > DECODE_MAX_QUERIES or k.shape[2] == 0:
+        return False
+    if tuple(k.shape) != (b, h, k.shape[2], d) or tuple(v.shape) != tuple(k.shape):
+        return False
+    for x in (q, k, v):
+        if x.stride(3) != 1 or any(s % 8 or s < 0 for s in x.stride()[:3]) or x.data_ptr() % 16:
+            return False
+    if attn_mask is not None:
+        if attn_mask.dtype != torch.bool or not attn_mask.is_cuda or attn_mask.dim() > 4:
+            return False
+        try:
+            torch.broadcast_shapes(tuple(attn_mask.shape), (b, h, t, k.shape[2]))
+        except RuntimeError:
+            return False
+        if tuple(torch.broadcast_shapes(tuple(attn_mask.shape), (b, h, t, k.shape[2]))) != (b, h, t, k.shape[2]):
+            return False
+    return True
+
+
+def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                     causal: bool, attn_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softmax(scale q kᵀ [masked]) v for a few queries per head in one launch; returns
+    [batch, heads, tokens, head_dim] contiguous."""
+    require_hip(q, k, v, attn_mask)
+    if not attention_decode_supported(q, k, v, attn_mask):
+        raise ValueError("attention_decode: unsupported operands (see attention_decode_supported)")
+    b, h, t, d = q.shape
+    out = torch.empty((b, h, t, d), dtype=q.dtype, device=q.device)
+    arr = lambda strides: (ctypes.c_int64 * len(strides))(*strides)  # noqa: E731
+    mask_ptr, mask_strides = None, None
+    if attn_mask is not None:
+        m4 = attn_mask.expand(b, h, t, k.shape[2])  # stride 0 where it broadcasts
+        mask_ptr, mask_strides = m4.data_ptr(), arr(m4.stride())
+    rc = _ek.lib().tmb_attention_decode(
+        out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), mask_ptr, b, h, t, k.shape[2], d,
+        arr(q.stride()[:3]), arr(k.stride()[:3]), arr(v.stride()[:3]), arr(out.stride()[:3]),
+        mask_strides, float(scale), int(bool(causal)), code_of(q.dtype), _stream())
+    _check("tmb_attention_decode", rc)
+    return out
+
+
 def attention_composed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
                        causal: bool, attn_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``softmax(q kᵀ · scale + mask) v`` for [..., tokens, head_dim] operands of any head size and
