@@ -80,6 +80,9 @@ struct GemmArgs {
   // i.e. what a separate elementwise add after the GEMM would store (MFMA kernels only)
   const void* residual;
   int64_t ldr, stride_r;
+  // persistent kernels with a streamed output: workgroups start in four phases this many 10 ns
+  // ticks apart, so that their store bursts do not all hit memory at the same moment
+  int stagger_ticks = 0;
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the

@@ -104,6 +104,15 @@ void gemm_ring_kernel(GemmArgs g) {
                 "tile does not split into whole 1 KiB loads per wave");
   __shared__ __attribute__((aligned(1024))) unsigned char ring[R * STAGE_BYTES];
 
+  // All workgroups of a persistent launch finish their tiles at the same time; with an output
+  // that streams to memory their store bursts then collide while the matrix pipes idle. A start
+  // offset of a few microseconds per phase keeps them apart for the whole launch (measured on a
+  // 32768 x 50257 x 768 product: 2.62 -> 2.44 ms with four phases 5 us apart; 8 or 12 us less).
+  if (g.stagger_ticks > 0) {
+    const uint64_t t0 = wall_clock64();
+    const uint64_t wait = static_cast<uint64_t>((blockIdx.x / 8) % 4) * g.stagger_ticks;
+    while (wall_clock64() - t0 < wait) __builtin_amdgcn_s_sleep(8);
+  }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   int64_t m0 = 0, n0 = 0;  // origin of the tile being worked on (set per tile below)
@@ -413,6 +422,8 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   const int64_t grid_x = (!kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R> || tiles < resident)
                              ? tiles
                              : resident;
+  // four start phases 5 us apart when every workgroup walks several tiles of a streamed output
+  g.stagger_ticks = (g.stream_c && !OUT_F32 && grid_x == resident && tiles >= 4 * resident) ? 500 : 0;
   gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR, OUT_F32>
       <<<dim3(static_cast<unsigned>(grid_x), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
