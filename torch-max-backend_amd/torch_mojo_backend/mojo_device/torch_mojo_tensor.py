@@ -31,9 +31,10 @@ class TorchMojoTensor(torch.Tensor):
             if t is not cls and not issubclass(cls, t):
                 return NotImplemented
         impl = DIRECT_IMPLS.get(func)
+        if impl is not None:
+            # the implementations work on the HIP holders, so nothing below re-enters this method
+            return impl(*args, **kwargs) if kwargs else impl(*args)
         with torch._C._DisableTorchDispatch():
-            if impl is not None:
-                return impl(*args, **kwargs) if kwargs else impl(*args)
             return func(*args, **(kwargs or {}))
 
     @classmethod
