@@ -35,6 +35,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "torch-max-backend_amd"))
 
 PEAK_BF16_DENSE_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
+PEAK_FP32_MFMA_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 
 # Bytes per launch of the headline GEMM kernel between L2 and the memory side, measured with
@@ -170,22 +171,24 @@ def main() -> int:
             return 1
     del a, b, bias
 
-    def gemm_row(name, m, n, k, batch=None, trans_b=False, steps=50):
+    def gemm_row(name, m, n, k, batch=None, trans_b=False, steps=50, dtype=torch.bfloat16):
         if batch:
-            x = gen((batch, m, k), 3, torch.bfloat16)
-            w = gen((batch, k, n), 4, torch.bfloat16)
+            x = gen((batch, m, k), 3, dtype)
+            w = gen((batch, k, n), 4, dtype)
             bs = None
         else:
-            x = gen((m, k), 3, torch.bfloat16)
-            w = gen((n, k), 4, torch.bfloat16).t() if trans_b else gen((k, n), 4, torch.bfloat16)
-            bs = gen((n,), 5, torch.bfloat16)
+            x = gen((m, k), 3, dtype)
+            w = gen((n, k), 4, dtype).t() if trans_b else gen((k, n), 4, dtype)
+            bs = gen((n,), 5, dtype)
         _, ms = timed(lambda: hip_ops.gemm(x, w, bs), steps, 10)
         bt = batch or 1
+        size = x.element_size()
+        peak = PEAK_FP32_MFMA_TFLOPS if dtype == torch.float32 else PEAK_BF16_DENSE_TFLOPS
         fl = 2.0 * bt * m * n * k
-        by = 2.0 * bt * (m * k + k * n + m * n) + (0 if batch else 2 * n)
+        by = size * (bt * (m * k + k * n + m * n) + (0 if batch else n))
         tf, gbs = fl / ms / 1e9, by / ms / 1e6
         sweep[name] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 2),
-                       "frac_mfma": round(tf / PEAK_BF16_DENSE_TFLOPS, 4),
+                       "frac_mfma": round(tf / peak, 4),
                        "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
 
     if want in ("all", "gemm"):
@@ -195,6 +198,10 @@ def main() -> int:
         for (m, n, k) in ((128, 768, 768), (1024, 3072, 768), (1024, 768, 3072), (4096, 4096, 4096)):
             gemm_row(f"addmm_bf16_{m}x{n}x{k}", m, n, k)
         gemm_row("bmm_bf16_48x1024x64x1024", 1024, 1024, 64, batch=48)
+        # fp32 storage: true fp32 products on the matrix cores (peak 157.3 TFLOP/s)
+        gemm_row("addmm_fp32_4096x4096x4096", 4096, 4096, 4096, steps=20, dtype=torch.float32)
+        gemm_row("addmm_fp32_128x3072x768", 128, 3072, 768, dtype=torch.float32)
+        gemm_row("linear_fp32_128x50257x768", 128, 50257, 768, trans_b=True, dtype=torch.float32)
 
     # ------------------------------------------------------------------ memory-bound rows
     # Launched straight through the C ABI with preallocated outputs, so the timed region holds

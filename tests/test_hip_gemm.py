@@ -371,9 +371,77 @@ def test_split_k_is_reproducible_and_needs_scratch_only_when_it_pays():
     assert lib.tmb_gemm_workspace_bytes(1, 8192, 8192, 8192, code) == 0      # plenty of tiles
     assert lib.tmb_gemm_workspace_bytes(1, 1024, 768, 768, code) == 0        # short K
     assert lib.tmb_gemm_workspace_bytes(4, 1024, 768, 4096, code) == 0       # batched
-    assert lib.tmb_gemm_workspace_bytes(1, 1024, 768, 4096, _ops().code_of(torch.float32)) == 0
+    f32 = _ops().code_of(torch.float32)
+    assert lib.tmb_gemm_workspace_bytes(1, 4096, 4096, 4096, f32) == 0       # fp32: plenty of tiles
+    assert lib.tmb_gemm_workspace_bytes(1, 1024, 768, 4096, f32) == 8 * 1024 * 768 * 4
     a = _dev(seeded((512, 4096), seed=31, dtype=torch.bfloat16))
     b = _dev(seeded((4096, 384), seed=32, dtype=torch.bfloat16))
     first = _ops().gemm(a, b)
     for _ in range(3):
         assert torch.equal(first, _ops().gemm(a, b))
+
+
+# ---- fp32 on the matrix cores --------------------------------------------------------------------
+F32_LAYOUTS = [  # (m, n, k, trans_a, trans_b): aligned for the MFMA kernel, edges in every direction
+    (128, 128, 16, False, False), (132, 260, 36, False, True), (132, 260, 36, True, False),
+    (132, 260, 36, True, True), (4, 8, 4, False, False), (1, 772, 768, False, True),
+    (300, 50257, 768, False, True), (257, 516, 1028, False, False), (257, 516, 1028, True, True),
+    (128, 768, 3072, False, True), (128, 3072, 768, False, False), (16, 4096, 4096, False, True),
+    (768, 768, 2048, True, False),
+    (130, 131, 72, False, False), (130, 132, 70, False, True),   # unaligned: the SIMT kernel
+]
+
+
+@pytest.mark.parametrize("case", F32_LAYOUTS)
+def test_fp32_mfma_all_layouts_match_float64(case):
+    m, n, k, ta, tb = case
+    a = seeded((k, m) if ta else (m, k), seed=41, dtype=torch.float32)
+    b = seeded((n, k) if tb else (k, n), seed=42, dtype=torch.float32)
+    bias = seeded((n,), seed=43, dtype=torch.float32)
+    av = _dev(a).t() if ta else _dev(a)
+    bv = _dev(b).t() if tb else _dev(b)
+    got = _ops().gemm(av, bv, _dev(bias))
+    a64 = as64(a).T if ta else as64(a)
+    b64 = as64(b).T if tb else as64(b)
+    want = a64 @ b64 + as64(bias)
+    # fp32 products are exact in the accumulator's input; k additions round at 2^-24 each
+    bound = k * 2.0 ** -24 * (np.abs(a64) @ np.abs(b64) + np.abs(as64(bias)))
+    assert_close64(got, want, extra_abs=bound, what=f"fp32 gemm {case}")
+    assert rel_frobenius(got, want) <= 2e-6
+
+
+def test_fp32_mfma_batched_strided_and_gelu():
+    a = _dev(seeded((6, 200, 96), seed=44, dtype=torch.float32))
+    b = _dev(seeded((6, 96, 136), seed=45, dtype=torch.float32))
+    got = _ops().gemm(a, b)
+    want = as64(a) @ as64(b)
+    assert rel_frobenius(got, want) <= 2e-6
+    # rows of a wider buffer (lda > k) and a GELU epilogue against the separate kernel
+    wide = _dev(seeded((200, 160), seed=46, dtype=torch.float32))
+    a2 = wide[:, 32:128]
+    w = _dev(seeded((136, 96), seed=47, dtype=torch.float32))
+    bias = _dev(seeded((136,), seed=48, dtype=torch.float32))
+    fused = _ops().gemm(a2, w.t(), bias, _ek().EPI_GELU_TANH)
+    unfused = _ops().gelu(_ops().gemm(a2, w.t(), bias), "tanh")
+    assert torch.equal(fused, unfused)
+    want = as64(a2) @ as64(w).T + as64(bias)
+    assert rel_frobenius(_ops().gemm(a2, w.t(), bias), want) <= 2e-6
+
+
+def test_fp32_split_k_is_reproducible_and_close_to_the_unsplit_kernel():
+    m, n, k = 128, 768, 3072
+    lib, ek = _ek().lib(), _ek()
+    assert lib.tmb_gemm_workspace_bytes(1, m, n, k, ek.F32) == 16 * m * n * 4
+    a = _dev(seeded((m, k), seed=51, dtype=torch.float32))
+    w = _dev(seeded((n, k), seed=52, dtype=torch.float32))
+    bias = _dev(seeded((n,), seed=53, dtype=torch.float32))
+    first = _ops().gemm(a, w.t(), bias)
+    for _ in range(3):
+        assert torch.equal(first, _ops().gemm(a, w.t(), bias))
+    plain = torch.empty_like(first)
+    rc = lib.tmb_gemm(plain.data_ptr(), a.data_ptr(), w.data_ptr(), bias.data_ptr(), 1, m, n, k,
+                      k, k, n, 0, 0, m * n, 0, 1, ek.F32, ek.EPI_NONE,
+                      torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    want = as64(a) @ as64(w).T + as64(bias)
+    assert rel_frobenius(first, want) <= 2e-6 and rel_frobenius(plain, want) <= 2e-6

@@ -20,6 +20,7 @@
 
 #include "gemm_mfma.h"
 #include "gemm_ring.h"
+#include "gemm_f32.h"
 
 namespace tmb {
 
@@ -232,6 +233,44 @@ static int launch_splitk(const GemmArgs& g, const SplitKPlan& plan, int trans_a,
   return check_launch();
 }
 
+// fp32 products run 16 times slower on the matrix cores than 16-bit ones, so a 128 x 128 tile
+// with a few hundred K already takes tens of microseconds and the split pays from much shorter K.
+// Chunks are whole 16-byte groups of K so that every chunk keeps the operands' alignment.
+static SplitKPlan splitk_plan_f32(int64_t batch, int64_t m, int64_t n, int64_t k) {
+  SplitKPlan p{0, 0};
+  if (batch != 1 || k < 128 || m < 1 || n < 1) return p;
+  const int64_t tiles = ((m + kF32BM - 1) / kF32BM) * ((n + kF32BN - 1) / kF32BN);
+  if (tiles >= 256) return p;
+  int64_t splits = 512 / tiles;
+  if (splits > 16) splits = 16;
+  if (splits > k / 64) splits = k / 64;
+  while (splits >= 2 && k % (splits * 4) != 0) --splits;
+  if (splits < 2) return p;
+  p.splits = static_cast<int>(splits);
+  p.k_chunk = k / splits;
+  return p;
+}
+
+template <int EPI>
+static int launch_splitk_f32(const GemmArgs& g, const SplitKPlan& plan, int trans_a, int trans_b,
+                             float* workspace, hipStream_t stream) {
+  GemmArgs part = g;
+  part.c = workspace;
+  part.bias = nullptr;
+  part.k = plan.k_chunk;
+  part.ldc = g.n;
+  part.stride_c = g.m * g.n;
+  part.stride_a = trans_a ? plan.k_chunk * g.lda : plan.k_chunk;
+  part.stride_b = trans_b ? plan.k_chunk : plan.k_chunk * g.ldb;
+  const int rc = launch_f32_mfma<TMB_EPI_NONE>(part, plan.splits, trans_a, trans_b, stream);
+  if (rc != 0) return rc;
+  const int64_t total = g.m * g.n;
+  splitk_reduce_kernel<float, EPI><<<dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream>>>(
+      static_cast<float*>(g.c), workspace, static_cast<const float*>(g.bias), g.m, g.n, g.ldc,
+      plan.splits);
+  return check_launch();
+}
+
 template <typename T, int EPI>
 static int gemm_typed(const GemmArgs& g, int64_t batch, int trans_a, int trans_b, bool half,
                       hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0) {
@@ -251,6 +290,16 @@ static int gemm_typed(const GemmArgs& g, int64_t batch, int trans_a, int trans_b
     if (half && mfma_eligible(g, batch, trans_a, trans_b)) {
       return trans_b ? mfma_pick_tile<T, true, EPI>(g, batch, stream)
                      : mfma_pick_tile<T, false, EPI>(g, batch, stream);
+    }
+  }
+  if constexpr (__is_same(T, float)) {
+    if (g.residual == nullptr && f32_mfma_eligible(g, batch, trans_a, trans_b)) {
+      const SplitKPlan plan = splitk_plan_f32(batch, g.m, g.n, g.k);
+      if (plan.splits > 0 && workspace != nullptr && g.m * g.n < (int64_t{1} << 31) &&
+          workspace_bytes >= static_cast<size_t>(plan.splits) * g.m * g.n * 4)
+        return launch_splitk_f32<EPI>(g, plan, trans_a, trans_b, static_cast<float*>(workspace),
+                                      stream);
+      return launch_f32_mfma<EPI>(g, batch, trans_a, trans_b, stream);
     }
   }
   return launch_simt<T, EPI>(g, batch, trans_a, trans_b, stream);
@@ -340,8 +389,9 @@ extern "C" int tmb_gemm(void* c, const void* a, const void* b, const void* bias,
 
 extern "C" size_t tmb_gemm_workspace_bytes(int64_t batch, int64_t m, int64_t n, int64_t k,
                                            int dtype) {
-  if (dtype != TMB_F16 && dtype != TMB_BF16) return 0;
-  const tmb::SplitKPlan plan = tmb::splitk_plan(batch, m, n, k);
+  if (dtype != TMB_F32 && dtype != TMB_F16 && dtype != TMB_BF16) return 0;
+  const tmb::SplitKPlan plan = dtype == TMB_F32 ? tmb::splitk_plan_f32(batch, m, n, k)
+                                                : tmb::splitk_plan(batch, m, n, k);
   if (plan.splits == 0 || m * n >= (int64_t{1} << 31)) return 0;
   return static_cast<size_t>(plan.splits) * static_cast<size_t>(m) * static_cast<size_t>(n) * 4;
 }
