@@ -184,26 +184,49 @@ static bool mfma_eligible(const GemmArgs& g, int64_t batch, int trans_a, int tra
 }
 
 // Split-K: products with few output tiles and a long K (weight gradients, narrow projections)
-// leave most CUs idle. K is cut into `splits` equal chunks that run as the batch dimension of one
-// launch of the 128x128 ring kernel and store fp32 partials [splits][M][N] into a workspace; a
-// second kernel adds them in split order and applies bias, epilogue and the one cast, so the
-// result is still "fp32 accumulation, one rounding" and depends on the shape only.
+// leave most CUs idle. K is cut into `splits` runs of whole stages (equal to within one stage)
+// that run as the y dimension of one launch of a ring kernel and store fp32 partials
+// [splits][M][N] into a workspace; a second kernel adds them in split order and applies bias,
+// epilogue and the one cast, so the result is still "fp32 accumulation, one rounding" and depends
+// on the shape only.
+//
+// Tile and split count come from a small cost model (all in microseconds): the 256 x 256 x 64
+// kernel sustains about 1240 TFLOP/s over 256 one-per-CU workgroups, the 128 x 128 x 32 kernel
+// about 900 TFLOP/s over 512 two-per-CU workgroups; the launch takes ceil(units / slots) rounds of
+// one unit's time, the reduction reads splits * M * N * 4 bytes at about 4 TB/s.
 struct SplitKPlan {
-  int splits;       // 0: not used
-  int64_t k_chunk;
+  int splits;  // 0: not used
+  int tile;    // 128 or 256
+  int64_t k_chunk;  // fp32 kernel only: equal chunks
 };
 static SplitKPlan splitk_plan(int64_t batch, int64_t m, int64_t n, int64_t k) {
-  SplitKPlan p{0, 0};
+  SplitKPlan p{0, 0, 0};
   if (batch != 1 || k < 2048 || k % 32 != 0 || n <= 64 || m < 1) return p;
-  const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128);
-  if (tiles >= 256) return p;  // at least one tile per CU: no split
-  int64_t splits = 512 / tiles;
-  if (splits > 16) splits = 16;
-  if (splits > k / 512) splits = k / 512;
-  while (splits >= 2 && k % (splits * 32) != 0) --splits;
-  if (splits < 2) return p;
-  p.splits = static_cast<int>(splits);
-  p.k_chunk = k / splits;
+  const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
+  if (t128 >= 256) return p;  // at least one tile per CU: no split
+  const int64_t t256 = ((m + 255) / 256) * ((n + 255) / 256);
+  double best = 0.0;
+  for (int tile = 128; tile <= 256; tile += 128) {
+    const int bk = tile == 128 ? 32 : 64;
+    if (k % bk != 0) continue;
+    if (tile == 256 && (m <= 128 || n <= 128)) continue;
+    const int64_t tiles = tile == 128 ? t128 : t256;
+    const int64_t slots = tile == 128 ? 512 : 256;
+    const double unit_rate = tile == 128 ? 900e6 / 512 : 1240e6 / 256;  // FLOP per us per workgroup
+    for (int64_t splits = 2; splits <= 16; ++splits) {
+      if (k / bk / splits < 8) break;  // at least 8 stages per split
+      const double chunk = static_cast<double>(k) / splits;
+      const double unit = 2.0 * tile * tile * chunk / unit_rate;
+      const double rounds = static_cast<double>((tiles * splits + slots - 1) / slots);
+      const double reduce = 3.0 + static_cast<double>(splits) * m * n * 4.0 / 4e6;
+      const double cost = rounds * unit + reduce;
+      if (p.splits == 0 || cost < best) {
+        best = cost;
+        p.splits = static_cast<int>(splits);
+        p.tile = tile;
+      }
+    }
+  }
   return p;
 }
 
@@ -214,22 +237,29 @@ static int launch_splitk(const GemmArgs& g, const SplitKPlan& plan, int trans_a,
   part.c = workspace;
   part.bias = nullptr;
   part.residual = nullptr;
-  part.k = plan.k_chunk;
   part.ldc = g.n;
   part.stride_c = g.m * g.n;
-  part.stride_a = trans_a ? plan.k_chunk * g.lda : plan.k_chunk;
-  part.stride_b = trans_b ? plan.k_chunk : plan.k_chunk * g.ldb;
+  part.stride_a = 0;
+  part.stride_b = 0;
+  part.splits = plan.splits;
   int rc;
-  if (trans_a)
+  if (plan.tile == 256) {
+    if (trans_a)
+      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, true, true>(part, plan.splits, stream);
+    else if (trans_b)
+      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, true, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+    else
+      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+  } else if (trans_a) {
     rc = launch_ring<T, 128, 128, 32, 2, 2, 4, false, TMB_EPI_NONE, true, true>(part, plan.splits, stream);
-  else if (trans_b)
+  } else if (trans_b) {
     rc = launch_ring<T, 128, 128, 32, 2, 2, 4, true, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
-  else
+  } else {
     rc = launch_ring<T, 128, 128, 32, 2, 2, 4, false, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+  }
   if (rc != 0) return rc;
-  const int64_t total = g.m * g.n;
-  splitk_reduce_kernel<T, EPI><<<dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream>>>(
-      static_cast<T*>(g.c), workspace, static_cast<const T*>(g.bias), g.m, g.n, g.ldc, plan.splits);
+  launch_splitk_reduce<T, EPI>(static_cast<T*>(g.c), workspace, static_cast<const T*>(g.bias), g.m,
+                               g.n, g.ldc, plan.splits, stream);
   return check_launch();
 }
 
@@ -237,7 +267,7 @@ static int launch_splitk(const GemmArgs& g, const SplitKPlan& plan, int trans_a,
 // with a few hundred K already takes tens of microseconds and the split pays from much shorter K.
 // Chunks are whole 16-byte groups of K so that every chunk keeps the operands' alignment.
 static SplitKPlan splitk_plan_f32(int64_t batch, int64_t m, int64_t n, int64_t k) {
-  SplitKPlan p{0, 0};
+  SplitKPlan p{0, 0, 0};
   if (batch != 1 || k < 128 || m < 1 || n < 1) return p;
   const int64_t tiles = ((m + kF32BM - 1) / kF32BM) * ((n + kF32BN - 1) / kF32BN);
   if (tiles >= 256) return p;
@@ -247,6 +277,7 @@ static SplitKPlan splitk_plan_f32(int64_t batch, int64_t m, int64_t n, int64_t k
   while (splits >= 2 && k % (splits * 4) != 0) --splits;
   if (splits < 2) return p;
   p.splits = static_cast<int>(splits);
+  p.tile = 128;
   p.k_chunk = k / splits;
   return p;
 }
@@ -264,10 +295,9 @@ static int launch_splitk_f32(const GemmArgs& g, const SplitKPlan& plan, int tran
   part.stride_b = trans_b ? plan.k_chunk : plan.k_chunk * g.ldb;
   const int rc = launch_f32_mfma<TMB_EPI_NONE>(part, plan.splits, trans_a, trans_b, stream);
   if (rc != 0) return rc;
-  const int64_t total = g.m * g.n;
-  splitk_reduce_kernel<float, EPI><<<dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream>>>(
-      static_cast<float*>(g.c), workspace, static_cast<const float*>(g.bias), g.m, g.n, g.ldc,
-      plan.splits);
+  launch_splitk_reduce<float, EPI>(static_cast<float*>(g.c), workspace,
+                                   static_cast<const float*>(g.bias), g.m, g.n, g.ldc, plan.splits,
+                                   stream);
   return check_launch();
 }
 

@@ -83,6 +83,9 @@ struct GemmArgs {
   // persistent kernels with a streamed output: workgroups start in four phases this many 10 ns
   // ticks apart, so that their store bursts do not all hit memory at the same moment
   int stagger_ticks = 0;
+  // fp32-partial launches (split-K): blockIdx.y is the split; split z of `splits` multiplies the
+  // K stages [stages * z / splits, stages * (z + 1) / splits) and stores partial z (0: not split)
+  int splits = 0;
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
@@ -331,19 +334,51 @@ __device__ __forceinline__ void store_wave_tile_f32(f32x16_t (&acc)[TM][TN], flo
 }
 
 // c[m, n] = epilogue(sum over the splits (in order) of partial[s][m][n] + bias[n]), one cast.
-template <typename T, int EPI>
+// VEC = 4: four consecutive columns per thread (n % 4 == 0 keeps them in one row).
+template <typename T, int EPI, int VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(T* __restrict__ c,
                                                             const float* __restrict__ partial,
                                                             const T* __restrict__ bias, int64_t m,
                                                             int64_t n, int64_t ldc, int splits) {
   const int64_t total = m * n;
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
   if (i >= total) return;
-  float sum = partial[i];
-  for (int s = 1; s < splits; ++s) sum += partial[s * total + i];
+  float sum[VEC];
+  if constexpr (VEC == 4) {
+    typedef float f32x4_aligned_t __attribute__((ext_vector_type(4)));
+    f32x4_aligned_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_aligned_t*>(partial + i));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[e] = v[e];
+    for (int s = 1; s < splits; ++s) {
+      v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_aligned_t*>(partial + s * total + i));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum[e] += v[e];
+    }
+  } else {
+    sum[0] = partial[i];
+    for (int s = 1; s < splits; ++s) sum[0] += partial[s * total + i];
+  }
   const int64_t row = i / n, col = i - row * n;
-  if (bias != nullptr) sum += to_f32(bias[col]);
-  c[row * ldc + col] = finish<T, EPI>(sum);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    if (bias != nullptr) sum[e] += to_f32(bias[col + e]);
+    c[row * ldc + col + e] = finish<T, EPI>(sum[e]);
+  }
+}
+
+// Launches the reduction over `splits` partials (workspace is 16-byte aligned or the scalar form runs).
+template <typename T, int EPI>
+static inline void launch_splitk_reduce(T* c, const float* partial, const T* bias, int64_t m,
+                                        int64_t n, int64_t ldc, int splits, hipStream_t stream) {
+  const int64_t total = m * n;
+  if (n % 4 == 0 && (reinterpret_cast<uintptr_t>(partial) & 15) == 0) {
+    const int64_t threads = total / 4;
+    splitk_reduce_kernel<T, EPI, 4><<<dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream>>>(
+        c, partial, bias, m, n, ldc, splits);
+  } else {
+    splitk_reduce_kernel<T, EPI, 1><<<dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream>>>(
+        c, partial, bias, m, n, ldc, splits);
+  }
 }
 
 // B_KMAJOR: B is stored [N, K] (ldb = pitch of an N-row); otherwise [K, N].

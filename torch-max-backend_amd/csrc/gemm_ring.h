@@ -303,7 +303,15 @@ void gemm_ring_kernel(GemmArgs g) {
   };
 
   // The launcher guarantees k % BK == 0 and at least R-1 stages of k.
-  const int64_t k_tiles = g.k / BK;
+  int64_t k_tiles = g.k / BK;
+  if constexpr (OUT_F32) {
+    if (g.splits > 0) {
+      const int64_t first = k_tiles * batch / g.splits, last = k_tiles * (batch + 1) / g.splits;
+      a_base += first * BK * a_kstep;
+      b_base += first * BK * b_kstep;
+      k_tiles = last - first;
+    }
+  }
   // Persistent workgroups: the grid covers the CUs once and each workgroup walks the tile list
   // with the grid's stride, which hands every XCD the same sequence of tiles as one launch per
   // tile would. The stores of a tile drain while the next tile's operands are already being
@@ -419,9 +427,11 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   int64_t resident = static_cast<int64_t>(compute_units()) * kWgPerCu / batch;
   resident = resident / 8 * 8;
   if (resident < 8) resident = 8;
-  const int64_t grid_x = (!kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R> || tiles < resident)
-                             ? tiles
-                             : resident;
+  // (a launch whose workgroups all fit the device at once gets one workgroup per tile)
+  const bool fits = tiles * batch <= static_cast<int64_t>(compute_units()) * kWgPerCu;
+  const int64_t grid_x =
+      (!kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R> || tiles < resident || fits) ? tiles
+                                                                                       : resident;
   // four start phases 5 us apart when every workgroup walks several tiles of a streamed output
   g.stagger_ticks = (g.stream_c && !OUT_F32 && grid_x == resident && tiles >= 4 * resident) ? 500 : 0;
   gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR, OUT_F32>
