@@ -6,7 +6,9 @@
 // spent on the operands. K is walked in stages of BK (32 or 64); R stages form a ring in LDS
 // and up to R-1 of them are in flight while one is multiplied. Each wave waits only for its own
 // loads of the stage needed next (s_waitcnt vmcnt(N) with N = the loads of the younger
-// stages), then one s_barrier makes every wave's part of that stage visible.
+// stages), then one s_barrier makes every wave's part of that stage visible. The 256 x 256 x 64
+// tile, whose two whole stages would fill 128 KB, keeps two buffers for A and three for B instead
+// (160 KB): B is requested two stages ahead, so only half of a stage has to land within one step.
 //
 // LDS stage layout of a K-major operand: one line of BK*2 bytes per matrix row, its 16-byte
 // chunks XOR-swizzled (ring_swizzle): a ds_read_b128 is served sixteen lanes at a time from 64
@@ -98,11 +100,17 @@ void gemm_ring_kernel(GemmArgs g) {
   constexpr int A_GROUPS = A_BYTES / 1024 / NW, B_GROUPS = B_BYTES / 1024 / NW;  // loads per wave
   constexpr int PER_STAGE = A_GROUPS + B_GROUPS;
   static_assert(BK == 32 || BK == 64, "a stage is 32 or 64 deep");
-  static_assert(R >= 2 && R * STAGE_BYTES <= 160 * 1024, "ring does not fit the 160 KB LDS");
+  // The 256 x 256 x 64 tile fills 128 KB with two whole stages, which leaves a stage's loads less
+  // than one step to arrive. Its ring is therefore split: two buffers for A (requested one stage
+  // ahead) and three for B (two stages ahead), 160 KB in all. Halving the burst that has to land
+  // within one step is worth 3-9 % at K = 8192 and nothing at short K.
+  constexpr bool SPLIT_RING = (R == 2 && BM == 256 && BN == 256 && BK == 64);
+  constexpr int RING_BYTES = SPLIT_RING ? 2 * A_BYTES + 3 * B_BYTES : R * STAGE_BYTES;
+  static_assert(R >= 2 && RING_BYTES <= 160 * 1024, "ring does not fit the 160 KB LDS");
   static_assert(A_GROUPS >= 1 && B_GROUPS >= 1 && A_BYTES % (1024 * NW) == 0 &&
                     B_BYTES % (1024 * NW) == 0,
                 "tile does not split into whole 1 KiB loads per wave");
-  __shared__ __attribute__((aligned(1024))) unsigned char ring[R * STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[RING_BYTES];
 
   // All workgroups of a persistent launch finish their tiles at the same time; with an output
   // that streams to memory their store bursts then collide while the matrix pipes idle. A start
@@ -186,13 +194,19 @@ void gemm_ring_kernel(GemmArgs g) {
                  : "s"(m0), "v"(voff), "s"(sbase)
                  : "memory");
   };
-  auto fetch_stage = [&](uint32_t stage_off, int64_t k0) {
+  auto fetch_a = [&](uint32_t off, int64_t k0) {
     const unsigned char* ak = a_base + k0 * a_kstep;
+#pragma unroll
+    for (int j = 0; j < A_GROUPS; ++j) dma16(a_m0 + off + j * 1024, a_off[j], ak);
+  };
+  auto fetch_b = [&](uint32_t off, int64_t k0) {
     const unsigned char* bk = b_base + k0 * b_kstep;
 #pragma unroll
-    for (int j = 0; j < A_GROUPS; ++j) dma16(a_m0 + stage_off + j * 1024, a_off[j], ak);
-#pragma unroll
-    for (int j = 0; j < B_GROUPS; ++j) dma16(b_m0 + stage_off + j * 1024, b_off[j], bk);
+    for (int j = 0; j < B_GROUPS; ++j) dma16(b_m0 + off + j * 1024, b_off[j], bk);
+  };
+  auto fetch_stage = [&](uint32_t stage_off, int64_t k0) {
+    fetch_a(stage_off, k0);
+    fetch_b(stage_off, k0);
   };
 
   f32x16_t acc[TM][TN];
@@ -235,8 +249,11 @@ void gemm_ring_kernel(GemmArgs g) {
   typedef __attribute__((address_space(3))) u32x4_t lds_u32x4_t;
   u32x4_t af[2][TM], bf[2][TN];
   // ks is a compile-time constant at every call site (the k-step loop is unrolled).
-  auto load_frags = [&](uint32_t stage_off, int ks, int s) {
-    lds_u8* stage = (lds_u8*)ring + stage_off;
+  // (a_stage_off, b_stage_off): where the stage's A and B parts start; b_lane / bt_lane and b_m0
+  // already carry the A_BYTES that separate the two inside a whole stage
+  auto load_frags2 = [&](uint32_t a_stage_off, uint32_t b_stage_off, int ks, int s) {
+    lds_u8* stage = (lds_u8*)ring + a_stage_off;
+    lds_u8* stage_b = (lds_u8*)ring + b_stage_off;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       if constexpr (!A_MMAJOR) {
@@ -253,9 +270,9 @@ void gemm_ring_kernel(GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if constexpr (B_KMAJOR) {
-        bf[s][j] = *(const lds_u32x4_t*)(stage + b_lane[ks] + j * (32 * LINE));
+        bf[s][j] = *(const lds_u32x4_t*)(stage_b + b_lane[ks] + j * (32 * LINE));
       } else {
-        lds_u8* src = stage + bt_lane[j] + ks * 16 * (BN * 2);
+        lds_u8* src = stage_b + bt_lane[j] + ks * 16 * (BN * 2);
         const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
         const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src + 4 * (BN * 2)));
         typedef short i16x8_t __attribute__((ext_vector_type(8)));
@@ -263,6 +280,9 @@ void gemm_ring_kernel(GemmArgs g) {
         bf[s][j] = __builtin_bit_cast(u32x4_t, both);
       }
     }
+  };
+  auto load_frags = [&](uint32_t stage_off, int ks, int s) {
+    load_frags2(stage_off, stage_off, ks, s);
   };
   auto mfma_step = [&](int s) {
 #pragma unroll
@@ -331,6 +351,57 @@ void gemm_ring_kernel(GemmArgs g) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
   }
+  if constexpr (SPLIT_RING) {
+    // A buffer i at i * A_BYTES, B buffer j at 2 * A_BYTES + j * B_BYTES (offsets below leave out
+    // the A_BYTES that b_m0 / b_lane carry). Step t requests A of stage t+1 into the buffer of
+    // stage t-1 and B of stage t+2 into the buffer of stage t-1; both were released by the
+    // barrier of step t-1. The launcher guarantees at least two stages of k.
+    constexpr uint32_t B0 = A_BYTES;
+    auto a_next = [](uint32_t o) { return o == 0 ? static_cast<uint32_t>(A_BYTES) : 0u; };
+    auto b_next = [](uint32_t o) {
+      return o + B_BYTES == B0 + 3 * B_BYTES ? B0 : o + static_cast<uint32_t>(B_BYTES);
+    };
+    fetch_a(0, 0);
+    fetch_b(B0, 0);
+    fetch_b(B0 + B_BYTES, BK);
+    wait_vm_lgkm0<B_GROUPS>();
+    __builtin_amdgcn_s_barrier();
+    load_frags2(0, B0, 0, 0);
+    uint32_t a_cur = 0, b_cur = B0;
+    auto split_step = [&](int64_t t, auto issue_b_tag) {
+      constexpr bool ISSUE_B = decltype(issue_b_tag)::value;
+      const uint32_t a_n = a_next(a_cur), b_n = b_next(b_cur);
+      fetch_a(a_n, (t + 1) * BK);
+      if constexpr (ISSUE_B) fetch_b(b_next(b_n), (t + 2) * BK);
+      static_for<KSTEPS - 1>([&](auto ks_tag) {
+        constexpr int ks = decltype(ks_tag)::value;
+        load_frags2(a_cur, b_cur, ks + 1, (ks + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step(ks & 1);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // A of the next stage is older than B of the one after it: only the latter may be pending
+      wait_vm_lgkm0<ISSUE_B ? B_GROUPS : 0>();
+      __builtin_amdgcn_s_barrier();
+      load_frags2(a_n, b_n, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step((KSTEPS - 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      a_cur = a_n;
+      b_cur = b_n;
+    };
+#pragma unroll 1
+    for (int64_t t = 0; t + 2 < k_tiles; ++t) split_step(t, std::true_type{});
+    split_step(k_tiles - 2, std::false_type{});
+    static_for<KSTEPS - 1>([&](auto ks_tag) {
+      constexpr int ks = decltype(ks_tag)::value;
+      load_frags2(a_cur, b_cur, ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step(ks & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    mfma_step((KSTEPS - 1) & 1);
+  } else {
   {
     uint32_t off = 0;
 #pragma unroll
@@ -367,6 +438,7 @@ void gemm_ring_kernel(GemmArgs g) {
     __builtin_amdgcn_sched_barrier(0);
   });
   mfma_step((KSTEPS - 1) & 1);
+  }  // whole-stage ring
 
   if constexpr (OUT_F32) {
     float* P = static_cast<float*>(g.c) + batch * g.stride_c;
@@ -375,7 +447,7 @@ void gemm_ring_kernel(GemmArgs g) {
   }
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
   __syncthreads();  // every wave is done with the ring: reuse it for the output
-  static_assert(NW * BandLayout<WN>::BYTES <= R * STAGE_BYTES, "band staging");
+  static_assert(NW * BandLayout<WN>::BYTES <= RING_BYTES, "band staging");
   lds_byte_t* band = (lds_byte_t*)ring + wave * BandLayout<WN>::BYTES;
   const T* resid = g.residual == nullptr
                        ? nullptr
