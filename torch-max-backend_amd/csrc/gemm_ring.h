@@ -182,17 +182,26 @@ void gemm_ring_kernel(GemmArgs g) {
   // through the compiler's own builtin, every later LDS wait in the loop degrades to
   // lgkmcnt(0) (it orders the DMA against all LDS traffic), which stalls each MFMA group on
   // loads issued for the next one. The compiler does not see these loads at all, so the
-  // vmcnt waits below are placed by hand.
+  // vmcnt waits below are placed by hand. In the 256 x 256 x 64
+  // kernel sc1 (agent scope) makes the load skip the per-CU cache, which these once-read lines
+  // only pass through: 2-8 % at K = 8192; the smaller tiles measured 2-8 % slower with it.
   typedef __attribute__((address_space(3))) unsigned char lds_u8;
   const uint32_t ring_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_u8*)ring));
   const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t a_m0 = ring_lds + wave_s * (A_GROUPS * 1024);
   const uint32_t b_m0 = ring_lds + A_BYTES + wave_s * (B_GROUPS * 1024);
   auto dma16 = [](uint32_t m0, uint32_t voff, const unsigned char* sbase) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(m0), "v"(voff), "s"(sbase)
-                 : "memory");
+    if constexpr (SPLIT_RING) {
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
+                   :
+                   : "s"(m0), "v"(voff), "s"(sbase)
+                   : "memory");
+    } else {
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(m0), "v"(voff), "s"(sbase)
+                   : "memory");
+    }
   };
   auto fetch_a = [&](uint32_t off, int64_t k0) {
     const unsigned char* ak = a_base + k0 * a_kstep;
@@ -371,11 +380,22 @@ void gemm_ring_kernel(GemmArgs g) {
     auto split_step = [&](int64_t t, auto issue_b_tag) {
       constexpr bool ISSUE_B = decltype(issue_b_tag)::value;
       const uint32_t a_n = a_next(a_cur), b_n = b_next(b_cur);
+      // A (needed at the end of this step) is requested at once, B (needed a step later) one
+      // load per k-step, which keeps the request queue shorter (1-2 %)
       fetch_a(a_n, (t + 1) * BK);
-      if constexpr (ISSUE_B) fetch_b(b_next(b_n), (t + 2) * BK);
+      const uint32_t b_t = b_next(b_n);
+      const unsigned char* bk2 = b_base + (t + 2) * BK * b_kstep;
+      if constexpr (ISSUE_B) {
+        dma16(b_m0 + b_t, b_off[0], bk2);
+#pragma unroll
+        for (int j = KSTEPS; j < B_GROUPS; ++j) dma16(b_m0 + b_t + j * 1024, b_off[j], bk2);
+      }
       static_for<KSTEPS - 1>([&](auto ks_tag) {
         constexpr int ks = decltype(ks_tag)::value;
         load_frags2(a_cur, b_cur, ks + 1, (ks + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (ISSUE_B && ks + 1 < B_GROUPS && ks + 1 < KSTEPS)
+          dma16(b_m0 + b_t + (ks + 1) * 1024, b_off[ks + 1], bk2);
         __builtin_amdgcn_sched_barrier(0);
         mfma_step(ks & 1);
         __builtin_amdgcn_sched_barrier(0);
