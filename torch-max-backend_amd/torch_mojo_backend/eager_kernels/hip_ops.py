@@ -91,6 +91,9 @@ def _matrix_layout(t: torch.Tensor) -> Optional[Tuple[int, int]]:
     return None
 
 
+_GEMM_WS_BYTES: dict = {}
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
          epilogue: int = _ek.EPI_NONE, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``epilogue(a @ b + bias)`` for 2-D operands, or 3-D operands with equal batch sizes.
@@ -133,7 +136,10 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
         return out
     lib = _ek.lib()
     # few output tiles and a long K: the library splits K when it is handed scratch memory
-    ws_bytes = lib.tmb_gemm_workspace_bytes(batch, m, n, k, code_of(a.dtype))
+    key = (batch, m, n, k, a.dtype)
+    ws_bytes = _GEMM_WS_BYTES.get(key)
+    if ws_bytes is None:  # a pure function of the shape: asked once per shape
+        ws_bytes = _GEMM_WS_BYTES[key] = lib.tmb_gemm_workspace_bytes(batch, m, n, k, code_of(a.dtype))
     if residual is not None and ws_bytes:
         # the split kernels have no residual step; the separate add has the same bits
         return gemm(a, b, bias, epilogue) + residual

@@ -229,6 +229,33 @@ def _resolve_overload(op_name: str):
     return getattr(packet, overload or "default")
 
 
+_PLAIN_ARG_TYPES = frozenset((int, float, bool, str, type(None), torch.dtype, torch.memory_format,
+                              torch.layout))
+
+
+def _unwrap_arg(x, owners: list):
+    """Nested / uncommon arguments: lists of tensors, mojo devices."""
+    if isinstance(x, TorchMojoTensor):
+        owners.append(x)
+        return x._holder
+    if isinstance(x, (list, tuple)):
+        return type(x)(_unwrap_arg(y, owners) for y in x)
+    if isinstance(x, torch.device) and x.type == "mojo":
+        return hip_device_of(x)
+    return x
+
+
+def _wrap_result(y, owners: list):
+    if isinstance(y, torch.Tensor):
+        for owner in owners:  # in-place and out= forms hand back one of the inputs
+            if owner._holder is y:
+                return owner
+        return TorchMojoTensor._wrap(y)
+    if isinstance(y, (list, tuple)):
+        return type(y)(_wrap_result(z, owners) for z in y)
+    return y
+
+
 def holder_impl(op_name: str) -> Callable:
     """The op on the HIP holders of its mojo arguments; results are wrapped (an output that is
     one of the inputs' holders — in-place and out= forms — comes back as that input)."""
@@ -238,29 +265,27 @@ def holder_impl(op_name: str) -> Callable:
         nonlocal op
         if op is None:
             op = _resolve_overload(op_name)
-        owners = {}
-
-        def unwrap(x):
-            if isinstance(x, TorchMojoTensor):
-                owners[id(x._holder)] = x
-                return x._holder
-            if isinstance(x, (list, tuple)):
-                return type(x)(unwrap(y) for y in x)
-            if isinstance(x, torch.device) and x.type == "mojo":
-                return hip_device_of(x)
-            return x
-
-        def wrap(y):
-            if isinstance(y, torch.Tensor):
-                owner = owners.get(id(y))
-                return owner if owner is not None else TorchMojoTensor._wrap(y)
-            if isinstance(y, (list, tuple)):
-                return type(y)(wrap(z) for z in y)
-            return y
-
+        owners = []
+        call = []
+        for a in args:  # this loop runs once per cold eager op: plain cases first
+            t = type(a)
+            if t is TorchMojoTensor:
+                owners.append(a)
+                call.append(a._holder)
+            elif t in _PLAIN_ARG_TYPES:
+                call.append(a)
+            else:
+                call.append(_unwrap_arg(a, owners))
         if kwargs:
-            return wrap(op(*[unwrap(a) for a in args], **{k: unwrap(v) for k, v in kwargs.items()}))
-        return wrap(op(*[unwrap(a) for a in args]))
+            out = op(*call, **{k: _unwrap_arg(v, owners) for k, v in kwargs.items()})
+        else:
+            out = op(*call)
+        if type(out) is torch.Tensor:
+            for owner in owners:
+                if owner._holder is out:
+                    return owner
+            return TorchMojoTensor._wrap(out)
+        return _wrap_result(out, owners)
 
     return impl
 

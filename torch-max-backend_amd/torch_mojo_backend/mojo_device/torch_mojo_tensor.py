@@ -2,8 +2,8 @@
 
 Same shape as the reference's class (torch_mojo_backend/mojo_device/torch_mojo_tensor.py:255-588):
 a storage-less ``PrivateUse1`` wrapper subclass whose payload is a ``_holder`` owning the device
-allocation plus layout metadata as plain attributes (``_ptr``, ``_shape``, ``_strides``,
-``_offset``, ``_dtype``, ``_numel``, ``_itemsize``, ``_device``, ``_is_contiguous``). Views share
+allocation plus layout metadata (``_ptr``, ``_shape``, ``_strides``, ``_offset``, ``_dtype``,
+``_numel``, ``_itemsize``, ``_device``, ``_is_contiguous``; read-only properties here). Views share
 the holder's allocation. Here the holder is a PyTorch-ROCm tensor (its caching allocator is
 stream-ordered, the job the reference's ``TensorHolder`` does, op_utils/__init__.mojo:250-263),
 already viewed with this tensor's shape/strides/offset, so kernels take ``_ptr`` directly.
@@ -20,6 +20,15 @@ MAX_RANK = 8  # reference :243
 # register_mojo_devices(); lets __torch_dispatch__ call the implementation directly instead of
 # going through the dispatcher a second time (about a third of the per-op host cost).
 DIRECT_IMPLS: dict = {}
+
+_MOJO_DEVICES: dict = {}
+
+
+def _mojo_device(index: int) -> torch.device:
+    dev = _MOJO_DEVICES.get(index)
+    if dev is None:
+        dev = _MOJO_DEVICES[index] = torch.device("mojo", index)
+    return dev
 
 
 class TorchMojoTensor(torch.Tensor):
@@ -40,23 +49,33 @@ class TorchMojoTensor(torch.Tensor):
     @classmethod
     def _wrap(cls, holder: torch.Tensor) -> "TorchMojoTensor":
         """Adopt a HIP tensor (zero-copy) as a mojo tensor with the same view."""
-        if holder.device.type != "cuda":
-            raise TypeError(f"a mojo tensor is backed by HIP memory, got {holder.device}")
-        if holder.dim() > MAX_RANK:
-            raise NotImplementedError(f"mojo tensors support at most rank {MAX_RANK}, got {holder.dim()}")
+        device = holder.device
+        if device.type != "cuda":
+            raise TypeError(f"a mojo tensor is backed by HIP memory, got {device}")
+        shape = holder.shape
+        if len(shape) > MAX_RANK:
+            raise NotImplementedError(f"mojo tensors support at most rank {MAX_RANK}, got {len(shape)}")
         if holder.requires_grad or holder.grad_fn is not None:
             holder = holder.detach()
         res = torch.Tensor._make_wrapper_subclass(
-            cls, holder.shape, strides=holder.stride(), storage_offset=holder.storage_offset(),
-            dtype=holder.dtype, layout=torch.strided,
-            device=torch.device("mojo", holder.device.index or 0), requires_grad=False)
-        # one dictionary update instead of ten attribute stores: this runs once per eager op
-        res.__dict__.update(
-            _holder=holder, _ptr=holder.data_ptr(), _shape=tuple(holder.shape),
-            _strides=tuple(holder.stride()), _offset=holder.storage_offset(), _dtype=holder.dtype,
-            _itemsize=holder.element_size(), _numel=holder.numel(), _device=holder.device,
-            _is_contiguous=holder.is_contiguous())
+            cls, shape, strides=holder.stride(), storage_offset=holder.storage_offset(),
+            dtype=holder.dtype, layout=torch.strided, device=_mojo_device(device.index or 0),
+            requires_grad=False)
+        # This runs once per eager op: only the holder is stored, the layout attributes below
+        # are read from it when an implementation asks for them.
+        res._holder = holder
         return res
+
+    # Layout metadata of the reference's class (:255-337), derived from the holder.
+    _ptr = property(lambda self: self._holder.data_ptr())
+    _shape = property(lambda self: tuple(self._holder.shape))
+    _strides = property(lambda self: tuple(self._holder.stride()))
+    _offset = property(lambda self: self._holder.storage_offset())
+    _dtype = property(lambda self: self._holder.dtype)
+    _itemsize = property(lambda self: self._holder.element_size())
+    _numel = property(lambda self: self._holder.numel())
+    _device = property(lambda self: self._holder.device)
+    _is_contiguous = property(lambda self: self._holder.is_contiguous())
 
     @classmethod
     def _alloc(cls, shape, dtype: torch.dtype, device) -> "TorchMojoTensor":
