@@ -182,6 +182,15 @@ int tmb_attention_decode(void* out, const void* q, const void* k, const void* v,
                          const int64_t* mask_strides, float scale, int causal, int dtype,
                          void* stream);
 
+/* Embedding lookup: out[i, :] = table[indices[i], :] for a contiguous [num_rows, row_len] table of
+ * type `dtype` and `num_indices` contiguous indices of type `index_dtype` (TMB_I64 or TMB_I32).
+ * Replaces `Gather0(out, table, indices, idx_dtype, num_indices, row_len, dtype, ctx)`
+ * (eager_kernels/nn_ops.mojo:1153-1176, 3098-3099; called from aten_fast.py:5336-5371) and
+ * `aten_embedding` (aten_functions.py:1780-1795). An index outside [0, num_rows) reads the
+ * nearest valid row instead of memory outside the table (the reference leaves it undefined). */
+int tmb_gather_rows(void* out, const void* table, const void* indices, int64_t num_indices,
+                    int64_t row_len, int64_t num_rows, int dtype, int index_dtype, void* stream);
+
 /* Elementwise GELU over `numel` contiguous elements, fp32 inside, one cast.
  * `approximate_tanh` != 0 selects the tanh form. Replaces activation_forward_kernels.mojo:22-56
  * (used when the GELU cannot be fused into the producing GEMM's epilogue). */

@@ -77,6 +77,8 @@ def lib() -> ctypes.CDLL:
         L.orc_argmax.argtypes = [vp, vp, i64, i64, ci]
         L.orc_gelu.argtypes = [vp, vp, i64, ci, ci]
         L.orc_gelu_backward.argtypes = [vp, vp, vp, i64, ci, ci]
+        L.orc_gather_rows.argtypes = [vp, vp, vp, i64, i64, i64, ci, ci]
+        L.orc_gather_rows.restype = ci
         L.orc_softmax_backward.argtypes = [vp, vp, vp, i64, i64, ci, ci]
         L.orc_layer_norm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, vp]
         for f in (L.orc_gelu_backward, L.orc_softmax_backward, L.orc_layer_norm_backward):
@@ -237,6 +239,18 @@ def gelu(x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
     if x.numel():
         _check(lib().orc_gelu(out.data_ptr(), x.data_ptr(), x.numel(), _code(x.dtype),
                               int(approximate == "tanh")), "gelu")
+    return out
+
+
+def embedding(table: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    """``table[indices]`` (reference: nn_ops.mojo:1153-1176 through aten_fast.py:5336-5371)."""
+    table, indices = _cpu(table).contiguous(), _cpu(indices).contiguous()
+    out = torch.empty(tuple(indices.shape) + (table.shape[1],), dtype=table.dtype)
+    if out.numel():
+        _check(lib().orc_gather_rows(out.data_ptr(), table.data_ptr(), indices.data_ptr(),
+                                     indices.numel(), table.shape[1], table.shape[0],
+                                     _code(table.dtype), 3 if indices.dtype == torch.int64 else 4),
+               "embedding")
     return out
 
 

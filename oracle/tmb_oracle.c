@@ -24,6 +24,8 @@
  *                   reference's scan only keeps a NaN that sits at index 0.
  *   orc_gelu        activation_forward_kernels.mojo:22-56 (fp32 inside, one cast)
  *   orc_gelu_backward       activation_backward_ops.mojo:50-73 (`_exact_grad`, `_tanh_grad`)
+ *   orc_gather_rows         nn_ops.mojo:1153-1176 (`_gather0`: out[i] = table[idx[i / row_len] *
+ *                           row_len + i % row_len]); out-of-range indices read the nearest row
  *   orc_softmax_backward    ../aten_functions.py:788-833 (grad - exp(out) * sum(grad)) and its
  *                           softmax twin out * (grad - sum(grad * out))
  *   orc_layer_norm_backward aten_fast.py:2797-2913 (LayerNormBackwardF32: grad_input from the
@@ -421,4 +423,22 @@ void orc_convert_to_f32(float* out, const void* in, int64_t n, int dtype) {
 }
 void orc_convert_from_f32(void* out, const float* in, int64_t n, int dtype) {
   for (int64_t i = 0; i < n; ++i) store_f(out, i, dtype, in[i]);
+}
+
+/* Element-by-element restatement of the reference's flat gather loop. index_dtype: 3 = int64,
+ * 4 = int32. */
+int orc_gather_rows(void* out, const void* table, const void* indices, int64_t num_indices,
+                    int64_t row_len, int64_t num_rows, int dtype, int index_dtype) {
+  const int64_t esize = dtype == 0 ? 4 : 2;
+  if (num_rows <= 0 && num_indices * row_len > 0) return 1;
+  for (int64_t i = 0; i < num_indices * row_len; ++i) {
+    int64_t row = index_dtype == 3 ? ((const int64_t*)indices)[i / row_len]
+                                   : (int64_t)((const int32_t*)indices)[i / row_len];
+    if (row < 0) row = 0;
+    if (row >= num_rows) row = num_rows - 1;
+    const char* src = (const char*)table + (row * row_len + i % row_len) * esize;
+    char* dst = (char*)out + i * esize;
+    for (int64_t b = 0; b < esize; ++b) dst[b] = src[b];
+  }
+  return 0;
 }

@@ -113,3 +113,70 @@ extern "C" int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* str
       static_cast<const unsigned char*>(in) + nvec * 16, tail);
   return tmb::check_launch();
 }
+
+namespace tmb {
+
+// out[i, :] = table[indices[i], :]: 16-byte chunks when a row is whole chunks and everything is
+// aligned, single elements otherwise. An index outside [0, num_rows) reads row 0 or the last row
+// instead (the reference's kernel and PyTorch's leave that case undefined / trap; a stray read
+// must not fault the device).
+template <typename IDX, typename CHUNK>
+__global__ __launch_bounds__(256) void gather_rows_kernel(CHUNK* __restrict__ out,
+                                                          const CHUNK* __restrict__ table,
+                                                          const IDX* __restrict__ indices,
+                                                          int64_t num_indices, int64_t chunks_per_row,
+                                                          int64_t num_rows) {
+  const int64_t total = num_indices * chunks_per_row;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * 256) {
+    const int64_t r = i / chunks_per_row, c = i - r * chunks_per_row;
+    int64_t row = static_cast<int64_t>(indices[r]);
+    row = row < 0 ? 0 : (row >= num_rows ? num_rows - 1 : row);
+    out[i] = table[row * chunks_per_row + c];
+  }
+}
+
+template <typename IDX>
+static int launch_gather_rows(void* out, const void* table, const void* indices,
+                              int64_t num_indices, int64_t row_bytes, int64_t num_rows,
+                              hipStream_t stream) {
+  const IDX* idx = static_cast<const IDX*>(indices);
+  auto blocks_for = [](int64_t total) {
+    int64_t b = (total + 255) / 256;
+    return static_cast<unsigned>(b > 65536 * 4 ? 65536 * 4 : (b < 1 ? 1 : b));
+  };
+  if (row_bytes % 16 == 0 && aligned16(out) && aligned16(table)) {
+    const int64_t cpr = row_bytes / 16;
+    gather_rows_kernel<IDX, uint4><<<dim3(blocks_for(num_indices * cpr)), dim3(256), 0, stream>>>(
+        static_cast<uint4*>(out), static_cast<const uint4*>(table), idx, num_indices, cpr, num_rows);
+  } else if (row_bytes % 4 == 0) {
+    const int64_t cpr = row_bytes / 4;
+    gather_rows_kernel<IDX, uint32_t><<<dim3(blocks_for(num_indices * cpr)), dim3(256), 0, stream>>>(
+        static_cast<uint32_t*>(out), static_cast<const uint32_t*>(table), idx, num_indices, cpr,
+        num_rows);
+  } else {
+    const int64_t cpr = row_bytes / 2;  // 16-bit elements, odd row length
+    gather_rows_kernel<IDX, uint16_t><<<dim3(blocks_for(num_indices * cpr)), dim3(256), 0, stream>>>(
+        static_cast<uint16_t*>(out), static_cast<const uint16_t*>(table), idx, num_indices, cpr,
+        num_rows);
+  }
+  return check_launch();
+}
+
+}  // namespace tmb
+
+extern "C" int tmb_gather_rows(void* out, const void* table, const void* indices,
+                               int64_t num_indices, int64_t row_len, int64_t num_rows, int dtype,
+                               int index_dtype, void* stream) {
+  if (num_indices < 0 || row_len < 0 || num_rows < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (dtype != TMB_F32 && dtype != TMB_F16 && dtype != TMB_BF16) return TMB_ERR_UNSUPPORTED;
+  if (index_dtype != TMB_I64 && index_dtype != TMB_I32) return TMB_ERR_UNSUPPORTED;
+  if (num_indices == 0 || row_len == 0) return TMB_OK;
+  if (num_rows == 0) return TMB_ERR_INVALID_ARGUMENT;  // nothing to read from
+  if (out == nullptr || table == nullptr || indices == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  const int64_t row_bytes = row_len * (dtype == TMB_F32 ? 4 : 2);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return index_dtype == TMB_I64
+             ? tmb::launch_gather_rows<int64_t>(out, table, indices, num_indices, row_bytes, num_rows, s)
+             : tmb::launch_gather_rows<int32_t>(out, table, indices, num_indices, row_bytes, num_rows, s);
+}

@@ -256,6 +256,16 @@ def aten_argmax(input: torch.Tensor, dim: Optional[int] = None, keepdim: bool = 
     return hip_ops.argmax(input, dim, keepdim)
 
 
+@map_to(aten.embedding)
+def aten_embedding(weight: torch.Tensor, indices: torch.Tensor, padding_idx: int = -1,
+                   scale_grad_by_freq: bool = False, sparse: bool = False) -> torch.Tensor:
+    """reference :1780-1795 (the remaining arguments only matter to the backward)."""
+    if weight.dim() == 2 and weight.dtype in hip_ops.FLOAT_DTYPES and weight.shape[0] > 0 \
+            and indices.dtype in (torch.int32, torch.int64):
+        return hip_ops.embedding(weight, indices)
+    return torch.ops.aten.embedding(weight, indices, padding_idx, scale_grad_by_freq, sparse)
+
+
 @map_to(aten.gelu)
 def aten_gelu(input: torch.Tensor, approximate: str = "none") -> torch.Tensor:
     """reference :2063-2067."""
@@ -373,7 +383,7 @@ _scaled_dot_product_efficient_attention _scaled_dot_product_flash_attention
 _to_copy abs acos add addcdiv addcmul alias amin any arange
 argmin asinh atanh avg_pool2d bitwise_and.Scalar bitwise_and.Tensor bitwise_not bitwise_or.Scalar
 bitwise_or.Tensor bitwise_xor.Scalar bitwise_xor.Tensor cat ceil clamp clone constant_pad_nd
-convolution copy cos cosh cumsum detach div embedding empty.memory_format empty_strided empty_like
+convolution copy cos cosh cumsum detach div empty.memory_format empty_strided empty_like
 empty_permuted eq erf exp expand fill fill_ floor full full_like ge gt index isin
 isnan le lift_fresh_copy log log1p logical_and logical_not logical_xor lt
 max max_pool2d_with_indices maximum mean.out min minimum mul native_batch_norm native_group_norm

@@ -41,6 +41,7 @@ SIGNATURES = {
                                 _flt, _ci, _ci, _ci, _vp]),
     "tmb_attention_decode": (_ci, [_vp] * 5 + [_i64] * 5 + [_vp] * 5 + [_flt, _ci, _ci, _vp]),
     "tmb_gelu": (_ci, [_vp, _vp, _i64, _ci, _ci, _vp]),
+    "tmb_gather_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _vp]),
     "tmb_gelu_backward": (_ci, [_vp, _vp, _vp, _i64, _ci, _ci, _vp]),
     "tmb_softmax_backward_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _ci, _ci, _vp]),
     "tmb_layer_norm_backward_workspace_bytes": (_sz, [_i64, _i64, _ci]),

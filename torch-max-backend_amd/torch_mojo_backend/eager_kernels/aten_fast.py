@@ -349,6 +349,16 @@ def fast_aten_gelu(input, approximate="none"):
     return _wrap(hip_ops.gelu(a._holder, approximate))
 
 
+def fast_aten_embedding(input, weight, padding_idx=-1, scale_grad_by_freq=False, sparse=False):
+    """``input`` is the table and ``weight`` the indices (aten naming, reference :5336-5371)."""
+    table, idx = _t(input), _t(weight)
+    if table is None or idx is None or table._device != idx._device \
+            or table._dtype not in _FLOAT_DTYPES or idx._dtype not in (torch.int32, torch.int64) \
+            or len(table._shape) != 2 or (table._shape[0] == 0 and idx._numel > 0):
+        return NOT_HANDLED
+    return _wrap(hip_ops.embedding(table._holder, idx._holder))
+
+
 # ---------------------------------------------------------------------------
 # Backward twins (reference :1413-1447, :2797-2913, :3237-3330, :4939-5031)
 # ---------------------------------------------------------------------------

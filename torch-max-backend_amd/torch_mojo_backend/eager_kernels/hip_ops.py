@@ -481,6 +481,29 @@ def argmax(x: torch.Tensor, dim: Optional[int], keepdim: bool) -> torch.Tensor:
     return out
 
 
+def embedding(table: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    """``table[indices]`` for a 2-D float table and int32 / int64 indices of any shape
+    (reference: aten_fast.py:5336-5371). Indices outside the table read the nearest valid row."""
+    require_hip(table, indices)
+    if table.dim() != 2 or table.dtype not in FLOAT_DTYPES:
+        raise TypeError(f"embedding: table must be a 2-D float tensor, got {tuple(table.shape)} {table.dtype}")
+    if indices.dtype not in (torch.int64, torch.int32):
+        raise TypeError(f"embedding: indices must be int32 or int64, got {indices.dtype}")
+    rows, row_len = table.shape
+    out = torch.empty(tuple(indices.shape) + (row_len,), dtype=table.dtype, device=table.device)
+    if out.numel() == 0:
+        return out
+    if rows == 0:
+        raise IndexError("embedding: lookup in an empty table")
+    t = table if table.is_contiguous() else table.contiguous()
+    i = indices if indices.is_contiguous() else indices.contiguous()
+    rc = _ek.lib().tmb_gather_rows(out.data_ptr(), t.data_ptr(), i.data_ptr(), i.numel(), row_len,
+                                   rows, code_of(table.dtype),
+                                   _ek.I64 if indices.dtype == torch.int64 else _ek.I32, _stream())
+    _check("tmb_gather_rows", rc)
+    return out
+
+
 def gelu(x: torch.Tensor, approximate: str = "none") -> torch.Tensor:
     require_hip(x)
     if x.dtype not in FLOAT_DTYPES:

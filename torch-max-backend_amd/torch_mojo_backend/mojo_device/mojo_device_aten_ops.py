@@ -119,6 +119,7 @@ _register_fast("aten::amax", "fast_aten_amax")
 _register_fast("aten::argmax", "fast_aten_argmax")
 _register_fast("aten::bmm", "fast_aten_bmm")
 _register_fast("aten::gelu", "fast_aten_gelu")
+_register_fast("aten::embedding", "fast_aten_embedding")
 _register_fast("aten::linear", "fast_aten_linear")
 _register_fast("aten::mean", "fast_aten_mean")
 _register_fast("aten::mean.dim", "fast_aten_mean")
@@ -308,7 +309,7 @@ _HOLDER_OPS = (
     "aten::max", "aten::max.dim", "aten::min", "aten::cumsum", "aten::topk", "aten::sort",
     "aten::multinomial",
     # indexing, gathering, concatenation
-    "aten::embedding", "aten::index_select", "aten::gather", "aten::index.Tensor",
+    "aten::index_select", "aten::gather", "aten::index.Tensor",
     "aten::index_put_", "aten::cat", "aten::stack", "aten::split.Tensor",
     "aten::split_with_sizes", "aten::unbind.int", "aten::squeeze", "aten::flatten.using_ints",
     "aten::tril", "aten::triu", "aten::repeat", "aten::roll",
