@@ -7,7 +7,8 @@ Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] b
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
 W untimed warm-up steps, then exactly K steps between two ``torch.cuda.synchronize()`` calls.
 Defaults are the reference's own protocol (25 warm-ups, 100 timed launches, ``bench_gemm.py``):
-the first ~25 ms after idle run about 6 % slower while the clocks settle.
+the first ~25 ms after idle run about 6 % slower while the clocks settle, so 50 untimed launches
+precede the W warm-up steps whatever W is (``config.preheat_launches``).
 
 The same line carries
   * ``roofline``   — the GEMM kernel against the MI355X dense bf16 MFMA peak (2.5 PFLOP/s):
@@ -138,6 +139,11 @@ def main() -> int:
     b = gen((K, N), 1, torch.bfloat16)
     bias = gen((N,), 2, torch.bfloat16)
     flops = 2.0 * M * N * K
+    # The first ~25 ms after idle run about 6 % slower while the clocks settle: 50 untimed launches
+    # come before the W warm-up steps whatever W is (reported as config.preheat_launches).
+    PREHEAT = 50
+    for _ in range(PREHEAT):
+        hip_ops.gemm(a, b, bias)
     wall_ms, ev_ms = timed(lambda: hip_ops.gemm(a, b, bias), args.steps, args.warmup)
     value = flops / (wall_ms * 1e-3) / 1e12
     achieved = flops / (ev_ms * 1e-3) / 1e12
@@ -546,7 +552,7 @@ def main() -> int:
         "config": {"workload": "standalone op sweep: aten.addmm bf16, (M,N,K)=(8192,8192,8192), "
                                "bias [N], seeded N(0,1) inputs resident in HBM",
                    "device": props.name, "compute_units": props.multi_processor_count,
-                   "host_threads": cpu_threads},
+                   "host_threads": cpu_threads, "preheat_launches": PREHEAT},
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "sweep": sweep,
