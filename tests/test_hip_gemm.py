@@ -445,3 +445,16 @@ def test_fp32_split_k_is_reproducible_and_close_to_the_unsplit_kernel():
     assert rc == 0
     want = as64(a) @ as64(w).T + as64(bias)
     assert rel_frobenius(first, want) <= 2e-6 and rel_frobenius(plain, want) <= 2e-6
+
+
+def test_fp32_mfma_output_larger_than_the_infinity_cache():
+    """8192 x 8200 fp32 = 269 MB: the kernel's streaming-store path. Sampled rows against float64."""
+    m, n, k = 8192, 8200, 64
+    a = _dev(seeded((m, k), seed=61, dtype=torch.float32))
+    w = _dev(seeded((n, k), seed=62, dtype=torch.float32))
+    bias = _dev(seeded((n,), seed=63, dtype=torch.float32))
+    got = _ops().gemm(a, w.t(), bias)
+    rows = torch.tensor([0, 1, 127, 128, 4095, 4096, 8190, 8191], device="cuda")
+    want = as64(a[rows]) @ as64(w).T + as64(bias)
+    assert rel_frobenius(got[rows], want) <= 2e-6
+    assert torch.isfinite(got).all()
