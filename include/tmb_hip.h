@@ -35,7 +35,8 @@ typedef enum tmb_status {
   TMB_OK = 0,
   TMB_ERR_INVALID_ARGUMENT = -1, /* null pointer, negative size, unknown enum */
   TMB_ERR_UNSUPPORTED = -2,      /* well-formed request this build has no kernel for */
-  TMB_ERR_WORKSPACE = -3         /* workspace missing or too small */
+  TMB_ERR_WORKSPACE = -3,        /* workspace missing or too small */
+  TMB_ERR_SCRATCH_LIMIT = -4     /* shape needs more scratch than the library's static array holds */
 } tmb_status;
 
 typedef enum tmb_reduce_op { TMB_SUM = 0, TMB_MEAN = 1, TMB_AMAX = 2 } tmb_reduce_op;
@@ -93,6 +94,24 @@ size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dtype);
  * (`_mean_rows`) behind SumSpec/MeanSpec/AmaxSpec (reduction_ops.mojo:1094-1184). */
 int tmb_reduce_rows(void* out, const void* in, int64_t rows, int64_t cols, int op, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* tmb_reduce_rows for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same kernels, same partition and
+ * therefore the same bits, but the partials of a split reduction go to a static array of
+ * TMB_REDUCE_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
+ * ends) instead of a caller's workspace. Allocates and frees nothing. Shapes whose
+ * tmb_reduce_workspace_bytes exceeds the array are refused with TMB_ERR_SCRATCH_LIMIT before
+ * anything is enqueued (a split reduction has at most rows + 8192 partials of 16 bytes, and only
+ * for rows < 4096, so every shape that fits the device's memory fits). The first call on a device
+ * looks the array's address up (hipGetSymbolAddress); make that call outside graph capture.
+ * All calls on one GPU share the array: calls that overlap there (two streams, two threads)
+ * race; calls on one stream are ordered and safe. Nothing in it needs clearing between calls:
+ * the first stage writes every partial the second stage reads.
+ * No counterpart in the reference, whose spec ops allocate their scratch inside the call
+ * (op_utils/__init__.mojo:389-447). */
+#define TMB_REDUCE_STATIC_SCRATCH_BYTES (256 * 1024)
+int tmb_reduce_rows_static(void* out, const void* in, int64_t rows, int64_t cols, int op,
+                           int dtype, void* stream);
 
 /* First-occurrence argmax of every row of [rows, cols] to int64 [rows]; NaN counts as the
  * maximum (first NaN wins), otherwise greater value wins and equal values keep the lower index

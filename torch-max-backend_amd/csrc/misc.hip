@@ -78,6 +78,7 @@ extern "C" const char* tmb_status_string(int code) {
     case TMB_ERR_INVALID_ARGUMENT: return "invalid argument";
     case TMB_ERR_UNSUPPORTED: return "unsupported dtype/shape for this build";
     case TMB_ERR_WORKSPACE: return "workspace missing or too small";
+    case TMB_ERR_SCRATCH_LIMIT: return "shape needs more scratch than the library's static array holds";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

@@ -13,7 +13,16 @@
 // every combine step.
 #include "tmb_common.h"
 
+#include <mutex>
+
 namespace tmb {
+
+// Scratch of the entry point that allocates nothing (tmb_reduce_rows_static): the partials of a
+// split reduction live in this array instead of a caller's workspace. Every GPU the library runs
+// on holds its own copy until the process ends. In host code the name `scratch` is only a handle
+// for hipGetSymbolAddress; kernels get the per-device address that call returns.
+constexpr size_t kStaticScratchBytes = TMB_REDUCE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kRedBlock = 256;
 constexpr int kRedWaves = kRedBlock / kWave;
@@ -557,6 +566,47 @@ extern "C" int tmb_reduce_rows(void* out, const void* in, int64_t rows, int64_t 
     default:
       return TMB_ERR_UNSUPPORTED;
   }
+}
+
+namespace tmb {
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kMaxDevices) return TMB_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return TMB_OK;
+}
+
+}  // namespace tmb
+
+extern "C" int tmb_reduce_rows_static(void* out, const void* in, int64_t rows, int64_t cols, int op,
+                                      int dtype, void* stream) {
+  if (rows < 0 || cols < 0) return TMB_ERR_INVALID_ARGUMENT;
+  const size_t need = tmb_reduce_workspace_bytes(rows, cols, dtype);
+  if (need > tmb::kStaticScratchBytes) return TMB_ERR_SCRATCH_LIMIT;
+  if (need == 0) return tmb_reduce_rows(out, in, rows, cols, op, dtype, nullptr, 0, stream);
+  if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  void* ws = nullptr;
+  const int rc = tmb::static_scratch(&ws);
+  if (rc != TMB_OK) return rc;
+  // Every partial the second stage reads is written by the first stage of the same call, so
+  // nothing in the array has to start at zero.
+  return tmb_reduce_rows(out, in, rows, cols, op, dtype, ws, tmb::kStaticScratchBytes, stream);
 }
 
 extern "C" int tmb_argmax_rows(int64_t* out, const void* in, int64_t rows, int64_t cols,

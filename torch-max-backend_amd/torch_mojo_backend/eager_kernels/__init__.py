@@ -32,6 +32,7 @@ SIGNATURES = {
     "tmb_layer_norm_rows": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _dbl, _ci, _vp]),
     "tmb_reduce_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
+    "tmb_reduce_rows_static": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp]),
     "tmb_argmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_gemm": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp]),
     "tmb_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _ci]),
