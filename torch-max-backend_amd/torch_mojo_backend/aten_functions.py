@@ -221,33 +221,54 @@ def aten_native_layer_norm(input: torch.Tensor, normalized_shape, weight: Option
 _INT_PROMOTE = (torch.bool, torch.uint8, torch.int8, torch.int16, torch.int32)
 
 
+def _reduced_shape(shape, dims, keepdim: bool) -> List[int]:
+    if keepdim:
+        return [1 if d in dims else s for d, s in enumerate(shape)]
+    return [s for d, s in enumerate(shape) if d not in dims]
+
+
 @map_to(aten.sum)
 def aten_sum(input: torch.Tensor, dim=None, keepdim: bool = False, *, dtype=None) -> torch.Tensor:
-    """reference :3311-3346: small integer / bool inputs are summed as int64."""
+    """reference :3311-3346: small integer / bool inputs are summed as int64; an empty reduction
+    is 0 (eager twin: aten_fast.py:3033-3037)."""
     if dtype is not None:
         input = input.to(dtype)
     elif input.dtype in _INT_PROMOTE:
         input = input.to(torch.int64)
     dims = _normalize_dims(dim, input.dim())
     if input.numel() == 0:
-        shape = [1 if d in dims else s for d, s in enumerate(input.shape)] if keepdim else \
-            [s for d, s in enumerate(input.shape) if d not in dims]
-        return torch.zeros(shape, dtype=input.dtype, device=input.device)
+        return torch.zeros(_reduced_shape(input.shape, dims, keepdim), dtype=input.dtype,
+                           device=input.device)
     return hip_ops.reduce(input, dims, keepdim, _ek.SUM)
 
 
 @map_to(aten.mean)
 def aten_mean(input: torch.Tensor, dim=None, keepdim: bool = False, *, dtype=None) -> torch.Tensor:
-    """reference :2556-2590."""
+    """reference :2556-2590. The mean of no elements is NaN (0/0), as in ATen."""
     if dtype is not None:
         input = input.to(dtype)
-    return hip_ops.reduce(input, _normalize_dims(dim, input.dim()), keepdim, _ek.MEAN)
+    if not input.dtype.is_floating_point:
+        raise TypeError(f"mean(): could not infer output dtype. Input dtype must be floating point, "
+                        f"got {input.dtype}")
+    dims = _normalize_dims(dim, input.dim())
+    if input.numel() == 0:
+        return torch.full(_reduced_shape(input.shape, dims, keepdim), float("nan"),
+                          dtype=input.dtype, device=input.device)
+    return hip_ops.reduce(input, dims, keepdim, _ek.MEAN)
 
 
 @map_to(aten.amax)
 def aten_amax(input: torch.Tensor, dim=[], keepdim: bool = False) -> torch.Tensor:
-    """reference :1002-1020."""
-    return hip_ops.reduce(input, _normalize_dims(dim, input.dim()), keepdim, _ek.AMAX)
+    """reference :1002-1020. A maximum over no elements does not exist: ValueError, unless the
+    result itself is empty."""
+    dims = _normalize_dims(dim, input.dim())
+    if input.numel() == 0:
+        if any(input.shape[d] == 0 for d in dims):
+            raise ValueError(f"amax(): expected every reduced dim of {tuple(input.shape)} to have "
+                             f"non-zero size, got dims {dims}")
+        return torch.empty(_reduced_shape(input.shape, dims, keepdim), dtype=input.dtype,
+                           device=input.device)
+    return hip_ops.reduce(input, dims, keepdim, _ek.AMAX)
 
 
 @map_to(aten.argmax)
