@@ -41,10 +41,40 @@ PEAK_BF16_DENSE_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
 PEAK_FP32_MFMA_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 
-# Bytes per launch of the headline GEMM kernel between L2 and the memory side, measured with
-# rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the factors being what the same
-# counters read for tmb_copy_bytes moving 1 GiB: `--only copy`).
-GEMM_TRAFFIC_BYTES = 1.760e9
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "gemm_ring_bf16_addmm_8192_counters.txt")
+
+
+def gemm_counters(path: str = COUNTERS_FILE) -> dict:
+    """What the committed rocprofv3 --pmc summary of the headline says, per launch:
+    ``traffic``: bytes between L2 and the memory side = FETCH_SIZE and WRITE_SIZE of the GEMM
+    kernel, each scaled by what the same counter reads for tmb_copy_bytes moving exactly 1 GiB each
+    way (the calibration lines of the same file); ``active_cycles``: GRBM_GUI_ACTIVE / 8 XCDs.
+    Missing file or line -> the key is absent."""
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return {}
+    reads: dict = {}
+    for ln in lines:
+        if ln.startswith("#") or "(per dispatch" not in ln:
+            continue
+        head = ln.split("(per dispatch")[0].split()
+        if len(head) < 3:
+            continue
+        kernel, counter, value = " ".join(head[:-2]), head[-2], float(head[-1])
+        kind = "copy" if "copy_kernel" in kernel else ("gemm" if "gemm_ring_kernel" in kernel else None)
+        if kind:
+            reads[(kind, counter)] = value
+    out: dict = {}
+    need = [("gemm", "FETCH_SIZE"), ("gemm", "WRITE_SIZE"), ("copy", "FETCH_SIZE"), ("copy", "WRITE_SIZE")]
+    if all(k in reads for k in need):
+        gib_kib = float(1 << 20)
+        kib = reads[("gemm", "FETCH_SIZE")] * (gib_kib / reads[("copy", "FETCH_SIZE")]) + \
+            reads[("gemm", "WRITE_SIZE")] * (gib_kib / reads[("copy", "WRITE_SIZE")])
+        out["traffic"] = round(kib * 1024.0)
+    if ("gemm", "GRBM_GUI_ACTIVE") in reads:
+        out["active_cycles"] = reads[("gemm", "GRBM_GUI_ACTIVE")] / 8.0
+    return out
 
 
 def _parse():
@@ -135,51 +165,64 @@ def main() -> int:
 
     # ------------------------------------------------------------------ GEMM (headline)
     M = N = K = 8192
-    a = gen((M, K), 0, torch.bfloat16)
-    b = gen((K, N), 1, torch.bfloat16)
-    bias = gen((N,), 2, torch.bfloat16)
-    flops = 2.0 * M * N * K
-    # The first ~25 ms after idle run about 6 % slower while the clocks settle: 50 untimed launches
-    # come before the W warm-up steps whatever W is (reported as config.preheat_launches).
     PREHEAT = 50
-    for _ in range(PREHEAT):
-        hip_ops.gemm(a, b, bias)
-    wall_ms, ev_ms = timed(lambda: hip_ops.gemm(a, b, bias), args.steps, args.warmup)
-    value = flops / (wall_ms * 1e-3) / 1e12
-    achieved = flops / (ev_ms * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_DENSE_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
-                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_ring_kernel<bf16,256x256x64,2x4 waves,2 A + 3 B buffers,N-major B>",
-                "launch_ms": round(ev_ms, 4), "algorithmic_flops": flops}
 
-    cpu_baseline = None
-    if not args.no_cpu:
-        import oracle  # the checker, timed here as the reported CPU baseline only
+    def run_headline():
+        a = gen((M, K), 0, torch.bfloat16)
+        b = gen((K, N), 1, torch.bfloat16)
+        bias = gen((N,), 2, torch.bfloat16)
+        flops = 2.0 * M * N * K
+        # The first ~25 ms after idle run about 6 % slower while the clocks settle: 50 untimed launches
+        # come before the W warm-up steps whatever W is (reported as config.preheat_launches).
+        for _ in range(PREHEAT):
+            hip_ops.gemm(a, b, bias)
+        wall_ms, ev_ms = timed(lambda: hip_ops.gemm(a, b, bias), args.steps, args.warmup)
+        value = flops / (wall_ms * 1e-3) / 1e12
+        achieved = flops / (ev_ms * 1e-3) / 1e12
+        counters = gemm_counters()
+        roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_DENSE_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
+                    "traffic": counters.get("traffic"), "kernel": "gemm_ring_kernel<bf16,256x256x64,2x4 waves,2 A + 3 B buffers,N-major B>",
+                    "launch_ms": round(ev_ms, 4), "algorithmic_flops": flops}
+        if "active_cycles" in counters:
+            # the same FLOPs against the cycles the chip was active for in the committed counter
+            # run: 2.5 PFLOP/s is 2.5e15 / 2.4e9 FLOP per cycle at the 2.4 GHz the peak assumes
+            roofline["frac_at_sustained_clock"] = round(
+                flops / (counters["active_cycles"] * (PEAK_BF16_DENSE_TFLOPS * 1e12 / 2.4e9)), 4)
 
-        # bounded sample: the [0:4096, 0:2048] slab of the same product (1/8 of the FLOPs, about
-        # 15 s on 16 host threads)
-        sm, sn = 4096, 2048
-        a_h, b_h, bias_h = a[:sm].cpu(), b[:, :sn].contiguous().cpu(), bias[:sn].cpu()
-        t0 = time.perf_counter()
-        ref = oracle.gemm(a_h, b_h, bias_h).float()  # one run: timed and kept as the check below
-        t = time.perf_counter() - t0
-        cpu_baseline = {"value": round(2.0 * sm * sn * K / t / 1e12, 5), "unit": "TFLOP/s",
-                        "cores": cpu_threads, "kind": "port",
-                        "sample": f"C[0:{sm},0:{sn}] slab of the same 8192^3 bf16 addmm (1/8 of "
-                                  f"the work), oracle/tmb_oracle.c orc_gemm, OpenMP over rows, "
-                                  f"{t:.2f} s"}
-        # context: a tuned CPU BLAS on the same slab (PyTorch CPU, fp32 math on bf16-rounded data)
-        a32, b32, bias32 = a_h.float(), b_h.float(), bias_h.float()
-        t_blas = cpu_time(lambda: torch.addmm(bias32, a32, b32), iters=3, warmup=1)
-        cpu_baseline["torch_cpu_fp32_tflops_same_slab"] = round(2.0 * sm * sn * K / t_blas / 1e12, 4)
-        # check the GPU result on that slab against the oracle while we are here
-        got = hip_ops.gemm(a, b, bias)[:sm, :sn].float().cpu()
-        rel = ((got - ref).norm() / ref.norm()).item()
-        cpu_baseline["gpu_vs_oracle_rel_frobenius"] = rel
-        if not rel < 1e-2:
-            print(f"bench: GEMM result deviates from the oracle (rel Frobenius {rel})", file=sys.stderr)
-            return 1
-    del a, b, bias
+        cpu_baseline = None
+        if not args.no_cpu:
+            import oracle  # the checker, timed here as the reported CPU baseline only
+
+            # bounded sample: the [0:4096, 0:2048] slab of the same product (1/8 of the FLOPs, about
+            # 15 s on 16 host threads)
+            sm, sn = 4096, 2048
+            a_h, b_h, bias_h = a[:sm].cpu(), b[:, :sn].contiguous().cpu(), bias[:sn].cpu()
+            t0 = time.perf_counter()
+            ref = oracle.gemm(a_h, b_h, bias_h).float()  # one run: timed and kept as the check below
+            t = time.perf_counter() - t0
+            cpu_baseline = {"value": round(2.0 * sm * sn * K / t / 1e12, 5), "unit": "TFLOP/s",
+                            "cores": cpu_threads, "kind": "port",
+                            "sample": f"C[0:{sm},0:{sn}] slab of the same 8192^3 bf16 addmm (1/8 of "
+                                      f"the work), oracle/tmb_oracle.c orc_gemm, OpenMP over rows, "
+                                      f"{t:.2f} s"}
+            # context: a tuned CPU BLAS on the same slab (PyTorch CPU, fp32 math on bf16-rounded data)
+            a32, b32, bias32 = a_h.float(), b_h.float(), bias_h.float()
+            t_blas = cpu_time(lambda: torch.addmm(bias32, a32, b32), iters=3, warmup=1)
+            cpu_baseline["torch_cpu_fp32_tflops_same_slab"] = round(2.0 * sm * sn * K / t_blas / 1e12, 4)
+            # check the GPU result on that slab against the oracle while we are here
+            got = hip_ops.gemm(a, b, bias)[:sm, :sn].float().cpu()
+            rel = ((got - ref).norm() / ref.norm()).item()
+            cpu_baseline["gpu_vs_oracle_rel_frobenius"] = rel
+            if not rel < 1e-2:
+                print(f"bench: GEMM result deviates from the oracle (rel Frobenius {rel})", file=sys.stderr)
+                raise SystemExit(1)
+        del a, b, bias
+        return value, wall_ms, ev_ms, achieved, roofline, cpu_baseline
+
+    value = wall_ms = ev_ms = achieved = roofline = cpu_baseline = None
+    if want in ("all", "headline", "gemm"):
+        value, wall_ms, ev_ms, achieved, roofline, cpu_baseline = run_headline()
 
     def gemm_row(name, m, n, k, batch=None, trans_b=False, steps=50, dtype=torch.bfloat16):
         if batch:
@@ -191,6 +234,11 @@ def main() -> int:
             w = gen((n, k), 4, dtype).t() if trans_b else gen((k, n), 4, dtype)
             bs = gen((n,), 5, dtype)
         _, ms = timed(lambda: hip_ops.gemm(x, w, bs), steps, 10)
+        # yardstick, not part of the product: PyTorch-ROCm's own library GEMM on the same tensors
+        if batch:
+            _, yard = timed(lambda: torch.bmm(x, w), max(steps // 2, 5), 5)
+        else:
+            _, yard = timed(lambda: torch.addmm(bs, x, w), max(steps // 2, 5), 5)
         bt = batch or 1
         size = x.element_size()
         peak = PEAK_FP32_MFMA_TFLOPS if dtype == torch.float32 else PEAK_BF16_DENSE_TFLOPS
@@ -199,7 +247,8 @@ def main() -> int:
         tf, gbs = fl / ms / 1e9, by / ms / 1e6
         sweep[name] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 2),
                        "frac_mfma": round(tf / peak, 4),
-                       "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+                       "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+                       "pytorch_rocm_us": round(yard * 1e3, 2)}
 
     if want in ("all", "gemm"):
         sweep["addmm_bf16_8192x8192x8192"] = {"us": round(ev_ms * 1e3, 2), "TFLOP/s": round(achieved, 2),
@@ -540,12 +589,12 @@ def main() -> int:
 
     line = {
         "metric": "GEMM TFLOP/s (bf16 addmm M=N=K=8192, fp32 accumulate)",
-        "value": round(value, 2),
+        "value": None if value is None else round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 4),
+        "ms_per_step": None if wall_ms is None else round(wall_ms, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -20,7 +20,7 @@ aten = torch.ops.aten
 
 def test_public_names():
     for name in ("mojo_backend", "MAPPING_TORCH_ATEN_TO_MOJO", "MojoCompilerError",
-                 "get_accelerators", "log_aten_calls"):
+                 "get_accelerators"):
         assert hasattr(torch_mojo_backend, name)
     assert torch_mojo_backend.get_accelerators()[-1] == torch.device("cpu")
 

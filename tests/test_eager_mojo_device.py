@@ -212,3 +212,23 @@ def test_eager_argmax_vocab_planted_max():
     planted = torch.randint(0, 50257, (256,))
     x[torch.arange(256), planted] = 100.0
     assert torch.equal(torch.argmax(x.to("mojo"), dim=-1).cpu(), planted)
+
+
+@gpu
+def test_eager_sdpa_decode_step_takes_the_decode_kernel(monkeypatch):
+    """One query per head, no mask: the eager twin must launch the memory-bound decode kernel, not
+    the 128-query MFMA kernel that also accepts the shapes."""
+    hip_ops = aten_fast.hip_ops
+    decode_calls, fused_calls = [], []
+    real_decode, real_fused = hip_ops.attention_decode, hip_ops.attention
+    monkeypatch.setattr(hip_ops, "attention_decode",
+                        lambda *a, **kw: decode_calls.append(1) or real_decode(*a, **kw))
+    monkeypatch.setattr(hip_ops, "attention", lambda *a, **kw: fused_calls.append(1) or real_fused(*a, **kw))
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(3, 12, 1, 64, generator=g).bfloat16()
+    k = torch.randn(3, 12, 208, 64, generator=g).bfloat16()
+    v = torch.randn(3, 12, 208, 64, generator=g).bfloat16()
+    got = torch.nn.functional.scaled_dot_product_attention(q.to("mojo"), k.to("mojo"), v.to("mojo"))
+    assert len(decode_calls) == 1 and not fused_calls
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    _close(got.float(), want, rtol=2e-2, atol=2e-2)

@@ -283,3 +283,28 @@ def test_sdpa_surfaces_route_decode_shapes_to_the_decode_kernel(monkeypatch):
     assert calls and got.shape == (2, 4, 1, 64)
     want = _sdpa64(q.cpu(), k.cpu(), v.cpu(), 0.125, False, mask.cpu())
     assert np.abs(as64(got) - want).max() <= 2e-2
+
+
+def test_unmasked_decode_step_takes_the_decode_kernel(monkeypatch):
+    """is_causal=False, no mask, one query per head: the graph mapping must
+    pick the memory-bound decode kernel, not the 128-query MFMA kernel (which also accepts the
+    shapes)."""
+    from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO
+    from torch_mojo_backend.eager_kernels import hip_ops
+    decode_calls, fused_calls = [], []
+    real_decode, real_fused = hip_ops.attention_decode, hip_ops.attention
+    monkeypatch.setattr(hip_ops, "attention_decode",
+                        lambda *a, **kw: decode_calls.append(1) or real_decode(*a, **kw))
+    monkeypatch.setattr(hip_ops, "attention", lambda *a, **kw: fused_calls.append(1) or real_fused(*a, **kw))
+    q = seeded((3, 12, 1, 64), seed=4, dtype=torch.bfloat16).cuda()
+    k = seeded((3, 12, 208, 64), seed=5, dtype=torch.bfloat16).cuda()
+    v = seeded((3, 12, 208, 64), seed=6, dtype=torch.bfloat16).cuda()
+    assert hip_ops.attention_supported(q, k, v)                 # the MFMA kernel would take it too
+    want = _sdpa64(q.cpu(), k.cpu(), v.cpu(), 0.125, False, None)
+    got = MAPPING_TORCH_ATEN_TO_MOJO[torch.ops.aten.scaled_dot_product_attention](q, k, v)
+    assert len(decode_calls) == 1 and not fused_calls
+    assert np.abs(as64(got) - want).max() <= 2e-2
+    # 17 queries: past the decode kernel's limit, the MFMA kernel takes over
+    q17 = seeded((3, 12, 17, 64), seed=7, dtype=torch.bfloat16).cuda()
+    MAPPING_TORCH_ATEN_TO_MOJO[torch.ops.aten.scaled_dot_product_attention](q17, k, v)
+    assert len(fused_calls) == 1

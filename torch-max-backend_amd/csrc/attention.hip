@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(m0), "v"(voff), "s"(sbase)
-                 : "memory");
+                 : "memory", "m0");
   };
   auto fetch_block = [&](int blk, uint32_t buf_off) {
 #pragma unroll

@@ -195,12 +195,12 @@ void gemm_ring_kernel(GemmArgs g) {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
                    :
                    : "s"(m0), "v"(voff), "s"(sbase)
-                   : "memory");
+                   : "memory", "m0");
     } else {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :
                    : "s"(m0), "v"(voff), "s"(sbase)
-                   : "memory");
+                   : "memory", "m0");
     }
   };
   auto fetch_a = [&](uint32_t off, int64_t k0) {

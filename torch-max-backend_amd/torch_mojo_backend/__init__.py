@@ -8,7 +8,6 @@
 Public names follow torch_mojo_backend/__init__.py:11-33 of the reference.
 """
 
-from torch_mojo_backend.mojo_device.log_aten_calls import log_aten_calls
 from torch_mojo_backend.mojo_device.register import register_mojo_devices
 from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
 from torch_mojo_backend.torch_compile_backend.compiler import (
@@ -25,5 +24,4 @@ __all__ = [
     "MojoCompilerError",
     "register_mojo_devices",
     "TorchMojoTensor",
-    "log_aten_calls",
 ]

@@ -308,12 +308,12 @@ def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout
         and not (attn_mask is not None and is_causal)
     if plain:
         s = float(scale) if scale is not None else 1.0 / math.sqrt(query.shape[-1])
-        if attn_mask is None and s > 0.0 and query.dim() == 4 \
-                and hip_ops.attention_supported(query, key, value):
-            return hip_ops.attention(query, key, value, s, bool(is_causal)).transpose(1, 2)
         if query.dim() == 4 and query.shape[2] <= hip_ops.DECODE_MAX_QUERIES \
                 and hip_ops.attention_decode_supported(query, key, value, attn_mask):
             return hip_ops.attention_decode(query, key, value, s, bool(is_causal), attn_mask)
+        if attn_mask is None and s > 0.0 and query.dim() == 4 \
+                and hip_ops.attention_supported(query, key, value):
+            return hip_ops.attention(query, key, value, s, bool(is_causal)).transpose(1, 2)
         return hip_ops.attention_composed(query, key, value, s, bool(is_causal), attn_mask)
     return aten.scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal,
                                              scale=scale, enable_gqa=enable_gqa)

@@ -186,15 +186,17 @@ def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dr
         if mask is None or not _same_device(q, mask) or is_causal:
             return NOT_HANDLED
     s = float(scale) if scale is not None else 1.0 / math.sqrt(q._shape[-1])
-    if mask is None and s > 0.0 and len(q._shape) == 4 \
-            and hip_ops.attention_supported(q._holder, k._holder, v._holder):
-        out = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal))
-        return _wrap(out.transpose(1, 2))  # [batch, heads, tokens, head_dim] view, as ATen returns it
+    # a few queries per head (a decode step): the memory-bound kernel that reads K and V once,
+    # before the 128-query MFMA kernel gets to run tiles with 1-16 live rows
     mask_h = None if mask is None else mask._holder
     if len(q._shape) == 4 and q._shape[2] <= hip_ops.DECODE_MAX_QUERIES \
             and hip_ops.attention_decode_supported(q._holder, k._holder, v._holder, mask_h):
         return _wrap(hip_ops.attention_decode(q._holder, k._holder, v._holder, s, bool(is_causal),
                                               mask_h))
+    if mask is None and s > 0.0 and len(q._shape) == 4 \
+            and hip_ops.attention_supported(q._holder, k._holder, v._holder):
+        out = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal))
+        return _wrap(out.transpose(1, 2))  # [batch, heads, tokens, head_dim] view, as ATen returns it
     # other head sizes, fp32, additive masks: GEMM + softmax + GEMM
     return _wrap(hip_ops.attention_composed(q._holder, k._holder, v._holder, s, bool(is_causal),
                                             None if mask is None else mask._holder))

@@ -21,15 +21,15 @@ def get_accelerators() -> list:
 
 
 def get_fully_qualified_name(func: Callable | str) -> str:
+    """How an FX call target is named in error messages: ``module.qualname of type <type> `` for
+    callables (aten overloads print as ``torch._ops.aten.<op>``-style names), ``torch.Tensor.<m>``
+    for method names (reference utils.py:21-33; tests match on the op name inside)."""
     if isinstance(func, str):
-        return f"torch.Tensor.{func}"
-    result = ""
-    if hasattr(func, "__module__"):
-        result += func.__module__ + "."
-    if hasattr(func, "__qualname__"):
-        result += func.__qualname__
-    result += " of type " + str(type(func)) + " "
-    return result
+        return "torch.Tensor." + func
+    parts = [getattr(func, "__module__", None), getattr(func, "__qualname__", None)]
+    module, qualname = parts
+    name = (module + "." if module is not None else "") + (qualname if qualname is not None else "")
+    return f"{name} of type {type(func)} "
 
 
 def _describe(value) -> str:
