@@ -389,7 +389,7 @@ def main() -> int:
                 hbm_row(f"layer_norm_{dn}_{rows}x{cols}", len(bufs),
                         lambda i: lib.tmb_layer_norm_rows(ptrs[i][0], mean.data_ptr(), rstd.data_ptr(),
                                                           ptrs[i][1], g_.data_ptr(), b_.data_ptr(),
-                                                          rows, cols, 1e-5, code, stream),
+                                                          rows, cols, 1e-5, code, code, stream),
                         2 * nbytes + 2 * cols * es + 2 * rows * 4, cpu_fn=cpu_ln)
                 assert torch.equal(outs[0], hip_ops.layer_norm(bufs[0], [cols], g_, b_, 1e-5)[0])
                 del bufs, outs

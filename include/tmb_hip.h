@@ -75,13 +75,16 @@ int tmb_softmax_rows_scaled(void* out, const void* in, int64_t rows, int64_t col
 
 /* Layer norm over the last dimension of [rows, cols]: two-pass fp32 statistics
  * (mean = sum(x)/cols, var = sum((x-mean)^2)/cols biased, rstd = 1/sqrt(var+eps)),
- * out = (x-mean)*rstd*gamma + beta cast once. `gamma`/`beta` may be NULL (no affine);
- * `mean`/`rstd` ([rows] fp32) may be NULL when the caller proved them dead.
+ * out = (x-mean)*rstd*gamma + beta cast once. `dtype` in {F32,F16,BF16} is the type of `out`,
+ * `gamma` and `beta`; `in_dtype` is `dtype`, or F32 for fp32 rows normalised into a 16-bit
+ * tensor (a residual stream kept in fp32 between the blocks of a 16-bit model). `gamma`/`beta`
+ * may be NULL (no affine); `mean`/`rstd` ([rows] fp32) may be NULL when the caller proved them
+ * dead.
  * Replaces normalization_forward_ops.mojo `LayerNormForwardF32`
  * (called at aten_fast.py:2763-2776) and nn_ops.mojo:208-346 `LayerNorm` (aten_fast.py:2783-2793). */
 int tmb_layer_norm_rows(void* out, float* mean, float* rstd, const void* x, const void* gamma,
-                        const void* beta, int64_t rows, int64_t cols, double eps, int dtype,
-                        void* stream);
+                        const void* beta, int64_t rows, int64_t cols, double eps, int in_dtype,
+                        int dtype, void* stream);
 
 /* Bytes of device workspace `tmb_reduce_rows` / `tmb_argmax_rows` need for a shape (may be 0). */
 size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dtype);

@@ -48,7 +48,9 @@ def test_host_side_argument_validation_needs_no_gpu():
     assert L.tmb_softmax_rows(None, None, -1, 4, ek.F32, ek.F32, 0, None) == -1
     assert L.tmb_softmax_rows(None, None, 3, 4, ek.F32, ek.F32, 0, None) == -1
     assert L.tmb_softmax_rows(None, None, 0, 4, ek.F32, ek.F32, 0, None) == 0   # empty: nothing to do
-    assert L.tmb_layer_norm_rows(None, None, None, None, None, None, 2, 2, 1e-5, ek.F32, None) == -1
+    assert L.tmb_layer_norm_rows(None, None, None, None, None, None, 2, 2, 1e-5, ek.F32, ek.F32, None) == -1
+    assert L.tmb_layer_norm_rows(None, None, None, None, None, None, 2, 2, 1e-5, ek.BF16, ek.F32, None) == -2   # never widens
+    assert L.tmb_layer_norm_rows(None, None, None, None, None, None, 2, 2, 1e-5, ek.F16, ek.BF16, None) == -2
     assert L.tmb_reduce_rows(None, None, 2, 2, 7, ek.F32, None, 0, None) == -1  # unknown op
     assert L.tmb_reduce_rows(None, None, 2, 0, ek.SUM, ek.F32, None, 0, None) == -1
     assert L.tmb_argmax_rows(None, None, 2, 0, ek.F32, None, 0, None) == -1

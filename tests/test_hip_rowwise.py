@@ -123,6 +123,67 @@ def test_layer_norm_matches_oracle(shape, dtype):
                    what="rstd vs C oracle")
 
 
+# Row widths on both sides of every geometry switch of the kernel (lanes per row x vectors per
+# lane, in 16-byte input vectors: 16x1 .. 1024x16), for 4- and 2-byte inputs, with row counts that
+# leave the last workgroup and the last iteration of the persistent walk partly empty.
+LN_WIDTHS_VEC = [1, 15, 16, 17, 32, 33, 48, 49, 64, 65, 96, 97, 128, 129, 192, 193, 256, 257, 384,
+                 385, 512, 513, 768, 769, 1024, 1025, 2048, 2049, 4096, 4100]
+
+
+@pytest.mark.parametrize("nvec", LN_WIDTHS_VEC)
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32),
+                                                (torch.bfloat16, torch.bfloat16),
+                                                (torch.float32, torch.bfloat16),
+                                                (torch.float32, torch.float16)])
+def test_layer_norm_every_geometry_and_the_widening_input(nvec, in_dtype, out_dtype):
+    cols = nvec * (4 if in_dtype == torch.float32 else 8)
+    rows = 37 if cols <= 4096 else 5
+    x = seeded((rows, cols), seed=nvec, scale=2.0, shift=0.25, dtype=in_dtype)
+    g = seeded((cols,), seed=1, scale=0.1, shift=1.0, dtype=out_dtype)
+    b = seeded((cols,), seed=2, scale=0.1, dtype=out_dtype)
+    out, mean, rstd = _ops().layer_norm(_dev(x), [cols], _dev(g), _dev(b), 1e-5, out_dtype=out_dtype)
+    assert out.dtype == out_dtype and mean.dtype == torch.float32 and tuple(mean.shape) == (rows, 1)
+    w_out, w_mean, w_rstd = cf.layer_norm(as64(x), as64(g), as64(b), 1e-5)
+    scale = np.abs(as64(x) - w_mean) * w_rstd * np.abs(as64(g)) + np.abs(as64(b))
+    assert_close64(out, w_out, extra_abs=1e-5 * scale, what=f"ln out {rows}x{cols}")
+    assert_close64(mean, w_mean, atol=2e-6, what="ln mean")
+    assert_close64(rstd, w_rstd, rtol=1e-5, what="ln rstd")
+
+
+def test_layer_norm_widening_input_rejects_other_combinations():
+    x = _dev(seeded((4, 64), dtype=torch.bfloat16))
+    with pytest.raises(TypeError, match="cannot be normalised"):
+        _ops().layer_norm(x, [64], None, None, 1e-5, out_dtype=torch.float32)
+    xf = _dev(seeded((4, 64)))
+    w16 = _dev(seeded((64,), dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="weight must be"):
+        _ops().layer_norm(xf, [64], w16, None, 1e-5)                       # fp32 out wants fp32 weight
+    out, _, _ = _ops().layer_norm(xf, [64], w16, None, 1e-5, out_dtype=torch.bfloat16)
+    assert out.dtype == torch.bfloat16
+
+
+def test_layer_norm_full_size_rows_walk_whole_tensor():
+    """The persistent walk at the benchmark shapes: every row is written exactly once and matches
+    a float64 reference on sampled rows (first, last, and the rows around each workgroup's stride)."""
+    for rows, cols, dtype in ((32768, 768, torch.bfloat16), (16384, 4096, torch.float32),
+                              (32768, 768, torch.float32)):
+        g_ = torch.Generator(device="cuda").manual_seed(rows + cols)
+        x = (torch.randn(rows, cols, generator=g_, device="cuda") * 1.5 + 0.3).to(dtype)
+        w = (1 + 0.1 * torch.randn(cols, generator=g_, device="cuda")).to(dtype)
+        b = (0.1 * torch.randn(cols, generator=g_, device="cuda")).to(dtype)
+        out, mean, rstd = _ops().layer_norm(x, [cols], w, b, 1e-5)
+        assert not torch.isnan(out).any()
+        pick = torch.tensor([0, 1, 7, 8, 1023, 1024, 4095, 4096, 8191, 8192, rows // 2, rows - 2, rows - 1])
+        xs = x[pick].double().cpu()
+        want = torch.nn.functional.layer_norm(xs, [cols], w.double().cpu(), b.double().cpu(), 1e-5)
+        tol = 2e-2 if dtype == torch.bfloat16 else 2e-5
+        torch.testing.assert_close(out[pick].double().cpu(), want, rtol=tol, atol=tol)
+        torch.testing.assert_close(mean[pick, 0].double().cpu(), xs.mean(-1), rtol=1e-5, atol=2e-6)
+        # every row normalised: per-row mean of (out - b) / w is ~0
+        z = ((out.float() - b.float()) / w.float()).mean(-1).abs().max().item()
+        assert z < (3e-2 if dtype == torch.bfloat16 else 1e-4)
+
+
 @pytest.mark.parametrize("has_weight,has_bias", [(False, False), (True, False), (False, True)])
 @pytest.mark.parametrize("shape,normalized,eps", [((3, 7), (7,), 1e-5), ((2, 3, 4), (3, 4), 0.5)])
 def test_layer_norm_optional_affine(shape, normalized, eps, has_weight, has_bias):

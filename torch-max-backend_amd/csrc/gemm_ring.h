@@ -489,20 +489,6 @@ void gemm_ring_kernel(GemmArgs g) {
 #endif
 }
 
-// CUs of the current device (queried once per process).
-static int compute_units() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cus = n;
-    else
-      cus = 256;
-  }
-  return cus;
-}
-
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
           bool A_MMAJOR = false, bool OUT_F32 = false>
 static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {

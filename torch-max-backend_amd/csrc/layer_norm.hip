@@ -12,165 +12,170 @@
 
 namespace tmb {
 
-// Same work decomposition as the softmax kernel: WPR waves per row, or (WPR == 1) RPW rows per
-// wave with all loads issued up front. gamma/beta are fetched before the statistics so their
-// latency hides behind the reductions.
-//
-// AFFINE_LDS (long rows): gamma and beta are copied into LDS once per workgroup, the workgroup
-// then walks many rows (grid-stride), so the affine parameters cost LDS reads instead of a
-// second and third pass through L2 for every row.
-template <typename T, int WPR, int VPL, int RPW, bool STREAM, bool AFFINE_LDS, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void layer_norm_regs_kernel(
-    T* __restrict__ out, float* __restrict__ mean_out, float* __restrict__ rstd_out,
-    const T* __restrict__ in, const T* __restrict__ gamma, const T* __restrict__ beta,
-    int64_t rows, int cols, float eps, int64_t row_span) {
-  constexpr int EPV = Vec16<T>::N;
-  constexpr int WAVES = BLOCK / kWave;
-  constexpr int GROUPS = WAVES / WPR;
-  static_assert(WPR == 1 || RPW == 1, "several rows per wave only without cross-wave reductions");
-  __shared__ float slot[WAVES];
+// Sum over the G lanes (16, 32 or 64, aligned) that share a row; every one of them gets the
+// result. DPP butterflies inside 16 lanes, cross-lane permutes above that: a fixed order.
+template <int G>
+__device__ __forceinline__ float lanes_sum(float v) {
+  v += dpp_f32<kDppQuadXor1>(v);
+  v += dpp_f32<kDppQuadXor2>(v);
+  v += dpp_f32<kDppRowHalfMirror>(v);
+  v += dpp_f32<kDppRowMirror>(v);
+  if constexpr (G >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (G >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
 
-  const int wave = threadIdx.x >> 6;
-  const int lane = threadIdx.x & 63;
-  const int group = wave / WPR;
-  const int wave_in_row = wave - group * WPR;
+// A row is owned by G consecutive lanes: part of a wave (16 or 32 lanes: short rows keep every
+// lane busy, a wave then works on 4 or 2 rows at once), one wave, or G/64 waves that meet in LDS.
+// Each lane holds VPL 16-byte vectors of the row (G * VPL >= cols / EPV; the vectors of a row
+// are interleaved so that one load instruction of the group covers G * 16 consecutive bytes), so
+// the row is read once and both statistics passes run on registers.
+//
+// The grid is persistent: about 16 waves per CU, each group walking rows with the grid's
+// stride, gamma and beta fetched once per lane (kept packed in their storage type) instead of
+// once per row. The input may be wider than the output (fp32 rows normalised into a 16-bit
+// tensor: the residual stream of a 16-bit model kept in fp32); gamma and beta have the output's
+// type.
+template <typename TIn, typename TOut, int G, int VPL, bool STREAM, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void layer_norm_rows_kernel(
+    TOut* __restrict__ out, float* __restrict__ mean_out, float* __restrict__ rstd_out,
+    const TIn* __restrict__ in, const TOut* __restrict__ gamma, const TOut* __restrict__ beta,
+    int64_t rows, int cols, float eps) {
+  constexpr int EPV = Vec16<TIn>::N;
+  constexpr int GPB = BLOCK / G;            // rows a workgroup works on at once
+  constexpr int WPR = G > 64 ? G / 64 : 1;  // waves per row
+  constexpr int SUB = G > 64 ? 64 : G;
+  static_assert(BLOCK % G == 0 && GPB >= 1, "workgroup holds whole row groups");
+  static_assert(sizeof(TOut) <= sizeof(TIn), "the output is never wider than the input");
+  __shared__ float slot[2][BLOCK / kWave];
+
+  const int tid = threadIdx.x;
+  const int g = tid / G, l = tid % G;
+  const int wave = tid >> 6;
   const int nvec = cols / EPV;
   const float n = static_cast<float>(cols);
+  const int64_t total = static_cast<int64_t>(gridDim.x) * GPB;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * GPB + g;
+  const int64_t iters = (rows + total - 1) / total;  // the same for every group: barriers stay matched
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char affine_lds[];
-  T* lds_gamma = reinterpret_cast<T*>(affine_lds);
-  T* lds_beta = lds_gamma + cols;
-  if constexpr (AFFINE_LDS) {
-    for (int vi = threadIdx.x; vi < nvec; vi += BLOCK) {
-      if (gamma != nullptr) store_vec16(lds_gamma + vi * EPV, load_vec16(gamma + vi * EPV));
-      if (beta != nullptr) store_vec16(lds_beta + vi * EPV, load_vec16(beta + vi * EPV));
-    }
-    __syncthreads();
+  typedef TOut param_t __attribute__((ext_vector_type(EPV)));
+  typedef param_t __attribute__((aligned(sizeof(TOut)))) param_unaligned_t;
+  param_t gv[VPL], bv[VPL];
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = v * G + l;
+    const int at = (vi < nvec ? vi : 0) * EPV;
+    if (gamma != nullptr) gv[v] = *reinterpret_cast<const param_unaligned_t*>(gamma + at);
+    if (beta != nullptr) bv[v] = *reinterpret_cast<const param_unaligned_t*>(beta + at);
   }
 
-  // Short rows: gamma/beta are fetched once, before the first row's statistics (their latency
-  // hides behind the reductions), and stay in registers for every row the workgroup walks.
-  // Long rows would pay for that with occupancy; they fetch them (from LDS or L2) in groups of
-  // four vectors right before use.
-  constexpr bool PREFETCH_AFFINE = !AFFINE_LDS && VPL <= 4;
-  constexpr int AFF = PREFETCH_AFFINE ? VPL : (VPL < 4 ? VPL : 4);  // vectors held at a time
-  Vec16<T> gv[AFF], bv[AFF];
-  auto load_affine = [&](int v_first) {
-#pragma unroll
-    for (int u = 0; u < AFF; ++u) {
-      const int vi = ((v_first + u) * WPR + wave_in_row) * kWave + lane;
-      const int64_t at = static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
-      if constexpr (AFFINE_LDS) {
-        if (gamma != nullptr) gv[u] = load_vec16(lds_gamma + at);
-        if (beta != nullptr) bv[u] = load_vec16(lds_beta + at);
-      } else {
-        if (gamma != nullptr) gv[u] = load_vec16(gamma + at);
-        if (beta != nullptr) bv[u] = load_vec16(beta + at);
-      }
-    }
-  };
-  if constexpr (PREFETCH_AFFINE) load_affine(0);
-
-  // A workgroup walks `row_span` consecutive rows (a whole number of its row groups).
-  const int64_t rows_per_block = static_cast<int64_t>(GROUPS) * RPW;
-  const int64_t span_begin = static_cast<int64_t>(blockIdx.x) * row_span;
-  const int64_t span_end = span_begin + row_span < rows ? span_begin + row_span : rows;
-  for (int64_t block_row = span_begin; block_row < span_end; block_row += rows_per_block) {
-  const int64_t row0 = block_row + static_cast<int64_t>(group) * RPW;
-
-  float x[RPW][VPL][EPV];
-#pragma unroll
-  for (int r = 0; r < RPW; ++r) {
-    int64_t row = row0 + r;
-    if (row >= rows) row = rows - 1;
-    const T* src = in + row * static_cast<int64_t>(cols);
+  auto load_row = [&](int64_t row, Vec16<TIn> (&raw)[VPL]) {
+    if (row >= rows) row = rows - 1;  // keeps the groups in lock step; stores are masked
+    const TIn* src = in + row * static_cast<int64_t>(cols);
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
-      // Lanes past the end of the row re-read vector 0 (always valid) and discard it: no
-      // branch, so all of a wave's loads are issued back to back.
-      const int vi = (v * WPR + wave_in_row) * kWave + lane;
-      const bool ok = vi < nvec;
-      const int64_t at = static_cast<int64_t>(ok ? vi : 0) * EPV;
-      // the row is read exactly once: non-temporal whatever the size (measured: 36 -> 26 us on
-      // 32768 x 768 bf16); STREAM only decides how the output is stored
-      const Vec16<T> t = load_vec16_stream(src + at);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) x[r][v][e] = ok ? to_f32(t.v[e]) : 0.0f;
+      // lanes past the end of the row re-read vector 0 (always valid) and discard it: no branch,
+      // all loads of the group are issued back to back; the row is read exactly once, so the
+      // loads are non-temporal whatever the size (STREAM only decides how the output is stored)
+      const int vi = v * G + l;
+      raw[v] = load_vec16_stream(src + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV);
     }
-  }
-#pragma unroll
-  for (int r = 0; r < RPW; ++r) {
+  };
+  Vec16<TIn> raw[VPL];
+  load_row(gid, raw);
+  for (int64_t it = 0; it < iters; ++it) {
+    const int64_t row = it * total + gid;
+    float x[VPL][EPV];
     float s = 0.0f;
 #pragma unroll
-    for (int v = 0; v < VPL; ++v)
+    for (int v = 0; v < VPL; ++v) {
+      const bool ok = v * G + l < nvec;
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) s += x[r][v][e];
-    s = wave_sum(s);
-    s = group_reduce(s, slot, wave, group * WPR, WPR, SumOp{});
+      for (int e = 0; e < EPV; ++e) {
+        x[v][e] = ok ? to_f32(raw[v].v[e]) : 0.0f;
+        s += x[v][e];
+      }
+    }
+    s = lanes_sum<SUB>(s);
+    if constexpr (WPR > 1) {
+      if ((tid & 63) == 0) slot[0][wave] = s;
+      __syncthreads();
+      s = slot[0][g * WPR];
+#pragma unroll
+      for (int w = 1; w < WPR; ++w) s += slot[0][g * WPR + w];
+    }
     float mean = s / n;
-
     float q = 0.0f;
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
-      const int vi = (v * WPR + wave_in_row) * kWave + lane;
-      const bool ok = vi < nvec;
+      const bool ok = v * G + l < nvec;
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
-        const float d = ok ? x[r][v][e] - mean : 0.0f;
-        x[r][v][e] = d;
+        const float d = ok ? x[v][e] - mean : 0.0f;
+        x[v][e] = d;
         q += d * d;
       }
     }
-    q = wave_sum(q);
-    q = group_reduce(q, slot, wave, group * WPR, WPR, SumOp{});
+    q = lanes_sum<SUB>(q);
+    if constexpr (WPR > 1) {
+      if ((tid & 63) == 0) slot[1][wave] = q;
+      __syncthreads();
+      q = slot[1][g * WPR];
+#pragma unroll
+      for (int w = 1; w < WPR; ++w) q += slot[1][g * WPR + w];
+    }
     const float var = q / n;
     const float rstd = 1.0f / sqrtf(var + eps);
     if (var != var) mean = var;
-
-    const int64_t row = row0 + r;
     if (row < rows) {
-      if (wave_in_row == 0 && lane == 0) {
+      if (l == 0) {
         if (mean_out) mean_out[row] = mean;
         if (rstd_out) rstd_out[row] = rstd;
       }
-      T* dst = out + row * static_cast<int64_t>(cols);
+      TOut* dst = out + row * static_cast<int64_t>(cols);
 #pragma unroll
-      for (int v0 = 0; v0 < VPL; v0 += AFF) {
-        if constexpr (!PREFETCH_AFFINE) load_affine(v0);
+      for (int v = 0; v < VPL; ++v) {
+        const int vi = v * G + l;
+        float y[EPV];
 #pragma unroll
-        for (int u = 0; u < AFF; ++u) {
-          const int v = v0 + u;
-          const int vi = (v * WPR + wave_in_row) * kWave + lane;
-          float y[EPV];
-          if (gamma != nullptr) {
-#pragma unroll
-            for (int e = 0; e < EPV; ++e) y[e] = x[r][v][e] * rstd * to_f32(gv[u].v[e]);
+        for (int e = 0; e < EPV; ++e) {
+          y[e] = x[v][e] * rstd;
+          if (gamma != nullptr) y[e] *= to_f32(gv[v][e]);
+          if (beta != nullptr) y[e] += to_f32(bv[v][e]);
+        }
+        if (vi < nvec) {
+          TOut* at = dst + static_cast<int64_t>(vi) * EPV;
+          if constexpr (sizeof(TOut) == sizeof(TIn)) {
+            store_converted<TOut, EPV, STREAM>(at, y);
           } else {
+            // four fp32 values in, four 16-bit values out: one 8-byte store per vector
+            param_t o;
 #pragma unroll
-            for (int e = 0; e < EPV; ++e) y[e] = x[r][v][e] * rstd;
+            for (int e = 0; e < EPV; ++e) o[e] = from_f32<TOut>(y[e]);
+            if constexpr (STREAM) {
+              __builtin_nontemporal_store(o, reinterpret_cast<param_t*>(at));
+            } else {
+              *reinterpret_cast<param_t*>(at) = o;
+            }
           }
-          if (beta != nullptr) {
-#pragma unroll
-            for (int e = 0; e < EPV; ++e) y[e] += to_f32(bv[u].v[e]);
-          }
-          if (vi < nvec) store_converted<T, EPV, STREAM>(dst + static_cast<int64_t>(vi) * EPV, y);
         }
       }
     }
+    if (it + 1 < iters) load_row(row + total, raw);
+    if constexpr (WPR > 1) __syncthreads();  // the slots are written again for the next row
   }
-  }  // rows of this workgroup's span
 }
 
-template <typename T>
+template <typename TIn, typename TOut>
 __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
-    T* __restrict__ out, float* __restrict__ mean_out, float* __restrict__ rstd_out,
-    const T* __restrict__ in, const T* __restrict__ gamma, const T* __restrict__ beta,
+    TOut* __restrict__ out, float* __restrict__ mean_out, float* __restrict__ rstd_out,
+    const TIn* __restrict__ in, const TOut* __restrict__ gamma, const TOut* __restrict__ beta,
     int64_t rows, int64_t cols, float eps) {
   __shared__ float slot[4];
   const int wave = threadIdx.x >> 6;
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    const T* src = in + row * cols;
-    T* dst = out + row * cols;
+    const TIn* src = in + row * cols;
+    TOut* dst = out + row * cols;
     float s = 0.0f;
     for (int64_t j = threadIdx.x; j < cols; j += 256) s += to_f32(src[j]);
     s = wave_sum(s);
@@ -195,85 +200,77 @@ __global__ __launch_bounds__(256) void layer_norm_generic_kernel(
       float y = (to_f32(src[j]) - center) * rstd;
       if (gamma != nullptr) y *= to_f32(gamma[j]);
       if (beta != nullptr) y += to_f32(beta[j]);
-      dst[j] = from_f32<T>(y);
+      dst[j] = from_f32<TOut>(y);
     }
   }
 }
 
-template <typename T, int WPR, int VPL, int BLOCK>
-static int launch_ln(T* out, float* mean, float* rstd, const T* x, const T* g, const T* b,
+template <typename TIn, typename TOut, int G, int VPL, int BLOCK>
+static int launch_ln(TOut* out, float* mean, float* rstd, const TIn* x, const TOut* g, const TOut* b,
                      int64_t rows, int64_t cols, float eps, hipStream_t stream) {
-  constexpr int EPV = Vec16<T>::N;
-  constexpr int RPW = 1;
-  constexpr int ROWS_PER_BLOCK = (BLOCK / kWave) / WPR * RPW;
-  const int64_t groups = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;  // row groups of a workgroup
-  const bool stream_hint = rows * cols * static_cast<int64_t>(2 * sizeof(T)) >= (int64_t{256} << 20);
-  const dim3 block(BLOCK);
-  const int c = static_cast<int>(cols);
-  // `walk` row groups per workgroup, consecutive in memory
-  auto launch = [&](auto lds_tag, int64_t walk, size_t lds_bytes) {
-    constexpr bool LDS = decltype(lds_tag)::value;
-    const int64_t blocks = (groups + walk - 1) / walk;
-    const dim3 grid(static_cast<unsigned>(blocks));
-    const int64_t span = walk * ROWS_PER_BLOCK;
-    if (stream_hint)
-      layer_norm_regs_kernel<T, WPR, VPL, RPW, true, LDS, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps, span);
-    else
-      layer_norm_regs_kernel<T, WPR, VPL, RPW, false, LDS, BLOCK><<<grid, block, lds_bytes, stream>>>(out, mean, rstd, x, g, b, rows, c, eps, span);
-    return check_launch();
-  };
-  // Long 16-bit rows with affine parameters: gamma/beta staged in LDS by a few workgroups that
-  // each walk many rows (for fp32 the LDS reads would cost as much as the L2 re-reads they
-  // replace).
-  const size_t lds_bytes = static_cast<size_t>(cols) * sizeof(T) * 2;
-  if constexpr (VPL >= 8 && sizeof(T) == 2) {
-    if ((g != nullptr || b != nullptr) && lds_bytes <= 65536) {
-      const int64_t persistent = 256 * (BLOCK >= 1024 ? 2 : 8);
-      return launch(std::true_type{}, (groups + persistent - 1) / persistent, lds_bytes);
-    }
+  constexpr int GPB = BLOCK / G;
+  const int64_t max_grid = (rows + GPB - 1) / GPB;
+  // about 16 waves per CU, every workgroup walking the same number of rows (measured on
+  // 32768 x 768 and 16384 x 4096: fewer waves leave the memory system short of requests, more
+  // only add ramp and tail)
+  int64_t grid = static_cast<int64_t>(compute_units()) * 16 / (BLOCK / kWave);
+  if (grid >= max_grid) {
+    grid = max_grid;
+  } else {
+    const int64_t walk = (max_grid + grid - 1) / grid;
+    grid = (max_grid + walk - 1) / walk;
   }
-  // Short rows keep gamma/beta in registers: a workgroup that walks a few consecutive row
-  // groups re-uses them (more than four measured slower: too few workgroups in flight).
-  const int64_t walk = VPL <= 4 ? (groups >= 16384 ? 4 : (groups >= 4096 ? 2 : 1)) : 1;
-  return launch(std::false_type{}, walk, 0);
+  const bool stream_hint =
+      rows * cols * static_cast<int64_t>(sizeof(TIn) + sizeof(TOut)) >= (int64_t{256} << 20);
+  const dim3 grid3(static_cast<unsigned>(grid)), block(BLOCK);
+  const int c = static_cast<int>(cols);
+  if (stream_hint)
+    layer_norm_rows_kernel<TIn, TOut, G, VPL, true, BLOCK><<<grid3, block, 0, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
+  else
+    layer_norm_rows_kernel<TIn, TOut, G, VPL, false, BLOCK><<<grid3, block, 0, stream>>>(out, mean, rstd, x, g, b, rows, c, eps);
+  return check_launch();
 }
 
-template <typename T>
+template <typename TIn, typename TOut>
 static int layer_norm_dispatch(void* out_, float* mean, float* rstd, const void* x_,
                                const void* g_, const void* b_, int64_t rows, int64_t cols,
                                float eps, hipStream_t stream) {
-  T* out = static_cast<T*>(out_);
-  const T* x = static_cast<const T*>(x_);
-  const T* g = static_cast<const T*>(g_);
-  const T* b = static_cast<const T*>(b_);
-  constexpr int EPV = Vec16<T>::N;
+  TOut* out = static_cast<TOut*>(out_);
+  const TIn* x = static_cast<const TIn*>(x_);
+  const TOut* g = static_cast<const TOut*>(g_);
+  const TOut* b = static_cast<const TOut*>(b_);
+  constexpr int EPV = Vec16<TIn>::N;
   constexpr int MAXV = 64 / EPV;  // at most 64 fp32 values of a row per lane
-  const bool vec_ok = (cols % EPV == 0) && aligned16(x) && aligned16(out) &&
-                      (g == nullptr || aligned16(g)) && (b == nullptr || aligned16(b)) &&
-                      rows < (int64_t{1} << 31);
+  constexpr uintptr_t kOutAlign = EPV * sizeof(TOut) - 1;  // one output vector per input vector
+  const bool vec_ok = (cols % EPV == 0) && aligned16(x) &&
+                      (reinterpret_cast<uintptr_t>(out) & kOutAlign) == 0 && rows < (int64_t{1} << 31);
   const int64_t nvec = cols / EPV;
-#define TMB_LN(WPR, VPL, BLOCK) \
-  return launch_ln<T, WPR, VPL, BLOCK>(out, mean, rstd, x, g, b, rows, cols, eps, stream)
-  if (vec_ok && nvec <= 16 * 64 * MAXV) {
-    if (nvec <= 64) TMB_LN(1, 1, 256);
-    if (nvec <= 128) TMB_LN(1, 2, 256);
-    if (nvec <= 256) TMB_LN(1, 4, 256);
-    if constexpr (MAXV >= 16) {
-      // fp32: rows shared by four waves, two or four vectors per lane (measured 5-10 % faster
-      // than one wave per row)
-      if (nvec <= 512) TMB_LN(4, 2, 256);
-      if (nvec <= 1024) TMB_LN(4, 4, 256);
-    } else {
-      if (nvec <= 512) TMB_LN(1, 8, 256);  // 16-bit: gamma/beta through LDS
-    }
-    if (nvec <= 4 * 64 * MAXV / 2) TMB_LN(4, MAXV / 2, 256);
-    if (nvec <= 4 * 64 * MAXV) TMB_LN(4, MAXV, 256);
-    if (nvec <= 16 * 64 * MAXV / 2) TMB_LN(16, MAXV / 2, 1024);
-    TMB_LN(16, MAXV, 1024);
+#define TMB_LN(G, VPL, BLOCK) \
+  return launch_ln<TIn, TOut, G, VPL, BLOCK>(out, mean, rstd, x, g, b, rows, cols, eps, stream)
+  if (vec_ok && nvec <= 1024 * MAXV) {
+    // the narrowest group that holds the row in at most four vectors per lane; measured on
+    // 768- and 4096-column rows, where 32 x 3 / 64 x 3 and 256 x 2 / 256 x 4 run at the speed
+    // of a plain copy of the same bytes
+    if (nvec <= 16) TMB_LN(16, 1, 256);
+    if (nvec <= 32) TMB_LN(16, 2, 256);
+    if (nvec <= 48) TMB_LN(16, 3, 256);
+    if (nvec <= 64) TMB_LN(32, 2, 256);
+    if (nvec <= 96) TMB_LN(32, 3, 256);
+    if (nvec <= 128) TMB_LN(64, 2, 256);
+    if (nvec <= 192) TMB_LN(64, 3, 256);
+    if (nvec <= 256) TMB_LN(64, 4, 256);
+    if (nvec <= 384) TMB_LN(128, 3, 256);
+    if (nvec <= 512) TMB_LN(256, 2, 512);
+    if (nvec <= 768) TMB_LN(256, 3, 512);
+    if (nvec <= 1024) TMB_LN(256, 4, 512);
+    if (nvec <= 2048) TMB_LN(512, 4, 512);
+    if (nvec <= 4096) TMB_LN(1024, 4, 1024);
+    if (nvec <= 8192) TMB_LN(1024, 8, 1024);
+    if constexpr (MAXV >= 16) TMB_LN(1024, 16, 1024);
   }
 #undef TMB_LN
   const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
-  layer_norm_generic_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(
+  layer_norm_generic_kernel<TIn, TOut><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(
       out, mean, rstd, x, g, b, rows, cols, eps);
   return check_launch();
 }
@@ -282,20 +279,23 @@ static int layer_norm_dispatch(void* out_, float* mean, float* rstd, const void*
 
 extern "C" int tmb_layer_norm_rows(void* out, float* mean, float* rstd, const void* x,
                                    const void* gamma, const void* beta, int64_t rows,
-                                   int64_t cols, double eps, int dtype, void* stream) {
+                                   int64_t cols, double eps, int in_dtype, int dtype, void* stream) {
+  using namespace tmb;
   if (rows < 0 || cols < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (dtype != TMB_F32 && dtype != TMB_F16 && dtype != TMB_BF16) return TMB_ERR_UNSUPPORTED;
+  if (in_dtype != dtype && in_dtype != TMB_F32) return TMB_ERR_UNSUPPORTED;
   if (rows == 0 || cols == 0) return TMB_OK;
   if (out == nullptr || x == nullptr) return TMB_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float e = static_cast<float>(eps);
-  switch (dtype) {
-    case TMB_F32:
-      return tmb::layer_norm_dispatch<float>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
-    case TMB_F16:
-      return tmb::layer_norm_dispatch<tmb::f16_t>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
-    case TMB_BF16:
-      return tmb::layer_norm_dispatch<tmb::bf16_t>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
-    default:
-      return TMB_ERR_UNSUPPORTED;
+  if (in_dtype == TMB_F32) {
+    switch (dtype) {
+      case TMB_F32: return layer_norm_dispatch<float, float>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
+      case TMB_F16: return layer_norm_dispatch<float, f16_t>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
+      default: return layer_norm_dispatch<float, bf16_t>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
+    }
   }
+  if (dtype == TMB_F16)
+    return layer_norm_dispatch<f16_t, f16_t>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
+  return layer_norm_dispatch<bf16_t, bf16_t>(out, mean, rstd, x, gamma, beta, rows, cols, e, s);
 }

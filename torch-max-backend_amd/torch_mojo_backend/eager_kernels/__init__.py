@@ -29,7 +29,7 @@ SIGNATURES = {
     "tmb_status_string": (ctypes.c_char_p, [_ci]),
     "tmb_softmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _ci, _vp]),
     "tmb_softmax_rows_scaled": (_ci, [_vp, _vp, _i64, _i64, _ci, _flt, _ci, _i64, _vp]),
-    "tmb_layer_norm_rows": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _dbl, _ci, _vp]),
+    "tmb_layer_norm_rows": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _dbl, _ci, _ci, _vp]),
     "tmb_reduce_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
     "tmb_reduce_rows_static": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp]),

@@ -385,22 +385,28 @@ def attention_composed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale:
 
 
 def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optional[torch.Tensor],
-               bias: Optional[torch.Tensor], eps: float, need_stats: bool = True):
+               bias: Optional[torch.Tensor], eps: float, need_stats: bool = True,
+               out_dtype: Optional[torch.dtype] = None):
     """(out, mean, rstd); mean/rstd are float32 with shape ``x.shape[:-k] + (1,)*k`` or None
-    when ``need_stats`` is False."""
+    when ``need_stats`` is False. ``out_dtype`` (default: the input's) may be a 16-bit type for
+    a float32 input: the row is read in float32 and the result cast once; weight and bias then
+    have the output's type."""
     require_hip(x, weight, bias)
     k = len(normalized_shape)
+    out_dtype = x.dtype if out_dtype is None else out_dtype
     if x.dtype not in FLOAT_DTYPES or k < 1 or x.dim() < k or \
             tuple(x.shape[x.dim() - k:]) != tuple(normalized_shape):
         raise ValueError(f"layer_norm: input {tuple(x.shape)} {x.dtype} vs normalized_shape "
                          f"{tuple(normalized_shape)}")
+    if out_dtype != x.dtype and not (x.dtype == torch.float32 and out_dtype in FLOAT_DTYPES):
+        raise TypeError(f"layer_norm: {x.dtype} input cannot be normalised into {out_dtype}")
     for name, p in (("weight", weight), ("bias", bias)):
-        if p is not None and (p.dtype != x.dtype or tuple(p.shape) != tuple(normalized_shape)):
-            raise ValueError(f"layer_norm: {name} must be {tuple(normalized_shape)} {x.dtype}")
+        if p is not None and (p.dtype != out_dtype or tuple(p.shape) != tuple(normalized_shape)):
+            raise ValueError(f"layer_norm: {name} must be {tuple(normalized_shape)} {out_dtype}")
     cols = math.prod(normalized_shape)
     xc = x if x.is_contiguous() else x.contiguous()
     rows = xc.numel() // cols if cols else 0
-    out = torch.empty_like(xc)
+    out = torch.empty(xc.shape, dtype=out_dtype, device=x.device)
     stat_shape = tuple(x.shape[: x.dim() - k]) + (1,) * k
     mean = rstd = None
     if need_stats:
@@ -413,7 +419,7 @@ def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optiona
             out.data_ptr(), None if mean is None else mean.data_ptr(),
             None if rstd is None else rstd.data_ptr(), xc.data_ptr(),
             None if w is None else w.data_ptr(), None if b is None else b.data_ptr(),
-            rows, cols, float(eps), code_of(x.dtype), _stream())
+            rows, cols, float(eps), code_of(x.dtype), code_of(out_dtype), _stream())
         _check("tmb_layer_norm_rows", rc)
     return out, mean, rstd
 
