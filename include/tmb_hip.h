@@ -47,6 +47,14 @@ typedef enum tmb_epilogue {
   TMB_EPI_GELU_ERF = 2   /* 0.5*x*(1+erf(x/sqrt(2))) applied after bias */
 } tmb_epilogue;
 
+/* Flag or-ed into an `epilogue` argument. Without it a fused epilogue stays in fp32 from the
+ * accumulator to the one cast: T(gelu(acc + bias)), T(acc + bias + residual) - the reference's
+ * rule for what it fuses into a GEMM (matmul_ops.mojo:2651-2657: "forming A@B + bias in fp32 and
+ * casting to the output dtype exactly once"). With it every fused step rounds to the storage
+ * type where a separate kernel would have stored its result: T(gelu(T(acc + bias))),
+ * T(T(acc + bias) + residual), the bits of the unfused sequence of kernels. */
+#define TMB_EPI_ROUND_LIKE_UNFUSED 0x100
+
 /* Library/ABI version (major*1000 + minor). */
 int tmb_version(void);
 
@@ -130,7 +138,8 @@ int tmb_argmax_rows(int64_t* out, const void* in, int64_t rows, int64_t cols, in
  * row-major as its logical shape ([m,k] with lda / [k,n] with ldb); = 1: stored as the
  * transpose ([k,m] with lda / [n,k] with ldb — the layout of a torch `weight.t()` view).
  * stride_* are element strides between batch entries (stride 0 broadcasts an operand).
- * `dtype` in {F32,F16,BF16} for A, B, bias and C alike.
+ * `dtype` in {F32,F16,BF16} for A, B, bias and C alike. `epilogue` is a tmb_epilogue, optionally
+ * or-ed with TMB_EPI_ROUND_LIKE_UNFUSED.
  * Replaces the raw-pointer GEMM bridges `Bf16GemmBF16` (aten_fast.py:4588-4600),
  * `Bf16BmmBF16` (aten_fast.py:4707-4721) and MatmulSpec/MatmulBiasSpec/BmmSpec
  * (matmul_ops.mojo:3451-3636). */
@@ -155,19 +164,24 @@ int tmb_gemm_ws(void* c, const void* a, const void* b, const void* bias, int64_t
                 int epilogue, void* workspace, size_t workspace_bytes, void* stream);
 
 /* tmb_gemm followed by an elementwise add of `residual` [batch][m, n] (row pitch `ldr`, batch
- * stride `stride_r`) in the same launch: c = T(float(T(epilogue(a b + bias))) + float(residual)),
- * rounded twice exactly as a GEMM kernel followed by an add kernel would (the residual
- * connection of a transformer block: demo_scripts/gpt2.py:85-86 `x = x + self.attn(...)`,
- * which reaches the graph as addmm -> view -> add). 16-bit dtypes on the MFMA path only;
- * TMB_ERR_UNSUPPORTED otherwise (fp32, k == 0, transposed A, unaligned operands): the caller then
- * launches tmb_gemm and adds separately.
+ * stride `stride_r`) in the same launch (the residual connection of a transformer block:
+ * demo_scripts/gpt2.py:85-86 `x = x + self.attn(...)`, which reaches the graph as
+ * addmm -> view -> add): c = OUT(a b + bias + residual), summed in fp32 and cast once; with
+ * TMB_EPI_ROUND_LIKE_UNFUSED c = T(T(epilogue(a b + bias)) + residual), rounded twice exactly as a
+ * GEMM kernel followed by an add kernel would.
+ * `residual_dtype` and `out_dtype` are `dtype` or TMB_F32: a 16-bit model may keep its residual
+ * stream in fp32 (fp32 residual in, fp32 sum out, nothing rounded in between; not together
+ * with TMB_EPI_ROUND_LIKE_UNFUSED). 16-bit A and B on the MFMA path only; TMB_ERR_UNSUPPORTED
+ * otherwise (fp32 A/B, k == 0, transposed A, unaligned operands, a GELU epilogue unless
+ * TMB_EPI_ROUND_LIKE_UNFUSED): the caller then launches tmb_gemm and adds separately.
  * Replaces `AddF32Bf16Spec` / the residual add of aten_fast.py:657-687 together with the GEMM
  * in front of it. */
 int tmb_gemm_residual(void* c, const void* a, const void* b, const void* bias,
                       const void* residual, int64_t batch, int64_t m, int64_t n, int64_t k,
                       int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr, int64_t stride_a,
                       int64_t stride_b, int64_t stride_c, int64_t stride_r, int trans_a,
-                      int trans_b, int dtype, int epilogue, void* stream);
+                      int trans_b, int dtype, int residual_dtype, int out_dtype, int epilogue,
+                      void* stream);
 
 /* Fused attention forward: out[b,t,h,:] = softmax_j(scale * q[b,h,t,:] . k[b,h,j,:]) v[b,h,j,:],
  * with `causal` != 0 only keys j <= t take part. The [batch, heads, q_len, kv_len] scores never

@@ -67,6 +67,10 @@ def lib() -> ctypes.CDLL:
         L = ctypes.CDLL(_LIB_PATH)
         i64, vp, ci, dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_double
         L.orc_gemm.argtypes = [vp, vp, vp, vp] + [i64] * 10 + [ci] * 4
+        L.orc_gemm_residual.argtypes = [vp, vp, vp, vp, vp] + [i64] * 12 + [ci] * 6
+        L.orc_gemm_residual.restype = ci
+        L.orc_layer_norm_mixed.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ci, ci]
+        L.orc_layer_norm_mixed.restype = ci
         L.orc_softmax.argtypes = [vp, vp, i64, i64, ci, ci, ci]
         L.orc_softmax_scaled.argtypes = [vp, vp, i64, i64, ci, ctypes.c_float, ci, i64]
         L.orc_softmax_scaled.restype = ci
@@ -118,9 +122,17 @@ def _check(rc: int, what: str) -> None:
 # ---------------------------------------------------------------------------
 # Row-level kernels (thin wrappers over the C functions)
 # ---------------------------------------------------------------------------
+EPI_ROUND_LIKE_UNFUSED = 0x100
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
-         epilogue: int = EPI_NONE) -> torch.Tensor:
-    """``epilogue(a @ b + bias)`` for 2-D or 3-D (batched) operands of any strides.
+         epilogue: int = EPI_NONE, residual: Optional[torch.Tensor] = None,
+         out_dtype: Optional[torch.dtype] = None, round_like_unfused: bool = False) -> torch.Tensor:
+    """``epilogue(a @ b + bias) [+ residual]`` for 2-D or 3-D (batched) operands of any strides,
+    formed in float32 and cast once (matmul_ops.mojo:2651-2657); ``round_like_unfused`` rounds
+    to the operands' dtype after the bias and after the GELU, as separate kernels would.
+    ``residual`` has the result's shape and the operands' dtype or float32; ``out_dtype``
+    defaults to the operands' dtype.
 
     Strided views are passed through as they are (transpose flags / leading dimensions) when
     each matrix is dense row-major or dense column-major, otherwise materialised first.
@@ -148,14 +160,20 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None, 
 
     a3, ta, lda, sa = layout(a3)
     b3, tb, ldb, sb = layout(b3)
-    out = torch.empty((batch, m, n), dtype=a.dtype)
+    out = torch.empty((batch, m, n), dtype=out_dtype or a.dtype)
     if bias is not None:
         assert bias.dtype == a.dtype and tuple(bias.shape) == (n,)
         bias = _cpu(bias)
+    res = None
+    if residual is not None:
+        res = _cpu(residual).reshape(batch, m, n).contiguous()
+        assert res.dtype in (a.dtype, torch.float32)
+    flags = epilogue | (EPI_ROUND_LIKE_UNFUSED if round_like_unfused else 0)
     if out.numel():
-        _check(lib().orc_gemm(out.data_ptr(), a3.data_ptr(), b3.data_ptr(), _ptr(bias), batch, m,
-                              n, k, lda, ldb, n, sa, sb, m * n, ta, tb, _code(a.dtype), epilogue),
-               "gemm")
+        _check(lib().orc_gemm_residual(
+            out.data_ptr(), a3.data_ptr(), b3.data_ptr(), _ptr(bias), _ptr(res), batch, m, n, k,
+            lda, ldb, n, n, sa, sb, m * n, m * n, ta, tb, _code(a.dtype),
+            _code(res.dtype if res is not None else a.dtype), _code(out.dtype), flags), "gemm")
     return out if batched else out[0]
 
 
@@ -197,19 +215,20 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
 
 
 def layer_norm_rows(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
-                    eps: float):
+                    eps: float, out_dtype: Optional[torch.dtype] = None):
     x = _cpu(x)
     assert x.dim() == 2
     rows, cols = x.shape
-    out = torch.empty_like(x)
+    out = torch.empty(x.shape, dtype=out_dtype or x.dtype)
     mean = torch.empty(rows, dtype=torch.float32)
     rstd = torch.empty(rows, dtype=torch.float32)
     g = None if gamma is None else _cpu(gamma.reshape(-1))
     b = None if beta is None else _cpu(beta.reshape(-1))
+    assert all(p is None or p.dtype == out.dtype for p in (g, b))
     if x.numel():
-        _check(lib().orc_layer_norm(out.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(),
-                                    _ptr(g), _ptr(b), rows, cols, float(eps), _code(x.dtype)),
-               "layer_norm")
+        _check(lib().orc_layer_norm_mixed(out.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                          x.data_ptr(), _ptr(g), _ptr(b), rows, cols, float(eps),
+                                          _code(x.dtype), _code(out.dtype)), "layer_norm")
     return out, mean, rstd
 
 

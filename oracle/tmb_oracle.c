@@ -117,11 +117,22 @@ static float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811
 
 /* C[b] = epi(op(A[b]) op(B[b]) + bias). The GELU epilogue acts on the value already rounded to
  * the storage dtype, i.e. exactly what an unfused addmm followed by gelu produces. */
-int orc_gemm(void* c, const void* a, const void* b, const void* bias, int64_t batch, int64_t m,
-             int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
-             int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
-             int epilogue) {
+/* epilogue = ORC_EPI_* | ORC_EPI_ROUND_LIKE_UNFUSED. The value is formed in fp32 from the
+ * accumulator to the one cast (matmul_ops.mojo:2651-2657: "forming A@B + bias in fp32 and casting
+ * to the output dtype exactly once"), also through a GELU and a residual add that a caller fuses
+ * into the product; with the flag it is rounded to `dtype` wherever a separate kernel would have
+ * stored it (after the bias, after the GELU). `residual` ([batch][m][n], pitch ldr, type
+ * residual_dtype) may be NULL; `out_dtype` is the type of c. */
+enum { ORC_EPI_ROUND_LIKE_UNFUSED = 0x100 };
+
+int orc_gemm_residual(void* c, const void* a, const void* b, const void* bias, const void* residual,
+                      int64_t batch, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                      int64_t ldc, int64_t ldr, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                      int64_t stride_r, int trans_a, int trans_b, int dtype, int residual_dtype,
+                      int out_dtype, int epilogue_flags) {
   if (dtype != ORC_F32 && dtype != ORC_F16 && dtype != ORC_BF16) return -2;
+  const int epilogue = epilogue_flags & 0xff;
+  const int twice = (epilogue_flags & ORC_EPI_ROUND_LIKE_UNFUSED) != 0;
   const int64_t sa_m = trans_a ? 1 : lda, sa_k = trans_a ? lda : 1;
   const int64_t sb_k = trans_b ? 1 : ldb, sb_n = trans_b ? ldb : 1;
   const int64_t total_rows = batch * m;
@@ -136,13 +147,25 @@ int orc_gemm(void* c, const void* a, const void* b, const void* bias, int64_t ba
       }
       if (bias) acc += load_f(bias, j, dtype);
       if (epilogue != ORC_EPI_NONE) {
-        acc = round_to(acc, dtype);
+        if (twice) acc = round_to(acc, dtype);
         acc = epilogue == ORC_EPI_GELU_TANH ? gelu_tanh(acc) : gelu_erf(acc);
       }
-      store_f(c, bz * stride_c + i * ldc + j, dtype, acc);
+      if (residual) {
+        if (twice) acc = round_to(acc, dtype);
+        acc += load_f(residual, bz * stride_r + i * ldr + j, residual_dtype);
+      }
+      store_f(c, bz * stride_c + i * ldc + j, out_dtype, acc);
     }
   }
   return 0;
+}
+
+int orc_gemm(void* c, const void* a, const void* b, const void* bias, int64_t batch, int64_t m,
+             int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+             int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, int dtype,
+             int epilogue) {
+  return orc_gemm_residual(c, a, b, bias, 0, batch, m, n, k, lda, ldb, ldc, 0, stride_a, stride_b,
+                           stride_c, 0, trans_a, trans_b, dtype, dtype, dtype, epilogue);
 }
 
 int orc_softmax(void* out, const void* in, int64_t rows, int64_t cols, int in_dtype,
@@ -241,24 +264,28 @@ int orc_attention(void* out, const void* q, const void* k, const void* v, int64_
   return 0;
 }
 
-int orc_layer_norm(void* out, float* mean_out, float* rstd_out, const void* x, const void* gamma,
-                   const void* beta, int64_t rows, int64_t cols, double eps, int dtype) {
+/* `in_dtype` is the type of x, `dtype` the type of out, gamma and beta (the same, or a 16-bit
+ * output normalised from an fp32 row: the statistics and the normalisation then use the fp32
+ * values and the result is cast once). */
+int orc_layer_norm_mixed(void* out, float* mean_out, float* rstd_out, const void* x,
+                         const void* gamma, const void* beta, int64_t rows, int64_t cols,
+                         double eps, int in_dtype, int dtype) {
   const float e = (float)eps;
 #pragma omp parallel for schedule(static)
   for (int64_t r = 0; r < rows; ++r) {
     const int64_t base = r * cols;
     float total = 0.0f;
-    for (int64_t j = 0; j < cols; ++j) total += load_f(x, base + j, dtype);
+    for (int64_t j = 0; j < cols; ++j) total += load_f(x, base + j, in_dtype);
     float mean = total / (float)cols;
     float var_sum = 0.0f;
     for (int64_t j = 0; j < cols; ++j) {
-      const float d = load_f(x, base + j, dtype) - mean;
+      const float d = load_f(x, base + j, in_dtype) - mean;
       var_sum += d * d;
     }
     const float var = var_sum / (float)cols;
     const float rstd = 1.0f / sqrtf(var + e);
     for (int64_t j = 0; j < cols; ++j) {
-      float y = (load_f(x, base + j, dtype) - mean) * rstd;
+      float y = (load_f(x, base + j, in_dtype) - mean) * rstd;
       if (gamma) y *= load_f(gamma, j, dtype);
       if (beta) y += load_f(beta, j, dtype);
       store_f(out, base + j, dtype, y);
@@ -268,6 +295,11 @@ int orc_layer_norm(void* out, float* mean_out, float* rstd_out, const void* x, c
     if (rstd_out) rstd_out[r] = rstd;
   }
   return 0;
+}
+
+int orc_layer_norm(void* out, float* mean_out, float* rstd_out, const void* x, const void* gamma,
+                   const void* beta, int64_t rows, int64_t cols, double eps, int dtype) {
+  return orc_layer_norm_mixed(out, mean_out, rstd_out, x, gamma, beta, rows, cols, eps, dtype, dtype);
 }
 
 int orc_reduce(void* out, const void* in, int64_t rows, int64_t cols, int op, int dtype) {

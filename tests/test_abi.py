@@ -65,7 +65,18 @@ def test_host_side_argument_validation_needs_no_gpu():
     assert L.tmb_attention_fwd(None, None, None, None, 1, 1, 4, 4, 64, strides, strides, strides,
                                strides, 0.125, 0, 0, ek.BF16, None) == -1
     assert L.tmb_gemm_residual(None, None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, 0,
-                               ek.BF16, 0, None) == -1
+                               ek.BF16, ek.BF16, ek.BF16, 0, None) == -1
+    # epilogue flags: only the rounding flag may be or-ed in; the float32 stream excludes it
+    assert L.tmb_gemm(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 0x200, None) == -1
+    assert L.tmb_gemm(None, None, None, None, 0, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32,
+                      ek.EPI_GELU_TANH | ek.EPI_ROUND_LIKE_UNFUSED, None) == 0
+    assert L.tmb_gemm_residual(None, None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, 0,
+                               ek.BF16, ek.F16, ek.BF16, 0, None) == -1   # NULL residual comes first
+    fake = ctypes.c_void_p(4096)   # never dereferenced: rejected on the host
+    assert L.tmb_gemm_residual(fake, fake, fake, None, fake, 1, 2, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, 0,
+                               ek.BF16, ek.F16, ek.BF16, 0, None) == -2   # residual type: T or fp32
+    assert L.tmb_gemm_residual(fake, fake, fake, None, fake, 1, 2, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, 0,
+                               ek.F32, ek.F32, ek.F32, 0, None) == -2     # fp32 A/B: caller adds separately
     assert L.tmb_gemm_ws(None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, ek.F32, 0, None, 0,
                          None) == -1
     assert L.tmb_gelu_backward(None, None, None, 8, ek.F32, 0, None) == -1

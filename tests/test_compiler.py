@@ -136,8 +136,9 @@ def cpu_hot_ops(monkeypatch):
     # the fusion pass keys on the built-in entries; point it at the stand-ins
     monkeypatch.setattr(compiler, "_BUILTIN_ADDMM", fake[aten.addmm])
     monkeypatch.setattr(compiler, "_BUILTIN_GELU", fake[aten.gelu])
+    monkeypatch.setattr(compiler, "_BUILTIN_LAYER_NORM", ln)
     monkeypatch.setattr(af, "addmm_gelu",
-                        rec("addmm_gelu", lambda i, a, b, approx: torch.nn.functional.gelu(
+                        rec("addmm_gelu", lambda i, a, b, approx, twice=False: torch.nn.functional.gelu(
                             torch.addmm(i, a, b), approximate=approx)))
     return log
 
@@ -154,6 +155,74 @@ def test_executor_runs_a_model_and_fuses_bias_gelu(cpu_hot_ops):
     assert "addmm_gelu" in cpu_hot_ops and "gelu" not in cpu_hot_ops
     assert cpu_hot_ops.count("addmm") == 1          # the second Linear
     assert "ln_first_only" in cpu_hot_ops           # inference graph: statistics are dead
+
+
+class _TwoBlocks(torch.nn.Module):
+    """x <- x + proj(norm(x)), twice, then a final norm: the residual stream of a decoder."""
+
+    def __init__(self):
+        super().__init__()
+        self.n1, self.n2, self.nf = (torch.nn.LayerNorm(16) for _ in range(3))
+        self.p1, self.p2 = torch.nn.Linear(16, 16), torch.nn.Linear(16, 16)
+        self.head = torch.nn.Linear(16, 4, bias=False)
+
+    def forward(self, x):
+        x = x + self.p1(self.n1(x))
+        x = x + self.p2(self.n2(x))
+        return self.head(self.nf(x))
+
+
+def _plans_of(model, x, monkeypatch):
+    seen = []
+    real = compiler._GraphFactory._widen_residual_stream
+
+    def spy(plans):
+        real(plans)
+        seen.append({n.name: p for n, p in plans.items() if p is not None})
+
+    monkeypatch.setattr(compiler._GraphFactory, "_widen_residual_stream", staticmethod(spy))
+    with torch.no_grad():
+        out = torch.compile(model, backend=mojo_backend, fullgraph=True)(x)
+    return out, (seen[-1] if seen else {})
+
+
+def test_residual_stream_of_a_16_bit_graph_is_kept_in_float32(cpu_hot_ops, monkeypatch):
+    torch.manual_seed(0)
+    model = _TwoBlocks().eval().to(torch.bfloat16)
+    x = torch.randn(2, 5, 16).to(torch.bfloat16)
+    out, plans = _plans_of(model, x, monkeypatch)
+    residual = [p for p in plans.values() if p[0] == "residual"]
+    norms = [p for p in plans.values() if p[0] == "wide_ln"]
+    # both residual adds hand float32 on (their consumers are the next add and layer norms);
+    # the two layer norms behind them read float32 and produce bfloat16
+    assert len(residual) == 2 and all(p[6] is torch.float32 for p in residual)
+    assert len(norms) == 2 and all(p[1] is torch.bfloat16 for p in norms)
+    assert out.dtype == torch.bfloat16
+    with torch.no_grad():
+        torch.testing.assert_close(out.float(), model.float()(x.float()), rtol=5e-2, atol=5e-2)
+
+
+def test_residual_stream_stays_narrow_when_something_else_reads_it(cpu_hot_ops, monkeypatch):
+    class Leaky(_TwoBlocks):
+        def forward(self, x):
+            x = x + self.p1(self.n1(x))
+            y = x + self.p2(self.n2(x))
+            return self.head(self.nf(y)), x          # the first stream value is a graph output
+
+    torch.manual_seed(0)
+    model = Leaky().eval().to(torch.bfloat16)
+    (out, leaked), plans = _plans_of(model, torch.randn(2, 5, 16).to(torch.bfloat16), monkeypatch)
+    residual = [p for p in plans.values() if p[0] == "residual"]
+    assert sorted(str(p[6]) for p in residual) == ["None", "torch.float32"]
+    assert leaked.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+    # float32 graphs and the bit-identical mode leave the graph's dtypes alone
+    _, plans32 = _plans_of(_TwoBlocks().eval(), torch.randn(2, 5, 16), monkeypatch)
+    assert all(p[6] is None for p in plans32.values() if p[0] == "residual")
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED", "1")
+    torch.compiler.reset()
+    _, plans_twice = _plans_of(_TwoBlocks().eval().to(torch.bfloat16),
+                               torch.randn(2, 5, 16).to(torch.bfloat16), monkeypatch)
+    assert plans_twice == {}                          # the widening pass is not even entered
 
 
 def test_fusion_can_be_switched_off(cpu_hot_ops, monkeypatch):

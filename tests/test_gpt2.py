@@ -54,15 +54,15 @@ def test_gpt2_small_fp32_batch1_seq128_matches_cpu_eager():
 
 
 def test_gpt2_small_bf16_logits_vs_fp32_oracle():
-    """bf16 weights/activations on the GPU vs float32 CPU eager on the same bf16-rounded weights.
+    """bf16 weights/activations on the GPU vs float32 CPU eager on the same bf16-rounded weights:
+    max-abs logit error <= 2e-2, the bound the workload definition states.
 
-    The workload definition asks for max-abs 2e-2. Measured on MI355X this graph lands at
-    2.9e-2 .. 3.2e-2 — and so does PyTorch-ROCm's own bf16 eager run of the same module
-    (3.1e-2): with logits up to |3| the final bf16 rounding alone costs 7.8e-3 and the rest is the
-    bf16 storage rounding between the graph's ~700 ops, which belongs to the graph, not to a
-    kernel. The test therefore pins what a kernel can be held to: no worse than the vendor's
-    bf16 pipeline on the same input (10% slack), a hard cap of 4e-2, and a mean error of 6e-3
-    (the vendor's is 4.6e-3)."""
+    What makes the bound reachable is the graph executor, not a kernel: a bf16 pipeline that
+    rounds the residual stream to bf16 after each of its 24 adds lands at 2.9e-2 .. 3.6e-2
+    (PyTorch-ROCm's bf16 eager run and PyTorch's CPU bf16 eager run of the same module, both
+    printed below, as well as this backend with TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED=1). The
+    executor keeps that stream in float32 between the fused residual GEMMs and the layer norms
+    that read it, and evaluates fused GELU / residual epilogues in float32 up to their one cast."""
     from torch_mojo_backend import mojo_backend
 
     model = build_gpt2_small(seed=0)
@@ -70,6 +70,7 @@ def test_gpt2_small_bf16_logits_vs_fp32_oracle():
     idx = seeded_tokens(2, 256, seed=1)
     with torch.no_grad():
         want_logits, _ = model(idx)
+        cpu_bf16_logits, _ = build_gpt2_small(seed=0).to(torch.bfloat16)(idx)
     gpu_model = build_gpt2_small(seed=0).to(torch.bfloat16).to("cuda")
     with torch.no_grad():
         vendor_logits, _ = gpu_model(idx.to("cuda"))
@@ -79,20 +80,121 @@ def test_gpt2_small_bf16_logits_vs_fp32_oracle():
     assert logits.dtype == torch.bfloat16
     err = (logits.float().cpu() - want_logits).abs()
     vendor_err = (vendor_logits.float().cpu() - want_logits).abs()
-    print(f"max-abs logit error: ours {err.max().item():.4f}, PyTorch-ROCm bf16 eager "
-          f"{vendor_err.max().item():.4f}; mean {err.mean().item():.5f} vs {vendor_err.mean().item():.5f}")
-    assert err.max().item() <= max(2e-2, 1.1 * vendor_err.max().item())
-    assert err.max().item() <= 4e-2
-    assert err.mean().item() <= 6e-3
+    cpu16_err = (cpu_bf16_logits.float() - want_logits).abs()
+    vs_cpu16 = (logits.float().cpu() - cpu_bf16_logits.float()).abs()
+    print(f"max-abs logit error vs the float32 model: ours {err.max().item():.4f} (mean "
+          f"{err.mean().item():.5f}); PyTorch-ROCm bf16 eager {vendor_err.max().item():.4f} "
+          f"({vendor_err.mean().item():.5f}); PyTorch CPU bf16 eager {cpu16_err.max().item():.4f} "
+          f"({cpu16_err.mean().item():.5f}); ours vs CPU bf16 eager {vs_cpu16.max().item():.4f}")
+    assert err.max().item() <= 2e-2
+    assert err.mean().item() <= 3e-3
+    # two bf16 pipelines differ from each other by more than either differs from float32 (their
+    # storage roundings are independent): the reference's same-dtype check against CPU eager
+    # (torch_mojo_backend/testing.py:186-229) holds at its own bf16 tolerance, not at 2e-2
+    assert vs_cpu16.max().item() <= 1.25 * cpu16_err.max().item() + 1e-2
     assert torch.equal(nxt.cpu(), torch.argmax(logits[:, -1, :], dim=-1).cpu())
 
 
+def test_gpt2_small_bf16_bit_identical_mode_matches_the_vendor_pipeline(monkeypatch):
+    """TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED=1: every tensor of the graph is rounded where the
+    unfused kernels would have stored it; the logit error is then that of any bf16 pipeline."""
+    from torch_mojo_backend import mojo_backend
+
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED", "1")
+    model = build_gpt2_small(seed=0).to(torch.bfloat16).to(torch.float32)
+    idx = seeded_tokens(2, 256, seed=1)
+    with torch.no_grad():
+        want_logits, _ = model(idx)
+    gpu_model = build_gpt2_small(seed=0).to(torch.bfloat16).to("cuda")
+    with torch.no_grad():
+        vendor_logits, _ = gpu_model(idx.to("cuda"))
+        logits, _ = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx.to("cuda"))
+    err = (logits.float().cpu() - want_logits).abs()
+    vendor_err = (vendor_logits.float().cpu() - want_logits).abs()
+    print(f"bit-identical mode: ours {err.max().item():.4f}, PyTorch-ROCm {vendor_err.max().item():.4f}")
+    assert err.max().item() <= 1.1 * vendor_err.max().item()
+    assert err.max().item() <= 3.6e-2
+    assert err.mean().item() <= 5e-3
+
+
+def test_gpt2_small_bf16_full_size_graph_routes_every_hot_op():
+    """The benchmark configuration itself (B=32, T=1024, bf16): every GEMM, layer norm, the
+    attention and the argmax run on the HIP kernels (call counts of the mapping functions and of
+    the fused steps), the argmax is exact on the graph's own logits, and rows sampled from the
+    logits equal those of the same graph without the attention rewrite up to the reordered
+    storage roundings."""
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+    import os
+
+    B, T = 32, 1024
+    gpu_model = build_gpt2_small(seed=0).to(torch.bfloat16).to("cuda")
+    idx = seeded_tokens(B, T, seed=0).to("cuda")
+    hip_ops = compiler.aten_functions.hip_ops
+    counts = {"gemm": 0, "attention": 0, "layer_norm": 0, "argmax": 0, "embedding": 0, "residual": 0,
+              "gelu_epilogue": 0, "wide_out": 0, "wide_ln": 0}
+    real = {n: getattr(hip_ops, n) for n in ("gemm", "attention", "layer_norm", "argmax", "embedding")}
+
+    def gemm(a, b, bias=None, epilogue=0, residual=None, out_dtype=None, round_like_unfused=False):
+        counts["gemm"] += 1
+        counts["residual"] += residual is not None
+        counts["gelu_epilogue"] += epilogue != 0
+        counts["wide_out"] += out_dtype is torch.float32
+        return real["gemm"](a, b, bias, epilogue, residual, out_dtype, round_like_unfused)
+
+    def layer_norm(x, shape, w, b, eps, need_stats=True, out_dtype=None):
+        counts["layer_norm"] += 1
+        counts["wide_ln"] += x.dtype == torch.float32 and out_dtype == torch.bfloat16
+        return real["layer_norm"](x, shape, w, b, eps, need_stats, out_dtype)
+
+    def counted(name):
+        def run(*a, **k):
+            counts[name] += 1
+            return real[name](*a, **k)
+        return run
+
+    patched = {"gemm": gemm, "layer_norm": layer_norm, "attention": counted("attention"),
+               "argmax": counted("argmax"), "embedding": counted("embedding")}
+    for n, f in patched.items():
+        setattr(hip_ops, n, f)
+    try:
+        with torch.no_grad():
+            logits, nxt = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    finally:
+        for n, f in real.items():
+            setattr(hip_ops, n, f)
+    assert logits.shape == (B, T, 50257) and logits.dtype == torch.bfloat16
+    # per layer: c_attn, c_proj (+residual), c_fc (+gelu), c_proj (+residual); plus lm_head
+    assert counts["gemm"] == 12 * 4 + 1
+    assert counts["residual"] == 24 and counts["gelu_epilogue"] == 12
+    assert counts["wide_out"] == 24 and counts["wide_ln"] == 24       # float32 residual stream
+    assert counts["attention"] == 12 and counts["layer_norm"] == 25
+    assert counts["argmax"] == 1 and counts["embedding"] == 2
+    assert torch.equal(nxt, torch.argmax(logits[:, -1, :].float(), dim=-1))
+    rows = [(0, 0), (0, 1023), (7, 511), (31, 0), (31, 1023)]
+    picked = torch.stack([logits[b, t] for b, t in rows]).float()
+    del logits
+    os.environ["TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION"] = "1"
+    try:
+        torch.compiler.reset()
+        with torch.no_grad():
+            plain, nxt_plain = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)(idx)
+    finally:
+        del os.environ["TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION"]
+    other = torch.stack([plain[b, t] for b, t in rows]).float()
+    diff = (picked - other).abs()
+    assert diff.max().item() <= 3e-2 and diff.mean().item() <= 2.0 ** -8
+    assert (nxt == nxt_plain).float().mean().item() >= 0.9
+
+
 def test_fusion_is_bit_identical_to_unfused(monkeypatch):
-    """The addmm->gelu and mul+masked_fill+softmax rewrites must not change a single bit of the
-    logits (the attention rewrite reorders roundings and is checked to a tolerance below)."""
+    """With TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED=1 the addmm->gelu, addmm->add and
+    mul+masked_fill+softmax rewrites must not change a single bit of the logits (the attention
+    rewrite reorders roundings and is checked to a tolerance below)."""
     from torch_mojo_backend import mojo_backend
 
     monkeypatch.setenv("TORCH_MOJO_BACKEND_NO_ATTENTION_FUSION", "1")
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED", "1")
     gpu_model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).to("cuda")
     idx = seeded_tokens(2, 64, seed=2).to("cuda")
     with torch.no_grad():
@@ -193,7 +295,9 @@ def test_attention_fusion_stays_within_the_storage_rounding(monkeypatch):
         want, _ = ref_model(idx.cpu())
     err_fused = (fused.float().cpu() - want).abs()
     err_plain = (plain.float().cpu() - want).abs()
-    assert err_fused.max().item() <= max(2e-2, 1.25 * err_plain.max().item())
+    print(f"attention fusion: max-abs error fused {err_fused.max().item():.4f}, unfused "
+          f"{err_plain.max().item():.4f}")
+    assert err_fused.max().item() <= 2e-2
     assert err_fused.mean().item() <= 1.1 * err_plain.mean().item() + 1e-4
     # and the two agree to about one bf16 spacing of a logit of magnitude ~1 (2^-7) on average
     diff = (fused.float() - plain.float()).abs()
@@ -206,6 +310,7 @@ def test_attention_fusion_falls_back_for_a_non_causal_buffer(monkeypatch):
     from torch_mojo_backend import mojo_backend
     from torch_mojo_backend.torch_compile_backend import compiler
 
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED", "1")
     gpu_model = build_gpt2_small(seed=0, n_layer=1).to(torch.bfloat16).to("cuda")
     for block in gpu_model.transformer.h:
         block.attn.bias[0, 0, 5, 40] = 1.0      # one key above the diagonal becomes visible

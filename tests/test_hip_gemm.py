@@ -176,7 +176,8 @@ def test_bmm_benchmark_shape_bf16():
 @pytest.mark.parametrize("approximate", ["tanh", "none"])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_gelu_epilogue_equals_unfused(dtype, approximate, trans_b):
-    """The fused epilogue must be bit-identical to addmm followed by the standalone GELU."""
+    """round_like_unfused: bit-identical to addmm followed by the standalone GELU. Default: the
+    GELU of the float32 sum, one cast - within one rounding of the float64 closed form."""
     m, n, k = 200, 3072, 768
     a, b, bias = _abc(m, n, k, dtype, seed=9)
     b = (b * 0.05).to(dtype)
@@ -184,13 +185,20 @@ def test_gelu_epilogue_equals_unfused(dtype, approximate, trans_b):
         b = b.t().contiguous().t()
     ek = _ek()
     epi = ek.EPI_GELU_TANH if approximate == "tanh" else ek.EPI_GELU_ERF
-    fused = _ops().gemm(_dev(a), _dev(b), _dev(bias), epilogue=epi)
+    fused = _ops().gemm(_dev(a), _dev(b), _dev(bias), epilogue=epi, round_like_unfused=True)
     unfused = _ops().gelu(_ops().gemm(_dev(a), _dev(b), _dev(bias)), approximate)
     assert torch.equal(fused, unfused)
     pre = (a.double() @ b.double() + bias.double()).numpy()
     want = cf.gelu_tanh(pre) if approximate == "tanh" else cf.gelu_erf(pre)
     assert_close64(fused, want, rtol=2e-2 if dtype != torch.float32 else 1e-4, atol=2e-3,
                    what="gelu epilogue vs closed form")
+    # one cast: the float32 accumulation error (k products of magnitude ~0.05) goes through a
+    # function of slope <= 1.13, then half a unit of the storage type
+    once = _ops().gemm(_dev(a), _dev(b), _dev(bias), epilogue=epi)
+    acc_err = 1.13 * k * 2.0 ** -24 * (a.double().abs() @ b.double().abs()).numpy()
+    assert_close64(once, want, rtol=1e-5, atol=1e-6, extra_abs=acc_err, what="gelu of the fp32 sum")
+    if dtype == torch.float32:
+        assert torch.equal(once, fused)          # nothing to round in between
 
 
 @pytest.mark.parametrize("dtype", [torch.float32] + HALF)
@@ -249,9 +257,11 @@ def test_queued_launches_are_bit_identical():
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
 
 
-# residual added in the GEMM's own epilogue: must give the bits of gemm(...) + residual. Shapes
-# cover the ring configurations (see KMAJOR), the register-staged kernel (K = 128) and an odd
-# row pitch; float32 has no fused path and takes the separate add inside the same call.
+# residual added in the GEMM's own epilogue. With round_like_unfused it must give the bits of
+# gemm(...) + residual; by default the sum is formed in float32 and cast once, and residual and
+# result may be float32 next to 16-bit operands. Shapes cover the ring configurations (see
+# KMAJOR), the register-staged kernel (K = 128) and an odd row pitch; float32 operands have no
+# fused path and take the separate add inside the same call.
 RESIDUAL = [(3900, 4000, 320), (4000, 4104, 448), (600, 1000, 352), (8000, 2200, 352),
             (1000, 5000, 128), (512, 50257, 768), (32768, 768, 768)]
 
@@ -267,9 +277,65 @@ def test_residual_epilogue_equals_separate_add(mnk, dtype, trans_b):
     b = b.t() if trans_b else b.t().contiguous()
     bias = torch.randn(n, generator=g, device="cuda").to(dtype)
     res = torch.randn(m, n, generator=g, device="cuda").to(dtype)
-    fused = _ops().gemm(a, b, bias, residual=res)
+    fused = _ops().gemm(a, b, bias, residual=res, round_like_unfused=True)
     plain = _ops().gemm(a, b, bias) + res
     assert torch.equal(fused, plain)
+
+
+def _residual_reference(a, b, bias, rows):
+    """float64 a[rows] @ b + bias on the device, plus the fp32 accumulation bound."""
+    a64, b64 = a[rows].double(), b.double()
+    exact = a64 @ b64 + bias.double()
+    bound = a.shape[1] * 2.0 ** -24 * (a64.abs() @ b64.abs())
+    return exact, bound
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", RESIDUAL)
+@pytest.mark.parametrize("resid_f32,out_f32", [(False, False), (True, True), (True, False), (False, True)])
+def test_residual_epilogue_in_float32_one_cast(mnk, dtype, resid_f32, out_f32):
+    """Default mode: c = OUT(acc + bias + residual), everything in float32 up to the one cast;
+    residual and result in the operands' type or float32. Checked on sampled rows against
+    float64 (the accumulation bound plus half a unit of the output type)."""
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(23)
+    a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
+    b = (torch.randn(n, k, generator=g, device="cuda") * 0.1).to(dtype).t()
+    bias = torch.randn(n, generator=g, device="cuda").to(dtype)
+    res = torch.randn(m, n, generator=g, device="cuda") * 3
+    res = res if resid_f32 else res.to(dtype)
+    out = _ops().gemm(a, b, bias, residual=res, out_dtype=torch.float32 if out_f32 else None)
+    assert out.dtype == (torch.float32 if out_f32 else dtype) and tuple(out.shape) == (m, n)
+    rows = torch.tensor(sorted({0, 1, 31, 32, 127, 128, 255, 256, m // 2, m - 129, m - 2, m - 1}),
+                        device="cuda")
+    exact, bound = _residual_reference(a, b, bias, rows)
+    want = (exact + res[rows].double()).cpu().numpy()
+    assert_close64(out[rows], want, rtol=1e-6, atol=1e-6, extra_abs=bound.cpu().numpy(),
+                   what=f"residual epilogue {mnk} resid_f32={resid_f32} out_f32={out_f32}")
+    if not resid_f32 and not out_f32:
+        # and it is closer to the truth than the unfused order, which rounds the product first
+        twice = _ops().gemm(a, b, bias, residual=res, round_like_unfused=True)
+        e_once = (out[rows].double() - torch.from_numpy(want).cuda()).abs().mean().item()
+        e_twice = (twice[rows].double() - torch.from_numpy(want).cuda()).abs().mean().item()
+        assert e_once <= e_twice
+
+
+def test_float32_stream_rejects_the_bit_identical_mode_and_composes_with_layer_norm():
+    g = torch.Generator(device="cuda").manual_seed(24)
+    a = torch.randn(512, 768, generator=g, device="cuda").bfloat16()
+    w = (torch.randn(768, 768, generator=g, device="cuda") * 0.02).bfloat16()
+    bias = torch.zeros(768, device="cuda").bfloat16()
+    x32 = torch.randn(512, 768, generator=g, device="cuda")
+    with pytest.raises(ValueError, match="round_like_unfused"):
+        _ops().gemm(a, w.t(), bias, residual=x32, round_like_unfused=True)
+    with pytest.raises(TypeError, match="residual only"):
+        _ops().gemm(a, w.t(), bias, out_dtype=torch.float32)
+    y32 = _ops().gemm(a, w.t(), bias, residual=x32, out_dtype=torch.float32)
+    gamma = torch.ones(768, device="cuda").bfloat16()
+    h, _, _ = _ops().layer_norm(y32, [768], gamma, bias, 1e-5, need_stats=False, out_dtype=torch.bfloat16)
+    want = torch.nn.functional.layer_norm(a.double() @ w.double().t() + x32.double(), [768])
+    assert h.dtype == torch.bfloat16
+    torch.testing.assert_close(h.double(), want, rtol=2.0 ** -8, atol=2.0 ** -8)
 
 
 def test_residual_with_gelu_batches_and_fallbacks():
@@ -278,14 +344,23 @@ def test_residual_with_gelu_batches_and_fallbacks():
     a = torch.randn(6, 300, 256, generator=g, device="cuda").bfloat16()
     b = (torch.randn(6, 256, 200, generator=g, device="cuda") * 0.1).bfloat16()
     res = torch.randn(6, 300, 200, generator=g, device="cuda").bfloat16()
-    assert torch.equal(_ops().gemm(a, b, residual=res), _ops().gemm(a, b) + res)
+    assert torch.equal(_ops().gemm(a, b, residual=res, round_like_unfused=True), _ops().gemm(a, b) + res)
+    # batched, one cast, float32 residual and result
+    got = _ops().gemm(a, b, residual=res.float(), out_dtype=torch.float32)
+    want = torch.bmm(a.double(), b.double()) + res.double()
+    torch.testing.assert_close(got.double(), want, rtol=1e-5, atol=1e-4)
     a2, b2, r2 = a[0], b[0], res[0]
     bias = torch.randn(200, generator=g, device="cuda").bfloat16()
-    fused = _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH, residual=r2)
-    assert torch.equal(fused, _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH) + r2)
+    fused = _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH, residual=r2, round_like_unfused=True)
+    assert torch.equal(fused, _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH,
+                                          round_like_unfused=True) + r2)
+    # GELU in front of a float32 add: no kernel, composed inside the same call, summed in float32
+    both = _ops().gemm(a2, b2, bias, epilogue=ek.EPI_GELU_TANH, residual=r2)
+    want = torch.nn.functional.gelu(a2.double() @ b2.double() + bias.double(), approximate="tanh") + r2.double()
+    torch.testing.assert_close(both.double(), want, rtol=2.0 ** -7, atol=2.0 ** -7)
     # a residual that is a column slice of something wider (row pitch > n)
     wide = torch.randn(300, 512, generator=g, device="cuda").bfloat16()
-    assert torch.equal(_ops().gemm(a2, b2, bias, residual=wide[:, 100:300]),
+    assert torch.equal(_ops().gemm(a2, b2, bias, residual=wide[:, 100:300], round_like_unfused=True),
                        _ops().gemm(a2, b2, bias) + wide[:, 100:300])
     # float32: no fused kernel, same call, same bits as the two ops
     a32, b32, r32 = a2.float(), b2.float(), r2.float()
@@ -421,9 +496,10 @@ def test_fp32_mfma_batched_strided_and_gelu():
     a2 = wide[:, 32:128]
     w = _dev(seeded((136, 96), seed=47, dtype=torch.float32))
     bias = _dev(seeded((136,), seed=48, dtype=torch.float32))
-    fused = _ops().gemm(a2, w.t(), bias, _ek().EPI_GELU_TANH)
+    fused = _ops().gemm(a2, w.t(), bias, _ek().EPI_GELU_TANH, round_like_unfused=True)
     unfused = _ops().gelu(_ops().gemm(a2, w.t(), bias), "tanh")
     assert torch.equal(fused, unfused)
+    assert torch.equal(fused, _ops().gemm(a2, w.t(), bias, _ek().EPI_GELU_TANH))   # float32: one mode
     want = as64(a2) @ as64(w).T + as64(bias)
     assert rel_frobenius(_ops().gemm(a2, w.t(), bias), want) <= 2e-6
 

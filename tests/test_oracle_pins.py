@@ -118,13 +118,86 @@ def test_gemm_bias_is_added_in_fp32_before_the_cast():
 
 
 @pytest.mark.parametrize("dtype", FLOATS)
-def test_gemm_gelu_epilogue_is_gelu_of_the_rounded_sum(dtype):
+def test_gemm_gelu_epilogue_both_rounding_modes(dtype):
     a, b, bias = seeded((9, 16), 1, dtype=dtype), seeded((16, 12), 2, dtype=dtype), seeded((12,), 3, dtype=dtype)
     pre = oracle.gemm(a, b, bias)
+    exact = as64(a) @ as64(b) + as64(bias)
     for epi, approx in ((oracle.EPI_GELU_TANH, "tanh"), (oracle.EPI_GELU_ERF, "none")):
-        fused = oracle.gemm(a, b, bias, epilogue=epi)
-        assert torch.equal(fused, oracle.gelu(pre, approx))
-        torch.testing.assert_close(fused, torch.nn.functional.gelu(pre, approximate=approx))
+        # like the unfused pair: gelu of the sum as a separate addmm kernel would have stored it
+        twice = oracle.gemm(a, b, bias, epilogue=epi, round_like_unfused=True)
+        assert torch.equal(twice, oracle.gelu(pre, approx))
+        torch.testing.assert_close(twice, torch.nn.functional.gelu(pre, approximate=approx))
+        # default: gelu of the float32 sum, one cast -> the correctly rounded gelu of the exact sum
+        once = oracle.gemm(a, b, bias, epilogue=epi)
+        want = torch.nn.functional.gelu(torch.from_numpy(exact), approximate=approx).numpy()
+        assert_close64(once, want, what=f"gelu({approx}) of the fp32 sum")
+    if dtype != torch.float32:
+        # a case where the two differ: acc + bias = 1 + 2^-9 is no bf16/fp16-tie-free number
+        a1 = torch.tensor([[1.0, 2.0 ** -9 if dtype == torch.bfloat16 else 2.0 ** -12]], dtype=dtype)
+        b1 = torch.ones(2, 1, dtype=dtype)
+        z = torch.zeros(1, dtype=dtype)
+        x = a1.double().sum().item()
+        once = oracle.gemm(a1, b1, z, epilogue=oracle.EPI_GELU_ERF).double().item()
+        twice = oracle.gemm(a1, b1, z, epilogue=oracle.EPI_GELU_ERF, round_like_unfused=True).double().item()
+        g = lambda v: 0.5 * v * (1 + math.erf(v / math.sqrt(2)))  # noqa: E731
+        assert once == torch.tensor(g(x), dtype=torch.float64).to(dtype).double().item()
+        assert twice == torch.tensor(g(1.0), dtype=torch.float64).to(dtype).double().item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_residual_rounding_modes_and_float32_stream(dtype):
+    a, b = seeded((7, 24), 4, dtype=dtype), seeded((24, 10), 5, dtype=dtype)
+    bias = seeded((10,), 6, dtype=dtype)
+    r32 = seeded((7, 10), 7, scale=3.0)
+    r16 = r32.to(dtype)
+    exact = as64(a) @ as64(b) + as64(bias)
+    # float32 residual in, float32 out: nothing is rounded to 16 bits anywhere
+    wide = oracle.gemm(a, b, bias, residual=r32, out_dtype=torch.float32)
+    assert wide.dtype == torch.float32
+    np.testing.assert_allclose(as64(wide), exact + as64(r32), rtol=1e-6, atol=1e-6)
+    # float32 residual in, 16-bit out; 16-bit residual in, float32 out; 16-bit both: one rounding
+    assert_close64(oracle.gemm(a, b, bias, residual=r32), exact + as64(r32), what="f32 residual")
+    np.testing.assert_allclose(as64(oracle.gemm(a, b, bias, residual=r16, out_dtype=torch.float32)),
+                               exact + as64(r16), rtol=1e-6, atol=1e-6)
+    once = oracle.gemm(a, b, bias, residual=r16)
+    assert_close64(once, exact + as64(r16), what="one rounding")
+    # like the unfused pair: PyTorch CPU's addmm (fp32 accumulate, one cast) followed by add
+    twice = oracle.gemm(a, b, bias, residual=r16, round_like_unfused=True)
+    assert torch.equal(twice, oracle.gemm(a, b, bias) + r16)
+    torch.testing.assert_close(twice, torch.addmm(bias, a, b) + r16)
+    # the two orders are told apart: the product 1 + eps (half a spacing of the storage type at 1)
+    # rounds to 1 before the residual eps is added in the unfused order; in float32 the sum
+    # 1 + 2 eps is exact and representable
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    a1, b1 = torch.tensor([[1.0, eps]], dtype=dtype), torch.ones(2, 1, dtype=dtype)
+    res = torch.tensor([[eps]], dtype=dtype)
+    assert oracle.gemm(a1, b1, None, residual=res).double().item() == 1.0 + 2 * eps
+    assert oracle.gemm(a1, b1, None, residual=res, round_like_unfused=True).double().item() == 1.0
+    # batched, and a transposed operand
+    a3, b3 = seeded((3, 5, 8), 8, dtype=dtype), seeded((3, 6, 8), 9, dtype=dtype).transpose(1, 2)
+    rr = seeded((3, 5, 6), 10)
+    got = oracle.gemm(a3, b3, None, residual=rr, out_dtype=torch.float32)
+    np.testing.assert_allclose(as64(got), np.einsum("bmk,bkn->bmn", as64(a3), as64(b3)) + as64(rr),
+                               rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_layer_norm_float32_rows_into_16_bit_output(out_dtype):
+    x = seeded((6, 200), 11, scale=2.0, shift=0.5)
+    g = seeded((200,), 12, scale=0.1, shift=1.0, dtype=out_dtype)
+    b = seeded((200,), 13, scale=0.1, dtype=out_dtype)
+    out, mean, rstd = oracle.layer_norm_rows(x, g, b, 1e-5, out_dtype=out_dtype)
+    assert out.dtype == out_dtype and mean.dtype == torch.float32
+    w_out, w_mean, w_rstd = cf.layer_norm(as64(x), as64(g), as64(b), 1e-5)
+    scale = np.abs(as64(x) - w_mean) * w_rstd * np.abs(as64(g)) + np.abs(as64(b))
+    assert_close64(out, w_out, extra_abs=1e-5 * scale)
+    assert_close64(mean.reshape(-1, 1), w_mean, atol=1e-6)
+    assert_close64(rstd.reshape(-1, 1), w_rstd, rtol=1e-5)
+    # the statistics come from the float32 values, not from values rounded to the output type
+    rounded, m16, _ = oracle.layer_norm_rows(x.to(out_dtype), g, b, 1e-5)
+    assert not torch.equal(m16, mean)
+    same, m32, _ = oracle.layer_norm_rows(x, g.float(), b.float(), 1e-5)
+    assert torch.equal(m32, mean) and torch.equal(same.to(out_dtype), out)
 
 
 # ---------------------------------------------------------------------------

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void gemm_simt_kernel(
     T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b,
     const T* __restrict__ bias, int64_t m, int64_t n, int64_t k, int64_t sa_m, int64_t sa_k,
     int64_t sb_k, int64_t sb_n, int64_t ldc, int64_t stride_a, int64_t stride_b,
-    int64_t stride_c, int64_t tiles_n) {
+    int64_t stride_c, int64_t tiles_n, bool twice) {
   constexpr int TM = 64, TN = 64, TK = 16;
   __shared__ float As[TK][TM + 4];
   __shared__ float Bs[TK][TN + 4];
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void gemm_simt_kernel(
       if (gn >= n) continue;
       float v = acc[i][j];
       if (bias != nullptr) v += to_f32(bias[gn]);
-      c[gm * ldc + gn] = finish<T, EPI>(v);
+      c[gm * ldc + gn] = finish<T, EPI>(v, twice);
     }
   }
 }
@@ -148,7 +148,7 @@ static int launch_simt(const GemmArgs& g, int64_t batch, int trans_a, int trans_
   gemm_simt_kernel<T, EPI><<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(256), 0, stream>>>(
       static_cast<T*>(g.c), static_cast<const T*>(g.a), static_cast<const T*>(g.b),
       static_cast<const T*>(g.bias), g.m, g.n, g.k, sa_m, sa_k, sb_k, sb_n, g.ldc, g.stride_a,
-      g.stride_b, g.stride_c, tiles_n);
+      g.stride_b, g.stride_c, tiles_n, g.round_like_unfused != 0);
   return check_launch();
 }
 
@@ -262,7 +262,7 @@ static int launch_splitk(const GemmArgs& g, const SplitKPlan& plan, int trans_a,
   }
   if (rc != 0) return rc;
   launch_splitk_reduce<T, EPI>(static_cast<T*>(g.c), workspace, static_cast<const T*>(g.bias), g.m,
-                               g.n, g.ldc, plan.splits, stream);
+                               g.n, g.ldc, plan.splits, g.round_like_unfused != 0, stream);
   return check_launch();
 }
 
@@ -300,7 +300,7 @@ static int launch_splitk_f32(const GemmArgs& g, const SplitKPlan& plan, int tran
   if (rc != 0) return rc;
   launch_splitk_reduce<float, EPI>(static_cast<float*>(g.c), workspace,
                                    static_cast<const float*>(g.bias), g.m, g.n, g.ldc, plan.splits,
-                                   stream);
+                                   false, stream);
   return check_launch();
 }
 
@@ -352,14 +352,14 @@ static int gemm_epi(const GemmArgs& g, int64_t batch, int ta, int tb, int epilog
 // Fills C with epilogue(bias) (or zeros) when k == 0.
 template <typename T, int EPI>
 __global__ void gemm_k0_kernel(T* c, const T* bias, int64_t m, int64_t n, int64_t ldc,
-                               int64_t stride_c) {
+                               int64_t stride_c, bool twice) {
   T* cb = c + static_cast<int64_t>(blockIdx.y) * stride_c;
   const int64_t total = m * n;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const int64_t r = i / n, col = i - r * n;
     const float v = bias != nullptr ? to_f32(bias[col]) : 0.0f;
-    cb[r * ldc + col] = finish<T, EPI>(v);
+    cb[r * ldc + col] = finish<T, EPI>(v, twice);
   }
 }
 
@@ -369,12 +369,24 @@ static int gemm_entry(void* c, const void* a, const void* b, const void* bias,
                       const void* residual, int64_t batch, int64_t m, int64_t n, int64_t k,
                       int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr, int64_t stride_a,
                       int64_t stride_b, int64_t stride_c, int64_t stride_r, int trans_a,
-                      int trans_b, int dtype, int epilogue, void* stream,
-                      void* workspace = nullptr, size_t workspace_bytes = 0) {
+                      int trans_b, int dtype, int epilogue_flags, void* stream,
+                      void* workspace = nullptr, size_t workspace_bytes = 0,
+                      int residual_dtype = -1, int out_dtype = -1) {
   using namespace tmb;
   if (batch < 0 || m < 0 || n < 0 || k < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (epilogue_flags < 0 || (epilogue_flags & ~(0xff | TMB_EPI_ROUND_LIKE_UNFUSED)) != 0)
+    return TMB_ERR_INVALID_ARGUMENT;
+  const int epilogue = epilogue_flags & 0xff;
+  const bool twice = (epilogue_flags & TMB_EPI_ROUND_LIKE_UNFUSED) != 0;
   if (epilogue < TMB_EPI_NONE || epilogue > TMB_EPI_GELU_ERF) return TMB_ERR_INVALID_ARGUMENT;
   if (dtype != TMB_F32 && dtype != TMB_F16 && dtype != TMB_BF16) return TMB_ERR_UNSUPPORTED;
+  if (residual_dtype < 0) residual_dtype = dtype;
+  if (out_dtype < 0) out_dtype = dtype;
+  if ((residual_dtype != dtype && residual_dtype != TMB_F32) ||
+      (out_dtype != dtype && out_dtype != TMB_F32))
+    return TMB_ERR_UNSUPPORTED;
+  const bool resid_f32 = residual != nullptr && residual_dtype == TMB_F32 && dtype != TMB_F32;
+  const bool out_f32 = out_dtype == TMB_F32 && dtype != TMB_F32;
   if (batch == 0 || m == 0 || n == 0) return TMB_OK;
   if (c == nullptr) return TMB_ERR_INVALID_ARGUMENT;
   if (k > 0 && (a == nullptr || b == nullptr)) return TMB_ERR_INVALID_ARGUMENT;
@@ -387,19 +399,26 @@ static int gemm_entry(void* c, const void* a, const void* b, const void* bias,
   if (batch > 65535) return TMB_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   GemmArgs g{c, a, b, bias, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, 0, 0, 0, residual, ldr, stride_r};
+  g.round_like_unfused = twice ? 1 : 0;
+  g.resid_f32 = resid_f32 ? 1 : 0;
+  g.out_f32 = out_f32 ? 1 : 0;
+  if (out_f32 && residual == nullptr) return TMB_ERR_UNSUPPORTED;  // fp32 C exists for the residual form only
   if (residual != nullptr) {
     // only the MFMA kernels carry the second epilogue step; the caller adds separately otherwise
     if (dtype == TMB_F32 || k == 0 || ldr < n || !mfma_eligible(g, batch, trans_a, trans_b))
       return TMB_ERR_UNSUPPORTED;
+    // fp32 operands of the epilogue and an epilogue that stays in fp32 exist without GELU only
+    if ((resid_f32 || out_f32 || !twice) && epilogue != TMB_EPI_NONE) return TMB_ERR_UNSUPPORTED;
+    if ((resid_f32 || out_f32) && twice) return TMB_ERR_INVALID_ARGUMENT;
   }
   if (k == 0) {
     const unsigned blocks = static_cast<unsigned>((m * n + 255) / 256 > 4096 ? 4096 : (m * n + 255) / 256);
     dim3 grid(blocks, static_cast<unsigned>(batch));
 #define TMB_K0(T)                                                                                   \
   switch (epilogue) {                                                                               \
-    case TMB_EPI_NONE: gemm_k0_kernel<T, TMB_EPI_NONE><<<grid, 256, 0, s>>>((T*)c, (const T*)bias, m, n, ldc, stride_c); break; \
-    case TMB_EPI_GELU_TANH: gemm_k0_kernel<T, TMB_EPI_GELU_TANH><<<grid, 256, 0, s>>>((T*)c, (const T*)bias, m, n, ldc, stride_c); break; \
-    default: gemm_k0_kernel<T, TMB_EPI_GELU_ERF><<<grid, 256, 0, s>>>((T*)c, (const T*)bias, m, n, ldc, stride_c); break; \
+    case TMB_EPI_NONE: gemm_k0_kernel<T, TMB_EPI_NONE><<<grid, 256, 0, s>>>((T*)c, (const T*)bias, m, n, ldc, stride_c, twice); break; \
+    case TMB_EPI_GELU_TANH: gemm_k0_kernel<T, TMB_EPI_GELU_TANH><<<grid, 256, 0, s>>>((T*)c, (const T*)bias, m, n, ldc, stride_c, twice); break; \
+    default: gemm_k0_kernel<T, TMB_EPI_GELU_ERF><<<grid, 256, 0, s>>>((T*)c, (const T*)bias, m, n, ldc, stride_c, twice); break; \
   }
     if (dtype == TMB_F32) { TMB_K0(float) } else if (dtype == TMB_F16) { TMB_K0(f16_t) } else { TMB_K0(bf16_t) }
 #undef TMB_K0
@@ -444,8 +463,10 @@ extern "C" int tmb_gemm_residual(void* c, const void* a, const void* b, const vo
                                  int64_t k, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr,
                                  int64_t stride_a, int64_t stride_b, int64_t stride_c,
                                  int64_t stride_r, int trans_a, int trans_b, int dtype,
-                                 int epilogue, void* stream) {
+                                 int residual_dtype, int out_dtype, int epilogue, void* stream) {
   if (residual == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  if (residual_dtype < 0 || out_dtype < 0) return TMB_ERR_INVALID_ARGUMENT;
   return gemm_entry(c, a, b, bias, residual, batch, m, n, k, lda, ldb, ldc, ldr, stride_a,
-                    stride_b, stride_c, stride_r, trans_a, trans_b, dtype, epilogue, stream);
+                    stride_b, stride_c, stride_r, trans_a, trans_b, dtype, epilogue, stream, nullptr,
+                    0, residual_dtype, out_dtype);
 }

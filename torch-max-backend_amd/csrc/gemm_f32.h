@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const GemmArgs g) {
         for (int e = 0; e < 4; ++e) {
           float v = acc[i][j][4 * q + e];
           if (bias != nullptr && col + e < g.n) v += bias[col + e];
-          out[e] = finish<float, EPI>(v);
+          out[e] = finish<float, EPI>(v, false);
         }
         if (col + 4 <= g.n) {
           const f32x4_unaligned_t v = {out[0], out[1], out[2], out[3]};

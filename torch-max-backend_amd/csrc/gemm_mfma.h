@@ -21,16 +21,18 @@
 
 namespace tmb {
 
-// Bias has already been added in fp32. With a GELU epilogue the sum is first rounded to the
-// storage type, so that the fused kernel returns exactly what addmm followed by a separate
-// gelu returns; then one final cast.
+// Bias has already been added in fp32. A GELU epilogue works on that fp32 sum and the result is
+// cast once (the reference's rule for everything it fuses into a GEMM: form the value in fp32,
+// cast exactly once, matmul_ops.mojo:2651-2657). With `twice` the sum is first rounded to the
+// storage type, so that the fused kernel returns exactly the bits of addmm followed by a
+// separate gelu kernel.
 template <typename T, int EPI>
-__device__ __forceinline__ T finish(float v) {
+__device__ __forceinline__ T finish(float v, bool twice) {
   v = pin_f32(v);  // acc + bias is an fp32 sum; it is rounded to T as a separate step
   if constexpr (EPI == TMB_EPI_NONE) {
     return from_f32<T>(v);
   } else {
-    const float r = to_f32(from_f32<T>(v));
+    const float r = twice ? to_f32(from_f32<T>(v)) : v;
     return from_f32<T>(EPI == TMB_EPI_GELU_TANH ? gelu_tanh_f32(r) : gelu_erf_f32(r));
   }
 }
@@ -80,6 +82,13 @@ struct GemmArgs {
   // i.e. what a separate elementwise add after the GEMM would store (MFMA kernels only)
   const void* residual;
   int64_t ldr, stride_r;
+  // round_like_unfused: every fused step rounds to the storage type where a separate kernel
+  // would have stored (bit-identical to the unfused graph); otherwise the epilogue stays in fp32
+  // up to the one cast. resid_f32 / out_f32: the residual operand / C are fp32 although A and B
+  // are 16-bit (a residual stream kept in fp32); both need round_like_unfused == 0.
+  int round_like_unfused = 0;
+  int resid_f32 = 0;
+  int out_f32 = 0;
   // persistent kernels with a streamed output: workgroups start in four phases this many 10 ns
   // ticks apart, so that their store bursts do not all hit memory at the same moment
   int stagger_ticks = 0;
@@ -161,30 +170,55 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 }
 
 template <typename T, int EPI>
-__device__ __forceinline__ uint32_t finish2(float a, float b) {
+__device__ __forceinline__ uint32_t finish2(float a, float b, bool twice) {
   a = pin_f32(a);  // acc + bias is an fp32 sum; it is rounded to T as a separate step
   b = pin_f32(b);
-  uint32_t p = pack2<T>(a, b);
-  if constexpr (EPI != TMB_EPI_NONE) {
-    const float ra = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(p)));
-    const float rb = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(p >> 16)));
-    p = EPI == TMB_EPI_GELU_TANH ? pack2<T>(gelu_tanh_f32(ra), gelu_tanh_f32(rb))
-                                 : pack2<T>(gelu_erf_f32(ra), gelu_erf_f32(rb));
+  if constexpr (EPI == TMB_EPI_NONE) {
+    return pack2<T>(a, b);
+  } else {
+    if (twice) {  // wave-uniform
+      const uint32_t p = pack2<T>(a, b);
+      a = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(p)));
+      b = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(p >> 16)));
+    }
+    return EPI == TMB_EPI_GELU_TANH ? pack2<T>(gelu_tanh_f32(a), gelu_tanh_f32(b))
+                                    : pack2<T>(gelu_erf_f32(a), gelu_erf_f32(b));
   }
-  return p;
 }
 
 // One 32x32 accumulator tile into the band: +bias (fp32) -> optional GELU -> one cast, 4 x 8
 // bytes per lane. `bias` holds the lane's 16 bias values as fp32 (zeros without a bias).
 template <typename T, int EPI>
 __device__ __forceinline__ void stage_tile(const f32x16_t& acc, lds_byte_t* dst,
-                                           const float (&bias)[16]) {
+                                           const float (&bias)[16], bool twice) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     u32x2_t packed;
-    packed[0] = finish2<T, EPI>(acc[4 * q + 0] + bias[4 * q + 0], acc[4 * q + 1] + bias[4 * q + 1]);
-    packed[1] = finish2<T, EPI>(acc[4 * q + 2] + bias[4 * q + 2], acc[4 * q + 3] + bias[4 * q + 3]);
+    packed[0] = finish2<T, EPI>(acc[4 * q + 0] + bias[4 * q + 0], acc[4 * q + 1] + bias[4 * q + 1], twice);
+    packed[1] = finish2<T, EPI>(acc[4 * q + 2] + bias[4 * q + 2], acc[4 * q + 3] + bias[4 * q + 3], twice);
     *(lds_u32x2_t*)(dst + 16 * q) = packed;
+  }
+}
+
+// The fp32 form of the band, for epilogues that go on in fp32 after the bias (a residual added
+// before the one cast, or an fp32 output): 16 bytes per lane and 8-column group, row pitch
+// WN * 4 + 16 bytes, which keeps both the 16-byte writes (16 lanes = 16 rows, 4 banks apart)
+// and the row-wise 16-byte reads free of bank conflicts.
+template <int WN>
+struct BandLayoutF32 {
+  static constexpr int PITCH = WN * 4 + 16;
+  static constexpr int BYTES = 32 * PITCH;
+};
+typedef float f32x4_lds_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) f32x4_lds_t lds_f32x4_t;
+
+__device__ __forceinline__ void stage_tile_f32(const f32x16_t& acc, lds_byte_t* dst,
+                                               const float (&bias)[16]) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const f32x4_lds_t v = {acc[4 * q + 0] + bias[4 * q + 0], acc[4 * q + 1] + bias[4 * q + 1],
+                           acc[4 * q + 2] + bias[4 * q + 2], acc[4 * q + 3] + bias[4 * q + 3]};
+    *(lds_f32x4_t*)(dst + 32 * q) = v;
   }
 }
 
@@ -252,18 +286,116 @@ __device__ __forceinline__ void flush_band(const lds_byte_t* band, T* __restrict
   }
 }
 
+// What the epilogue does after bias (and GELU): nothing, or "+ residual", in the storage type
+// (twice) or in fp32 before the one cast.
+struct EpilogueArgs {
+  const void* residual;  // [M, N] with pitch ldr (already offset to the batch entry) or nullptr
+  int64_t ldr;
+  bool twice;            // round to the storage type after every fused step
+  bool resid_f32;        // residual elements are fp32 (else T)
+  bool out_f32;          // C elements are fp32 (else T)
+  // the fp32 band is needed unless everything is rounded step by step in T
+  __device__ __forceinline__ bool wide() const {
+    return residual != nullptr && (!twice || resid_f32 || out_f32);
+  }
+};
+
+typedef float f32x4_g_t __attribute__((ext_vector_type(4)));
+typedef f32x4_g_t __attribute__((aligned(4))) f32x4_g_unaligned_t;
+
+// Writes the staged fp32 band (32 x WN) to C: a lane takes 8 columns of a row, adds the residual
+// (8 x T or 8 x fp32) in fp32 and stores 8 x T (one 16-byte store) or 8 x fp32.
+template <typename T, int WN, bool STREAM>
+__device__ __forceinline__ void flush_band_wide(const lds_byte_t* band, void* __restrict__ Cv,
+                                                int64_t ldc, int64_t row0, int64_t col0, int64_t M,
+                                                int64_t N, const EpilogueArgs& ep, int lane) {
+  constexpr int PITCH = BandLayoutF32<WN>::PITCH;
+  constexpr int LPR = WN / 8;    // lanes per row
+  constexpr int RPP = 64 / LPR;  // rows per pass
+#pragma unroll
+  for (int p = 0; p < 32 / RPP; ++p) {
+    const int r = p * RPP + lane / LPR;
+    const int c = (lane % LPR) * 8;
+    const f32x4_lds_t lo = *(const lds_f32x4_t*)(band + r * PITCH + c * 4);
+    const f32x4_lds_t hi = *(const lds_f32x4_t*)(band + r * PITCH + c * 4 + 16);
+    float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    const int64_t row = row0 + r, col = col0 + c;
+    if (row >= M || col >= N) continue;
+    const bool whole = col + 8 <= N;
+    if (ep.resid_f32) {
+      const float* rsrc = static_cast<const float*>(ep.residual) + row * ep.ldr + col;
+      if (whole) {
+        const f32x4_g_t r0 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc);
+        const f32x4_g_t r1 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] += r0[e];
+          v[4 + e] += r1[e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) v[e] += rsrc[e];
+      }
+    } else {
+      const T* rsrc = static_cast<const T*>(ep.residual) + row * ep.ldr + col;
+      if (whole) {
+        const u32x4_t rv = *reinterpret_cast<const u32x4_unaligned_t*>(rsrc);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          v[e] += to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(rv[e >> 1] >> (16 * (e & 1)))));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) v[e] += to_f32(rsrc[e]);
+      }
+    }
+    if (ep.out_f32) {
+      float* dst = static_cast<float*>(Cv) + row * ldc + col;
+      if (whole) {
+        const f32x4_g_t o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+        if constexpr (STREAM) {
+          __builtin_nontemporal_store(o0, reinterpret_cast<f32x4_g_unaligned_t*>(dst));
+          __builtin_nontemporal_store(o1, reinterpret_cast<f32x4_g_unaligned_t*>(dst + 4));
+        } else {
+          *reinterpret_cast<f32x4_g_unaligned_t*>(dst) = o0;
+          *reinterpret_cast<f32x4_g_unaligned_t*>(dst + 4) = o1;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) dst[e] = v[e];
+      }
+    } else {
+      T* dst = static_cast<T*>(Cv) + row * ldc + col;
+      if (whole) {
+        const u32x4_t o = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]), pack2<T>(v[4], v[5]),
+                           pack2<T>(v[6], v[7])};
+        if constexpr (STREAM) {
+          __builtin_nontemporal_store(o, reinterpret_cast<u32x4_unaligned_t*>(dst));
+        } else {
+          *reinterpret_cast<u32x4_unaligned_t*>(dst) = o;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) dst[e] = from_f32<T>(v[e]);
+      }
+    }
+  }
+}
+
 // The whole wave tile (TM x TN tiles of 32x32), one 32-row band at a time through `band`
-// (wave-private, BandLayout<WN>::BYTES). The caller has synchronised the workgroup so that
-// nobody still reads operands from the LDS that `band` overlays.
+// (wave-private, BandLayout<WN>::BYTES, or BandLayoutF32<WN>::BYTES when ep.wide()). The caller
+// has synchronised the workgroup so that nobody still reads operands from the LDS that `band`
+// overlays.
 template <typename T, int EPI, int TM, int TN, bool STREAM>
 __device__ __forceinline__ void store_wave_tile_impl(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
-                                                T* __restrict__ C, int64_t ldc, int64_t row0,
+                                                void* __restrict__ Cv, int64_t ldc, int64_t row0,
                                                 int64_t col0, int64_t M, int64_t N,
                                                 const T* __restrict__ bias,
-                                                const T* __restrict__ R, int64_t ldr, int lane) {
+                                                const EpilogueArgs& ep, int lane) {
   constexpr int WN = TN * 32;
-  constexpr int PITCH = BandLayout<WN>::PITCH;
-  lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
   // The bias a lane adds depends on its columns only: fetched once for the whole wave tile
   // (the operand fragments' registers are free by now).
   float bias_f[TN][16];
@@ -275,29 +407,56 @@ __device__ __forceinline__ void store_wave_tile_impl(f32x16_t (&acc)[TM][TN], ld
 #pragma unroll
       for (int e = 0; e < 4; ++e) bias_f[j][4 * q + e] = unpack_elem<T>(b4, e);
     }
+  if constexpr (EPI == TMB_EPI_NONE) {
+    if (ep.wide()) {  // wave-uniform
+      constexpr int PITCH = BandLayoutF32<WN>::PITCH;
+      lds_byte_t* mine = band + (lane & 31) * PITCH + 16 * (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        if (row0 + i * 32 >= M) break;  // wave-uniform
+#pragma unroll
+        for (int j = 0; j < TN; ++j) stage_tile_f32(acc[i][j], mine + j * 128, bias_f[j]);
+        flush_band_wide<T, WN, STREAM>(band, Cv, ldc, row0 + i * 32, col0, M, N, ep, lane);
+      }
+      return;
+    }
+  }
+  constexpr int PITCH = BandLayout<WN>::PITCH;
+  lds_byte_t* mine = band + (lane & 31) * PITCH + 8 * (lane >> 5);
+  T* __restrict__ C = static_cast<T*>(Cv);
+  const T* __restrict__ R = static_cast<const T*>(ep.residual);
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     if (row0 + i * 32 >= M) break;  // wave-uniform
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      stage_tile<T, EPI>(acc[i][j], mine + j * 64, bias_f[j]);
-    flush_band<T, WN, STREAM>(band, C, ldc, row0 + i * 32, col0, M, N, R, ldr, lane);
+      stage_tile<T, EPI>(acc[i][j], mine + j * 64, bias_f[j], ep.twice);
+    flush_band<T, WN, STREAM>(band, C, ldc, row0 + i * 32, col0, M, N, R, ep.ldr, lane);
   }
 }
 
 template <typename T, int EPI, int TM, int TN>
 __device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byte_t* band,
-                                                T* __restrict__ C, int64_t ldc, int64_t row0,
+                                                void* __restrict__ C, int64_t ldc, int64_t row0,
                                                 int64_t col0, int64_t M, int64_t N,
                                                 const T* __restrict__ bias, bool stream,
-                                                const T* __restrict__ R, int64_t ldr, int lane) {
+                                                const EpilogueArgs& ep, int lane) {
   if (stream) {
-    store_wave_tile_impl<T, EPI, TM, TN, true>(acc, band, C, ldc, row0, col0, M, N, bias, R, ldr,
-                                               lane);
+    store_wave_tile_impl<T, EPI, TM, TN, true>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane);
   } else {
-    store_wave_tile_impl<T, EPI, TM, TN, false>(acc, band, C, ldc, row0, col0, M, N, bias, R, ldr,
-                                                lane);
+    store_wave_tile_impl<T, EPI, TM, TN, false>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane);
   }
+}
+
+// The batch entry's epilogue description out of the launch arguments.
+template <typename T>
+__device__ __forceinline__ EpilogueArgs epilogue_args(const GemmArgs& g, int64_t batch) {
+  const void* r = nullptr;
+  if (g.residual != nullptr) {
+    r = g.resid_f32 ? static_cast<const void*>(static_cast<const float*>(g.residual) + batch * g.stride_r)
+                    : static_cast<const void*>(static_cast<const T*>(g.residual) + batch * g.stride_r);
+  }
+  return EpilogueArgs{r, g.ldr, g.round_like_unfused != 0, g.resid_f32 != 0, g.out_f32 != 0};
 }
 
 // Split-K partials: the wave tile's fp32 accumulators go to P [M, N] (pitch ldp, in floats) as
@@ -339,7 +498,8 @@ template <typename T, int EPI, int VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(T* __restrict__ c,
                                                             const float* __restrict__ partial,
                                                             const T* __restrict__ bias, int64_t m,
-                                                            int64_t n, int64_t ldc, int splits) {
+                                                            int64_t n, int64_t ldc, int splits,
+                                                            bool twice) {
   const int64_t total = m * n;
   const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
   if (i >= total) return;
@@ -362,22 +522,23 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(T* __restrict__ c,
 #pragma unroll
   for (int e = 0; e < VEC; ++e) {
     if (bias != nullptr) sum[e] += to_f32(bias[col + e]);
-    c[row * ldc + col + e] = finish<T, EPI>(sum[e]);
+    c[row * ldc + col + e] = finish<T, EPI>(sum[e], twice);
   }
 }
 
 // Launches the reduction over `splits` partials (workspace is 16-byte aligned or the scalar form runs).
 template <typename T, int EPI>
 static inline void launch_splitk_reduce(T* c, const float* partial, const T* bias, int64_t m,
-                                        int64_t n, int64_t ldc, int splits, hipStream_t stream) {
+                                        int64_t n, int64_t ldc, int splits, bool twice,
+                                        hipStream_t stream) {
   const int64_t total = m * n;
   if (n % 4 == 0 && (reinterpret_cast<uintptr_t>(partial) & 15) == 0) {
     const int64_t threads = total / 4;
     splitk_reduce_kernel<T, EPI, 4><<<dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream>>>(
-        c, partial, bias, m, n, ldc, splits);
+        c, partial, bias, m, n, ldc, splits, twice);
   } else {
     splitk_reduce_kernel<T, EPI, 1><<<dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream>>>(
-        c, partial, bias, m, n, ldc, splits);
+        c, partial, bias, m, n, ldc, splits, twice);
   }
 }
 
@@ -596,12 +757,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmAr
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
   __syncthreads();  // every wave is done with the operand buffers: reuse them for the output
   static_assert(WAVES_M * WAVES_N * BandLayout<WN>::BYTES <= 2 * STAGE_BYTES, "band staging");
-  lds_byte_t* band = (lds_byte_t*)smem + wave * BandLayout<WN>::BYTES;
-  const T* resid = g.residual == nullptr
-                       ? nullptr
-                       : static_cast<const T*>(g.residual) + static_cast<int64_t>(blockIdx.y) * g.stride_r;
-  store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  g.stream_c != 0, resid, g.ldr, lane);
+  static_assert(WAVES_M * WAVES_N * BandLayoutF32<WN>::BYTES <= 2 * STAGE_BYTES, "fp32 band staging");
+  const EpilogueArgs ep = epilogue_args<T>(g, blockIdx.y);
+  lds_byte_t* band = (lds_byte_t*)smem +
+                     wave * (ep.wide() ? BandLayoutF32<WN>::BYTES : BandLayout<WN>::BYTES);
+  void* Cout = g.out_f32 ? static_cast<void*>(static_cast<float*>(g.c) + batch * g.stride_c)
+                         : static_cast<void*>(C);
+  store_wave_tile<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
+                                  g.stream_c != 0, ep, lane);
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KMAJOR, int EPI>
@@ -619,7 +782,7 @@ static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
-  g.stream_c = g.m * g.n * batch * 2 >= (int64_t{256} << 20);
+  g.stream_c = g.m * g.n * batch * (g.out_f32 ? 4 : 2) >= (int64_t{256} << 20);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), SMEM, stream>>>(g);

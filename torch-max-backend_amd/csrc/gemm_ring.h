@@ -468,12 +468,14 @@ void gemm_ring_kernel(GemmArgs g) {
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
   __syncthreads();  // every wave is done with the ring: reuse it for the output
   static_assert(NW * BandLayout<WN>::BYTES <= RING_BYTES, "band staging");
-  lds_byte_t* band = (lds_byte_t*)ring + wave * BandLayout<WN>::BYTES;
-  const T* resid = g.residual == nullptr
-                       ? nullptr
-                       : static_cast<const T*>(g.residual) + batch * g.stride_r;
-  store_wave_tile<T, EPI, TM, TN>(acc, band, C, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  g.stream_c != 0, resid, g.ldr, lane);
+  static_assert(NW * BandLayoutF32<WN>::BYTES <= RING_BYTES, "fp32 band staging");
+  const EpilogueArgs ep = epilogue_args<T>(g, batch);
+  lds_byte_t* band = (lds_byte_t*)ring +
+                     wave * (ep.wide() ? BandLayoutF32<WN>::BYTES : BandLayout<WN>::BYTES);
+  void* Cout = g.out_f32 ? static_cast<void*>(static_cast<float*>(g.c) + batch * g.stride_c)
+                         : static_cast<void*>(C);
+  store_wave_tile<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
+                                  g.stream_c != 0, ep, lane);
   };
   // Configurations compiled for four waves per SIMD have no registers to spare for the loop
   // state; their second resident workgroup already overlaps the tile boundaries.
@@ -495,7 +497,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
   g.tiles_n = static_cast<int>((g.n + BN - 1) / BN);
-  g.stream_c = g.m * g.n * batch * 2 >= (int64_t{256} << 20);
+  g.stream_c = g.m * g.n * batch * (g.out_f32 ? 4 : 2) >= (int64_t{256} << 20);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
   // as many workgroups as the device holds at once (a multiple of the 8 XCDs), shared between

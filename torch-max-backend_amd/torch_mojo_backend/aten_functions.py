@@ -153,21 +153,27 @@ def aten_addmm(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor, *, b
 
 
 def addmm_gelu(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor,
-               approximate: str = "none") -> torch.Tensor:
+               approximate: str = "none", round_like_unfused: bool = False) -> torch.Tensor:
     """``gelu(addmm(bias, mat1, mat2))`` in one kernel. Produced by the executor's
-    addmm -> view -> gelu fusion; the epilogue rounds to the storage dtype before the GELU, so
-    the result is bit-identical to the unfused pair."""
+    addmm -> view -> gelu fusion. The GELU works on the float32 sum and the result is cast once
+    (the reference forms what it fuses into a GEMM in float32 and casts once,
+    matmul_ops.mojo:2651-2657); with ``round_like_unfused`` the sum is rounded to the storage
+    dtype first, which makes the result bit-identical to the unfused pair."""
     epi = _ek.EPI_GELU_TANH if approximate == "tanh" else _ek.EPI_GELU_ERF
-    return hip_ops.gemm(mat1, mat2, input, epilogue=epi)
+    return hip_ops.gemm(mat1, mat2, input, epilogue=epi, round_like_unfused=round_like_unfused)
 
 
 def addmm_residual(input: torch.Tensor, mat1: torch.Tensor, mat2: torch.Tensor,
-                   residual: torch.Tensor) -> torch.Tensor:
+                   residual: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                   round_like_unfused: bool = False) -> torch.Tensor:
     """``addmm(bias, mat1, mat2) + residual`` in one kernel (residual reshaped to the product's
-    [M, N]). Produced by the executor's addmm -> view -> add fusion; the sum is formed from the
-    rounded product, so the result is bit-identical to the unfused pair."""
+    [M, N]). Produced by the executor's addmm -> view -> add fusion. Summed in float32 and cast
+    once; ``residual`` and the result may be float32 for 16-bit operands (the residual stream of a
+    16-bit graph kept in float32). With ``round_like_unfused`` the product is rounded to the
+    storage dtype before the add: the bits of the unfused pair."""
     m, n = mat1.shape[0], mat2.shape[-1]
-    return hip_ops.gemm(mat1, mat2, input, residual=residual.reshape(m, n))
+    return hip_ops.gemm(mat1, mat2, input, residual=residual.reshape(m, n), out_dtype=out_dtype,
+                        round_like_unfused=round_like_unfused)
 
 
 @map_to(aten.linear)

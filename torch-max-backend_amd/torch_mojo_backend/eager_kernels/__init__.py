@@ -19,6 +19,7 @@ LIBRARY_PATH = os.path.join(_CSRC, "libtmb_hip.so")
 F32, F16, BF16, I64, I32 = 0, 1, 2, 3, 4
 SUM, MEAN, AMAX = 0, 1, 2
 EPI_NONE, EPI_GELU_TANH, EPI_GELU_ERF = 0, 1, 2
+EPI_ROUND_LIKE_UNFUSED = 0x100  # flag: fused steps round where separate kernels would store
 ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED = -1, -2  # tmb_status values of include/tmb_hip.h
 
 # Every symbol include/tmb_hip.h declares, with its ctypes signature.
@@ -37,7 +38,7 @@ SIGNATURES = {
     "tmb_gemm": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp]),
     "tmb_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _ci]),
     "tmb_gemm_ws": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp, _sz, _vp]),
-    "tmb_gemm_residual": (_ci, [_vp, _vp, _vp, _vp, _vp] + [_i64] * 12 + [_ci] * 4 + [_vp]),
+    "tmb_gemm_residual": (_ci, [_vp, _vp, _vp, _vp, _vp] + [_i64] * 12 + [_ci] * 6 + [_vp]),
     "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
                                 _flt, _ci, _ci, _ci, _vp]),
     "tmb_attention_decode": (_ci, [_vp] * 5 + [_i64] * 5 + [_vp] * 5 + [_flt, _ci, _ci, _vp]),

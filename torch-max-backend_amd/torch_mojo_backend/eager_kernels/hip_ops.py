@@ -96,19 +96,26 @@ _GEMM_PLANS: dict = {}
 
 
 def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         epilogue: int = _ek.EPI_NONE, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``epilogue(a @ b + bias)`` for 2-D operands, or 3-D operands with equal batch sizes.
+         epilogue: int = _ek.EPI_NONE, residual: Optional[torch.Tensor] = None,
+         out_dtype: Optional[torch.dtype] = None, round_like_unfused: bool = False) -> torch.Tensor:
+    """``epilogue(a @ b + bias) [+ residual]`` for 2-D operands, or 3-D operands with equal batch
+    sizes.
 
     Transposed views (``weight.t()``, ``k.transpose(-2, -1)``) are consumed in place through
     the kernel's transpose flags; other non-dense layouts are materialised once.
-    ``residual`` (same shape and dtype as the result) is added after the result has been rounded
-    to the storage type, in the same launch where the kernel supports it, otherwise by a separate
-    add: either way the bits of ``gemm(...) + residual``.
+
+    A fused epilogue is evaluated in float32 and cast once: ``T(gelu(acc + bias))``,
+    ``T(acc + bias + residual)``. ``round_like_unfused`` instead rounds to the storage type
+    wherever a separate kernel would have stored a tensor (the bits of ``gelu(addmm(...))`` and
+    of ``addmm(...) + residual``). ``residual`` has the result's shape and the operands' dtype or
+    float32; ``out_dtype`` (with a residual only) may be float32 for 16-bit operands: the residual
+    stream of a 16-bit model kept in float32.
     """
+    epi_flags = epilogue | (_ek.EPI_ROUND_LIKE_UNFUSED if round_like_unfused else 0)
     # Calls that repeat an operand layout already validated (every decode step of a model) go
     # straight to the launch: the key holds everything the checks below look at.
     key = None
-    if residual is None:
+    if residual is None and out_dtype is None:
         key = (a.shape, a.stride(), b.shape, b.stride(), a.dtype, b.dtype, a.device, b.device,
                None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device))
         plan = _GEMM_PLANS.get(key)
@@ -119,10 +126,10 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
             if ws_bytes:
                 ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
                 rc = _ek.lib().tmb_gemm_ws(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_ptr,
-                                           *dims, epilogue, ws.data_ptr(), ws_bytes, _stream())
+                                           *dims, epi_flags, ws.data_ptr(), ws_bytes, _stream())
             else:
                 rc = _ek.lib().tmb_gemm(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_ptr,
-                                        *dims, epilogue, _stream())
+                                        *dims, epi_flags, _stream())
             _check("tmb_gemm", rc)
             return out
     a_in, b_in, bias_in = a, b, bias
@@ -141,6 +148,10 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
             raise ValueError(f"gemm: bias must be [{n}] {a.dtype}, got {tuple(bias.shape)} {bias.dtype}")
         if not bias.is_contiguous():
             bias = bias.contiguous()
+    result_dtype = a.dtype if out_dtype is None else out_dtype
+    if result_dtype != a.dtype and (result_dtype != torch.float32 or residual is None):
+        raise TypeError(f"gemm: {a.dtype} operands cannot produce {result_dtype} "
+                        "(float32 results exist together with a residual only)")
 
     la = _matrix_layout(a)
     if la is None or (batched and batch > 1 and a.stride(0) < 0):
@@ -150,10 +161,16 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
     if lb is None or (batched and batch > 1 and b.stride(0) < 0):
         b = b.contiguous()
         lb = (0, max(n, 1))
-    out = torch.empty((batch, m, n) if batched else (m, n), dtype=a.dtype, device=a.device)
-    if residual is not None and (residual.dtype != a.dtype or tuple(residual.shape) != tuple(out.shape)):
-        raise ValueError(f"gemm: residual must be {tuple(out.shape)} {a.dtype}, got "
+    out_shape = (batch, m, n) if batched else (m, n)
+    if residual is not None and (residual.dtype not in (a.dtype, torch.float32)
+                                 or tuple(residual.shape) != out_shape):
+        raise ValueError(f"gemm: residual must be {out_shape} {a.dtype} or float32, got "
                          f"{tuple(residual.shape)} {residual.dtype}")
+    wide = residual is not None and (residual.dtype != a.dtype or result_dtype != a.dtype)
+    if wide and round_like_unfused:
+        raise ValueError("gemm: a float32 residual or result keeps the epilogue in float32; "
+                         "round_like_unfused does not apply")
+    out = torch.empty(out_shape, dtype=result_dtype, device=a.device)
     if out.numel() == 0:
         return out
     lib = _ek.lib()
@@ -162,9 +179,18 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
     ws_bytes = _GEMM_WS_BYTES.get(key)
     if ws_bytes is None:  # a pure function of the shape: asked once per shape
         ws_bytes = _GEMM_WS_BYTES[key] = lib.tmb_gemm_workspace_bytes(batch, m, n, k, code_of(a.dtype))
-    if residual is not None and ws_bytes:
-        # the split kernels have no residual step; the separate add has the same bits
-        return gemm(a, b, bias, epilogue) + residual
+
+    def unfused_residual():
+        # no kernel carries this epilogue for these operands: product first, then the add.
+        # Rounded twice when both live in the storage type, otherwise summed in float32.
+        prod = gemm(a, b, bias, epilogue, round_like_unfused=round_like_unfused)
+        if wide or not round_like_unfused:
+            return (prod.float() + residual.float()).to(result_dtype)
+        return prod + residual
+
+    if residual is not None and (ws_bytes or (epilogue != _ek.EPI_NONE and not round_like_unfused)):
+        # the split kernels have no residual step; a GELU in front of a float32 add neither
+        return unfused_residual()
     if residual is not None:
         res = residual if residual.stride(-1) == 1 and residual.stride(-2) >= n else residual.contiguous()
         rc = lib.tmb_gemm_residual(
@@ -172,24 +198,27 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
             res.data_ptr(), batch, m, n, k, la[1], lb[1], n, res.stride(-2),
             a.stride(0) if batched else 0, b.stride(0) if batched else 0, m * n,
             res.stride(0) if batched else 0,
-            la[0], lb[0], code_of(a.dtype), epilogue, _stream())
+            la[0], lb[0], code_of(a.dtype), code_of(res.dtype), code_of(result_dtype), epi_flags,
+            _stream())
         if rc == _ek.ERR_UNSUPPORTED:
-            return gemm(a, b, bias, epilogue) + residual
+            return unfused_residual()
         _check("tmb_gemm_residual", rc)
         return out
-    if key is not None and a is a_in and b is b_in and bias is bias_in:
+    if key is not None and a is a_in and b is b_in and bias is bias_in and out_dtype is None:
         # operands are consumed in place: remember the launch arguments for this layout
         if len(_GEMM_PLANS) >= 4096:
             _GEMM_PLANS.clear()
-        _GEMM_PLANS[key] = (tuple(out.shape),
-                            (batch, m, n, k, la[1], lb[1], n, a.stride(0) if batched else 0,
-                             b.stride(0) if batched else 0, m * n, la[0], lb[0], code_of(a.dtype)),
-                            ws_bytes)
+        plan_key = (a.shape, a.stride(), b.shape, b.stride(), a.dtype, b.dtype, a.device, b.device,
+                    None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device))
+        _GEMM_PLANS[plan_key] = (tuple(out.shape),
+                                 (batch, m, n, k, la[1], lb[1], n, a.stride(0) if batched else 0,
+                                  b.stride(0) if batched else 0, m * n, la[0], lb[0], code_of(a.dtype)),
+                                 ws_bytes)
     if ws_bytes:
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
         rc = lib.tmb_gemm_ws(
             out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
-            batch, m, n, k, la[1], lb[1], n, 0, 0, m * n, la[0], lb[0], code_of(a.dtype), epilogue,
+            batch, m, n, k, la[1], lb[1], n, 0, 0, m * n, la[0], lb[0], code_of(a.dtype), epi_flags,
             ws.data_ptr(), ws_bytes, _stream())
         _check("tmb_gemm_ws", rc)
         return out
@@ -197,7 +226,7 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
         out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
         batch, m, n, k, la[1], lb[1], n,
         a.stride(0) if batched else 0, b.stride(0) if batched else 0, m * n,
-        la[0], lb[0], code_of(a.dtype), epilogue, _stream())
+        la[0], lb[0], code_of(a.dtype), epi_flags, _stream())
     _check("tmb_gemm", rc)
     return out
 

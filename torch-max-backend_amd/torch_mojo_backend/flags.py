@@ -26,3 +26,11 @@ def verbose_enabled() -> bool:
 def debug_graph() -> bool:
     """Compare every node's output with the same aten op run by PyTorch-ROCm itself."""
     return _flag("DEBUG_GRAPH")
+
+
+def round_like_unfused() -> bool:
+    """Fused steps (GEMM + GELU, GEMM + residual add) round to the storage type wherever the
+    separate kernels would have stored a tensor, which makes a fused graph bit-identical to the
+    unfused one. Off by default: a fused epilogue stays in float32 up to its one cast, and a
+    16-bit graph keeps its residual stream in float32 between the blocks."""
+    return _flag("ROUND_LIKE_UNFUSED")

@@ -17,10 +17,14 @@ What differs is the engine underneath. The reference lowers the FX graph to a MA
 lets MAX compile and run it; here ``BaseMaxCompiler`` turns the FX graph into a flat program of
 (mapping function, argument slots) steps once, and ``__call__`` runs those steps in order on the
 current HIP stream: hot ops enqueue hand-written gfx950 kernels, everything stays asynchronous,
-intermediates are released at their last use. Two graph-level rewrites happen at build time:
-``addmm -> [view] -> gelu`` chains become one GEMM with a GELU epilogue, and
+intermediates are released at their last use. Graph-level rewrites happen at build time:
+``addmm -> [view] -> gelu`` chains become one GEMM with a GELU epilogue, ``addmm -> [view] -> add``
+one GEMM with the residual added in its epilogue, the attention score pipeline one kernel, and
 ``native_layer_norm`` nodes whose statistics are dead skip them (reference
-aten_functions.py:2837-2849).
+aten_functions.py:2837-2849). Fused epilogues stay in float32 up to their one cast, and the
+residual stream of a 16-bit graph is kept in float32 between the fused steps that produce and
+consume it (``TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED=1`` switches both off and makes every fused
+step bit-identical to the kernels it replaces).
 """
 
 from __future__ import annotations
@@ -43,7 +47,8 @@ from torch_mojo_backend.aten_functions import (
     DECOMPOSITION_TABLE,
     MAPPING_TORCH_ATEN_TO_MOJO,
 )
-from torch_mojo_backend.flags import debug_graph, profiling_enabled, verbose_enabled
+from torch_mojo_backend.flags import (debug_graph, profiling_enabled, round_like_unfused,
+                                      verbose_enabled)
 from torch_mojo_backend.torch_compile_backend.utils import get_accelerators, get_error_message
 
 __all__ = ["mojo_backend", "MojoCompilerError", "MAPPING_TORCH_ATEN_TO_MOJO", "get_accelerators",
@@ -100,6 +105,8 @@ def _step_name(step) -> str:
         return "attention: bmm+mul+masked_fill+_softmax+bmm (fused)"
     if step.fn is _skipped:
         return "fused-away"
+    if step.fn is _WIDE_LAYER_NORM:
+        return "aten.native_layer_norm (float32 residual in)"
     return str(step.key)
 
 
@@ -397,7 +404,9 @@ class _GraphFactory:
         """addmm (single user) -> optional view (single user) -> add.Tensor(x, .) or add(., x)
         with alpha 1 and x of the viewed shape and dtype: the residual connection after a
         projection. The add becomes the fused step; addmm and view are skipped.
-        Returns {node: None (skip) | ("residual", bias, mat1, mat2, x, out_shape)}."""
+        Returns {node: None (skip) | ("residual", bias, mat1, mat2, x, out_shape, out_dtype)};
+        out_dtype is None here (the graph's own dtype) and float32 where _widen_residual_stream
+        decides to keep the stream wide."""
         out: dict = {}
         if MAPPING_TORCH_ATEN_TO_MOJO.get(aten.addmm) is not _BUILTIN_ADDMM or \
                 MAPPING_TORCH_ATEN_TO_MOJO.get(aten.add) is not _BUILTIN_ADD:
@@ -428,21 +437,65 @@ class _GraphFactory:
                 if tuple(pv.shape) != tuple(ov.shape) or pv.dtype != ov.dtype or \
                         tuple(nv.shape) != tuple(pv.shape) or nv.dtype != pv.dtype:
                     continue
-                out[node] = ("residual", src.args[0], src.args[1], src.args[2], other, tuple(pv.shape))
+                out[node] = ("residual", src.args[0], src.args[1], src.args[2], other, tuple(pv.shape),
+                             None)
                 out[src] = None
                 if via is not None:
                     out[via] = None
                 break
         return out
 
+    @staticmethod
+    def _widen_residual_stream(plans: dict) -> None:
+        """A fused residual step of a 16-bit graph whose result only feeds other fused residual
+        steps (as their residual operand) and native_layer_norm nodes (as their input) hands that
+        result on in float32: the consumers read float32, and the stream x <- x + f(norm(x)) is
+        never rounded to 16 bits between the blocks (24 roundings per forward of a 12-layer
+        decoder otherwise, the largest single contribution to its logit error). Every consumer
+        still produces the dtype the graph says. Nodes with any other user (a graph output, a
+        tensor saved for backward, an elementwise op) keep the graph's dtype."""
+        if MAPPING_TORCH_ATEN_TO_MOJO.get(aten.native_layer_norm) is not _BUILTIN_LAYER_NORM:
+            return
+        for node, plan in list(plans.items()):
+            if plan is None or plan[0] != "residual":
+                continue
+            val = node.meta.get("val")
+            if val is None or val.dtype not in (torch.bfloat16, torch.float16):
+                continue
+            norms = []
+            ok = len(node.users) > 0
+            for user in node.users:
+                uplan = plans.get(user, 0)
+                if uplan not in (0, None) and uplan[0] == "residual":
+                    # only as the residual operand, never as bias / mat1 / mat2 as well
+                    if uplan[4] is node and all(x is not node for x in uplan[1:4]):
+                        continue
+                    ok = False
+                    break
+                if user.op == "call_function" and user.target is aten.native_layer_norm.default \
+                        and user not in plans and user.args[0] is node \
+                        and all(a is not node for a in user.args[1:]) and not user.kwargs:
+                    norms.append(user)
+                    continue
+                ok = False
+                break
+            if not ok:
+                continue
+            plans[node] = plan[:6] + (torch.float32,)
+            for user in norms:
+                plans[user] = ("wide_ln", val.dtype)
+
     def create_graph(self, graph: torch.fx.Graph):
         rewrites = self._fuse_bias_gelu(graph) if _fusion_enabled() else {}
         softmax_rewrites = self._fuse_masked_softmax(graph) if _fusion_enabled() else {}
         if softmax_rewrites and _attention_fusion_enabled():
             self._fuse_attention(softmax_rewrites)
+        twice = round_like_unfused()
         if _fusion_enabled():
             # same bookkeeping as the softmax/attention plans: None = skipped, tuple = fused step
             softmax_rewrites.update(self._fuse_residual_add(graph, {**rewrites, **softmax_rewrites}))
+            if not twice:
+                self._widen_residual_stream(softmax_rewrites)
         nodes = list(graph.nodes)
         # what each node reads after the rewrites (liveness must follow the rewritten program)
         reads: dict = {}
@@ -455,6 +508,8 @@ class _GraphFactory:
                     reads[node] = [plan[1], plan[3]]
                 elif plan[0] == "residual":
                     reads[node] = [plan[1], plan[2], plan[3], plan[4]]
+                elif plan[0] == "wide_ln":
+                    reads[node] = list(node.all_input_nodes)
                 else:
                     reads[node] = [plan[1], plan[2], plan[3], plan[5]]
             else:
@@ -485,8 +540,10 @@ class _GraphFactory:
                         fn, kwargs = _FUSED_MASKED_SOFTMAX, {}
                         args = (plan[1], plan[2], plan[3], plan[4], plan[5])
                     elif plan[0] == "residual":
-                        fn, kwargs = _FUSED_ADDMM_RESIDUAL, {}
+                        fn, kwargs = _FUSED_ADDMM_RESIDUAL, {"round_like_unfused": twice}
                         args = plan[1:]
+                    elif plan[0] == "wide_ln":
+                        fn, kwargs = _WIDE_LAYER_NORM, {"out_dtype": plan[1]}
                     else:
                         fn, kwargs = _FUSED_ATTENTION, {}
                         args = plan[1:]
@@ -495,7 +552,7 @@ class _GraphFactory:
                         fn, args, kwargs = _identity, (node.args[0],), {}
                     else:
                         fn = _FUSED_ADDMM_GELU
-                        kwargs = {"approximate": rewrites[node]}
+                        kwargs = {"approximate": rewrites[node], "round_like_unfused": twice}
                 if fn is _skipped:
                     # no step at all: a fused step later does this node's work
                     self.slots[node.name] = len(self.slots)
@@ -531,10 +588,10 @@ class _GraphFactory:
         return self
 
 
-def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none"):
+def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none", round_like_unfused=False):
     n = mat2.shape[-1]
     if input.dim() == 1 and input.shape[0] == n and input.dtype == mat1.dtype:
-        return aten_functions.addmm_gelu(input, mat1, mat2, approximate)
+        return aten_functions.addmm_gelu(input, mat1, mat2, approximate, round_like_unfused)
     return _BUILTIN_GELU(_BUILTIN_ADDMM(input, mat1, mat2), approximate=approximate)
 
 
@@ -591,13 +648,38 @@ def _fused_masked_softmax(x, scale, root, slices, dim):
     return _BUILTIN_SOFTMAX(filled, dim, False)
 
 
-def _fused_addmm_residual(bias, mat1, mat2, residual, out_shape):
-    """add(view(addmm(bias, mat1, mat2), out_shape), residual)"""
+def _fused_addmm_residual(bias, mat1, mat2, residual, out_shape, out_dtype, *,
+                          round_like_unfused=False):
+    """add(view(addmm(bias, mat1, mat2), out_shape), residual). ``residual`` arrives in the
+    graph's dtype or, from a widened producer, in float32; ``out_dtype`` is None (the graph's
+    dtype) or float32 (this step's consumers all read float32)."""
     n = mat2.shape[-1]
     if isinstance(mat1, torch.Tensor) and mat1.is_cuda and bias.dim() == 1 and bias.shape[0] == n \
-            and bias.dtype == mat1.dtype and residual.dtype == mat1.dtype:
-        return aten_functions.addmm_residual(bias, mat1, mat2, residual).view(out_shape)
-    return _BUILTIN_ADD(_BUILTIN_ADDMM(bias, mat1, mat2).view(out_shape), residual)
+            and bias.dtype == mat1.dtype and residual.dtype in (mat1.dtype, torch.float32):
+        return aten_functions.addmm_residual(bias, mat1, mat2, residual, out_dtype,
+                                             round_like_unfused).view(out_shape)
+    prod = _BUILTIN_ADDMM(bias, mat1, mat2).view(out_shape)
+    if residual.dtype != prod.dtype:   # a float32 stream next to a product this step cannot fuse
+        total = prod.float() + residual
+        return total if out_dtype is torch.float32 else total.to(prod.dtype)
+    total = _BUILTIN_ADD(prod, residual)
+    return total.float() if out_dtype is torch.float32 else total
+
+
+def _wide_layer_norm(input, normalized_shape, weight, bias, eps, *, out_dtype):
+    """native_layer_norm whose input is a float32 residual stream of a 16-bit graph: statistics
+    and normalisation from the float32 row, one cast to the graph's dtype."""
+    if not isinstance(input, torch.Tensor) or input.dtype == out_dtype:
+        return _BUILTIN_LAYER_NORM(input, normalized_shape, weight, bias, eps)
+    if not input.is_cuda:   # a stand-in registry on another device: the graph's own dtypes
+        return _BUILTIN_LAYER_NORM(input.to(out_dtype), normalized_shape, weight, bias, eps)
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    shape = [int(s) for s in normalized_shape]
+    need_stats = not aten_functions._only_first_output_used()
+    out, mean, rstd = hip_ops.layer_norm(input, shape, weight, bias, eps, need_stats=need_stats,
+                                         out_dtype=out_dtype)
+    return out, mean, rstd
 
 
 def _fused_attention(q, k, v, scale, root, slices):
@@ -623,6 +705,7 @@ _BUILTIN_ADDMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.addmm]
 _BUILTIN_BMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.bmm]
 _BUILTIN_ADD = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.add)
 _BUILTIN_GELU = MAPPING_TORCH_ATEN_TO_MOJO[aten.gelu]
+_BUILTIN_LAYER_NORM = MAPPING_TORCH_ATEN_TO_MOJO[aten.native_layer_norm]
 _BUILTIN_SOFTMAX = MAPPING_TORCH_ATEN_TO_MOJO[aten._softmax]
 _BUILTIN_MASKED_FILL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.masked_fill)
 _BUILTIN_MUL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.mul)
@@ -633,6 +716,7 @@ _FUSED_ADDMM_GELU = _fused_addmm_gelu
 _FUSED_MASKED_SOFTMAX = _fused_masked_softmax
 _FUSED_ATTENTION = _fused_attention
 _FUSED_ADDMM_RESIDUAL = _fused_addmm_residual
+_WIDE_LAYER_NORM = _wide_layer_norm
 
 
 class BaseMaxCompiler:
@@ -713,6 +797,10 @@ def _compare_with_torch(step: _Step, args, kwargs, out) -> None:
     try:
         if step.fn is _FUSED_ADDMM_GELU:
             expected = torch.nn.functional.gelu(target(*args), approximate=kwargs["approximate"])
+        elif step.fn is _WIDE_LAYER_NORM:
+            ref = target(args[0].float(), args[1], None if args[2] is None else args[2].float(),
+                         None if args[3] is None else args[3].float(), args[4])
+            expected = (ref[0].to(kwargs["out_dtype"]),) + tuple(ref[1:])
         else:
             expected = target(*args, **kwargs)
     except Exception as exc:  # noqa: BLE001
