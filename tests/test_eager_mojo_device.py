@@ -232,3 +232,128 @@ def test_eager_sdpa_decode_step_takes_the_decode_kernel(monkeypatch):
     assert len(decode_calls) == 1 and not fused_calls
     want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
     _close(got.float(), want, rtol=2e-2, atol=2e-2)
+
+
+@gpu
+def test_out_variants_follow_the_dtype_policy():
+    """out= overloads (reference mojo_device_aten_ops.py:155-207, aten::mean.out :761): compute,
+    then a strided, casting copy into out; safe_cast / exact policies; wrong device or shape."""
+    x = torch.randn(6, 10)
+    m = x.to("mojo")
+    out = torch.empty(6, device="mojo")
+    ret = torch.mean(m, dim=1, out=out)
+    assert ret is out
+    torch.testing.assert_close(out.cpu(), x.mean(dim=1), rtol=1e-5, atol=1e-6)
+    # safe_cast: a float32 mean may land in a float64 destination, not in an integer one
+    wide = torch.empty(6, dtype=torch.float64, device="mojo")
+    torch.mean(m, dim=1, out=wide)
+    torch.testing.assert_close(wide.cpu(), x.double().mean(dim=1), rtol=1e-5, atol=1e-6)
+    with pytest.raises(RuntimeError, match="can't be cast"):
+        torch.mean(m, dim=1, out=torch.empty(6, dtype=torch.int32, device="mojo"))
+    # a strided destination: every other column of a wider buffer
+    buf = torch.zeros(6, 2, device="mojo")
+    torch.sum(m, dim=[1], out=buf[:, 1])
+    got = buf.cpu()
+    torch.testing.assert_close(got[:, 1], x.sum(dim=1), rtol=1e-5, atol=1e-5)
+    assert bool((got[:, 0] == 0).all())
+    # exact policy
+    a, b = torch.randn(5, 7), torch.randn(7, 3)
+    dst = torch.empty(5, 3, device="mojo")
+    assert torch.mm(a.to("mojo"), b.to("mojo"), out=dst) is dst
+    torch.testing.assert_close(dst.cpu(), a @ b, rtol=1e-4, atol=1e-4)
+    with pytest.raises(RuntimeError, match="can't be cast"):
+        torch.mm(a.to("mojo"), b.to("mojo"), out=torch.empty(5, 3, dtype=torch.float64, device="mojo"))
+    idx = torch.empty(6, dtype=torch.int64, device="mojo")
+    torch.argmax(m, dim=1, out=idx)
+    assert torch.equal(idx.cpu(), x.argmax(dim=1))
+    with pytest.raises(RuntimeError, match="shape"):
+        torch.mean(m, dim=1, out=torch.empty(5, device="mojo"))
+    with pytest.raises((RuntimeError, TypeError)):
+        torch.mean(m, dim=1, out=torch.empty(6))             # a host destination
+
+
+@gpu
+def test_mojo_backend_over_mojo_tensors_returns_zero_copy_wrappers():
+    """torch.compile(backend=mojo_backend) over eager mojo tensors (reference
+    torch_compile_backend/compiler.py:496-532, tests/test_compile_mojo_device.py): inputs are
+    consumed in place, results are mojo tensors."""
+    from torch_mojo_backend import mojo_backend
+
+    def fn(x, w, b):
+        h = torch.nn.functional.linear(x, w, b)
+        return torch.softmax(h, dim=-1), h.sum(dim=0), None
+
+    x, w, b = torch.randn(9, 16), torch.randn(12, 16), torch.randn(12)
+    xm, wm, bm = x.to("mojo"), w.to("mojo"), b.to("mojo")
+    probs, sums, nothing = torch.compile(fn, backend=mojo_backend, fullgraph=True)(xm, wm, bm)
+    assert nothing is None
+    want = fn(x, w, b)
+    _close(probs, want[0], rtol=1e-4, atol=1e-5)
+    _close(sums, want[1], rtol=1e-4, atol=1e-4)
+    # a non-contiguous input view and an output that is a view of an input
+    def fn2(x):
+        return x + 1.0, x.t()
+
+    y, xt = torch.compile(fn2, backend=mojo_backend, fullgraph=True)(xm.t())
+    _close(y, x.t() + 1.0, rtol=0, atol=0)
+    _close(xt, x, rtol=0, atol=0)
+    assert xt._ptr == xm._ptr                                  # adopted, not copied
+
+
+@gpu
+def test_mojo_backend_over_host_tensors_copies_in_and_out():
+    """The workload's CPU-resident configuration: a float32 GPT-2-shaped module that lives on the
+    host, compiled with mojo_backend. There is no CPU kernel path: parameters and inputs cross to
+    the HIP device (parameters once, cached), results come back as host tensors."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    model = build_gpt2_small(seed=0, n_layer=2)
+    idx = seeded_tokens(1, 128, seed=0)
+    with torch.no_grad():
+        want_logits, want_next = model(idx)
+        compiled = torch.compile(model, backend=mojo_backend, fullgraph=True)
+        logits, nxt = compiled(idx)
+        made = compiler._DEVICE_COPIES["made"]
+        logits2, _ = compiled(idx)
+    assert logits.device.type == "cpu" and nxt.device.type == "cpu"
+    torch.testing.assert_close(logits, want_logits, rtol=1e-4, atol=1e-4)
+    assert torch.equal(nxt, torch.argmax(logits[:, -1, :], dim=-1))
+    assert made > 0 and compiler._DEVICE_COPIES["made"] == made       # parameters crossed once
+    assert torch.equal(logits, logits2)
+    # an in-place update of a host parameter is seen by the next call
+    with torch.no_grad():
+        model.transformer.ln_f.bias.add_(1.0)
+        logits3, _ = compiled(idx)
+        want3, _ = model(idx)
+    torch.testing.assert_close(logits3, want3, rtol=1e-4, atol=1e-4)
+
+
+def test_out_of_memory_launch_status_becomes_torch_out_of_memory_error(monkeypatch):
+    """Host-only: a launcher that reports hipErrorOutOfMemory (status 2) surfaces as
+    torch.OutOfMemoryError, any other failure as HipKernelError naming the op (the reference maps
+    its kernels' OOM markers the same way, aten_fast.py:730-751, tests/test_tensor_spec_oom.py)."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    with pytest.raises(torch.OutOfMemoryError, match="tmb_gemm"):
+        hip_ops._check("tmb_gemm", 2)
+    with pytest.raises(hip_ops.HipKernelError, match="tmb_softmax_rows failed.*invalid argument"):
+        hip_ops._check("tmb_softmax_rows", -1)
+    assert hip_ops._check("tmb_gemm", 0) is None
+
+    class _Lib:
+        def tmb_softmax_rows(self, *a):
+            return 2
+
+    class _T:
+        dtype, device, shape = torch.float32, torch.device("cuda", 0), (2, 4)
+
+    # through a real launcher: everything up to the launch is stubbed, the status is real
+    monkeypatch.setattr(hip_ops, "require_hip", lambda *t: torch.device("cuda", 0))
+    monkeypatch.setattr(hip_ops._ek, "lib", lambda: _Lib())
+    monkeypatch.setattr(hip_ops, "_stream", lambda: 0)
+    monkeypatch.setattr(hip_ops.torch, "empty", lambda *a, **k: torch.zeros(2, 4))
+    x = torch.zeros(2, 4)
+    with pytest.raises(torch.OutOfMemoryError, match="tmb_softmax_rows"):
+        hip_ops.softmax(x, -1)

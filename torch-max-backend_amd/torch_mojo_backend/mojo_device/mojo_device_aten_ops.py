@@ -136,6 +136,61 @@ _register_fast("aten::native_layer_norm_backward", "fast_aten_native_layer_norm_
 _register_fast("aten::linear_backward", "fast_aten_linear_backward")
 
 
+def _out_variant(op_name: str, fast_name: str, *, dtype_policy: str = "safe_cast"):
+    """An ``out=`` overload from the functional implementation: compute, check the destination,
+    then a strided, casting copy into ``out`` (reference :155-207). ``dtype_policy``:
+    "safe_cast" (``torch.can_cast(result, out)``), "exact", or "bool_or_uint8". A destination of
+    another shape is an error here (the reference resizes its payload; a wrapper over a HIP
+    tensor cannot change its sizes)."""
+    if dtype_policy not in ("safe_cast", "exact", "bool_or_uint8"):
+        raise AssertionError(f"unknown out dtype policy: {dtype_policy}")
+
+    def dispatcher(*args, out, **kwargs):
+        if not isinstance(out, TorchMojoTensor):
+            raise RuntimeError(f"{op_name}: expected out to be a mojo tensor")
+        input_device = next((a._device for a in args if isinstance(a, TorchMojoTensor)), None)
+        if input_device is not None and out._device != input_device:
+            raise RuntimeError(f"{op_name}: expected out and input tensors to be on the same device")
+        aten_fast = _fast()
+        result = getattr(aten_fast, fast_name)(*args, **kwargs)
+        if result is aten_fast.NOT_HANDLED:
+            raise _unsupported(op_name, args, kwargs)
+        if out._device != result._device:
+            raise RuntimeError(f"{op_name}: expected out and result tensors to be on the same device")
+        if dtype_policy == "exact":
+            valid = result._dtype == out._dtype
+        elif dtype_policy == "bool_or_uint8":
+            valid = out._dtype in (torch.bool, torch.uint8)
+        else:
+            valid = torch.can_cast(result._dtype, out._dtype)
+        if not valid:
+            raise RuntimeError(f"result type {result._dtype} can't be cast to the desired output "
+                               f"type {out._dtype}")
+        if tuple(result._shape) != tuple(out._shape):
+            raise RuntimeError(f"{op_name}: out has shape {tuple(out._shape)}, the result has "
+                               f"{tuple(result._shape)}; resizing a mojo tensor is not supported")
+        out._holder.copy_(result._holder)   # casts and follows out's strides
+        return out
+
+    return dispatcher
+
+
+# out= overloads of the hot ops (the reference registers aten::mean.out, :761; the others share
+# its machinery)
+for _op, _fast_name, _policy in (
+        ("aten::mean.out", "fast_aten_mean", "safe_cast"),
+        ("aten::sum.IntList_out", "fast_aten_sum", "safe_cast"),
+        ("aten::amax.out", "fast_aten_amax", "exact"),
+        ("aten::argmax.out", "fast_aten_argmax", "exact"),
+        ("aten::mm.out", "fast_aten_mm", "exact"),
+        ("aten::bmm.out", "fast_aten_bmm", "exact"),
+        ("aten::addmm.out", "fast_aten_addmm", "exact"),
+        ("aten::_softmax.out", "fast_aten__softmax", "exact"),
+        ("aten::_log_softmax.out", "fast_aten__log_softmax", "exact"),
+        ("aten::gelu.out", "fast_aten_gelu", "exact")):
+    register_aten_op(_op)(_out_variant(_op, _fast_name, dtype_policy=_policy))
+
+
 @register_aten_op("aten::sum")
 def _sum_default(self, *, dtype=None):
     result = _fast().fast_aten_sum(self, None, False, dtype=dtype)

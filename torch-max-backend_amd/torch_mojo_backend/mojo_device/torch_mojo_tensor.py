@@ -39,6 +39,13 @@ class TorchMojoTensor(torch.Tensor):
         for t in types:
             if t is not cls and not issubclass(cls, t):
                 return NotImplemented
+        # torch.compile traces through this class with stand-in (fake / functional) holders: no
+        # kernel can take those, the op is replayed on the holders instead (see _trace_dispatch)
+        for a in args:
+            if type(a) is cls:
+                if type(a._holder) is not torch.Tensor:
+                    return cls._trace_dispatch(func, args, kwargs or {})
+                break
         impl = DIRECT_IMPLS.get(func)
         if impl is not None:
             # the implementations work on the HIP holders, so nothing below re-enters this method
@@ -65,6 +72,40 @@ class TorchMojoTensor(torch.Tensor):
         # are read from it when an implementation asks for them.
         res._holder = holder
         return res
+
+    # torch.compile support: as a traceable wrapper subclass the tensor flattens to its HIP holder,
+    # so a compiled graph computes on the holders (zero-copy) and AOTAutograd wraps its outputs
+    # back into mojo tensors.
+    def __tensor_flatten__(self):
+        return ["_holder"], None
+
+    @staticmethod
+    def __tensor_unflatten__(inner_tensors, meta, outer_size, outer_stride):
+        return TorchMojoTensor._wrap(inner_tensors["_holder"])
+
+    @classmethod
+    def _trace_dispatch(cls, func, args, kwargs):
+        """The op on the holders, results wrapped again: what tracing records for an op on mojo
+        tensors (device arguments naming the mojo device become the holders' HIP device)."""
+        from torch.utils._pytree import tree_map
+
+        hip = [None]
+
+        def unwrap(x):
+            if isinstance(x, cls):
+                hip[0] = x._holder.device
+                return x._holder
+            return x
+
+        a, kw = tree_map(unwrap, args), tree_map(unwrap, kwargs)
+        if isinstance(kw.get("device"), torch.device) and kw["device"].type == "mojo":
+            kw["device"] = hip[0] or hip_device_of(kw["device"])
+        out = func(*a, **kw)
+        return tree_map(lambda t: cls._wrap(t) if isinstance(t, torch.Tensor) and t.device.type == "cuda"
+                        else t, out)
+
+    def __coerce_same_metadata_as_tangent__(self, expected_meta, expected_type=None):
+        return self if expected_type in (None, torch.Tensor, TorchMojoTensor) else None
 
     # Layout metadata of the reference's class (:255-337), derived from the holder.
     _ptr = property(lambda self: self._holder.data_ptr())

@@ -34,7 +34,6 @@ import operator
 import os
 import time
 import traceback
-import weakref
 from typing import Any, Callable, List, Optional
 
 import torch
@@ -185,7 +184,13 @@ class _GraphFactory:
     """Turns an FX graph into a step program (counterpart of the reference's ``_GraphFactory``,
     :154-403, which emits MAX graph ops instead)."""
 
-    def __init__(self):
+    def __init__(self, run_device: Optional[torch.device] = None, example_inputs: Optional[list] = None):
+        # real (not fake) example tensors by placeholder position: lets build-time checks that
+        # need values (is this mask buffer causal?) run once here instead of inside a step
+        self.example_inputs = list(example_inputs) if example_inputs is not None else []
+        # HIP device the steps run on when the graph's own tensors live elsewhere (host tensors
+        # or the eager `mojo` device): factory nodes with an explicit device are pointed there
+        self.run_device = run_device
         self.slots: dict = {}
         self.steps: List[_Step] = []
         self.input_slots: List[int] = []
@@ -485,6 +490,45 @@ class _GraphFactory:
             for user in norms:
                 plans[user] = ("wide_ln", val.dtype)
 
+    def _prewarm_causal_verdicts(self, graph: torch.fx.Graph, plans: dict) -> None:
+        """The fused softmax / attention steps ask whether their mask buffer is causal, which
+        costs one device synchronisation per buffer. Where the buffer's values are known while
+        the program is built (module attributes, real example inputs) the question is answered
+        here, so that no step of a running graph synchronises for it."""
+        from torch._subclasses.fake_tensor import FakeTensor
+
+        placeholders = [n for n in graph.nodes if n.op == "placeholder"]
+        for node, plan in plans.items():
+            if plan is None or plan[0] not in ("softmax", "attention"):
+                continue
+            root, slices = (plan[3], plan[4]) if plan[0] == "softmax" else (plan[5], plan[6])
+            value = None
+            if root.op == "get_attr":
+                value = graph.owning_module
+                for part in root.target.split("."):
+                    value = getattr(value, part, None)
+            elif root.op == "placeholder" and root in placeholders:
+                pos = placeholders.index(root)
+                if pos < len(self.example_inputs):
+                    value = self.example_inputs[pos]
+            if not isinstance(value, torch.Tensor) or isinstance(value, FakeTensor):
+                continue
+            if self.run_device is not None:
+                value = _on_device(value, self.run_device)
+            scores = (plan[1] if plan[0] == "softmax" else None)
+            val = scores.meta.get("val") if scores is not None else None
+            if plan[0] == "attention":
+                q, k = plan[1].meta.get("val"), plan[2].meta.get("val")
+                shape = None if q is None or k is None else (q.shape[2], k.shape[2])
+            else:
+                shape = None if val is None or val.dim() < 2 else tuple(val.shape[-2:])
+            if shape is None or not all(isinstance(d, int) for d in shape):
+                continue
+            try:
+                _causal_q_len(value, slices, shape)
+            except Exception:  # noqa: BLE001 - the step asks again at run time
+                pass
+
     def create_graph(self, graph: torch.fx.Graph):
         rewrites = self._fuse_bias_gelu(graph) if _fusion_enabled() else {}
         softmax_rewrites = self._fuse_masked_softmax(graph) if _fusion_enabled() else {}
@@ -528,6 +572,8 @@ class _GraphFactory:
                 value = owner
                 for part in node.target.split("."):
                     value = getattr(value, part)
+                if self.run_device is not None and isinstance(value, torch.Tensor):
+                    value = _on_device(value, self.run_device)
                 self.constants.append((self.slots[node.name], value))
             elif node.op == "call_function":
                 key, fn = self.resolve(idx, node)
@@ -553,6 +599,9 @@ class _GraphFactory:
                     else:
                         fn = _FUSED_ADDMM_GELU
                         kwargs = {"approximate": rewrites[node], "round_like_unfused": twice}
+                if self.run_device is not None and isinstance(kwargs.get("device"), torch.device) \
+                        and kwargs["device"].type in ("cpu", "mojo"):
+                    kwargs["device"] = self.run_device
                 if fn is _skipped:
                     # no step at all: a fused step later does this node's work
                     self.slots[node.name] = len(self.slots)
@@ -574,6 +623,7 @@ class _GraphFactory:
                 self.output_template = self._convert(node.args[0])
             else:
                 raise MojoCompilerError(f"Unsupported FX node kind {node.op!r} ({node.name})")
+        self._prewarm_causal_verdicts(graph, softmax_rewrites)
         # Release each value after the step that uses it last (never graph outputs).
         output_node = nodes[-1]
         keep = {n.name for n in _nodes_in(output_node.args)}
@@ -595,12 +645,13 @@ def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none", round_like_unfus
     return _BUILTIN_GELU(_BUILTIN_ADDMM(input, mat1, mat2), approximate=approximate)
 
 
-# id(buffer) -> (weak reference, version, slices and shapes, verdict); verdict = query length if
-# the sliced buffer is a causal mask (nonzero exactly where column <= row), else 0. Checking
-# costs one device sync, once per buffer object and shape. The weak reference guards against a
-# new tensor reusing the id (or the address) of a dead one, the version counter against
-# in-place edits of the buffer.
-_CAUSAL_VERDICTS: dict = {}
+# The verdict about a mask buffer rides on the buffer tensor itself as an attribute
+# (version counter, slices and shapes, verdict); verdict = query length if the sliced buffer is a
+# causal mask (nonzero exactly where column <= row), else 0. Checking costs one device sync, once
+# per buffer object and shape (at graph build time where the values are known by then). The
+# attribute dies with the tensor, so a new tensor that reuses the address of a dead one starts
+# without a verdict; the version counter catches in-place edits of the buffer.
+_CAUSAL_ATTR = "_tmb_causal_verdict"
 
 
 def _causal_q_len(root: torch.Tensor, slices: tuple, x) -> int:
@@ -614,9 +665,9 @@ def _causal_q_len(root: torch.Tensor, slices: tuple, x) -> int:
     if not (isinstance(root, torch.Tensor) and root.is_cuda):
         return 0
     what = (tuple(root.shape), tuple(root.stride()), root.dtype, root.data_ptr(), slices, x_shape)
-    entry = _CAUSAL_VERDICTS.get(id(root))
-    if entry is not None and entry[0]() is root and entry[1] == root._version and entry[2] == what:
-        return entry[3]
+    entry = getattr(root, _CAUSAL_ATTR, None)
+    if entry is not None and entry[0] == root._version and entry[1] == what:
+        return entry[2]
     sub = root
     for dim, start, end, step in slices:
         sub = sub[(slice(None),) * (dim % sub.dim()) + (slice(start, end, step),)]
@@ -626,9 +677,10 @@ def _causal_q_len(root: torch.Tensor, slices: tuple, x) -> int:
         keep = torch.ones(q, cols, dtype=torch.bool, device=sub.device).tril()
         if bool(torch.equal(sub.reshape(q, cols) != 0, keep)):
             verdict = q
-    if len(_CAUSAL_VERDICTS) > 256:
-        _CAUSAL_VERDICTS.clear()
-    _CAUSAL_VERDICTS[id(root)] = (weakref.ref(root), root._version, what, verdict)
+    try:
+        setattr(root, _CAUSAL_ATTR, (root._version, what, verdict))
+    except (AttributeError, RuntimeError):
+        pass
     return verdict
 
 
@@ -719,8 +771,68 @@ _FUSED_ADDMM_RESIDUAL = _fused_addmm_residual
 _WIDE_LAYER_NORM = _wide_layer_norm
 
 
+def _graph_home(gm: torch.fx.GraphModule, example_inputs: list) -> str:
+    """Where the graph's own tensors live: "mojo" (eager device wrappers: outputs are adopted
+    zero-copy as mojo tensors, reference :407-421), "cpu" (host tensors: copied to the HIP device
+    on the way in and back on the way out) or "cuda". Decided at build time from the example
+    inputs and the node metas (factory-only graphs have no tensor inputs)."""
+    devices = set()
+    for t in example_inputs:
+        if isinstance(t, torch.Tensor):
+            devices.add(t.device.type)
+    for node in gm.graph.nodes:
+        val = node.meta.get("val", node.meta.get("example_value"))
+        if isinstance(val, torch.Tensor):
+            devices.add(val.device.type)
+    if "mojo" in devices:
+        return "mojo"
+    if "cuda" in devices or not devices:
+        return "cuda"
+    return "cpu"
+
+
+# Parameters of a module that lives on the host are the same tensor objects on every call: they
+# cross PCIe once, not once per call (the reference caches its imported buffers per tensor object
+# as well, :535-566). The copy rides on the host tensor itself (an attribute: it dies with the
+# tensor, and no weak reference gets in the way of torch.utils.swap_tensors); the version counter
+# catches in-place updates, the data pointer a swapped storage.
+_COPY_ATTR = "_tmb_device_copy"
+_DEVICE_COPIES = {"made": 0, "reused": 0}   # counters, for tests and diagnostics
+
+
+def _on_device(t: torch.Tensor, device: torch.device) -> torch.Tensor:
+    """`t` as a HIP tensor: mojo wrappers hand over their holder (zero-copy), host tensors are
+    copied (parameters and large tensors keep their copy), HIP tensors pass through."""
+    kind = t.device.type
+    if kind == "cuda":
+        return t
+    if kind == "mojo":
+        return t._holder
+    entry = getattr(t, _COPY_ATTR, None)
+    if entry is not None and entry[0] == t.data_ptr() and entry[1] == t._version \
+            and entry[2].device == device:
+        _DEVICE_COPIES["reused"] += 1
+        return entry[2]
+    copy = t.detach().to(device)
+    if isinstance(t, torch.nn.Parameter) or t.numel() >= 4096:
+        try:
+            setattr(t, _COPY_ATTR, (t.data_ptr(), t._version, copy))
+            _DEVICE_COPIES["made"] += 1
+        except (AttributeError, RuntimeError):
+            pass
+    return copy
+
+
+def _hip_available() -> bool:
+    """Host-resident graphs are moved to the HIP device when there is one (a process without
+    one can still build and inspect step programs)."""
+    return torch.cuda.is_available()
+
+
 class BaseMaxCompiler:
-    """Executable form of one FX graph (the name is the reference's, :455-532)."""
+    """Executable form of one FX graph (the name is the reference's, :455-532). Inputs may live
+    on a HIP device, on the eager `mojo` device (wrappers over HIP memory: consumed and returned
+    zero-copy) or on the host (copied in, results copied back: there is no CPU kernel path)."""
 
     def __init__(self, gm: torch.fx.GraphModule, example_inputs: list, mode=None):
         self.gm = gm
@@ -729,7 +841,16 @@ class BaseMaxCompiler:
             print(f"Graph has {len(gm.graph.nodes)} nodes.")
             gather_stats_on_graph(gm)
             gm.graph.print_tabular()
-        self.program = _GraphFactory().create_graph(gm.graph)
+        self.home = _graph_home(gm, example_inputs)
+        self.run_device = None
+        if self.home == "mojo" or (self.home == "cpu" and _hip_available()):
+            index = 0
+            for t in example_inputs:
+                if isinstance(t, torch.Tensor) and t.device.type == "mojo":
+                    index = t.device.index or 0
+                    break
+            self.run_device = torch.device("cuda", index)
+        self.program = _GraphFactory(self.run_device, example_inputs).create_graph(gm.graph)
         self.num_slots = len(self.program.slots)
         if profiling_enabled():
             elapsed = dt.timedelta(microseconds=(time.time_ns() - start) / 1000)
@@ -750,8 +871,13 @@ class BaseMaxCompiler:
         if len(args) != len(program.input_slots):
             raise MojoCompilerError(
                 f"graph takes {len(program.input_slots)} inputs, got {len(args)}")
-        for slot, value in zip(program.input_slots, args):
-            env[slot] = value
+        run_device = self.run_device
+        if run_device is None:
+            for slot, value in zip(program.input_slots, args):
+                env[slot] = value
+        else:
+            for slot, value in zip(program.input_slots, args):
+                env[slot] = _on_device(value, run_device) if isinstance(value, torch.Tensor) else value
         for slot, value in program.constants:
             env[slot] = value
         check = debug_graph()
@@ -785,7 +911,20 @@ class BaseMaxCompiler:
             result = list(result)
         elif not isinstance(result, list):
             result = [result]
+        if run_device is not None:
+            result = [self._to_home(r) for r in result]
         return [int(r) if isinstance(r, torch.SymInt) else r for r in result]
+
+    def _to_home(self, value):
+        """A result back where the graph's tensors live: adopted as a mojo wrapper (zero-copy,
+        reference :504-518) or copied to the host."""
+        if not isinstance(value, torch.Tensor) or value.device.type != "cuda":
+            return value
+        if self.home == "mojo":
+            from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
+
+            return TorchMojoTensor._wrap(value)
+        return value.cpu()
 
 
 def _compare_with_torch(step: _Step, args, kwargs, out) -> None:
