@@ -534,3 +534,63 @@ def test_fp32_mfma_output_larger_than_the_infinity_cache():
     want = as64(a[rows]) @ as64(w).T + as64(bias)
     assert rel_frobenius(got[rows], want) <= 2e-6
     assert torch.isfinite(got).all()
+
+
+# ---- K = 64 products on whole 128 x 128 tiles: the stream kernel -----------------------------------
+# (batch, m, n): at least 512 tiles, so every persistent workgroup walks several of them; both
+# layouts of B, a bias, a broadcast (stride 0) operand, and the shapes next to the kernel's limits
+# that must take the general kernels instead.
+STREAM64 = [(48, 1024, 1024), (8, 2048, 4096), (1, 4096, 8192), (96, 256, 768)]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("bmn", STREAM64)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_k64_stream_kernel_matches_float64(bmn, dtype, trans_b):
+    batch, m, n = bmn
+    g = torch.Generator(device="cuda").manual_seed(31)
+    a = torch.randn(batch, m, 64, generator=g, device="cuda").to(dtype)
+    b = torch.randn(batch, n, 64, generator=g, device="cuda").to(dtype)
+    b = b.transpose(1, 2) if trans_b else b.transpose(1, 2).contiguous()
+    if batch == 1:
+        a, b = a[0], b[0]
+    got = _ops().gemm(a, b)
+    for sel in ((0,), (batch - 1,)) if batch > 1 else ((),):
+        rows = torch.tensor([0, 31, 32, 127, 128, m // 2 + 5, m - 1], device="cuda")
+        aa, bb, cc = (a[sel], b[sel], got[sel]) if batch > 1 else (a, b, got)
+        aa, bb, cc = aa.reshape(m, 64), bb.reshape(64, n), cc.reshape(m, n)
+        want = (aa[rows].double() @ bb.double()).cpu().numpy()
+        bound = 64 * 2.0 ** -24 * (aa[rows].double().abs() @ bb.double().abs()).cpu().numpy()
+        assert_close64(cc[rows], want, rtol=1e-6, atol=1e-6, extra_abs=bound, what=f"k64 {bmn} tb={trans_b}")
+    # every tile was written: compare the whole product with the library kernel for K != 64
+    # (same operands padded with zero columns take the general path)
+    pad = torch.zeros(*a.shape[:-1], 8, device="cuda", dtype=dtype)
+    a72 = torch.cat([a, pad], dim=-1)
+    b72 = torch.cat([b, torch.zeros(*b.shape[:-2], 8, n, device="cuda", dtype=dtype)], dim=-2)
+    assert torch.equal(got, _ops().gemm(a72, b72))
+
+
+def test_k64_stream_kernel_bias_broadcast_and_neighbouring_shapes():
+    g = torch.Generator(device="cuda").manual_seed(32)
+    a = torch.randn(64, 512, 64, generator=g, device="cuda").bfloat16()
+    w = torch.randn(64, 512, generator=g, device="cuda").bfloat16()       # one B for every batch entry
+    got = _ops().gemm(a, w.unsqueeze(0).expand(64, 64, 512))
+    want = (a.double() @ w.double())
+    torch.testing.assert_close(got.double(), want, rtol=2.0 ** -7, atol=2.0 ** -6)
+    # 2-D with a bias
+    a2 = torch.randn(8192, 64, generator=g, device="cuda").bfloat16()
+    b2 = torch.randn(64, 1024, generator=g, device="cuda").bfloat16()
+    bias = torch.randn(1024, generator=g, device="cuda").bfloat16()
+    got = _ops().gemm(a2, b2, bias)
+    want = a2.double() @ b2.double() + bias.double()
+    torch.testing.assert_close(got.double(), want, rtol=2.0 ** -7, atol=2.0 ** -6)
+    # m not a multiple of 128, n not a multiple of 128, K = 32: the general kernels, same numbers
+    for m, n, k in ((8200, 1024, 64), (8192, 1000, 64), (8192, 1024, 32)):
+        x = torch.randn(m, k, generator=g, device="cuda").bfloat16()
+        y = torch.randn(k, n, generator=g, device="cuda").bfloat16()
+        torch.testing.assert_close(_ops().gemm(x, y).double(), x.double() @ y.double(),
+                                   rtol=2.0 ** -7, atol=2.0 ** -6)
+    # deterministic: three queued launches, identical bits
+    outs = [_ops().gemm(a2, b2, bias) for _ in range(3)]
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])

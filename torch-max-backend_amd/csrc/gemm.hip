@@ -20,6 +20,7 @@
 
 #include "gemm_mfma.h"
 #include "gemm_ring.h"
+#include "gemm_stream64.h"
 #include "gemm_f32.h"
 
 namespace tmb {
@@ -320,6 +321,10 @@ static int gemm_typed(const GemmArgs& g, int64_t batch, int trans_a, int trans_b
     }
     if (half && mfma_transposed_a_eligible(g, batch, trans_a, trans_b, EPI))
       return mfma_transposed_a<T>(g, batch, stream);
+    if (half && !trans_a && stream64_eligible(g, batch, trans_b, EPI)) {
+      return trans_b ? launch_stream64<T, true>(g, batch, stream)
+                     : launch_stream64<T, false>(g, batch, stream);
+    }
     if (half && mfma_eligible(g, batch, trans_a, trans_b)) {
       return trans_b ? mfma_pick_tile<T, true, EPI>(g, batch, stream)
                      : mfma_pick_tile<T, false, EPI>(g, batch, stream);

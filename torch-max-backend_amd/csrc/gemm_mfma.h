@@ -785,7 +785,15 @@ static int launch_mfma(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   g.stream_c = g.m * g.n * batch * (g.out_f32 ? 4 : 2) >= (int64_t{256} << 20);
   const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (tiles >= (int64_t{1} << 31) || batch > 65535) return TMB_ERR_UNSUPPORTED;
-  kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), SMEM, stream>>>(g);
+  // A product whose whole K fits one stage (attention's q.k^T with head size 64) never touches
+  // the second buffer: with half the LDS twice as many workgroups share a CU, and the load,
+  // multiply and store phases of different tiles overlap (such products are bound by their
+  // output stores, not by the matrix cores). The output bands overlay the stage.
+  constexpr int WN = BN / WAVES_N;
+  constexpr int kBands = WAVES_M * WAVES_N * BandLayoutF32<WN>::BYTES;
+  constexpr int kOneStage = (BM + BN) * kLineBytes > kBands ? (BM + BN) * kLineBytes : kBands;
+  const int smem = g.k <= kBK ? kOneStage : SMEM;
+  kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), dim3(NT), smem, stream>>>(g);
   return check_launch();
 }
 
