@@ -1,0 +1,97 @@
+"""Autograd over eager ``mojo`` tensors.
+
+``TorchMojoTensor`` is a wrapper subclass, so PyTorch's generated autograd applies whenever an op
+has a derivative formula: the formulas run on mojo tensors and reach the backward twins of the hot
+ops (``linear_backward``, ``native_layer_norm_backward``, ``gelu_backward``,
+``_log_softmax_backward_data``, ``_softmax_backward_data``) through their PrivateUse1
+registrations. What is left for this module are the ops PyTorch would normally *decompose* before
+autograd sees them and which the eager device registers whole for speed (``softmax.int``,
+``contiguous``, ``scaled_dot_product_attention``): registered at the backend key they have no
+derivative, so each gets an ``AutogradPrivateUse1`` kernel that takes the differentiable route
+when a gradient is wanted and the registered fast kernel otherwise (the reference keeps the same
+split in mojo_device/mojo_device_autograd.py:1-60).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+_registered = False
+aten = torch.ops.aten
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(
+        isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
+def _below_autograd(op, *args, **kwargs):
+    with torch._C._AutoDispatchBelowAutograd():
+        return op(*args, **kwargs)
+
+
+def _softmax_int(self, dim, dtype=None):
+    if _wants_grad(self):
+        x = self if dtype is None or dtype == self.dtype else self.to(dtype)
+        return aten._softmax(x, dim, False)          # has a derivative: _softmax_backward_data
+    return _below_autograd(aten.softmax.int, self, dim, dtype)
+
+
+def _log_softmax_int(self, dim, dtype=None):
+    if _wants_grad(self):
+        x = self if dtype is None or dtype == self.dtype else self.to(dtype)
+        return aten._log_softmax(x, dim, False)
+    return _below_autograd(aten.log_softmax.int, self, dim, dtype)
+
+
+def _contiguous(self, *, memory_format=torch.contiguous_format):
+    if _wants_grad(self):
+        if self.is_contiguous(memory_format=memory_format):
+            return aten.alias(self)
+        return aten.clone(self, memory_format=memory_format)
+    return _below_autograd(aten.contiguous, self, memory_format=memory_format)
+
+
+def _sdpa(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None,
+          enable_gqa=False):
+    if not _wants_grad(query, key, value):
+        return _below_autograd(aten.scaled_dot_product_attention, query, key, value, attn_mask,
+                               dropout_p, is_causal, scale=scale, enable_gqa=enable_gqa)
+    if dropout_p != 0.0 or enable_gqa:
+        raise NotImplementedError("scaled_dot_product_attention with dropout or grouped-query "
+                                  "attention has no gradient on the mojo device")
+    # the differentiable route: matmul, scale, mask, softmax, matmul (each with a derivative)
+    s = float(scale) if scale is not None else 1.0 / math.sqrt(query.shape[-1])
+    scores = torch.matmul(query, key.transpose(-2, -1)) * s
+    t, n = query.shape[-2], key.shape[-2]
+    if is_causal:
+        keep = torch.ones(t, n, dtype=torch.bool, device=query.device).tril()
+        scores = scores.masked_fill(~keep, float("-inf"))
+    if attn_mask is not None:
+        if attn_mask.dtype == torch.bool:
+            scores = scores.masked_fill(~attn_mask, float("-inf"))
+        else:
+            scores = scores + attn_mask
+    return torch.matmul(aten._softmax(scores, -1, False), value)
+
+
+_AUTOGRAD_KERNELS = {
+    "aten::softmax.int": _softmax_int,
+    "aten::log_softmax.int": _log_softmax_int,
+    "aten::contiguous": _contiguous,
+    "aten::scaled_dot_product_attention": _sdpa,
+}
+
+
+def register_autograd_kernels(registered_ops) -> None:
+    """AutogradPrivateUse1 kernels for those of the composite ops above that the device
+    registers at its backend key (``registered_ops``: the names in the eager registry)."""
+    global _registered
+    if _registered:
+        return
+    for name, fn in _AUTOGRAD_KERNELS.items():
+        if name in registered_ops:
+            torch.library.impl(name, "AutogradPrivateUse1")(fn)
+    _registered = True

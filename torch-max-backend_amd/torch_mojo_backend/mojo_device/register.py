@@ -29,4 +29,7 @@ def register_mojo_devices() -> None:
         torch.library.impl(op_name, "privateuseone")(func)
         # "aten::mean" names the default overload, as torch.library resolves it
         DIRECT_IMPLS[_resolve_overload(op_name)] = func
+    from .mojo_device_autograd import register_autograd_kernels
+
+    register_autograd_kernels({name for name, _ in _aten_ops_registry})
     _registered = True
