@@ -424,3 +424,83 @@ def test_residual_add_rewrite(cpu_hot_ops):
     fused = next(s for s in programs[-1].steps if s.fn is compiler._FUSED_ADDMM_RESIDUAL)
     assert fused.args[4] == (2, 5, 16)
     assert cpu_hot_ops.count("addmm") == 2     # one inside the fused step's host branch, one plain
+
+
+def _partitioned_training_graphs(model, idx, targets, partition_fn):
+    """Runs one training step through aot_autograd with PyTorch's own kernels and the given
+    partitioner; returns ([forward graph, backward graph], parameter gradients)."""
+    import torch.nn.functional as F
+    from functorch.compile import make_boxed_func
+    from torch._dynamo.backends.common import aot_autograd
+
+    graphs = []
+
+    def keep(gm, example_inputs):
+        graphs.append(gm)
+        return make_boxed_func(gm.forward)
+
+    backend = aot_autograd(fw_compiler=keep, partition_fn=partition_fn,
+                           decompositions=af.DECOMPOSITION_TABLE)
+    logits, _ = torch.compile(model, backend=backend)(idx)
+    F.cross_entropy(logits.view(-1, logits.shape[-1]), targets.view(-1)).backward()
+    return graphs, [p.grad.clone() for p in model.parameters()]
+
+
+def test_training_partition_recomputes_attention_scores_and_forward_fuses():
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch._functorch.partitioners import default_partition
+
+    idx, targets = seeded_tokens(2, 8, seed=0), seeded_tokens(2, 8, seed=1)
+    make = lambda: build_gpt2_small(seed=0, n_layer=2).bfloat16()  # noqa: E731
+    plain, want = _partitioned_training_graphs(make(), idx, targets, default_partition)
+    graphs, got = _partitioned_training_graphs(make(), idx, targets,
+                                               compiler.attention_recompute_partition)
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, w, rtol=0, atol=0)  # same ops in the same order
+    fw, bw = graphs
+    # a float32 graph is split exactly as PyTorch would: the kernel only takes 16-bit heads
+    f32, _ = _partitioned_training_graphs(build_gpt2_small(seed=0, n_layer=2), idx, targets,
+                                          compiler.attention_recompute_partition)
+    assert len([n for n in f32[1].graph.nodes if n.target is aten._softmax.default]) == 0
+
+    def saved_score_matrices(gm):
+        outs = gm.graph.output_node().args[0]
+        return [o for o in outs if isinstance(o, torch.fx.Node)
+                and tuple(o.meta["val"].shape[-2:]) == (8, 8) and o.meta["val"].dim() >= 3
+                and o.meta["val"].dtype.is_floating_point]
+
+    # PyTorch's split hands the probabilities to backward; ours hands over none of the
+    # [.., tokens, tokens] matrices and the forward graph fuses both attentions
+    assert saved_score_matrices(plain[0]) and not saved_score_matrices(fw)
+    rewrites = compiler._GraphFactory._fuse_masked_softmax(fw.graph)
+    assert len(compiler._GraphFactory._fuse_attention(rewrites)) == 2
+    assert len(compiler._GraphFactory._fuse_attention(
+        compiler._GraphFactory._fuse_masked_softmax(plain[0].graph))) == 0
+    # backward rebuilds the probabilities: one softmax per block, fusable with its mask
+    softmaxes = [n for n in bw.graph.nodes if n.target is aten._softmax.default]
+    assert len(softmaxes) == 2
+    bw_rewrites = compiler._GraphFactory._fuse_masked_softmax(bw.graph)
+    assert sum(1 for p in bw_rewrites.values() if p is not None and p[0] == "softmax") == 2
+
+
+def test_training_partition_leaves_graphs_without_attention_alone():
+    from torch._functorch.partitioners import default_partition
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb, self.lin = torch.nn.Embedding(8, 8), torch.nn.Linear(8, 8)
+
+        def forward(self, idx):
+            return torch.softmax(self.lin(self.emb(idx)), -1), None
+
+    idx, targets = torch.tensor([1, 5, 2, 7]), torch.tensor([0, 3, 3, 6])
+    results = []
+    for partition in (default_partition, compiler.attention_recompute_partition):
+        torch.manual_seed(0)
+        results.append(_partitioned_training_graphs(Net(), idx, targets, partition))
+    (a_graphs, a), (b_graphs, b) = results
+    for g, w in zip(b, a):
+        torch.testing.assert_close(g, w)
+    for ga, gb in zip(a_graphs, b_graphs):
+        assert [n.target for n in ga.graph.nodes] == [n.target for n in gb.graph.nodes]

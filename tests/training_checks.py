@@ -48,6 +48,41 @@ def gpt2_training_step_gradients_match_cpu():
     assert grew == set(watched), f"not every backward twin ran: {grew}"
 
 
+def training_forward_runs_the_fused_attention_kernel():
+    """The training partitioner recomputes the attention scores in backward, so the forward graph
+    of a bf16 training step runs one fused attention per block; a float32 graph, which the
+    16-bit kernel does not take, is split as PyTorch would. Either way the gradients match float64
+    autograd of the same weights."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    calls = []
+    real = hip_ops.attention
+
+    def counted(*a, **k):
+        calls.append(a[0].dtype)
+        return real(*a, **k)
+
+    hip_ops.attention = counted
+    idx, targets = seeded_tokens(2, 64, seed=0), seeded_tokens(2, 64, seed=1)
+    ref = build_gpt2_small(seed=0, n_layer=2).double()
+    _loss(ref, idx, targets).backward()
+    for dtype, bound in ((torch.float32, 2e-4), (torch.bfloat16, 6e-2)):
+        calls.clear()
+        model = build_gpt2_small(seed=0, n_layer=2).to(dtype).cuda()
+        loss = _loss(torch.compile(model, backend=mojo_backend), idx.cuda(), targets.cuda())
+        expected = [dtype, dtype] if dtype is torch.bfloat16 else []
+        assert calls == expected, calls
+        loss.backward()
+        assert calls == expected, "backward must not run the forward kernel again"
+        for (name, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+            scale = q.grad.abs().max().item() + 1e-12
+            err = (p.grad.double().cpu() - q.grad).abs().max().item()
+            assert err <= bound * scale, (dtype, name, err / scale)
+        torch._dynamo.reset()
+
+
 def one_sgd_step_lowers_the_loss():
     from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
     from torch_mojo_backend import mojo_backend

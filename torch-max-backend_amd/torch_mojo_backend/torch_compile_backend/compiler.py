@@ -319,17 +319,19 @@ class _GraphFactory:
         return rewrites
 
     @staticmethod
-    def _fuse_attention(softmax_rewrites: dict) -> None:
+    def _fuse_attention(softmax_rewrites: dict) -> dict:
         """Grows a fused masked softmax into a fused attention when it sits in
             bmm(flat(q), flat(k^T)) -> view -> [mul, masked_fill, _softmax] -> expand -> view
               -> bmm(., flat(v)) -> view -> transpose(1, 2) -> clone(contiguous)
         with flat(x) = _unsafe_view(clone(expand(x))) and every link used once. The clone at the
         end becomes the fused step over (q, k, v, scale, mask buffer, slices) and returns the
         [batch, tokens, heads, head_dim] tensor; everything in between is skipped. The plan of
-        the _softmax node is replaced in place."""
+        the _softmax node is replaced in place. Returns {fused clone node: every node the fused
+        step stands for (the score chain, its mask nodes and the operand copies)}."""
         bmm_ops = (aten.bmm.default,)
+        absorbed: dict = {}
         if MAPPING_TORCH_ATEN_TO_MOJO.get(aten.bmm) is not _BUILTIN_BMM:
-            return
+            return absorbed
 
         def single(node, *targets):
             return (isinstance(node, torch.fx.Node) and node.op == "call_function"
@@ -400,9 +402,18 @@ class _GraphFactory:
             if not (len(shapes[0]) == 4 and shapes[1] == shapes[2]
                     and shapes[0][:2] == shapes[1][:2] and shapes[0][3] == shapes[1][3]):
                 continue
-            for node in [*qa[1], *kb[1], kt, bmm0, scores_view, sm_node, ex, pv, *va[1], bmm1, ov, tr]:
+            chain = [*qa[1], *kb[1], kt, bmm0, scores_view, sm_node, ex, pv, *va[1], bmm1, ov, tr]
+            for node in chain:
                 softmax_rewrites[node] = None
             softmax_rewrites[final] = ("attention", q4, k4, v4, scale, root, slices)
+            fill = sm_node.args[0]
+            chain += [fill, fill.args[0]]
+            link = fill.args[1]
+            while isinstance(link, torch.fx.Node) and link.op == "call_function":
+                chain.append(link)  # eq, then the slices / aliases down to the mask buffer
+                link = link.args[0]
+            absorbed[final] = chain
+        return absorbed
 
     @staticmethod
     def _fuse_residual_add(graph: torch.fx.Graph, taken: dict) -> dict:
@@ -957,10 +968,68 @@ def boxed_func(*args, **kwargs):
     return make_boxed_func(BaseMaxCompiler(*args, **kwargs).__call__)
 
 
+def _tag_attention_for_recompute(joint_module: torch.fx.GraphModule, num_fwd_outputs: int) -> list:
+    """Marks, in a joint forward + backward graph, every node that the fused attention step
+    would stand for in the forward graph as "recompute in the backward graph": attention
+    probabilities, scores, the mask comparison and the flattened operand copies are then not
+    saved for backward, the forward graph keeps the single-user chain the attention rewrite
+    needs, and the backward graph rebuilds the probabilities from q, k and the mask buffer
+    (fused masked softmax) before the usual softmax / bmm backward ops. Returns the tagged
+    nodes. The forward half is matched on a copy of the graph cut at the forward outputs, with
+    the same matchers the forward compile uses, so a chain is tagged only if it will fuse."""
+    import torch.utils._pytree as pytree
+    from torch.utils.checkpoint import CheckpointPolicy
+
+    graph = joint_module.graph
+    if any(n.op == "call_function" and n.is_impure(impure_random=False) for n in graph.nodes):
+        return []  # the partitioner refuses recompute tags next to impure ops
+    forward = torch.fx.Graph()  # node names carry over: they are how twins are found below
+    leaves = pytree.arg_tree_leaves(forward.graph_copy(graph, {}))
+    forward.output(tuple(leaves[:num_fwd_outputs]))
+    forward.eliminate_dead_code()
+    rewrites = _GraphFactory._fuse_masked_softmax(forward)
+    absorbed = _GraphFactory._fuse_attention(rewrites)
+    by_name = {n.name: n for n in graph.nodes}
+    tagged = []
+    for region, (final, chain) in enumerate(absorbed.items(), start=1):
+        q = rewrites[final][1].meta["val"]
+        if q.dtype not in (torch.bfloat16, torch.float16) or q.shape[-1] != 64:
+            continue  # the kernel takes 16-bit heads of 64: elsewhere recomputing buys nothing
+        for twin in chain:
+            node = by_name.get(twin.name)
+            if node is None or node.op != "call_function":
+                continue
+            node.meta["recompute"] = CheckpointPolicy.MUST_RECOMPUTE
+            node.meta["ac_graph_id"] = region
+            tagged.append(node)
+    # views of the probabilities that only the backward graph holds (detach) follow them
+    for node in list(tagged):
+        for user in node.users:
+            if user.target is aten.detach.default and "recompute" not in user.meta:
+                user.meta["recompute"] = CheckpointPolicy.MUST_RECOMPUTE
+                user.meta["ac_graph_id"] = node.meta["ac_graph_id"]
+                tagged.append(user)
+    return tagged
+
+
+def attention_recompute_partition(joint_module, joint_inputs, *, num_fwd_outputs, **kwargs):
+    """The partitioner of a training graph: PyTorch's default split (what is between the forward
+    inputs and outputs is the forward graph, everything it computed is available to backward;
+    the reference passes no partitioner and gets the same, compiler.py:573-577), after the
+    attention score chains were tagged for recomputation so that the forward graph runs the
+    fused attention kernel and saves q, k, v instead of the [heads, tokens, tokens] matrices."""
+    from torch._functorch.partitioners import default_partition
+
+    if _fusion_enabled() and _attention_fusion_enabled():
+        _tag_attention_for_recompute(joint_module, num_fwd_outputs)
+    return default_partition(joint_module, joint_inputs, num_fwd_outputs=num_fwd_outputs, **kwargs)
+
+
 class mojo_backend:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs: list):
         self.func_to_execute = aot_autograd(
-            fw_compiler=boxed_func, decompositions=DECOMPOSITION_TABLE
+            fw_compiler=boxed_func, partition_fn=attention_recompute_partition,
+            decompositions=DECOMPOSITION_TABLE
         )(gm, example_inputs)
 
     def __call__(self, *args) -> list:
