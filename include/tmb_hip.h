@@ -196,11 +196,37 @@ int tmb_gemm_residual(void* c, const void* a, const void* b, const void* bias,
  * caller then runs the unfused chain).
  * Replaces aten_functions.py:443-677 (`aten__scaled_dot_product_*`, built from matmul, softmax
  * and matmul graph ops) and aten_fast.py:5177-5285 (`fast_aten_scaled_dot_product_attention`). */
-int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v, int64_t batch,
-                      int64_t heads, int64_t q_len, int64_t kv_len, int64_t head_dim,
+int tmb_attention_fwd(void* out, void* lse, const void* q, const void* k, const void* v,
+                      int64_t batch, int64_t heads, int64_t q_len, int64_t kv_len, int64_t head_dim,
                       const int64_t* q_strides, const int64_t* k_strides,
                       const int64_t* v_strides, const int64_t* out_strides, float scale,
                       int causal, int round_like_unfused, int dtype, void* stream);
+
+/* Fused attention backward: dq, dk, dv of tmb_attention_fwd's `out` given its gradient `dout`,
+ * the forward's inputs, `out` itself and the `lse` it wrote. With p[t,j] = exp(scale * q_t . k_j -
+ * lse[t]) (0 where the causal rule hides key j) and delta[t] = sum_d dout[t,d] * out[t,d]:
+ *   dv[j] = sum_t p[t,j] dout[t],   ds[t,j] = p[t,j] * (dout[t] . v[j] - delta[t]) * scale,
+ *   dq[t] = sum_j ds[t,j] k[j],     dk[j] = sum_t ds[t,j] q[t].
+ * Nothing of size q_len x kv_len reaches memory; p and ds are rounded to `dtype` before they enter
+ * a product, all sums are float32, and no atomics are used (the same call gives the same bits).
+ * Tensors are addressed [batch, heads, tokens, 64] through three element strides {batch, head,
+ * token} each: multiples of 8 with 16-byte aligned bases for q, k, v, out, dout, multiples of 4
+ * with 8-byte aligned bases for dq, dk, dv. `workspace` is device memory of
+ * tmb_attention_bwd_workspace_bytes(batch, heads, q_len) bytes, 16-byte aligned, that the call
+ * overwrites (delta and lse in base-2 units). `dtype` in {F16, BF16}, head_dim 64, scale > 0.
+ * Returns TMB_ERR_UNSUPPORTED for anything else (the caller then differentiates the unfused
+ * chain). Replaces `fast_fa4_bf16_d64_causal_backward` (eager_kernels/aten_fast.py:4089-4170),
+ * the kernel behind aten::_scaled_dot_product_flash_attention_backward
+ * (mojo_device/mojo_device_aten_ops.py:881-882). */
+int64_t tmb_attention_bwd_workspace_bytes(int64_t batch, int64_t heads, int64_t q_len);
+int tmb_attention_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
+                      const void* v, const void* out, const void* lse, void* workspace,
+                      int64_t batch, int64_t heads, int64_t q_len, int64_t kv_len,
+                      int64_t head_dim, const int64_t* q_strides, const int64_t* k_strides,
+                      const int64_t* v_strides, const int64_t* out_strides,
+                      const int64_t* dout_strides, const int64_t* dq_strides,
+                      const int64_t* dk_strides, const int64_t* dv_strides, float scale,
+                      int causal, int dtype, void* stream);
 
 /* Attention for a few queries per (batch, head) — the decode step of a generation loop — as one
  * memory-bound launch (K and V are read once, nothing goes through MFMA): out = softmax(scale *

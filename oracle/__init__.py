@@ -76,6 +76,10 @@ def lib() -> ctypes.CDLL:
         L.orc_softmax_scaled.restype = ci
         L.orc_attention.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, ctypes.c_float, ci, ci]
         L.orc_attention.restype = ci
+        L.orc_attention_lse.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, ctypes.c_float, ci, ci]
+        L.orc_attention_lse.restype = ci
+        L.orc_attention_backward.argtypes = [vp] * 9 + [i64] * 5 + [ctypes.c_float, ci, ci]
+        L.orc_attention_backward.restype = ci
         L.orc_layer_norm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ci]
         L.orc_reduce.argtypes = [vp, vp, i64, i64, ci, ci]
         L.orc_argmax.argtypes = [vp, vp, i64, i64, ci]
@@ -212,6 +216,36 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
                                    t, k.shape[2], d, float(scale), int(bool(causal)),
                                    _code(q.dtype)), "attention")
     return out
+
+
+def attention_lse(q: torch.Tensor, k: torch.Tensor, scale: float, causal: bool) -> torch.Tensor:
+    """[B,H,T,D] x [B,H,S,D] -> float32 [B,H,T]: log-sum-exp of each query's scaled scores."""
+    q, k = _cpu(q).contiguous(), _cpu(k).contiguous()
+    b, h, t, d = q.shape
+    lse = torch.empty((b, h, t), dtype=torch.float32)
+    if lse.numel():
+        _check(lib().orc_attention_lse(lse.data_ptr(), q.data_ptr(), k.data_ptr(), b, h, t,
+                                       k.shape[2], d, float(scale), int(bool(causal)),
+                                       _code(q.dtype)), "attention_lse")
+    return lse
+
+
+def attention_backward(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                       out: torch.Tensor, lse: torch.Tensor, scale: float, causal: bool):
+    """Gradients (dq, dk, dv), each [B,H,T|S,D], of `attention`'s [B,T,H,D] output given its
+    gradient `dout` (same layout) and the float32 [B,H,T] log-sum-exp."""
+    q, k, v, out, dout = (_cpu(x).contiguous() for x in (q, k, v, out, dout))
+    lse = _cpu(lse).contiguous().float()
+    b, h, t, d = q.shape
+    assert tuple(out.shape) == (b, t, h, d) and tuple(dout.shape) == (b, t, h, d)
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    if q.numel() and k.numel():
+        _check(lib().orc_attention_backward(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                            dout.data_ptr(), q.data_ptr(), k.data_ptr(),
+                                            v.data_ptr(), out.data_ptr(), lse.data_ptr(), b, h, t,
+                                            k.shape[2], d, float(scale), int(bool(causal)),
+                                            _code(q.dtype)), "attention_backward")
+    return dq, dk, dv
 
 
 def layer_norm_rows(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],

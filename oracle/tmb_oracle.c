@@ -14,6 +14,13 @@
  *   orc_attention   aten_functions.py:443-677  (scaled dot product attention as the reference builds
  *                                               it: matmul, *scale, causal mask, softmax, matmul;
  *                                               every stage stored in the tensor dtype)
+ *   orc_attention_lse / orc_attention_backward
+ *                   aten_fast.py:4050-4170 (the fused attention's float32 log-sum-exp output and
+ *                   its backward: the kernel source is a vendored third-party Mojo port of
+ *                   FlashAttention, so the oracle restates the published algorithm, Dao 2023
+ *                   "FlashAttention-2" algorithm 2: P = exp(S - L), dV = P^T dO, dP = dO V^T,
+ *                   dS = P o (dP - rowsum(dO o O)), dQ = dS K, dK = dS^T Q, S scaled; P and dS
+ *                   are rounded to the tensor dtype before their products, sums are fp32)
  *   orc_layer_norm  nn_ops.mojo:299-326        (two-pass mean / centered variance, fp32) with the
  *                                               NaN-mean rule of normalization_forward_kernels.mojo:60-70
  *   orc_reduce      reduction_ops.mojo:161-194 (fp32 accumulator for floats, own type for ints,
@@ -43,6 +50,7 @@
  */
 #include <math.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 enum { ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2, ORC_I64 = 3, ORC_I32 = 4 };
@@ -260,6 +268,83 @@ int orc_attention(void* out, const void* q, const void* k, const void* v, int64_
         store_f(out, ((b * T + t) * H + h) * D + d, dtype, acc);
       }
     }
+  }
+  return 0;
+}
+
+/* lse[b,h,t] = log sum_j exp(scale * q[b,h,t,:].k[b,h,j,:]) over the keys the causal rule keeps
+ * (j <= t), in double from the stored operands, rounded to float once. */
+int orc_attention_lse(float* lse, const void* q, const void* k, int64_t B, int64_t H, int64_t T,
+                      int64_t S, int64_t D, float scale, int causal, int dtype) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t bh = 0; bh < B * H; ++bh) {
+    for (int64_t t = 0; t < T; ++t) {
+      const int64_t last = causal ? (t < S - 1 ? t : S - 1) : S - 1;
+      double sc[S > 0 ? S : 1];
+      double m = -INFINITY;
+      for (int64_t j = 0; j <= last; ++j) {
+        double acc = 0.0;
+        for (int64_t d = 0; d < D; ++d)
+          acc += (double)load_f(q, (bh * T + t) * D + d, dtype) * (double)load_f(k, (bh * S + j) * D + d, dtype);
+        sc[j] = acc * (double)scale;
+        if (sc[j] > m) m = sc[j];
+      }
+      double denom = 0.0;
+      for (int64_t j = 0; j <= last; ++j) denom += exp(sc[j] - m);
+      lse[bh * T + t] = (float)(m + log(denom));
+    }
+  }
+  return 0;
+}
+
+/* Gradients of orc_attention's output with respect to q, k, v. q, k, v, dq, dk, dv are
+ * [B,H,T|S,D] contiguous; out and dout are [B,T,H,D] contiguous as orc_attention writes them; lse
+ * is [B,H,T] float32. fp32 scores, P = exp(scale * s - lse) and dS = P * (dP - delta) * scale are
+ * rounded to dtype before the products that consume them, every sum is fp32 and each result is
+ * rounded once. */
+int orc_attention_backward(void* dq, void* dk, void* dv, const void* dout, const void* q,
+                           const void* k, const void* v, const void* out, const float* lse,
+                           int64_t B, int64_t H, int64_t T, int64_t S, int64_t D, float scale,
+                           int causal, int dtype) {
+#pragma omp parallel for schedule(static)
+  for (int64_t bh = 0; bh < B * H; ++bh) {
+    const int64_t b = bh / H, h = bh % H;
+    float* p = (float*)malloc(sizeof(float) * (size_t)(T * S > 0 ? T * S : 1));
+    float* ds = (float*)malloc(sizeof(float) * (size_t)(T * S > 0 ? T * S : 1));
+    for (int64_t t = 0; t < T; ++t) {
+      const int64_t orow = ((b * T + t) * H + h) * D;
+      float delta = 0.0f;
+      for (int64_t d = 0; d < D; ++d) delta += load_f(dout, orow + d, dtype) * load_f(out, orow + d, dtype);
+      for (int64_t j = 0; j < S; ++j) {
+        const int hidden = causal && j > t;
+        float s = 0.0f, dp = 0.0f;
+        for (int64_t d = 0; d < D; ++d) {
+          s += load_f(q, (bh * T + t) * D + d, dtype) * load_f(k, (bh * S + j) * D + d, dtype);
+          dp += load_f(dout, orow + d, dtype) * load_f(v, (bh * S + j) * D + d, dtype);
+        }
+        const float pr = hidden ? 0.0f : expf(s * scale - lse[bh * T + t]);
+        p[t * S + j] = round_to(pr, dtype);
+        ds[t * S + j] = round_to(pr * (dp - delta) * scale, dtype);
+      }
+    }
+    for (int64_t t = 0; t < T; ++t)
+      for (int64_t d = 0; d < D; ++d) {
+        float acc = 0.0f;
+        for (int64_t j = 0; j < S; ++j) acc += ds[t * S + j] * load_f(k, (bh * S + j) * D + d, dtype);
+        store_f(dq, (bh * T + t) * D + d, dtype, acc);
+      }
+    for (int64_t j = 0; j < S; ++j)
+      for (int64_t d = 0; d < D; ++d) {
+        float acc_k = 0.0f, acc_v = 0.0f;
+        for (int64_t t = 0; t < T; ++t) {
+          acc_k += ds[t * S + j] * load_f(q, (bh * T + t) * D + d, dtype);
+          acc_v += p[t * S + j] * load_f(dout, ((b * T + t) * H + h) * D + d, dtype);
+        }
+        store_f(dk, (bh * S + j) * D + d, dtype, acc_k);
+        store_f(dv, (bh * S + j) * D + d, dtype, acc_v);
+      }
+    free(p);
+    free(ds);
   }
   return 0;
 }

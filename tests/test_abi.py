@@ -62,8 +62,14 @@ def test_host_side_argument_validation_needs_no_gpu():
     # the entry points added later obey the same rules
     assert L.tmb_softmax_rows_scaled(None, None, 2, 2, ek.F32, 1.0, 0, 0, None) == -1
     strides = (ctypes.c_int64 * 3)(64, 64, 64)
-    assert L.tmb_attention_fwd(None, None, None, None, 1, 1, 4, 4, 64, strides, strides, strides,
+    assert L.tmb_attention_fwd(None, None, None, None, None, 1, 1, 4, 4, 64, strides, strides, strides,
                                strides, 0.125, 0, 0, ek.BF16, None) == -1
+    eight = [strides] * 8
+    assert L.tmb_attention_bwd(*[None] * 10, 1, 1, 4, 4, 64, *eight, 0.125, 1, ek.BF16, None) == -1
+    assert L.tmb_attention_bwd(*[None] * 10, 1, 1, 4, 4, 128, *eight, 0.125, 1, ek.BF16, None) == -2
+    assert L.tmb_attention_bwd(*[None] * 10, 1, 1, 4, 4, 64, *eight, 0.125, 1, ek.F32, None) == -2
+    assert L.tmb_attention_bwd(*[None] * 10, 0, 1, 4, 4, 64, *eight, 0.125, 1, ek.BF16, None) == 0
+    assert L.tmb_attention_bwd_workspace_bytes(2, 3, 5) == 2 * 2 * 3 * 5 * 4
     assert L.tmb_gemm_residual(None, None, None, None, None, 1, 2, 2, 2, 2, 2, 2, 2, 0, 0, 0, 0, 0, 0,
                                ek.BF16, ek.BF16, ek.BF16, 0, None) == -1
     # epilogue flags: only the rounding flag may be or-ed in; the float32 stream excludes it

@@ -582,3 +582,59 @@ def test_layer_norm_backward_oracle_vs_autograd_and_invariants(dtype, affine):
         assert dx.sum(-1).abs().max().item() <= 1e-4
         assert (dx * xhat).sum(-1).abs().max().item() <= 1e-3
         torch.testing.assert_close(db, g.sum(0), rtol=1e-5, atol=1e-5)
+
+
+# --- attention backward -------------------------------------------------------------------------
+def _attention_math_f64(q, k, v, scale, causal):
+    """float64 autograd chain: the definition the oracle's backward is pinned to."""
+    s = (q @ k.transpose(-1, -2)) * scale
+    if causal:
+        t, n = s.shape[-2:]
+        s = s.masked_fill(torch.ones(t, n, dtype=torch.bool).triu(1), float("-inf"))
+    return torch.softmax(s, -1) @ v, torch.logsumexp(s, -1)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1, 4), (2, 3, 7, 7, 8), (1, 2, 5, 9, 16)])
+def test_attention_lse_and_backward_match_float64_autograd(shape, causal):
+    b, h, t, s_len, d = shape
+    g = torch.Generator().manual_seed(sum(shape) + causal)
+    q, k, v = (torch.randn(b, h, n, d, generator=g) for n in (t, s_len, s_len))
+    dout = torch.randn(b, t, h, d, generator=g)
+    scale = 0.37
+    q64, k64, v64 = (x.double().requires_grad_(True) for x in (q, k, v))
+    out64, lse64 = _attention_math_f64(q64, k64, v64, scale, causal)
+    out64.backward(dout.double().transpose(1, 2))
+    lse = oracle.attention_lse(q, k, scale, causal)
+    torch.testing.assert_close(lse.double(), lse64.detach(), rtol=1e-6, atol=1e-6)
+    out = out64.detach().float().transpose(1, 2).contiguous()
+    dq, dk, dv = oracle.attention_backward(dout, q, k, v, out, lse, scale, causal)
+    for got, want in ((dq, q64.grad), (dk, k64.grad), (dv, v64.grad)):
+        torch.testing.assert_close(got.double(), want, rtol=2e-5, atol=2e-5)
+
+
+def test_attention_backward_oracle_catches_its_plausible_mistakes():
+    """Dropping delta, the scale on dS, or the causal rule each moves a gradient far outside the
+    tolerance above: the pin would notice."""
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(1, 2, 6, 8, generator=g) for _ in range(3))
+    dout = torch.randn(1, 6, 2, 8, generator=g)
+    scale = 0.5
+    out = oracle.attention(q, k, v, scale, True)
+    lse = oracle.attention_lse(q, k, scale, True)
+    dq, dk, dv = oracle.attention_backward(dout, q, k, v, out, lse, scale, True)
+    # delta dropped == out replaced by zeros; causal dropped == causal False with the causal lse
+    no_delta = oracle.attention_backward(dout, q, k, v, torch.zeros_like(out), lse, scale, True)
+    assert (no_delta[0] - dq).abs().max() > 1e-2
+    # dv of a hidden key row gets mass only if the causal rule is dropped: key 5 is seen by query 5 alone
+    not_causal = oracle.attention_backward(dout, q, k, v, out, lse, scale, False)
+    assert (not_causal[2] - dv).abs().max() > 1e-2
+    # linearity in dout (dq, dk, dv are linear maps of it for fixed q, k, v, out-consistent delta)
+    out2 = oracle.attention_backward(2 * dout, q, k, v, out, lse, scale, True)
+    for a2, a1 in zip(out2, (dq, dk, dv)):
+        torch.testing.assert_close(a2, 2 * a1, rtol=1e-5, atol=1e-6)
+    # sum over keys of dS is zero for every query (softmax rows sum to one), so adding a constant
+    # vector c to every key leaves dq unchanged up to rounding: dq = dS K
+    shifted = oracle.attention_backward(dout, q, k + 3.0, v, oracle.attention(q, k + 3.0, v, scale, True),
+                                        oracle.attention_lse(q, k + 3.0, scale, True), scale, True)
+    torch.testing.assert_close(shifted[0], dq, rtol=1e-3, atol=1e-4)

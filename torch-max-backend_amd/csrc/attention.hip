@@ -22,17 +22,13 @@
 // storage type too, as a separate bmm and mul kernel would have stored them. The one
 // difference that remains is that probabilities are rounded before, not after, the division by
 // the row sum.
-#include "gemm_mfma.h"
+#include "attention_tiles.h"
 
 namespace tmb {
 
-typedef __attribute__((address_space(3))) unsigned char attn_lds_u8;
-typedef __attribute__((address_space(3))) u32x4_t attn_lds_u32x4_t;
-typedef short attn_i16x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) attn_i16x4_t attn_lds_i16x4_t;
-
 struct AttnArgs {
   void* out;
+  float* lse;  // may be null: [batch, heads, q_len] log-sum-exp of the scaled, masked scores
   const void* q;
   const void* k;
   const void* v;
@@ -46,17 +42,7 @@ struct AttnArgs {
   int round_like_unfused;
 };
 
-constexpr int kAttnBQ = 128;     // queries per workgroup
-constexpr int kAttnBKV = 64;     // keys per block
-constexpr int kAttnRow = 128;    // bytes of one K or V row (head_dim 64)
-constexpr int kAttnTile = kAttnBKV * kAttnRow;  // 8 KiB: one K or V block
 constexpr int kAttnBuf = 2 * kAttnTile;         // K + V
-constexpr int kAttnStages = 3;                  // LDS ring: one block in use, two in flight
-
-__device__ __forceinline__ float other_half(float x, int lane) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2,
-                                                                __builtin_bit_cast(int, x)));
-}
 
 template <typename T>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attention_fwd_kernel(
@@ -270,6 +256,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   }
 
   // out[b, qi, h, d]: register r of tile dt is d = 32dt + 8(r/4) + 4*half + r%4
+  if (a.lse != nullptr && half == 0 && qi < a.q_len)
+    a.lse[(static_cast<int64_t>(b) * a.heads + h) * a.q_len + qi] =
+        m_run * (a.round_like_unfused ? 1.0f : a.scale) + logf(l_run);
   if (qi < a.q_len) {
     const float inv = 1.0f / l_run;
     T* dst = static_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + static_cast<int64_t>(qi) * a.o_st;
@@ -396,7 +385,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnDecodeArgs a)
 
 }  // namespace tmb
 
-extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const void* v,
+extern "C" int tmb_attention_fwd(void* out, void* lse, const void* q, const void* k, const void* v,
                                  int64_t batch, int64_t heads, int64_t q_len, int64_t kv_len,
                                  int64_t head_dim, const int64_t* q_strides,
                                  const int64_t* k_strides, const int64_t* v_strides,
@@ -427,7 +416,8 @@ extern "C" int tmb_attention_fwd(void* out, const void* q, const void* k, const 
   if ((kv_len * k_strides[2] + 64) * 2 >= (int64_t{1} << 32) ||
       (kv_len * v_strides[2] + 64) * 2 >= (int64_t{1} << 32))
     return TMB_ERR_UNSUPPORTED;
-  AttnArgs a{out, q, k, v,
+  if (lse != nullptr && (reinterpret_cast<uintptr_t>(lse) & 3)) return TMB_ERR_INVALID_ARGUMENT;
+  AttnArgs a{out, static_cast<float*>(lse), q, k, v,
              q_strides[0], q_strides[1], q_strides[2],
              k_strides[0], k_strides[1], k_strides[2],
              v_strides[0], v_strides[1], v_strides[2],

@@ -39,8 +39,10 @@ SIGNATURES = {
     "tmb_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _ci]),
     "tmb_gemm_ws": (_ci, [_vp, _vp, _vp, _vp] + [_i64] * 10 + [_ci] * 4 + [_vp, _sz, _vp]),
     "tmb_gemm_residual": (_ci, [_vp, _vp, _vp, _vp, _vp] + [_i64] * 12 + [_ci] * 6 + [_vp]),
-    "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
-                                _flt, _ci, _ci, _ci, _vp]),
+    "tmb_attention_fwd": (_ci, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp,
+                                _vp, _flt, _ci, _ci, _ci, _vp]),
+    "tmb_attention_bwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "tmb_attention_bwd": (_ci, [_vp] * 10 + [_i64] * 5 + [_vp] * 8 + [_flt, _ci, _ci, _vp]),
     "tmb_attention_decode": (_ci, [_vp] * 5 + [_i64] * 5 + [_vp] * 5 + [_flt, _ci, _ci, _vp]),
     "tmb_gelu": (_ci, [_vp, _vp, _i64, _ci, _ci, _vp]),
     "tmb_gather_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _vp]),

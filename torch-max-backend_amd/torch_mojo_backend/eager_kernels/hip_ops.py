@@ -306,10 +306,12 @@ def attention_supported(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> bo
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool,
-              round_like_unfused: bool = False) -> torch.Tensor:
+              round_like_unfused: bool = False, return_lse: bool = False):
     """softmax(scale * q k^T [causal]) v for [batch, heads, tokens, 64] tensors (any strides
     `attention_supported` accepts). Returns a [batch, q_len, heads, 64] contiguous tensor, i.e.
-    the layout `y.transpose(1, 2).contiguous()` would have produced."""
+    the layout `y.transpose(1, 2).contiguous()` would have produced; with `return_lse` also the
+    float32 [batch, heads, q_len] log-sum-exp of every query's scores, which
+    `attention_backward` needs."""
     require_hip(q, k, v)
     if not (scale > 0.0 and math.isfinite(scale)):
         raise ValueError(f"attention: scale must be positive and finite, got {scale}")
@@ -321,12 +323,68 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, c
     i64x3 = ctypes.c_int64 * 3
     strides = [i64x3(x.stride(0), x.stride(1), x.stride(2)) for x in (q, k, v)]
     o_str = i64x3(out.stride(0), out.stride(2), out.stride(1))
-    rc = _ek.lib().tmb_attention_fwd(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+    lse = torch.empty((b, h, t), dtype=torch.float32, device=q.device) if return_lse else None
+    rc = _ek.lib().tmb_attention_fwd(out.data_ptr(), lse.data_ptr() if return_lse else None,
+                                     q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                      b, h, t, k.shape[2], d, strides[0], strides[1], strides[2],
                                      o_str, float(scale), int(bool(causal)),
                                      int(bool(round_like_unfused)), code_of(q.dtype), _stream())
     _check("tmb_attention_fwd", rc)
-    return out
+    return (out, lse) if return_lse else out
+
+
+def attention_backward_supported(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor,
+                                 v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor) -> bool:
+    """True when `attention_backward` takes these tensors as they are: q, k, v as for `attention`,
+    `out` and `dout` [batch, heads, q_len, 64] views with the same stride rules, `lse` float32
+    [batch, heads, q_len] contiguous."""
+    if not attention_supported(q, k, v):
+        return False
+    b, h, t, d = q.shape
+    for x in (out, dout):
+        if not x.is_cuda or x.dtype != q.dtype or tuple(x.shape) != (b, h, t, d):
+            return False
+        if x.stride(3) != 1 or any(s % 8 or s < 0 for s in x.stride()[:3]) or x.data_ptr() % 16:
+            return False
+    if (t * dout.stride(2) + 64) * 2 >= 1 << 32 or (t * q.stride(2) + 64) * 2 >= 1 << 32:
+        return False
+    return (lse.is_cuda and lse.dtype == torch.float32 and tuple(lse.shape) == (b, h, t)
+            and lse.is_contiguous())
+
+
+def attention_backward(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                       out: torch.Tensor, lse: torch.Tensor, scale: float, causal: bool):
+    """(dq, dk, dv) of `attention`: `out` and `dout` are [batch, heads, q_len, 64] views (the
+    transposed view of what `attention` returned, and the gradient in the same layout), `lse` what
+    `attention(..., return_lse=True)` returned. The three gradients are [batch, heads, tokens, 64]
+    views of one packed [batch, tokens, 3, heads, 64] buffer when q_len == kv_len (so the gradient
+    of a packed q/k/v projection needs no concatenation), separate [batch, tokens, heads, 64]
+    buffers otherwise."""
+    require_hip(dout, q, k, v, out, lse)
+    if not (scale > 0.0 and math.isfinite(scale)):
+        raise ValueError(f"attention_backward: scale must be positive and finite, got {scale}")
+    if not attention_backward_supported(dout, q, k, v, out, lse):
+        raise ValueError("attention_backward: unsupported operands (see attention_backward_supported)")
+    b, h, t, d = q.shape
+    s_len = k.shape[2]
+    if t == s_len:
+        packed = torch.empty((b, t, 3, h, d), dtype=q.dtype, device=q.device)
+        dq, dk, dv = (packed[:, :, i].transpose(1, 2) for i in range(3))
+    else:
+        dq = torch.empty((b, t, h, d), dtype=q.dtype, device=q.device).transpose(1, 2)
+        dk = torch.empty((b, s_len, h, d), dtype=q.dtype, device=q.device).transpose(1, 2)
+        dv = torch.empty((b, s_len, h, d), dtype=q.dtype, device=q.device).transpose(1, 2)
+    lib = _ek.lib()
+    workspace = torch.empty(max(int(lib.tmb_attention_bwd_workspace_bytes(b, h, t)), 16),
+                            dtype=torch.uint8, device=q.device)
+    i64x3 = ctypes.c_int64 * 3
+    st = [i64x3(x.stride(0), x.stride(1), x.stride(2)) for x in (q, k, v, out, dout, dq, dk, dv)]
+    rc = lib.tmb_attention_bwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dout.data_ptr(),
+                               q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                               lse.data_ptr(), workspace.data_ptr(), b, h, t, s_len, d, *st,
+                               float(scale), int(bool(causal)), code_of(q.dtype), _stream())
+    _check("tmb_attention_bwd", rc)
+    return dq, dk, dv
 
 
 # Queries per (batch, head) up to which the decode kernel (one wave per query row, K and V read
