@@ -112,3 +112,35 @@ def test_training_step_on_the_eager_device_matches_cpu_gradients(mojo):
         for p in dev.parameters():
             p -= 0.5 * p.grad
     assert loss_of(dev, idx.to(mojo), target.to(mojo)).item() < got.item()
+
+
+def test_sdpa_gradients_on_the_eager_device_come_from_the_fused_backward(mojo):
+    """F.scaled_dot_product_attention with a gradient wanted, bf16 heads of 64: the autograd
+    kernel routes to aten::_scaled_dot_product_flash_attention (fused forward + log-sum-exp) and
+    PyTorch's derivative formula then calls the fused backward op; gradients match float64."""
+    from torch_mojo_backend.mojo_device.mojo_device_aten_ops import EAGER_CALL_COUNTERS
+
+    torch.manual_seed(3)
+    b, h, t = 2, 3, 140
+    qkv = torch.randn(b, t, 3 * h * 64).bfloat16()
+    g = torch.randn(b, h, t, 64).bfloat16()
+
+    def run(x, grad, dtype):
+        x = x.to(dtype).requires_grad_(True)
+        q, k, v = (y.view(b, t, h, 64).transpose(1, 2) for y in x.split(h * 64, dim=2))
+        out = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+        (out * grad.to(dtype)).sum().backward()
+        return out.detach(), x.grad
+
+    want_out, want_grad = run(qkv, g, torch.float64)
+    ops = ("aten::_scaled_dot_product_flash_attention", "aten::_scaled_dot_product_flash_attention_backward")
+    before = [EAGER_CALL_COUNTERS[op].call_count for op in ops]
+    got_out, got_grad = run(qkv.to(mojo), g.to(mojo), torch.bfloat16)
+    assert [EAGER_CALL_COUNTERS[op].call_count - n for op, n in zip(ops, before)] == [1, 1]
+    assert got_grad.device.type == "mojo" and got_grad.dtype == torch.bfloat16
+    assert (got_out.cpu().double() - want_out).abs().max().item() <= 3e-2
+    big = want_grad.abs().max().item()
+    assert (got_grad.cpu().double() - want_grad).abs().max().item() <= 2e-2 * big
+    # float32 heads keep the composed, differentiable route
+    _, grad32 = run(qkv.to(mojo), g.to(mojo), torch.float32)
+    assert (grad32.cpu().double() - want_grad).abs().max().item() <= 1e-4 * big

@@ -106,7 +106,7 @@ def test_attention_backward_reads_packed_projections_and_packs_its_gradients():
     ops = _ops()
     out, lse = ops.attention(qd, kd, vd, 0.125, True, return_lse=True)
     dq, dk, dv = ops.attention_backward(dout.cuda().transpose(1, 2), qd, kd, vd, out.transpose(1, 2),
-                                        lse, 0.125, True)
+                                        lse, 0.125, True, packed=True)
     assert dq.data_ptr() + h * 64 * 2 == dk.data_ptr() and dk.data_ptr() + h * 64 * 2 == dv.data_ptr()
     packed = torch.cat([g.transpose(1, 2).reshape(b, t, h * 64) for g in (dq, dk, dv)], dim=2)
     q, k, v = (x.view(b, t, h, 64).transpose(1, 2).contiguous() for x in qkv.split(h * 64, dim=2))
@@ -157,3 +157,50 @@ def test_attention_backward_rejects_what_it_cannot_take():
         ops.attention_backward(do[:, :, :8], q, k, v, o, lse, 0.125, True)
     with pytest.raises(TypeError):
         ops.attention_backward(do.cpu(), q, k, v, o, lse, 0.125, True)
+
+
+def test_registry_entries_for_the_flash_attention_ops_match_pytorch_rocm():
+    """The graph surface maps aten::_scaled_dot_product_flash_attention and its backward (what
+    torch.compile makes of F.scaled_dot_product_attention on 16-bit tensors) to the fused
+    kernels: same contract as PyTorch-ROCm's own ops, values against float64 autograd."""
+    from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO as mapping
+    aten = torch.ops.aten
+    b, h, t = 2, 3, 200
+    qkv = seeded((b, t, 3 * h * 64), seed=21, dtype=torch.bfloat16).cuda()
+    q, k, v = (x.view(b, t, h, 64).transpose(1, 2) for x in qkv.split(h * 64, dim=2))
+    dout = seeded((b, t, h, 64), seed=22, dtype=torch.bfloat16).cuda().transpose(1, 2)
+    got = mapping[aten._scaled_dot_product_flash_attention](q, k, v, 0.0, True, False, scale=0.125)
+    ref = aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False, scale=0.125)
+    assert len(got) == len(ref) == 9
+    for g, r in zip(got, ref):
+        if isinstance(r, torch.Tensor):
+            assert g.shape == r.shape and g.dtype == r.dtype and g.device == r.device
+            assert g.stride() == r.stride()
+        else:
+            assert g == r
+    out64, lse64, *want = _float64_reference(q.cpu(), k.cpu(), v.cpu(), dout.cpu().transpose(1, 2), 0.125, True)
+    assert np.abs(as64(got[0]) - out64.numpy()).max() <= 3e-2
+    np.testing.assert_allclose(as64(got[1]), lse64.numpy(), rtol=0, atol=1e-4)
+    np.testing.assert_allclose(as64(ref[1]), lse64.numpy(), rtol=0, atol=1e-3)  # same definition
+    grads = mapping[aten._scaled_dot_product_flash_attention_backward](
+        dout, q, k, v, got[0], got[1], None, None, t, t, 0.0, True, got[6], got[7], scale=0.125)
+    ref_grads = aten._scaled_dot_product_flash_attention_backward(
+        dout, q, k, v, ref[0], ref[1], None, None, t, t, 0.0, True, ref[6], ref[7], scale=0.125)
+    for name, g, r, w in zip("qkv", grads, ref_grads, want):
+        assert g.shape == r.shape and g.dtype == r.dtype and g.stride() == r.stride(), name
+        big = w.abs().max().item()
+        assert np.abs(as64(g) - w.numpy()).max() <= 2e-2 * big, name
+    # and our backward accepts PyTorch-ROCm's forward results (same log-sum-exp definition)
+    mixed = mapping[aten._scaled_dot_product_flash_attention_backward](
+        dout, q, k, v, ref[0], ref[1], None, None, t, t, 0.0, True, ref[6], ref[7], scale=0.125)
+    for name, g, w in zip("qkv", mixed, want):
+        assert np.abs(as64(g) - w.numpy()).max() <= 2e-2 * w.abs().max().item(), name
+    # dropout is PyTorch-ROCm's own op
+    calls = []
+    real = _ops().attention
+    try:
+        _ops().attention = lambda *a, **kw: calls.append(1) or real(*a, **kw)
+        mapping[aten._scaled_dot_product_flash_attention](q, k, v, 0.5, True, False, scale=0.125)
+    finally:
+        _ops().attention = real
+    assert not calls

@@ -83,6 +83,55 @@ def training_forward_runs_the_fused_attention_kernel():
         torch._dynamo.reset()
 
 
+def sdpa_training_graph_runs_the_fused_forward_and_backward():
+    """F.scaled_dot_product_attention on bf16 tensors reaches a training graph as
+    aten::_scaled_dot_product_flash_attention and its backward op: both run on the fused kernels
+    and the gradients match float64 autograd of the same module."""
+    from torch_mojo_backend import MAPPING_TORCH_ATEN_TO_MOJO as mapping
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    class Block(torch.nn.Module):
+        def __init__(self, heads=4):
+            super().__init__()
+            self.heads = heads
+            self.qkv = torch.nn.Linear(heads * 64, 3 * heads * 64)
+            self.proj = torch.nn.Linear(heads * 64, heads * 64)
+
+        def forward(self, x):
+            b, t, c = x.shape
+            q, k, v = (y.view(b, t, self.heads, 64).transpose(1, 2) for y in self.qkv(x).split(c, dim=2))
+            y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            return self.proj(y.transpose(1, 2).reshape(b, t, c))
+
+    torch.manual_seed(0)
+    ref = Block().double()
+    x = torch.randn(2, 150, 256, dtype=torch.float64)
+    g = torch.randn(2, 150, 256, dtype=torch.float64)
+    xr = x.clone().requires_grad_(True)
+    (ref(xr) * g).sum().backward()
+
+    fused = {"fwd": 0, "bwd": 0}
+    real_f, real_b = hip_ops.attention, hip_ops.attention_backward
+    hip_ops.attention = lambda *a, **k: (fused.__setitem__("fwd", fused["fwd"] + 1), real_f(*a, **k))[1]
+    hip_ops.attention_backward = lambda *a, **k: (fused.__setitem__("bwd", fused["bwd"] + 1), real_b(*a, **k))[1]
+    model = Block().bfloat16().cuda()
+    model.load_state_dict({k: v.bfloat16() for k, v in ref.state_dict().items()})
+    aten = torch.ops.aten
+    watched = (aten._scaled_dot_product_flash_attention, aten._scaled_dot_product_flash_attention_backward)
+    before = [mapping[op].call_count for op in watched]
+    xd = x.bfloat16().cuda().requires_grad_(True)
+    (torch.compile(model, backend=mojo_backend)(xd) * g.bfloat16().cuda()).sum().backward()
+    assert [mapping[op].call_count - n for op, n in zip(watched, before)] == [1, 1]
+    assert fused == {"fwd": 1, "bwd": 1}, fused
+    pairs = [("x", xd.grad, xr.grad)] + [(n, p.grad, q.grad) for (n, p), (_, q) in
+                                         zip(model.named_parameters(), ref.named_parameters())]
+    for name, got, want in pairs:
+        scale = want.abs().max().item()
+        err = (got.double().cpu() - want).abs().max().item()
+        assert err <= 4e-2 * scale, (name, err / scale)
+
+
 def one_sgd_step_lowers_the_loss():
     from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
     from torch_mojo_backend import mojo_backend

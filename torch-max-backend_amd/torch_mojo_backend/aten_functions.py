@@ -325,6 +325,63 @@ def aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout
                                              scale=scale, enable_gqa=enable_gqa)
 
 
+_FLASH_EXTRAS: dict = {}
+
+
+def _flash_extras(like: torch.Tensor) -> tuple:
+    """The outputs of aten::_scaled_dot_product_flash_attention that carry nothing without
+    dropout: the two random-number-state scalars (int64 on ROCm) and the empty debug mask.
+    Nothing ever writes them, so one set per (device, dtype) serves every call."""
+    key = (like.device, like.dtype)
+    if key not in _FLASH_EXTRAS:
+        _FLASH_EXTRAS[key] = (torch.zeros((), dtype=torch.int64, device=like.device),
+                              torch.zeros((), dtype=torch.int64, device=like.device),
+                              torch.empty(0, dtype=like.dtype, device=like.device))
+    return _FLASH_EXTRAS[key]
+
+
+def _flash_scale(query, scale) -> float:
+    return float(scale) if scale is not None else 1.0 / math.sqrt(query.shape[-1])
+
+
+@map_to(aten._scaled_dot_product_flash_attention)
+def aten__scaled_dot_product_flash_attention(query, key, value, dropout_p: float = 0.0,
+                                             is_causal: bool = False,
+                                             return_debug_mask: bool = False, *, scale=None):
+    """reference :540-677 (which returns a zero log-sum-exp: "we don't support training yet") and
+    eager_kernels/aten_fast.py:4211-4248 (which returns the real one). What torch.compile makes of
+    F.scaled_dot_product_attention on 16-bit CUDA tensors: output laid out like the query, the
+    float32 log-sum-exp the backward op needs, and the placeholders of the 9-value contract.
+    Dropout, a debug mask, other head sizes: PyTorch-ROCm's own op."""
+    s = _flash_scale(query, scale)
+    if dropout_p == 0.0 and not return_debug_mask and query.dim() == 4 and s > 0.0 \
+            and hip_ops.attention_supported(query, key, value):
+        out, lse = hip_ops.attention(query, key, value, s, bool(is_causal), return_lse=True,
+                                     like_query=True)
+        seed, offset, debug_mask = _flash_extras(query)
+        return (out, lse, None, None, query.shape[2], key.shape[2], seed, offset, debug_mask)
+    return aten._scaled_dot_product_flash_attention(query, key, value, dropout_p, is_causal,
+                                                    return_debug_mask, scale=scale)
+
+
+@map_to(aten._scaled_dot_product_flash_attention_backward)
+def aten__scaled_dot_product_flash_attention_backward(grad_out, query, key, value, out, logsumexp,
+                                                      cum_seq_q, cum_seq_k, max_q, max_k,
+                                                      dropout_p, is_causal, philox_seed,
+                                                      philox_offset, *, scale=None):
+    """eager_kernels/aten_fast.py:4251-4338 (the graph surface of the reference has no attention
+    backward). (grad_query, grad_key, grad_value), each laid out like its input."""
+    s = _flash_scale(query, scale)
+    if dropout_p == 0.0 and cum_seq_q is None and cum_seq_k is None and s > 0.0 \
+            and query.dim() == 4 and logsumexp.is_contiguous() \
+            and hip_ops.attention_backward_supported(grad_out, query, key, value, out, logsumexp):
+        return hip_ops.attention_backward(grad_out, query, key, value, out, logsumexp, s,
+                                          bool(is_causal))
+    return aten._scaled_dot_product_flash_attention_backward(
+        grad_out, query, key, value, out, logsumexp, cum_seq_q, cum_seq_k, max_q, max_k,
+        dropout_p, is_causal, philox_seed, philox_offset, scale=scale)
+
+
 # ---------------------------------------------------------------------------
 # Backward twins of the hot ops (reference :788-833, :2070-2102, :2323-2375; the layer-norm
 # backward is eager-only there, eager_kernels/aten_fast.py:2797-2913)
@@ -406,7 +463,7 @@ HOT_OPS = (aten.mm, aten.bmm, aten.addmm, aten.linear, aten._softmax, aten.softm
 _PASSTHROUGH = """
 floordiv _local_scalar_dense all _adaptive_avg_pool2d _adaptive_avg_pool2d_backward
 _native_batch_norm_legit_no_training _scaled_dot_product_attention_math
-_scaled_dot_product_efficient_attention _scaled_dot_product_flash_attention
+_scaled_dot_product_efficient_attention
 _to_copy abs acos add addcdiv addcmul alias amin any arange
 argmin asinh atanh avg_pool2d bitwise_and.Scalar bitwise_and.Tensor bitwise_not bitwise_or.Scalar
 bitwise_or.Tensor bitwise_xor.Scalar bitwise_xor.Tensor cat ceil clamp clone constant_pad_nd
@@ -434,6 +491,7 @@ index_put index_put_ gather scatter_add nll_loss_forward nll_loss_backward nll_l
 embedding_dense_backward tanh_backward sigmoid_backward threshold_backward new_zeros new_empty
 new_empty_strided zeros_like zeros ones sum_to_size expand_as squeeze_ unsqueeze_ mse_loss
 mse_loss_backward _softmax_backward_data.out log sqrt_ rsub addcmul_ addcdiv_ lerp
+_scaled_dot_product_efficient_attention_backward
 """.split()
 
 

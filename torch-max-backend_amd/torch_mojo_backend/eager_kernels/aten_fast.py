@@ -202,6 +202,56 @@ def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dr
                                             None if mask is None else mask._holder))
 
 
+def _flash_operands(query, key, value, dropout_p, scale):
+    """(q, k, v, scale) when the fused kernels take the call, else None."""
+    q, k, v = _t(query), _t(key), _t(value)
+    if q is None or k is None or v is None or not _same_device(q, k, v) or dropout_p != 0.0 \
+            or len(q._shape) != 4:
+        return None
+    s = float(scale) if scale is not None else 1.0 / math.sqrt(q._shape[-1])
+    if not (s > 0.0) or not hip_ops.attention_supported(q._holder, k._holder, v._holder):
+        return None
+    return q, k, v, s
+
+
+def fast_aten__scaled_dot_product_flash_attention(query, key, value, dropout_p=0.0,
+                                                  is_causal=False, return_debug_mask=False, *,
+                                                  scale=None):
+    """reference :4211-4248: output laid out like the query, the real float32 log-sum-exp (the
+    backward op needs it) and the placeholders of ATen's 9-value contract."""
+    ops = None if return_debug_mask else _flash_operands(query, key, value, dropout_p, scale)
+    if ops is None:
+        return NOT_HANDLED
+    q, k, v, s = ops
+    out, lse = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal),
+                                 return_lse=True, like_query=True)
+    seed = torch.zeros((), dtype=torch.int64, device=out.device)
+    return (_wrap(out), _wrap(lse), None, None, q._shape[2], k._shape[2], _wrap(seed),
+            _wrap(seed.clone()), _wrap(torch.empty(0, dtype=out.dtype, device=out.device)))
+
+
+def fast_aten__scaled_dot_product_flash_attention_backward(grad_out, query, key, value, out,
+                                                           logsumexp, cum_seq_q, cum_seq_k, max_q,
+                                                           max_k, dropout_p, is_causal,
+                                                           philox_seed, philox_offset, *,
+                                                           scale=None):
+    """reference :4251-4338 and :4089-4170: (grad_query, grad_key, grad_value) from the fused
+    backward kernels; a log-sum-exp view that is not contiguous is materialised first."""
+    ops = _flash_operands(query, key, value, dropout_p, scale)
+    g, o, lse = _t(grad_out), _t(out), _t(logsumexp)
+    if ops is None or g is None or o is None or lse is None or cum_seq_q is not None \
+            or cum_seq_k is not None:
+        return NOT_HANDLED
+    q, k, v, s = ops
+    lse_h = lse._holder if lse._holder.is_contiguous() else lse._holder.contiguous()
+    if not hip_ops.attention_backward_supported(g._holder, q._holder, k._holder, v._holder,
+                                                o._holder, lse_h):
+        return NOT_HANDLED
+    grads = hip_ops.attention_backward(g._holder, q._holder, k._holder, v._holder, o._holder,
+                                       lse_h, s, bool(is_causal), packed=True)
+    return tuple(_wrap(x) for x in grads)
+
+
 # ---------------------------------------------------------------------------
 # Layer norm (reference :2704-2794)
 # ---------------------------------------------------------------------------

@@ -306,12 +306,14 @@ def attention_supported(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> bo
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool,
-              round_like_unfused: bool = False, return_lse: bool = False):
+              round_like_unfused: bool = False, return_lse: bool = False,
+              like_query: bool = False):
     """softmax(scale * q k^T [causal]) v for [batch, heads, tokens, 64] tensors (any strides
     `attention_supported` accepts). Returns a [batch, q_len, heads, 64] contiguous tensor, i.e.
-    the layout `y.transpose(1, 2).contiguous()` would have produced; with `return_lse` also the
-    float32 [batch, heads, q_len] log-sum-exp of every query's scores, which
-    `attention_backward` needs."""
+    the layout `y.transpose(1, 2).contiguous()` would have produced; with `like_query` a
+    [batch, heads, q_len, 64] tensor laid out as `torch.empty_like(q)` (what ATen's fused attention
+    ops return). With `return_lse` also the float32 [batch, heads, q_len] log-sum-exp of every
+    query's scores, which `attention_backward` needs."""
     require_hip(q, k, v)
     if not (scale > 0.0 and math.isfinite(scale)):
         raise ValueError(f"attention: scale must be positive and finite, got {scale}")
@@ -319,10 +321,14 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, c
         raise ValueError(f"attention: unsupported operands q{tuple(q.shape)} {q.dtype} "
                          f"strides {q.stride()} / k{tuple(k.shape)} / v{tuple(v.shape)}")
     b, h, t, d = q.shape
-    out = torch.empty((b, t, h, d), dtype=q.dtype, device=q.device)
     i64x3 = ctypes.c_int64 * 3
     strides = [i64x3(x.stride(0), x.stride(1), x.stride(2)) for x in (q, k, v)]
-    o_str = i64x3(out.stride(0), out.stride(2), out.stride(1))
+    if like_query:
+        out = _gradient_like(q)
+        o_str = i64x3(out.stride(0), out.stride(1), out.stride(2))
+    else:
+        out = torch.empty((b, t, h, d), dtype=q.dtype, device=q.device)
+        o_str = i64x3(out.stride(0), out.stride(2), out.stride(1))
     lse = torch.empty((b, h, t), dtype=torch.float32, device=q.device) if return_lse else None
     rc = _ek.lib().tmb_attention_fwd(out.data_ptr(), lse.data_ptr() if return_lse else None,
                                      q.data_ptr(), k.data_ptr(), v.data_ptr(),
@@ -331,6 +337,16 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, c
                                      int(bool(round_like_unfused)), code_of(q.dtype), _stream())
     _check("tmb_attention_fwd", rc)
     return (out, lse) if return_lse else out
+
+
+def _gradient_like(x: torch.Tensor) -> torch.Tensor:
+    """A [batch, heads, tokens, 64] buffer laid out as `torch.empty_like(x)` when the kernels can
+    write that layout (rows of 64 contiguous, strides multiples of 4), token-major otherwise."""
+    like = torch.empty_like(x)
+    if like.stride(3) == 1 and all(s % 4 == 0 and s >= 0 for s in like.stride()[:3]):
+        return like
+    b, h, t, d = x.shape
+    return torch.empty((b, t, h, d), dtype=x.dtype, device=x.device).transpose(1, 2)
 
 
 def attention_backward_supported(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor,
@@ -353,13 +369,15 @@ def attention_backward_supported(dout: torch.Tensor, q: torch.Tensor, k: torch.T
 
 
 def attention_backward(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-                       out: torch.Tensor, lse: torch.Tensor, scale: float, causal: bool):
+                       out: torch.Tensor, lse: torch.Tensor, scale: float, causal: bool,
+                       packed: bool = False):
     """(dq, dk, dv) of `attention`: `out` and `dout` are [batch, heads, q_len, 64] views (the
     transposed view of what `attention` returned, and the gradient in the same layout), `lse` what
-    `attention(..., return_lse=True)` returned. The three gradients are [batch, heads, tokens, 64]
-    views of one packed [batch, tokens, 3, heads, 64] buffer when q_len == kv_len (so the gradient
-    of a packed q/k/v projection needs no concatenation), separate [batch, tokens, heads, 64]
-    buffers otherwise."""
+    `attention(..., return_lse=True)` returned. Each gradient is laid out as
+    `torch.empty_like` of its input (what ATen's fused attention backward returns); with `packed`
+    and q_len == kv_len the three are [batch, heads, tokens, 64] views of one
+    [batch, tokens, 3, heads, 64] buffer, so the gradient of a packed q/k/v projection needs no
+    concatenation."""
     require_hip(dout, q, k, v, out, lse)
     if not (scale > 0.0 and math.isfinite(scale)):
         raise ValueError(f"attention_backward: scale must be positive and finite, got {scale}")
@@ -367,13 +385,11 @@ def attention_backward(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: 
         raise ValueError("attention_backward: unsupported operands (see attention_backward_supported)")
     b, h, t, d = q.shape
     s_len = k.shape[2]
-    if t == s_len:
-        packed = torch.empty((b, t, 3, h, d), dtype=q.dtype, device=q.device)
-        dq, dk, dv = (packed[:, :, i].transpose(1, 2) for i in range(3))
+    if packed and t == s_len:
+        buf = torch.empty((b, t, 3, h, d), dtype=q.dtype, device=q.device)
+        dq, dk, dv = (buf[:, :, i].transpose(1, 2) for i in range(3))
     else:
-        dq = torch.empty((b, t, h, d), dtype=q.dtype, device=q.device).transpose(1, 2)
-        dk = torch.empty((b, s_len, h, d), dtype=q.dtype, device=q.device).transpose(1, 2)
-        dv = torch.empty((b, s_len, h, d), dtype=q.dtype, device=q.device).transpose(1, 2)
+        dq, dk, dv = _gradient_like(q), _gradient_like(k), _gradient_like(v)
     lib = _ek.lib()
     workspace = torch.empty(max(int(lib.tmb_attention_bwd_workspace_bytes(b, h, t)), 16),
                             dtype=torch.uint8, device=q.device)

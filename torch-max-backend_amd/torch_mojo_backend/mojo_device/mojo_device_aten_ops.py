@@ -126,6 +126,10 @@ _register_fast("aten::mean.dim", "fast_aten_mean")
 _register_fast("aten::mm", "fast_aten_mm")
 _register_fast("aten::native_layer_norm", "fast_aten_native_layer_norm")
 _register_fast("aten::scaled_dot_product_attention", "fast_aten_scaled_dot_product_attention")
+_register_fast("aten::_scaled_dot_product_flash_attention",
+               "fast_aten__scaled_dot_product_flash_attention")
+_register_fast("aten::_scaled_dot_product_flash_attention_backward",
+               "fast_aten__scaled_dot_product_flash_attention_backward")  # reference :881-882
 _register_fast("aten::softmax.int", "fast_aten_softmax")
 _register_fast("aten::sum.dim_IntList", "fast_aten_sum")
 # backward twins (reference :930-1000 registers the same op names)

@@ -54,6 +54,15 @@ def _contiguous(self, *, memory_format=torch.contiguous_format):
     return _below_autograd(aten.contiguous, self, memory_format=memory_format)
 
 
+def _fused_attention_takes(query, key, value, scale) -> bool:
+    from torch_mojo_backend.eager_kernels import hip_ops
+    from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
+
+    if not all(isinstance(x, TorchMojoTensor) for x in (query, key, value)) or not scale > 0.0:
+        return False
+    return query.dim() == 4 and hip_ops.attention_supported(query._holder, key._holder, value._holder)
+
+
 def _sdpa(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None,
           enable_gqa=False):
     if not _wants_grad(query, key, value):
@@ -62,8 +71,13 @@ def _sdpa(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, 
     if dropout_p != 0.0 or enable_gqa:
         raise NotImplementedError("scaled_dot_product_attention with dropout or grouped-query "
                                   "attention has no gradient on the mojo device")
-    # the differentiable route: matmul, scale, mask, softmax, matmul (each with a derivative)
     s = float(scale) if scale is not None else 1.0 / math.sqrt(query.shape[-1])
+    if attn_mask is None and _fused_attention_takes(query, key, value, s):
+        # one fused forward that also returns the log-sum-exp; PyTorch's derivative formula of
+        # this op calls _scaled_dot_product_flash_attention_backward, the fused backward
+        return aten._scaled_dot_product_flash_attention(query, key, value, 0.0, bool(is_causal),
+                                                        False, scale=s)[0]
+    # the differentiable route: matmul, scale, mask, softmax, matmul (each with a derivative)
     scores = torch.matmul(query, key.transpose(-2, -1)) * s
     t, n = query.shape[-2], key.shape[-2]
     if is_causal:
