@@ -307,6 +307,20 @@ def main() -> int:
             "frac_mfma": round(useful / ms / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4),
             "GB/s": round(algo_bytes / ms / 1e6, 1), "flops": useful, "bytes": algo_bytes,
             "note": "useful FLOPs (masked half not counted); scores never reach memory"}
+        # its backward: dq, dk, dv from q, k, v, out, dout and the forward's log-sum-exp, gradients
+        # written as the thirds of one packed buffer. Useful FLOPs = 2.5 x the forward's (five
+        # products against two); the kernels recompute scores and dP in both launches (seven).
+        out_f, lse_f = hip_ops.attention(q4, k4, v4, 0.125, True, return_lse=True)
+        dout = gen((Bq, Tq, Hq, 64), 34, torch.bfloat16).transpose(1, 2)
+        _, ms = timed(lambda: hip_ops.attention_backward(dout, q4, k4, v4, out_f.transpose(1, 2), lse_f,
+                                                         0.125, True, packed=True), 30, 8)
+        sweep["attention_backward_causal_bf16_32x12x1024x64"] = {
+            "us": round(ms * 1e3, 2), "TFLOP/s": round(2.5 * useful / ms / 1e9, 1),
+            "frac_mfma": round(2.5 * useful / ms / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4),
+            "flops": 2.5 * useful,
+            "note": "two launches (dq; dk and dv), no atomics; useful FLOPs = 5 products over the "
+                    "unmasked half"}
+        del out_f, lse_f, dout
         # a decode step of the eager generation benchmark (batch 512, 12 heads, 1 query, 208 keys):
         # K and V are read once; rotated over several caches so no cache level holds them
         Bd, Sd = 512, 208

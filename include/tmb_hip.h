@@ -288,6 +288,16 @@ int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_bet
                                  const float* rstd, const void* gamma, int64_t rows, int64_t cols,
                                  int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Concatenation of two contiguous row blocks: out[r] = a[r] ++ b[r] for `rows` rows of
+ * `a_row_bytes` and `b_row_bytes` bytes (any element type; the widest of 16/4/2/1-byte pieces that
+ * the lengths and the three addresses allow is moved). With rows = the product of the dims in
+ * front of the concatenated one this is aten::cat of two contiguous tensors, in particular the
+ * append of one token to a [batch, heads, tokens, head_dim] key/value cache.
+ * Replaces `Cat2` (eager_kernels/data_movement_ops.mojo:217-340, called from
+ * aten_fast.py:2203-2228). */
+int tmb_cat2_rows(void* out, const void* a, const void* b, int64_t rows, int64_t a_row_bytes,
+                  int64_t b_row_bytes, void* stream);
+
 /* Plain device copy kernel (16-byte vectors, grid-stride) — the bandwidth yardstick the
  * benchmark and the counter calibration use. No reference counterpart. */
 int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* stream);

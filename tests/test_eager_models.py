@@ -30,8 +30,9 @@ def test_demo_gpt2_forward_runs_eagerly_on_the_hip_kernels(mojo):
     assert torch.equal(nxt.cpu(), want_next)
     grew = {k for k, v in EAGER_CALL_COUNTERS.items() if v.call_count > before[k]}
     # every hot op of the forward went through its fast_aten_* twin
-    # (eagerly, nn.Linear is aten::linear and F.softmax is aten::softmax.int; nothing decomposes)
-    for op in ("aten::linear", "aten::native_layer_norm", "aten::bmm", "aten::softmax.int",
+    # (eagerly, nn.Linear is aten::linear, F.softmax is aten::softmax.int and F.layer_norm is
+    # aten::layer_norm, which skips the row statistics nobody reads without a gradient)
+    for op in ("aten::linear", "aten::layer_norm", "aten::bmm", "aten::softmax.int",
                "aten::gelu", "aten::argmax"):
         assert op in grew, f"{op} did not run on the mojo device ({sorted(grew)})"
 
@@ -144,3 +145,76 @@ def test_sdpa_gradients_on_the_eager_device_come_from_the_fused_backward(mojo):
     # float32 heads keep the composed, differentiable route
     _, grad32 = run(qkv.to(mojo), g.to(mojo), torch.float32)
     assert (grad32.cpu().double() - want_grad).abs().max().item() <= 1e-4 * big
+
+
+def test_cat_of_two_contiguous_tensors_is_one_launch_and_matches_torch(mojo):
+    """The key/value-cache append of a decode step, and every alignment class of the row-append
+    kernel (16-, 4-, 2- and 1-byte pieces); other inputs take PyTorch-ROCm's cat on the holders."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    calls = []
+    real = hip_ops.cat2
+    hip_ops.cat2 = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        cases = [((4, 3, 10, 64), (4, 3, 1, 64), 2, torch.bfloat16),   # cache append
+                 ((4, 3, 10, 64), (4, 3, 1, 64), -2, torch.float16),
+                 ((5, 6), (5, 2), 1, torch.float32),                    # 4-byte pieces
+                 ((5, 3), (5, 1), 1, torch.bfloat16),                   # 2-byte pieces
+                 ((7, 3), (7, 2), 1, torch.uint8),                      # single bytes
+                 ((2, 5), (3, 5), 0, torch.int64),                      # one row: plain append
+                 ((3, 0, 4), (3, 2, 4), 1, torch.float32)]              # an empty first operand
+        for sa, sb, dim, dtype in cases:
+            a = (torch.randn(sa) * 10).to(dtype) if dtype.is_floating_point else torch.randint(0, 100, sa).to(dtype)
+            b = (torch.randn(sb) * 10).to(dtype) if dtype.is_floating_point else torch.randint(0, 100, sb).to(dtype)
+            got = torch.cat([a.to(mojo), b.to(mojo)], dim=dim)
+            assert got.device.type == "mojo"
+            assert torch.equal(got.cpu(), torch.cat([a, b], dim=dim)), (sa, sb, dim, dtype)
+        assert len(calls) == len(cases)
+        # three inputs, and a strided input: PyTorch-ROCm's cat
+        x = torch.randn(4, 6)
+        got = torch.cat([x.to(mojo), x.to(mojo), x.to(mojo)], dim=0)
+        assert torch.equal(got.cpu(), torch.cat([x, x, x], dim=0))
+        got = torch.cat([x.to(mojo).t(), x.to(mojo).t()], dim=1)
+        assert torch.equal(got.cpu(), torch.cat([x.t(), x.t()], dim=1))
+        assert len(calls) == len(cases)
+    finally:
+        hip_ops.cat2 = real
+
+
+def test_lean_elementwise_and_split_match_torch(mojo):
+    x, y = torch.randn(3, 8), torch.randn(3, 8)
+    xm, ym = x.to(mojo), y.to(mojo)
+    for got, want in ((xm + ym, x + y), (xm * ym, x * y), (xm - ym, x - y), (xm * 0.5, x * 0.5),
+                      (2 + xm, 2 + x), (torch.pow(xm, 3.0), torch.pow(x, 3.0)), (torch.tanh(xm), torch.tanh(x)),
+                      (torch.add(xm, ym, alpha=2), torch.add(x, y, alpha=2)),
+                      (xm + ym[0], x + y[0]), (xm * torch.tensor(2.0), x * 2.0)):
+        assert got.device.type == "mojo"
+        torch.testing.assert_close(got.cpu(), want)
+    parts = xm.split(3, dim=1)
+    assert [tuple(p.shape) for p in parts] == [(3, 3), (3, 3), (3, 2)]
+    for p, w in zip(parts, x.split(3, dim=1)):
+        assert torch.equal(p.cpu(), w)
+
+
+def test_layer_norm_without_gradient_skips_the_statistics(mojo):
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    seen = []
+    real = hip_ops.layer_norm
+    hip_ops.layer_norm = lambda *a, **k: (seen.append(k.get("need_stats", True)), real(*a, **k))[1]
+    try:
+        x, w, b = torch.randn(4, 5, 48), torch.randn(48), torch.randn(48)
+        want = torch.nn.functional.layer_norm(x, (48,), w, b, 1e-5)
+        with torch.no_grad():
+            got = torch.nn.functional.layer_norm(x.to(mojo), (48,), w.to(mojo), b.to(mojo), 1e-5)
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+        assert seen == [False]
+        xg = x.to(mojo).requires_grad_(True)
+        out = torch.nn.functional.layer_norm(xg, (48,), w.to(mojo), b.to(mojo), 1e-5)
+        out.sum().backward()
+        assert seen == [False, True] and xg.grad is not None
+        xr = x.clone().requires_grad_(True)
+        torch.nn.functional.layer_norm(xr, (48,), w, b, 1e-5).sum().backward()
+        torch.testing.assert_close(xg.grad.cpu(), xr.grad, rtol=1e-4, atol=1e-5)
+    finally:
+        hip_ops.layer_norm = real

@@ -357,3 +357,4 @@ def test_out_of_memory_launch_status_becomes_torch_out_of_memory_error(monkeypat
     x = torch.zeros(2, 4)
     with pytest.raises(torch.OutOfMemoryError, match="tmb_softmax_rows"):
         hip_ops.softmax(x, -1)
+

@@ -68,7 +68,73 @@ __global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ out,
   if (blockIdx.x == 0 && threadIdx.x < tail) out_tail[threadIdx.x] = in_tail[threadIdx.x];
 }
 
+// out[r, :] = a[r, :] followed by b[r, :] for contiguous a [rows, a_units] and b [rows, b_units]
+// of UNIT-sized pieces: the append of a key/value cache (a long row and a short one) in one
+// launch. One thread moves four pieces of the output, 256 apart.
+template <typename UNIT, typename IDX>
+__global__ __launch_bounds__(256) void cat2_rows_kernel(UNIT* __restrict__ out,
+                                                        const UNIT* __restrict__ a,
+                                                        const UNIT* __restrict__ b, IDX total,
+                                                        IDX a_units, IDX b_units) {
+  const IDX out_units = a_units + b_units;
+  const IDX base = static_cast<IDX>(blockIdx.x) * 1024 + threadIdx.x;
+  UNIT v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const IDX i = base + u * 256;
+    if (i < total) {
+      const IDX row = i / out_units, c = i - row * out_units;
+      v[u] = c < a_units ? a[row * a_units + c] : b[row * b_units + (c - a_units)];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const IDX i = base + u * 256;
+    if (i < total) out[i] = v[u];
+  }
+}
+
+template <typename UNIT>
+int launch_cat2(void* out, const void* a, const void* b, int64_t rows, int64_t a_bytes,
+                int64_t b_bytes, hipStream_t s) {
+  const int64_t au = a_bytes / static_cast<int64_t>(sizeof(UNIT));
+  const int64_t bu = b_bytes / static_cast<int64_t>(sizeof(UNIT));
+  const int64_t total = rows * (au + bu);
+  const int64_t blocks = (total + 1023) / 1024;
+  if (blocks >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(blocks));
+  if (total + 1024 < (int64_t{1} << 32)) {
+    cat2_rows_kernel<UNIT, uint32_t><<<grid, dim3(256), 0, s>>>(
+        static_cast<UNIT*>(out), static_cast<const UNIT*>(a), static_cast<const UNIT*>(b),
+        static_cast<uint32_t>(total), static_cast<uint32_t>(au), static_cast<uint32_t>(bu));
+  } else {
+    cat2_rows_kernel<UNIT, uint64_t><<<grid, dim3(256), 0, s>>>(
+        static_cast<UNIT*>(out), static_cast<const UNIT*>(a), static_cast<const UNIT*>(b),
+        static_cast<uint64_t>(total), static_cast<uint64_t>(au), static_cast<uint64_t>(bu));
+  }
+  return check_launch();
+}
+
 }  // namespace tmb
+
+extern "C" int tmb_cat2_rows(void* out, const void* a, const void* b, int64_t rows,
+                             int64_t a_row_bytes, int64_t b_row_bytes, void* stream) {
+  if (rows < 0 || a_row_bytes < 0 || b_row_bytes < 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || a_row_bytes + b_row_bytes == 0) return TMB_OK;
+  if (!out || (a_row_bytes && !a) || (b_row_bytes && !b)) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows >= (int64_t{1} << 40) || a_row_bytes >= (int64_t{1} << 40) ||
+      b_row_bytes >= (int64_t{1} << 40))
+    return TMB_ERR_UNSUPPORTED;
+  // the widest piece that divides both row lengths and every base address
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(a) |
+                         reinterpret_cast<uintptr_t>(b) | static_cast<uintptr_t>(a_row_bytes) |
+                         static_cast<uintptr_t>(b_row_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if ((bits & 15) == 0) return tmb::launch_cat2<uint4>(out, a, b, rows, a_row_bytes, b_row_bytes, s);
+  if ((bits & 3) == 0) return tmb::launch_cat2<uint32_t>(out, a, b, rows, a_row_bytes, b_row_bytes, s);
+  if ((bits & 1) == 0) return tmb::launch_cat2<uint16_t>(out, a, b, rows, a_row_bytes, b_row_bytes, s);
+  return tmb::launch_cat2<uint8_t>(out, a, b, rows, a_row_bytes, b_row_bytes, s);
+}
 
 extern "C" int tmb_version(void) { return 1000; }
 

@@ -33,8 +33,7 @@ def _t(x):
     return x if isinstance(x, TorchMojoTensor) else None
 
 
-def _wrap(holder: torch.Tensor) -> TorchMojoTensor:
-    return TorchMojoTensor._wrap(holder)
+_wrap = TorchMojoTensor._adopt  # results of the kernels below: HIP tensors, never part of a graph
 
 
 def fast_filled(shape, value, dtype, device) -> TorchMojoTensor:
@@ -171,7 +170,22 @@ def fast_aten__log_softmax(input, dim, half_to_float=False):
 def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0,
                                            is_causal=False, *, scale=None, enable_gqa=False):
     q, k, v = _t(query), _t(key), _t(value)
-    if q is None or k is None or v is None or not _same_device(q, k, v):
+    if q is None or k is None or v is None:
+        return NOT_HANDLED
+    hq, hk, hv = q._holder, k._holder, v._holder
+    # a decode step first (a few queries per head, every layer of every generated token): its
+    # own support check covers dtypes, shapes and layouts, so the general checks below are skipped
+    if dropout_p == 0.0 and not enable_gqa and hq.dim() == 4 \
+            and hq.shape[2] <= hip_ops.DECODE_MAX_QUERIES and hk.device == hq.device \
+            and hv.device == hq.device and not (attn_mask is not None and is_causal):
+        mask0 = None if attn_mask is None else _t(attn_mask)
+        if (attn_mask is None or (mask0 is not None and mask0._holder.device == hq.device)) \
+                and hip_ops.attention_decode_supported(hq, hk, hv, None if mask0 is None else mask0._holder):
+            s0 = float(scale) if scale is not None else 1.0 / math.sqrt(hq.shape[-1])
+            return _wrap(hip_ops.attention_decode(hq, hk, hv, s0, bool(is_causal),
+                                                  None if mask0 is None else mask0._holder,
+                                                  checked=True))
+    if not _same_device(q, k, v):
         return NOT_HANDLED
     if dropout_p != 0.0 or enable_gqa or len(q._shape) < 2 or q._dtype not in _FLOAT_DTYPES \
             or k._dtype != q._dtype or v._dtype != q._dtype:
@@ -192,7 +206,7 @@ def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dr
     if len(q._shape) == 4 and q._shape[2] <= hip_ops.DECODE_MAX_QUERIES \
             and hip_ops.attention_decode_supported(q._holder, k._holder, v._holder, mask_h):
         return _wrap(hip_ops.attention_decode(q._holder, k._holder, v._holder, s, bool(is_causal),
-                                              mask_h))
+                                              mask_h, checked=True))
     if mask is None and s > 0.0 and len(q._shape) == 4 \
             and hip_ops.attention_supported(q._holder, k._holder, v._holder):
         out = hip_ops.attention(q._holder, k._holder, v._holder, s, bool(is_causal))
@@ -200,6 +214,29 @@ def fast_aten_scaled_dot_product_attention(query, key, value, attn_mask=None, dr
     # other head sizes, fp32, additive masks: GEMM + softmax + GEMM
     return _wrap(hip_ops.attention_composed(q._holder, k._holder, v._holder, s, bool(is_causal),
                                             None if mask is None else mask._holder))
+
+
+# ---------------------------------------------------------------------------
+# Concatenation of two contiguous tensors (reference :2173-2256): the key/value-cache append
+# ---------------------------------------------------------------------------
+def fast_aten_cat(tensors, dim=0):
+    """Two contiguous mojo tensors: one launch of the row-append kernel. Anything else (more
+    inputs, strided inputs, the legacy 1-D empty tensor PyTorch skips) is PyTorch-ROCm's cat on
+    the holders, as the other cold ops run."""
+    if len(tensors) == 2 and type(dim) is int:
+        a, b = _t(tensors[0]), _t(tensors[1])
+        if a is not None and b is not None:
+            ha, hb = a._holder, b._holder
+            rank = ha.dim()
+            if rank and -rank <= dim < rank and hip_ops.cat2_supported(ha, hb, dim % rank):
+                return _wrap(hip_ops.cat2(ha, hb, dim % rank))
+    holders = []
+    for x in tensors:
+        t = _t(x)
+        if t is None:
+            return NOT_HANDLED
+        holders.append(t._holder)
+    return _wrap(torch.cat(holders, dim))
 
 
 def _flash_operands(query, key, value, dropout_p, scale):
@@ -277,6 +314,26 @@ def fast_aten_native_layer_norm(input, normalized_shape, weight, bias, eps):
                                          None if gamma is None else gamma._holder,
                                          None if beta is None else beta._holder, float(eps))
     return _wrap(out), _wrap(mean), _wrap(rstd)
+
+
+def fast_aten_layer_norm(input, normalized_shape, weight=None, bias=None, eps=1e-5,
+                         cudnn_enable=True):
+    """aten::layer_norm registered whole: without a gradient nobody reads the row statistics, so
+    neither buffer is allocated or written (the composite would call native_layer_norm and drop
+    two of its three results)."""
+    a = _t(input)
+    gamma = None if weight is None else _t(weight)
+    beta = None if bias is None else _t(bias)
+    if a is None or (weight is not None and gamma is None) or (bias is not None and beta is None):
+        return NOT_HANDLED
+    try:
+        out, _, _ = hip_ops.layer_norm(a._holder, tuple(normalized_shape),
+                                       None if gamma is None else gamma._holder,
+                                       None if beta is None else beta._holder, float(eps),
+                                       need_stats=False)
+    except (ValueError, TypeError):
+        return NOT_HANDLED
+    return _wrap(out)
 
 
 # ---------------------------------------------------------------------------

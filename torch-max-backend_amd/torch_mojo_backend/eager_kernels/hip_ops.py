@@ -63,10 +63,14 @@ def require_hip(*tensors: Optional[torch.Tensor]) -> torch.device:
     return dev
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream
+_current_device = torch.cuda.current_device
+
+
 def _stream() -> int:
     """The raw hipStream_t of PyTorch's current stream on the current device (the private
     accessor costs a fraction of building a torch.cuda.Stream object per launch)."""
-    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    return _raw_stream(_current_device())
 
 
 def code_of(dtype: torch.dtype) -> int:
@@ -91,6 +95,7 @@ def _matrix_layout(t: torch.Tensor) -> Optional[Tuple[int, int]]:
     return None
 
 
+_I64X3 = ctypes.c_int64 * 3
 _GEMM_WS_BYTES: dict = {}
 _GEMM_PLANS: dict = {}
 
@@ -436,23 +441,28 @@ def attention_decode_supported(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
 
 
 def attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
-                     causal: bool, attn_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     causal: bool, attn_mask: Optional[torch.Tensor] = None,
+                     checked: bool = False) -> torch.Tensor:
     """softmax(scale q kᵀ [masked]) v for a few queries per head in one launch; returns
-    [batch, heads, tokens, head_dim] contiguous."""
-    require_hip(q, k, v, attn_mask)
-    if not attention_decode_supported(q, k, v, attn_mask):
-        raise ValueError("attention_decode: unsupported operands (see attention_decode_supported)")
+    [batch, heads, tokens, head_dim] contiguous. `checked`: the caller has just seen
+    `attention_decode_supported` accept exactly these operands."""
+    if not checked:
+        require_hip(q, k, v, attn_mask)
+        if not attention_decode_supported(q, k, v, attn_mask):
+            raise ValueError("attention_decode: unsupported operands (see attention_decode_supported)")
     b, h, t, d = q.shape
     out = torch.empty((b, h, t, d), dtype=q.dtype, device=q.device)
-    arr = lambda strides: (ctypes.c_int64 * len(strides))(*strides)  # noqa: E731
+    i64x3 = _I64X3
     mask_ptr, mask_strides = None, None
     if attn_mask is not None:
         m4 = attn_mask.expand(b, h, t, k.shape[2])  # stride 0 where it broadcasts
-        mask_ptr, mask_strides = m4.data_ptr(), arr(m4.stride())
+        mask_ptr, mask_strides = m4.data_ptr(), (ctypes.c_int64 * 4)(*m4.stride())
+    qs, ks, vs = q.stride(), k.stride(), v.stride()
     rc = _ek.lib().tmb_attention_decode(
         out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), mask_ptr, b, h, t, k.shape[2], d,
-        arr(q.stride()[:3]), arr(k.stride()[:3]), arr(v.stride()[:3]), arr(out.stride()[:3]),
-        mask_strides, float(scale), int(bool(causal)), code_of(q.dtype), _stream())
+        i64x3(qs[0], qs[1], qs[2]), i64x3(ks[0], ks[1], ks[2]), i64x3(vs[0], vs[1], vs[2]),
+        i64x3(h * t * d, t * d, d), mask_strides, float(scale), int(bool(causal)),
+        _CODES[q.dtype], _stream())
     _check("tmb_attention_decode", rc)
     return out
 
@@ -487,6 +497,9 @@ def attention_composed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale:
     return gemm(probs, v3).view(*lead, t, v.shape[-1])
 
 
+_LN_PLANS: dict = {}
+
+
 def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optional[torch.Tensor],
                bias: Optional[torch.Tensor], eps: float, need_stats: bool = True,
                out_dtype: Optional[torch.dtype] = None):
@@ -494,6 +507,25 @@ def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optiona
     when ``need_stats`` is False. ``out_dtype`` (default: the input's) may be a 16-bit type for
     a float32 input: the row is read in float32 and the result cast once; weight and bias then
     have the output's type."""
+    # a layout already validated (every layer of every decode step): straight to the launch
+    key = (x.shape, x.stride(), x.dtype, x.device, tuple(normalized_shape), out_dtype, need_stats,
+           None if weight is None else (weight.shape, weight.stride(), weight.dtype, weight.device),
+           None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device))
+    plan = _LN_PLANS.get(key)
+    if plan is not None:
+        rows, cols, stat_shape, in_code, out_code, odt = plan
+        out = torch.empty(x.shape, dtype=odt, device=x.device)
+        mean = rstd = None
+        if need_stats:
+            mean = torch.empty(stat_shape, dtype=torch.float32, device=x.device)
+            rstd = torch.empty(stat_shape, dtype=torch.float32, device=x.device)
+        rc = _ek.lib().tmb_layer_norm_rows(
+            out.data_ptr(), None if mean is None else mean.data_ptr(),
+            None if rstd is None else rstd.data_ptr(), x.data_ptr(),
+            None if weight is None else weight.data_ptr(), None if bias is None else bias.data_ptr(),
+            rows, cols, float(eps), in_code, out_code, _stream())
+        _check("tmb_layer_norm_rows", rc)
+        return out, mean, rstd
     require_hip(x, weight, bias)
     k = len(normalized_shape)
     out_dtype = x.dtype if out_dtype is None else out_dtype
@@ -524,6 +556,10 @@ def layer_norm(x: torch.Tensor, normalized_shape: Sequence[int], weight: Optiona
             None if w is None else w.data_ptr(), None if b is None else b.data_ptr(),
             rows, cols, float(eps), code_of(x.dtype), code_of(out_dtype), _stream())
         _check("tmb_layer_norm_rows", rc)
+        if xc is x and (weight is None or w is weight) and (bias is None or b is bias):
+            if len(_LN_PLANS) >= 1024:
+                _LN_PLANS.clear()
+            _LN_PLANS[key] = (rows, cols, stat_shape, code_of(x.dtype), code_of(out_dtype), out_dtype)
     return out, mean, rstd
 
 
@@ -610,6 +646,36 @@ def embedding(table: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
                                    rows, code_of(table.dtype),
                                    _ek.I64 if indices.dtype == torch.int64 else _ek.I32, _stream())
     _check("tmb_gather_rows", rc)
+    return out
+
+
+def cat2_supported(a: torch.Tensor, b: torch.Tensor, dim: int) -> bool:
+    """True when `cat2` takes these two tensors: same device, dtype and rank, equal sizes apart
+    from `dim` (already normalised), both contiguous, not both empty."""
+    if a.dtype != b.dtype or a.device != b.device or not a.is_cuda or a.dim() != b.dim() \
+            or not 0 <= dim < a.dim() or not (a.is_contiguous() and b.is_contiguous()):
+        return False
+    sa, sb = a.shape, b.shape
+    for i in range(a.dim()):
+        if i != dim and sa[i] != sb[i]:
+            return False
+    return a.numel() + b.numel() > 0
+
+
+def cat2(a: torch.Tensor, b: torch.Tensor, dim: int) -> torch.Tensor:
+    """``torch.cat([a, b], dim)`` for two contiguous tensors in one launch (reference:
+    aten_fast.py:2203-2228, the key/value-cache append of a decode step)."""
+    if not cat2_supported(a, b, dim):
+        raise ValueError(f"cat2: unsupported operands {tuple(a.shape)} {a.dtype} / "
+                         f"{tuple(b.shape)} {b.dtype}, dim {dim}")
+    shape = list(a.shape)
+    shape[dim] += b.shape[dim]
+    out = torch.empty(shape, dtype=a.dtype, device=a.device)
+    rows = math.prod(shape[:dim])
+    inner = math.prod(shape[dim + 1:]) * a.element_size()
+    rc = _ek.lib().tmb_cat2_rows(out.data_ptr(), a.data_ptr(), b.data_ptr(), rows,
+                                 a.shape[dim] * inner, b.shape[dim] * inner, _stream())
+    _check("tmb_cat2_rows", rc)
     return out
 
 

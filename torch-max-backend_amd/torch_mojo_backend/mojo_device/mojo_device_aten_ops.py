@@ -125,12 +125,14 @@ _register_fast("aten::mean", "fast_aten_mean")
 _register_fast("aten::mean.dim", "fast_aten_mean")
 _register_fast("aten::mm", "fast_aten_mm")
 _register_fast("aten::native_layer_norm", "fast_aten_native_layer_norm")
+_register_fast("aten::layer_norm", "fast_aten_layer_norm")
 _register_fast("aten::scaled_dot_product_attention", "fast_aten_scaled_dot_product_attention")
 _register_fast("aten::_scaled_dot_product_flash_attention",
                "fast_aten__scaled_dot_product_flash_attention")
 _register_fast("aten::_scaled_dot_product_flash_attention_backward",
                "fast_aten__scaled_dot_product_flash_attention_backward")  # reference :881-882
 _register_fast("aten::softmax.int", "fast_aten_softmax")
+_register_fast("aten::cat", "fast_aten_cat")  # reference :914
 _register_fast("aten::sum.dim_IntList", "fast_aten_sum")
 # backward twins (reference :930-1000 registers the same op names)
 _register_fast("aten::gelu_backward", "fast_aten_gelu_backward")
@@ -248,9 +250,11 @@ def _local_scalar_dense(self):
 
 
 def _view_op(op_name: str, fn: Callable):
+    adopt = TorchMojoTensor._adopt
+
     @register_aten_op(op_name)
     def view(self, *args, **kwargs):
-        return TorchMojoTensor._wrap(fn(self._holder, *args, **kwargs))
+        return adopt(fn(self._holder, *args, **kwargs))
 
     return view
 
@@ -369,7 +373,7 @@ _HOLDER_OPS = (
     "aten::multinomial",
     # indexing, gathering, concatenation
     "aten::index_select", "aten::gather", "aten::index.Tensor",
-    "aten::index_put_", "aten::cat", "aten::stack", "aten::split.Tensor",
+    "aten::index_put_", "aten::stack",
     "aten::split_with_sizes", "aten::unbind.int", "aten::squeeze", "aten::flatten.using_ints",
     "aten::tril", "aten::triu", "aten::repeat", "aten::roll",
     # fills, copies and factories
@@ -386,5 +390,52 @@ _HOLDER_OPS = (
     "aten::mul_.Scalar", "aten::add_.Scalar", "aten::addcmul_", "aten::addcdiv_", "aten::sqrt_",
     "aten::lerp_.Scalar", "aten::log", "aten::sum_to_size",
 )
+# The elementwise ops a decode loop issues by the hundred per token (HF's tanh-GELU alone is
+# eight of them per layer) skip the generic argument walk: tensor-with-tensor and
+# tensor-with-number calls go to the torch function of the same op on the holders.
+_LEAN_BINARY = {"aten::add.Tensor": torch.add, "aten::mul.Tensor": torch.mul,
+                "aten::sub.Tensor": torch.sub, "aten::pow.Tensor_Scalar": torch.pow}
+_LEAN_UNARY = {"aten::tanh": torch.tanh}
+
+
+def _lean_binary(op_name: str, fn: Callable) -> Callable:
+    generic = holder_impl(op_name)
+    adopt = TorchMojoTensor._adopt
+
+    def impl(self, other, *rest, **kwargs):
+        if not rest and not kwargs and type(self) is TorchMojoTensor:
+            t = type(other)
+            if t is TorchMojoTensor:
+                return adopt(fn(self._holder, other._holder))
+            if t is float or t is int:
+                return adopt(fn(self._holder, other))
+        return generic(self, other, *rest, **kwargs)
+
+    return impl
+
+
+def _lean_unary(op_name: str, fn: Callable) -> Callable:
+    generic = holder_impl(op_name)
+    adopt = TorchMojoTensor._adopt
+
+    def impl(self, *rest, **kwargs):
+        if not rest and not kwargs and type(self) is TorchMojoTensor:
+            return adopt(fn(self._holder))
+        return generic(self, *rest, **kwargs)
+
+    return impl
+
+
 for _name in _HOLDER_OPS:
-    register_aten_op(_name)(holder_impl(_name))
+    if _name in _LEAN_BINARY:
+        register_aten_op(_name)(_lean_binary(_name, _LEAN_BINARY[_name]))
+    elif _name in _LEAN_UNARY:
+        register_aten_op(_name)(_lean_unary(_name, _LEAN_UNARY[_name]))
+    else:
+        register_aten_op(_name)(holder_impl(_name))
+
+
+@register_aten_op("aten::split.Tensor")
+def _split_tensor(self, split_size, dim=0):
+    adopt = TorchMojoTensor._adopt
+    return [adopt(piece) for piece in self._holder.split(split_size, dim)]

@@ -6,7 +6,7 @@ ops (``linear_backward``, ``native_layer_norm_backward``, ``gelu_backward``,
 ``_log_softmax_backward_data``, ``_softmax_backward_data``) through their PrivateUse1
 registrations. What is left for this module are the ops PyTorch would normally *decompose* before
 autograd sees them and which the eager device registers whole for speed (``softmax.int``,
-``contiguous``, ``scaled_dot_product_attention``): registered at the backend key they have no
+``contiguous``, ``layer_norm``, ``scaled_dot_product_attention``): registered at the backend key they have no
 derivative, so each gets an ``AutogradPrivateUse1`` kernel that takes the differentiable route
 when a gradient is wanted and the registered fast kernel otherwise (the reference keeps the same
 split in mojo_device/mojo_device_autograd.py:1-60).
@@ -18,8 +18,18 @@ import math
 
 import torch
 
+from .torch_mojo_tensor import DIRECT_IMPLS, TorchMojoTensor
+
 _registered = False
 aten = torch.ops.aten
+
+
+# the overloads the eager registry (and with it DIRECT_IMPLS) is keyed by
+_SOFTMAX_INT = aten.softmax.int
+_LOG_SOFTMAX_INT = aten.log_softmax.int
+_CONTIGUOUS = aten.contiguous.default
+_LAYER_NORM = aten.layer_norm.default
+_SDPA = aten.scaled_dot_product_attention.default
 
 
 def _wants_grad(*tensors) -> bool:
@@ -28,6 +38,15 @@ def _wants_grad(*tensors) -> bool:
 
 
 def _below_autograd(op, *args, **kwargs):
+    """The registered kernel of `op` when no gradient is wanted. With real HIP holders behind the
+    first argument the eager implementation is called directly (one Python entry per op, as
+    without an autograd kernel); while torch.compile traces (stand-in holders) or for other
+    argument types the call is redispatched below the autograd keys."""
+    first = args[0]
+    if type(first) is TorchMojoTensor and type(first._holder) is torch.Tensor:
+        impl = DIRECT_IMPLS.get(op)
+        if impl is not None:
+            return impl(*args, **kwargs)
     with torch._C._AutoDispatchBelowAutograd():
         return op(*args, **kwargs)
 
@@ -36,14 +55,14 @@ def _softmax_int(self, dim, dtype=None):
     if _wants_grad(self):
         x = self if dtype is None or dtype == self.dtype else self.to(dtype)
         return aten._softmax(x, dim, False)          # has a derivative: _softmax_backward_data
-    return _below_autograd(aten.softmax.int, self, dim, dtype)
+    return _below_autograd(_SOFTMAX_INT, self, dim, dtype)
 
 
 def _log_softmax_int(self, dim, dtype=None):
     if _wants_grad(self):
         x = self if dtype is None or dtype == self.dtype else self.to(dtype)
         return aten._log_softmax(x, dim, False)
-    return _below_autograd(aten.log_softmax.int, self, dim, dtype)
+    return _below_autograd(_LOG_SOFTMAX_INT, self, dim, dtype)
 
 
 def _contiguous(self, *, memory_format=torch.contiguous_format):
@@ -51,12 +70,17 @@ def _contiguous(self, *, memory_format=torch.contiguous_format):
         if self.is_contiguous(memory_format=memory_format):
             return aten.alias(self)
         return aten.clone(self, memory_format=memory_format)
-    return _below_autograd(aten.contiguous, self, memory_format=memory_format)
+    return _below_autograd(_CONTIGUOUS, self, memory_format=memory_format)
+
+
+def _layer_norm(input, normalized_shape, weight=None, bias=None, eps=1e-5, cudnn_enable=True):
+    if _wants_grad(input, weight, bias):
+        return aten.native_layer_norm(input, normalized_shape, weight, bias, eps)[0]
+    return _below_autograd(_LAYER_NORM, input, normalized_shape, weight, bias, eps, cudnn_enable)
 
 
 def _fused_attention_takes(query, key, value, scale) -> bool:
     from torch_mojo_backend.eager_kernels import hip_ops
-    from torch_mojo_backend.mojo_device.torch_mojo_tensor import TorchMojoTensor
 
     if not all(isinstance(x, TorchMojoTensor) for x in (query, key, value)) or not scale > 0.0:
         return False
@@ -66,8 +90,8 @@ def _fused_attention_takes(query, key, value, scale) -> bool:
 def _sdpa(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None,
           enable_gqa=False):
     if not _wants_grad(query, key, value):
-        return _below_autograd(aten.scaled_dot_product_attention, query, key, value, attn_mask,
-                               dropout_p, is_causal, scale=scale, enable_gqa=enable_gqa)
+        return _below_autograd(_SDPA, query, key, value, attn_mask, dropout_p, is_causal,
+                               scale=scale, enable_gqa=enable_gqa)
     if dropout_p != 0.0 or enable_gqa:
         raise NotImplementedError("scaled_dot_product_attention with dropout or grouped-query "
                                   "attention has no gradient on the mojo device")
@@ -95,6 +119,7 @@ _AUTOGRAD_KERNELS = {
     "aten::softmax.int": _softmax_int,
     "aten::log_softmax.int": _log_softmax_int,
     "aten::contiguous": _contiguous,
+    "aten::layer_norm": _layer_norm,
     "aten::scaled_dot_product_attention": _sdpa,
 }
 

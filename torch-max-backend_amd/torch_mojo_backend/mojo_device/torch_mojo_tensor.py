@@ -31,14 +31,19 @@ def _mojo_device(index: int) -> torch.device:
     return dev
 
 
+_make_wrapper = torch.Tensor._make_wrapper_subclass
+_STRIDED = torch.strided
+
+
 class TorchMojoTensor(torch.Tensor):
     @classmethod
     def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
         # Let higher-priority wrappers (FakeTensor, FunctionalTensor) handle mixed calls, then
         # continue into the mojo implementation of the exact overload PyTorch chose.
-        for t in types:
-            if t is not cls and not issubclass(cls, t):
-                return NotImplemented
+        if len(types) != 1 or types[0] is not cls:
+            for t in types:
+                if t is not cls and not issubclass(cls, t):
+                    return NotImplemented
         # torch.compile traces through this class with stand-in (fake / functional) holders: no
         # kernel can take those, the op is replayed on the holders instead (see _trace_dispatch)
         for a in args:
@@ -64,12 +69,24 @@ class TorchMojoTensor(torch.Tensor):
             raise NotImplementedError(f"mojo tensors support at most rank {MAX_RANK}, got {len(shape)}")
         if holder.requires_grad or holder.grad_fn is not None:
             holder = holder.detach()
-        res = torch.Tensor._make_wrapper_subclass(
-            cls, shape, strides=holder.stride(), storage_offset=holder.storage_offset(),
-            dtype=holder.dtype, layout=torch.strided, device=_mojo_device(device.index or 0),
-            requires_grad=False)
+        # positional (size, strides, storage_offset, memory_format, dtype, layout, device,
+        # pin_memory): keyword parsing is a quarter of this call, which runs once per eager op
+        res = _make_wrapper(cls, shape, holder.stride(), holder.storage_offset(), None, holder.dtype,
+                            _STRIDED, _mojo_device(device.index or 0), False)
         # This runs once per eager op: only the holder is stored, the layout attributes below
         # are read from it when an implementation asks for them.
+        res._holder = holder
+        return res
+
+    @classmethod
+    def _adopt(cls, holder: torch.Tensor) -> "TorchMojoTensor":
+        """`_wrap` for what an implementation on this device has just computed from holders: a
+        HIP tensor outside any autograd graph by construction, so only the rank is checked."""
+        shape = holder.shape
+        if len(shape) > MAX_RANK:
+            raise NotImplementedError(f"mojo tensors support at most rank {MAX_RANK}, got {len(shape)}")
+        res = _make_wrapper(cls, shape, holder.stride(), holder.storage_offset(), None, holder.dtype,
+                            _STRIDED, _mojo_device(holder.device.index or 0), False)
         res._holder = holder
         return res
 
