@@ -35,6 +35,7 @@ def fake_backend(monkeypatch):
     launched = []
     monkeypatch.setattr(aten_fast, "_t", lambda x: x if isinstance(x, types.SimpleNamespace) else None)
     monkeypatch.setattr(aten_fast, "_wrap", lambda holder: ("wrapped", holder))
+    monkeypatch.setattr(aten_fast.hip_ops, "gemm_if_planned", lambda *a, **k: None)  # nothing planned yet
     for name in ("gemm", "softmax", "layer_norm", "reduce", "argmax", "gelu"):
         monkeypatch.setattr(aten_fast.hip_ops, name,
                             lambda *a, _n=name, **k: launched.append(_n) or (_n, _n, _n))

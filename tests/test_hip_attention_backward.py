@@ -117,8 +117,9 @@ def test_attention_backward_reads_packed_projections_and_packs_its_gradients():
 
 def test_attention_backward_is_deterministic_at_the_benchmark_shape():
     """32 x 12 heads x 1024 tokens, causal (one GPT-2 block of the largest benchmark config):
-    no atomics, so two calls agree to the bit; the gradients match float32 autograd of the unfused
-    chain on the same device."""
+    no atomics, so two calls agree to the bit; the gradients of the first and the last batch entry
+    match float32 autograd of the unfused chain (on the host: autograd over HIP tensors is not
+    available in a process that has registered the eager device)."""
     b, h, t = 32, 12, 1024
     g = torch.Generator(device="cuda").manual_seed(0)
     q, k, v = (torch.randn(b, h, t, 64, device="cuda", generator=g).bfloat16() for _ in range(3))
@@ -131,13 +132,13 @@ def test_attention_backward_is_deterministic_at_the_benchmark_shape():
         assert torch.equal(a1, a2)
     # the reference chain one batch entry at a time: [12, 1024, 1024] float32 scores
     for bi in (0, b - 1):
-        q32, k32, v32 = (x[bi].float().requires_grad_(True) for x in (q, k, v))
+        q32, k32, v32 = (x[bi].float().cpu().requires_grad_(True) for x in (q, k, v))
         s = (q32 @ k32.transpose(-1, -2)) * 0.125
-        s = s.masked_fill(torch.ones(t, t, dtype=torch.bool, device="cuda").triu(1), float("-inf"))
-        (torch.softmax(s, -1) @ v32).backward(dout[bi].float().transpose(0, 1))
+        s = s.masked_fill(torch.ones(t, t, dtype=torch.bool).triu(1), float("-inf"))
+        (torch.softmax(s, -1) @ v32).backward(dout[bi].float().cpu().transpose(0, 1))
         for name, got, want in zip("qkv", first, (q32.grad, k32.grad, v32.grad)):
             big = want.abs().max().item()
-            err = (got[bi].float() - want).abs()
+            err = (got[bi].float().cpu() - want).abs()
             assert err.max().item() <= 2e-2 * big, (name, err.max().item() / big)
             assert err.mean().item() <= 2e-2 * big / 16, name
 

@@ -66,6 +66,11 @@ def fast_aten_addmm(input, mat1, mat2, *, beta=1.0, alpha=1.0):
     if beta != 1 or alpha != 1:
         return NOT_HANDLED
     bias, a, b = _t(input), _t(mat1), _t(mat2)
+    if bias is not None and a is not None and b is not None:
+        # the layout of a previous call (same module, next decode step): checked then
+        out = hip_ops.gemm_if_planned(a._holder, b._holder, bias._holder)
+        if out is not None:
+            return _wrap(out)
     if bias is None or not _gemm_operands_ok(a, b, 2) or not _same_device(a, bias):
         return NOT_HANDLED
     n = b._shape[1]
@@ -229,7 +234,7 @@ def fast_aten_cat(tensors, dim=0):
             ha, hb = a._holder, b._holder
             rank = ha.dim()
             if rank and -rank <= dim < rank and hip_ops.cat2_supported(ha, hb, dim % rank):
-                return _wrap(hip_ops.cat2(ha, hb, dim % rank))
+                return _wrap(hip_ops.cat2(ha, hb, dim % rank, checked=True))
     holders = []
     for x in tensors:
         t = _t(x)

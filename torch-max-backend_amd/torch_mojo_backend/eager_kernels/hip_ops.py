@@ -100,6 +100,32 @@ _GEMM_WS_BYTES: dict = {}
 _GEMM_PLANS: dict = {}
 
 
+def gemm_if_planned(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                    epi_flags: int = _ek.EPI_NONE) -> Optional[torch.Tensor]:
+    """``gemm(a, b, bias)`` when exactly this operand layout (shapes, strides, dtypes, devices)
+    has been validated and launched before, else None: the plan holds the launch arguments, so a
+    repeated call (every layer of every decode step) costs one dictionary lookup, one allocation
+    and the launch."""
+    plan = _GEMM_PLANS.get(
+        (a.shape, a.stride(), b.shape, b.stride(), a.dtype, b.dtype, a.device, b.device,
+         None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device)))
+    if plan is None:
+        return None
+    out_shape, dims, ws_bytes = plan
+    out = torch.empty(out_shape, dtype=a.dtype, device=a.device)
+    bias_ptr = None if bias is None else bias.data_ptr()
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+        rc = _ek.lib().tmb_gemm_ws(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_ptr,
+                                   *dims, epi_flags, ws.data_ptr(), ws_bytes, _stream())
+    else:
+        rc = _ek.lib().tmb_gemm(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_ptr,
+                                *dims, epi_flags, _stream())
+    if rc:
+        _check("tmb_gemm", rc)
+    return out
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
          epilogue: int = _ek.EPI_NONE, residual: Optional[torch.Tensor] = None,
          out_dtype: Optional[torch.dtype] = None, round_like_unfused: bool = False) -> torch.Tensor:
@@ -121,22 +147,10 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
     # straight to the launch: the key holds everything the checks below look at.
     key = None
     if residual is None and out_dtype is None:
-        key = (a.shape, a.stride(), b.shape, b.stride(), a.dtype, b.dtype, a.device, b.device,
-               None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device))
-        plan = _GEMM_PLANS.get(key)
-        if plan is not None:
-            out_shape, dims, ws_bytes = plan
-            out = torch.empty(out_shape, dtype=a.dtype, device=a.device)
-            bias_ptr = None if bias is None else bias.data_ptr()
-            if ws_bytes:
-                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
-                rc = _ek.lib().tmb_gemm_ws(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_ptr,
-                                           *dims, epi_flags, ws.data_ptr(), ws_bytes, _stream())
-            else:
-                rc = _ek.lib().tmb_gemm(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_ptr,
-                                        *dims, epi_flags, _stream())
-            _check("tmb_gemm", rc)
+        out = gemm_if_planned(a, b, bias, epi_flags)
+        if out is not None:
             return out
+        key = True
     a_in, b_in, bias_in = a, b, bias
     require_hip(a, b, bias, residual)
     if a.dtype != b.dtype or a.dtype not in FLOAT_DTYPES:
@@ -662,10 +676,11 @@ def cat2_supported(a: torch.Tensor, b: torch.Tensor, dim: int) -> bool:
     return a.numel() + b.numel() > 0
 
 
-def cat2(a: torch.Tensor, b: torch.Tensor, dim: int) -> torch.Tensor:
+def cat2(a: torch.Tensor, b: torch.Tensor, dim: int, checked: bool = False) -> torch.Tensor:
     """``torch.cat([a, b], dim)`` for two contiguous tensors in one launch (reference:
-    aten_fast.py:2203-2228, the key/value-cache append of a decode step)."""
-    if not cat2_supported(a, b, dim):
+    aten_fast.py:2203-2228, the key/value-cache append of a decode step). `checked`: the caller
+    has just seen `cat2_supported` accept exactly these operands."""
+    if not checked and not cat2_supported(a, b, dim):
         raise ValueError(f"cat2: unsupported operands {tuple(a.shape)} {a.dtype} / "
                          f"{tuple(b.shape)} {b.dtype}, dim {dim}")
     shape = list(a.shape)

@@ -259,13 +259,28 @@ def _view_op(op_name: str, fn: Callable):
     return view
 
 
-_view_op("aten::view", lambda h, size: h.view(size))
-_view_op("aten::_unsafe_view", lambda h, size: h.view(size))
+def _direct_view_ops():
+    """view and transpose are two thirds of the views of a decode step: no lambda in between."""
+    adopt = TorchMojoTensor._adopt
+
+    @register_aten_op("aten::view")
+    def view(self, size):
+        return adopt(self._holder.view(size))
+
+    @register_aten_op("aten::_unsafe_view")
+    def unsafe_view(self, size):
+        return adopt(self._holder.view(size))
+
+    @register_aten_op("aten::transpose.int")
+    def transpose(self, dim0, dim1):
+        return adopt(self._holder.transpose(dim0, dim1))
+
+
+_direct_view_ops()
 _view_op("aten::_reshape_alias", lambda h, size, stride: h.as_strided(size, stride))
 _view_op("aten::as_strided", lambda h, size, stride, storage_offset=None:
          h.as_strided(size, stride, h.storage_offset() if storage_offset is None else storage_offset))
 _view_op("aten::t", lambda h: h.t())
-_view_op("aten::transpose.int", lambda h, d0, d1: h.transpose(d0, d1))
 _view_op("aten::permute", lambda h, dims: h.permute(dims))
 _view_op("aten::expand", lambda h, size, implicit=False: h.expand(size))
 _view_op("aten::unsqueeze", lambda h, dim: h.unsqueeze(dim))

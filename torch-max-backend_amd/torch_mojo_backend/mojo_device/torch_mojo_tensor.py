@@ -22,6 +22,7 @@ MAX_RANK = 8  # reference :243
 DIRECT_IMPLS: dict = {}
 
 _MOJO_DEVICES: dict = {}
+_MOJO_OF_HIP: dict = {}  # HIP device of a holder -> the mojo device of its wrapper
 
 
 def _mojo_device(index: int) -> torch.device:
@@ -85,8 +86,12 @@ class TorchMojoTensor(torch.Tensor):
         shape = holder.shape
         if len(shape) > MAX_RANK:
             raise NotImplementedError(f"mojo tensors support at most rank {MAX_RANK}, got {len(shape)}")
+        hip = holder.device
+        dev = _MOJO_OF_HIP.get(hip)
+        if dev is None:
+            dev = _MOJO_OF_HIP[hip] = _mojo_device(hip.index or 0)
         res = _make_wrapper(cls, shape, holder.stride(), holder.storage_offset(), None, holder.dtype,
-                            _STRIDED, _mojo_device(holder.device.index or 0), False)
+                            _STRIDED, dev, False)
         res._holder = holder
         return res
 
