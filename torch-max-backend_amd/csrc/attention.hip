@@ -50,19 +50,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(1024))) unsigned char lds[kAttnStages * kAttnBuf];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
-  // Workgroups are dealt to the 8 XCDs round-robin by their linear id, and under a causal mask
-  // a query block's cost grows with its index: with the query block as the fastest grid
-  // dimension and 8 of them, one XCD would get every heaviest block. Rotating the query block
-  // by the (batch, head) index gives each XCD an even mix.
-  //
-  // Under a causal mask a workgroup takes two query blocks of one (batch, head): block
-  // n-1-u and then block u, which together always walk the same number of key blocks, so every
-  // workgroup carries the same load and its fixed costs are spread over a long key loop.
+  // Under a causal mask a query block's cost grows with its index, so a workgroup takes two
+  // query blocks of one (batch, head): block n-1-u and then block u, which together always walk
+  // the same number of key blocks. Every workgroup then carries the same load, and the
+  // workgroups of one (batch, head), which read the same K and V, are numbered onto one XCD.
   const int n_qb = (a.q_len + kAttnBQ - 1) / kAttnBQ;
   const bool paired = a.causal && n_qb > 1;
   const int units = paired ? (n_qb + 1) / 2 : n_qb;
-  const int bh = blockIdx.x / units;
-  const int unit = static_cast<int>((blockIdx.x % units + bh) % units);
+  const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int bh = wg / units;
+  const int unit = wg % units;
   const int b = bh / a.heads, h = bh % a.heads;
   auto run_qblock = [&](const int qb) {
   const int q0 = qb * kAttnBQ, qw0 = q0 + wave * 32;

@@ -91,8 +91,9 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
   const int n_qb = (a.q_len + kAttnBQ - 1) / kAttnBQ;
   const bool paired = a.causal && n_qb > 1;
   const int units = paired ? (n_qb + 1) / 2 : n_qb;
-  const int bh = blockIdx.x / units;
-  const int unit = static_cast<int>((blockIdx.x % units + bh) % units);
+  const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int bh = wg / units;
+  const int unit = wg % units;
   const int b = bh / a.heads, h = bh % a.heads;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((attn_lds_u8*)lds));
   const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
@@ -254,8 +255,9 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
   const int n_kb = (a.kv_len + kAttnBQ - 1) / kAttnBQ;
   const bool paired = a.causal && n_kb > 1;
   const int units = paired ? (n_kb + 1) / 2 : n_kb;
-  const int bh = blockIdx.x / units;
-  const int unit = static_cast<int>((blockIdx.x % units + bh) % units);
+  const int wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int bh = wg / units;
+  const int unit = wg % units;
   const int b = bh / a.heads, h = bh % a.heads;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((attn_lds_u8*)lds));
   const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);

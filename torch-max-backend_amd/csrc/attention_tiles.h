@@ -76,6 +76,17 @@ __device__ __forceinline__ u32x4_t attn_tr_operand(attn_lds_u8* tile, int off_lo
   return __builtin_bit_cast(u32x4_t, both);
 }
 
+// Workgroups are dealt to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.
+// This renumbering gives every XCD one contiguous run of logical ids, so that the workgroups
+// that share operands (the query blocks of one (batch, head) all walk the same K and V; the key
+// blocks of one head all walk the same Q and dout) sit on one XCD at about the same time and the
+// operands come from memory once instead of once per XCD.
+__device__ __forceinline__ int xcd_contiguous_id(int id, int n) {
+  const int q = n >> 3, r = n & 7;
+  const int xcd = id & 7, slot = id >> 3;
+  return (xcd < r ? xcd * (q + 1) : r * (q + 1) + (xcd - r) * q) + slot;
+}
+
 template <typename T>
 __device__ __forceinline__ void unpack2(uint32_t v, float& a, float& b) {
   a = to_f32(__builtin_bit_cast(T, static_cast<unsigned short>(v)));
