@@ -594,10 +594,46 @@ def main() -> int:
 
             rocm = gen_rate(dev)
             ours = gen_rate("mojo")
+
+            def host_breakdown(steps=40):
+                """Host microseconds per call inside the registered implementations, by op, over
+                `steps` decoded tokens (the time between a call from __torch_dispatch__ and its
+                return; PyTorch's own dispatch and the model's Python come on top)."""
+                from torch_mojo_backend.mojo_device import torch_mojo_tensor as tmt
+
+                calls, spent = {}, {}
+                saved = dict(tmt.DIRECT_IMPLS)
+
+                def timed_impl(name, fn):
+                    def run(*a, **k):
+                        t = time.perf_counter()
+                        out = fn(*a, **k)
+                        spent[name] = spent.get(name, 0.0) + time.perf_counter() - t
+                        calls[name] = calls.get(name, 0) + 1
+                        return out
+                    return run
+
+                mdl, i, a = hf.to("mojo"), ids.to("mojo"), mask.to("mojo")
+                try:
+                    for op, fn in saved.items():
+                        tmt.DIRECT_IMPLS[op] = timed_impl(str(op), fn)
+                    with torch.no_grad():
+                        mdl.generate(i, max_new_tokens=steps, min_new_tokens=steps, do_sample=False,
+                                     pad_token_id=50256, attention_mask=a)
+                        sync()
+                finally:
+                    tmt.DIRECT_IMPLS.update(saved)
+                top = sorted(spent, key=spent.get, reverse=True)[:10]
+                return {"ops_per_step": round(sum(calls.values()) / steps, 1),
+                        "impl_ms_per_step": round(sum(spent.values()) / steps * 1e3, 3),
+                        "top": {n: {"calls_per_step": round(calls[n] / steps, 1),
+                                    "us_per_call": round(spent[n] / calls[n] * 1e6, 2)} for n in top}}
+
             sweep["gpt2_hf_generate_bf16_B512_eager"] = {
                 "tokens/s": round(ours, 1), "ms_per_decode_step": round(B / ours * 1e3, 3),
-                "pytorch_rocm_eager_tokens/s": round(rocm, 1), "batch": B, "prompt": P,
-                "new_tokens": NEW, "dtype": "bf16",
+                "pytorch_rocm_eager_tokens/s": round(rocm, 1),
+                "vs_pytorch_rocm_eager": round(ours / rocm, 4), "batch": B, "prompt": P,
+                "new_tokens": NEW, "dtype": "bf16", "host": host_breakdown(),
                 "note": "HF GPT2LMHeadModel.generate on the eager mojo device, random-init weights"}
             del hf
 
