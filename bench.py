@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot-op kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|backward|gpt2|generate|copy|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only headline|gemm|rows|reduce|attn|backward|gpt2|train|generate|copy|all]
 
 Headline (the JSON line's ``value``): bf16 ``addmm`` with M=N=K=8192 and a [N] bias, fp32
 accumulation — one *step* is one launch of that GEMM through the C ABI, inputs resident in HBM.
@@ -82,7 +82,7 @@ def _parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=100)
     p.add_argument("--warmup", type=int, default=25)
-    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "backward", "gpt2", "generate", "copy"])
+    p.add_argument("--only", default="all", choices=["all", "headline", "gemm", "rows", "reduce", "attn", "backward", "gpt2", "train", "generate", "copy"])
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     return p.parse_args()
 
@@ -559,6 +559,48 @@ def main() -> int:
             row["cpu_note"] = (f"PyTorch CPU eager fp32 of the same module at B={cb}, T={ct} "
                                f"(the workload's CPU configuration), {cpu_threads} threads")
         sweep[f"gpt2_small_fwd_bf16_B{B}_T{T}"] = row
+        del model, compiled
+
+    # ------------------------------------------------------------------ GPT-2 training step
+    # Forward + backward of the same module through mojo_backend (bf16, B=16, T=1024, mean
+    # cross-entropy over all positions; no optimizer step: the reference's training path ends at
+    # the gradients). The backward graph runs the backward twins of the hot ops and the GEMMs of
+    # linear_backward; PyTorch-ROCm's eager forward + backward of the same module is timed beside
+    # it. (Runs before the eager device is registered: afterwards PyTorch's autograd engine no
+    # longer takes plain HIP tensors in this process.)
+    if want in ("all", "train"):
+        import torch.nn.functional as F
+        from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+        from torch_mojo_backend import mojo_backend
+
+        B, T = 16, 1024
+        model = build_gpt2_small(seed=0).to(torch.bfloat16).to(dev)
+        idx, targets = seeded_tokens(B, T, seed=0).to(dev), seeded_tokens(B, T, seed=1).to(dev)
+
+        def train_step(m):
+            logits, _ = m(idx)
+            loss = F.cross_entropy(logits.view(-1, logits.shape[-1]), targets.view(-1))
+            loss.backward()
+            for p_ in model.parameters():
+                p_.grad = None
+            return loss
+
+        compiled = torch.compile(model, backend=mojo_backend)
+        t0 = time.perf_counter()
+        loss_c = train_step(compiled).item()
+        compile_s = time.perf_counter() - t0
+        wall, _ = timed(lambda: train_step(compiled), 5, 2)
+        loss_e = train_step(model).item()
+        wall_e, _ = timed(lambda: train_step(model), 5, 2)
+        # forward FLOPs of the projections and attention; backward = 2x
+        fwd_flops = 12 * (2 * B * T * 7077888) + 12 * (2 * 2 * B * 12 * T * T * 64) + 2 * B * T * 768 * 50257
+        sweep[f"gpt2_small_train_step_bf16_B{B}_T{T}"] = {
+            "tokens/s": round(B * T / (wall * 1e-3), 1), "ms_per_step": round(wall, 3),
+            "TFLOP/s_over_whole_step": round(3 * fwd_flops / (wall * 1e-3) / 1e12, 2),
+            "pytorch_rocm_eager_ms_per_step": round(wall_e, 3), "compile_s": round(compile_s, 2),
+            "loss": round(loss_c, 4), "pytorch_rocm_eager_loss": round(loss_e, 4),
+            "batch": B, "seq": T, "dtype": "bf16",
+            "note": "forward + backward through mojo_backend, no optimizer step"}
         del model, compiled
 
     # ------------------------------------------------------------------ eager decode loop

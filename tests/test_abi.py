@@ -147,3 +147,43 @@ def test_product_never_imports_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
                 assert "libtmb_oracle" not in text, f
+
+
+def test_relayout_rules_on_the_host():
+    """Pure host logic (no GPU): which layouts are re-laid, and into what."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    def prep(a, b):
+        la, lb = hip_ops._matrix_layout(a), hip_ops._matrix_layout(b)
+        m, k, n = a.shape[-2], a.shape[-1], b.shape[-1]
+        ok = hip_ops._mfma_layouts_ok(a, b, la, lb, m, n, k, a.dim() == 3)
+        return ok, (None if ok else hip_ops._relayout_for_mfma(a, b, la, lb, m, n, k, a.dim() == 3))
+
+    bf = torch.bfloat16
+    ok, _ = prep(torch.zeros(64, 256, dtype=bf), torch.zeros(256, 128, dtype=bf))
+    assert ok
+    # an odd contraction length (a vocabulary as K): both operands padded with zeros to 64 | K
+    a, b = torch.randn(16, 1001).to(bf), torch.randn(1001, 24).to(bf)
+    ok, (a2, b2, la, lb, k) = prep(a, b)
+    assert not ok and k == 1024 and tuple(a2.shape) == (16, 1024) and tuple(b2.shape) == (1024, 24)
+    assert la == (0, 1024) and lb == (0, 24)
+    assert torch.equal(a2[:, :1001], a) and not a2[:, 1001:].any() and not b2[1001:].any()
+    assert hip_ops._mfma_layouts_ok(a2, b2, la, lb, 16, 24, k, False)
+    # the weight-gradient form with an odd M: A becomes row-major, B stays
+    a, b = torch.randn(512, 1001).to(bf).t(), torch.randn(512, 96).to(bf)
+    ok, (a2, b2, la, lb, k) = prep(a, b)
+    assert not ok and a2.is_contiguous() and torch.equal(a2, a) and b2 is b and k == 512
+    # ... and the same form when it is eligible is left alone
+    ok, _ = prep(torch.randn(512, 1024).to(bf).t(), torch.randn(512, 96).to(bf))
+    assert ok
+    # a narrow product behind a transposed A (attention's dV = P^T dO)
+    ok, (a2, b2, la, lb, k) = prep(torch.randn(3, 256, 128).to(bf).transpose(1, 2), torch.randn(3, 256, 64).to(bf))
+    assert not ok and la == (0, 256) and b2.shape == (3, 256, 64)
+    # N-major B with an odd pitch becomes K-major; float32 counts in vectors of four
+    a, b = torch.randn(32, 64).to(bf), torch.randn(64, 77).to(bf)
+    ok, (a2, b2, la, lb, k) = prep(a, b)
+    assert not ok and lb == (1, 64) and torch.equal(b2, b)
+    ok, _ = prep(torch.zeros(8, 36), torch.zeros(36, 20))
+    assert ok
+    ok, (a2, b2, la, lb, k) = prep(torch.randn(8, 50), torch.randn(50, 20))
+    assert not ok and k == 64 and la == (0, 64)

@@ -1,5 +1,7 @@
 """GPU parity of the GEMM family (mm / addmm / bmm / linear, bias + GELU epilogue)."""
 
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -594,3 +596,33 @@ def test_k64_stream_kernel_bias_broadcast_and_neighbouring_shapes():
     outs = [_ops().gemm(a2, b2, bias) for _ in range(3)]
     torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+
+
+# ---- operands the matrix-core kernels cannot read as they lie ------------------------------------
+@pytest.mark.parametrize("case", [
+    # (dtype, a shape, a transposed?, b shape, b transposed?)
+    (torch.bfloat16, (700, 1001), False, (1001, 384), False),   # odd K: padded
+    (torch.bfloat16, (1024, 1001), True, (1024, 256), False),   # weight-gradient form, odd M
+    (torch.float16, (700, 1001), False, (384, 1001), True),     # odd K, K-major B
+    (torch.bfloat16, (6, 512, 640), True, (6, 512, 64), False),  # transposed A, 64 columns
+    (torch.float32, (600, 1001), False, (1001, 200), False),    # fp32, K not a multiple of 4
+    (torch.float32, (1024, 1001), True, (1024, 128), False),    # fp32 weight-gradient form, odd M
+])
+def test_large_products_with_awkward_layouts_match_float64(case):
+    """Above the re-layout threshold these run on the matrix-core kernels after one padded or
+    transposed copy; the result is that of the product as given."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+    dtype, ashape, ta, bshape, tb = case
+    a = seeded(ashape, seed=41, dtype=dtype).cuda()
+    b = seeded(bshape, seed=42, dtype=dtype).cuda()
+    av = a.transpose(-1, -2) if ta else a
+    bv = b.transpose(-1, -2) if tb else b
+    m, k, n = av.shape[-2], av.shape[-1], bv.shape[-1]
+    assert math.prod(av.shape[:-2]) * m * n * k >= hip_ops._RELAYOUT_MIN_WORK
+    got = hip_ops.gemm(av, bv)
+    want = as64(av) @ as64(bv)
+    scale = np.abs(want).max()
+    tol = {torch.float32: 2e-6, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}[dtype]
+    assert np.abs(as64(got) - want).max() <= tol * scale
+    ref = oracle.gemm(av.cpu(), bv.cpu())
+    assert np.abs(as64(got) - as64(ref)).max() <= tol * scale

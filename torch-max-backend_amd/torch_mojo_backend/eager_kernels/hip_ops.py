@@ -95,6 +95,63 @@ def _matrix_layout(t: torch.Tensor) -> Optional[Tuple[int, int]]:
     return None
 
 
+# Products smaller than this many multiply-adds run as they are: the kernel that takes any layout
+# is quick enough there, and re-laying an operand costs launches of its own.
+_RELAYOUT_MIN_WORK = 1 << 26
+
+
+def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
+    """`x` with its last dimension zero-padded to `size`, contiguous (one copy, one small fill)."""
+    out = torch.empty(tuple(x.shape[:-1]) + (size,), dtype=x.dtype, device=x.device)
+    out[..., : x.shape[-1]].copy_(x)
+    if size > x.shape[-1]:
+        out[..., x.shape[-1]:].zero_()
+    return out
+
+
+def _mfma_layouts_ok(a, b, la, lb, m, n, k, batched, plain_epilogue=True) -> bool:
+    """Whether the matrix-core kernels take these operands as they lie (mirrors the library's
+    own checks; when it says no, the library would run its any-layout kernel, which is one to two
+    orders of magnitude slower on large products)."""
+    unit = 16 // a.element_size()  # elements per 16-byte vector: 8 (16-bit) or 4 (fp32)
+    if la[1] % unit or lb[1] % unit or a.data_ptr() % 16 or b.data_ptr() % 16:
+        return False
+    if batched and a.shape[0] > 1 and (a.stride(0) % unit or b.stride(0) % unit):
+        return False
+    if a.element_size() == 4:
+        return (m if la[0] else k) % 4 == 0 and (k if lb[0] else n) % 4 == 0
+    if la[0]:  # A stored [K, M]: the weight-gradient form, with B stored [K, N] and no epilogue
+        return plain_epilogue and not lb[0] and k % 32 == 0 and k >= 256 and m % 8 == 0 \
+            and n % 8 == 0 and n > 64
+    return k % 8 == 0
+
+
+def _relayout_for_mfma(a, b, la, lb, m, n, k, batched):
+    """Re-lays the operands of a large product so that the matrix-core kernels take it: a
+    transposed A the weight-gradient kernel cannot read becomes row-major, a contraction length
+    or pitch that is not whole 16-byte vectors (a 50257-wide vocabulary as K) is zero-padded, B
+    becomes K-major where its own pitch is the obstacle. Returns (a, b, la, lb, k)."""
+    unit = 16 // a.element_size()
+    if la[0]:
+        a = a.contiguous()                      # [.., M, K] row-major
+    kp = k if k % unit == 0 else (k + 63) // 64 * 64
+    if a.shape[-1] != kp or a.stride(-2) % unit or a.data_ptr() % 16 or not a.is_contiguous():
+        a = _pad_last(a, kp)
+    bt = b.transpose(-1, -2)                    # [.., N, K]
+    n_major_ok = not lb[0] and lb[1] % unit == 0 and b.data_ptr() % 16 == 0 and \
+        (a.element_size() == 2 or n % 4 == 0)
+    k_major_ok = bool(lb[0]) and lb[1] % unit == 0 and b.data_ptr() % 16 == 0 and kp == k
+    if n_major_ok:
+        if kp != k:                             # rows of zeros below the last k
+            grown = torch.empty(tuple(b.shape[:-2]) + (kp, n), dtype=b.dtype, device=b.device)
+            grown[..., :k, :].copy_(b)
+            grown[..., k:, :].zero_()
+            b = grown
+    elif not k_major_ok:
+        b = _pad_last(bt, kp).transpose(-1, -2)  # K-major, padded along K
+    return a, b, _matrix_layout(a), _matrix_layout(b), kp
+
+
 _I64X3 = ctypes.c_int64 * 3
 _GEMM_WS_BYTES: dict = {}
 _GEMM_PLANS: dict = {}
@@ -180,6 +237,9 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
     if lb is None or (batched and batch > 1 and b.stride(0) < 0):
         b = b.contiguous()
         lb = (0, max(n, 1))
+    if batch * m * n * k >= _RELAYOUT_MIN_WORK and not _mfma_layouts_ok(
+            a, b, la, lb, m, n, k, batched, epilogue == _ek.EPI_NONE):
+        a, b, la, lb, k = _relayout_for_mfma(a, b, la, lb, m, n, k, batched)
     out_shape = (batch, m, n) if batched else (m, n)
     if residual is not None and (residual.dtype not in (a.dtype, torch.float32)
                                  or tuple(residual.shape) != out_shape):

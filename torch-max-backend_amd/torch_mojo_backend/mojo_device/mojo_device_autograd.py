@@ -37,13 +37,17 @@ def _wants_grad(*tensors) -> bool:
         isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
 
 
+_dispatch_modes_active = torch._C._len_torch_dispatch_stack
+
+
 def _below_autograd(op, *args, **kwargs):
     """The registered kernel of `op` when no gradient is wanted. With real HIP holders behind the
     first argument the eager implementation is called directly (one Python entry per op, as
     without an autograd kernel); while torch.compile traces (stand-in holders) or for other
     argument types the call is redispatched below the autograd keys."""
     first = args[0]
-    if type(first) is TorchMojoTensor and type(first._holder) is torch.Tensor:
+    if type(first) is TorchMojoTensor and type(first._holder) is torch.Tensor \
+            and _dispatch_modes_active() == 0:  # a mode (profiler, fake tensors) must see the op
         impl = DIRECT_IMPLS.get(op)
         if impl is not None:
             return impl(*args, **kwargs)

@@ -1021,7 +1021,14 @@ def attention_recompute_partition(joint_module, joint_inputs, *, num_fwd_outputs
     from torch._functorch.partitioners import default_partition
 
     if _fusion_enabled() and _attention_fusion_enabled():
-        _tag_attention_for_recompute(joint_module, num_fwd_outputs)
+        try:
+            _tag_attention_for_recompute(joint_module, num_fwd_outputs)
+        except Exception as exc:  # noqa: BLE001 - the untagged split is always valid
+            for node in joint_module.graph.nodes:
+                if node.meta.get("recompute") is not None and "ac_graph_id" in node.meta:
+                    del node.meta["recompute"], node.meta["ac_graph_id"]
+            if verbose_enabled():
+                print(f"[mojo_backend] attention chains left to the default split: {exc!r}")
     return default_partition(joint_module, joint_inputs, num_fwd_outputs=num_fwd_outputs, **kwargs)
 
 
