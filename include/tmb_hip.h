@@ -298,6 +298,16 @@ int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_bet
 int tmb_cat2_rows(void* out, const void* a, const void* b, int64_t rows, int64_t a_row_bytes,
                   int64_t b_row_bytes, void* stream);
 
+/* Row copy with zero padding: out[r, 0:row_len] = in[r, 0:row_len], out[r, row_len:out_pitch] = 0
+ * for `rows` rows of 2- or 4-byte elements (`itemsize`); pitches in elements. The source needs
+ * element alignment only, the destination 16-byte aligned rows (out_pitch * itemsize % 16 == 0).
+ * It turns an operand whose rows are not whole 16-byte vectors (K = 50257 in the backward of a
+ * vocabulary projection) into one the matrix-core GEMM kernels read, at copy speed. No counterpart
+ * entry in the reference: its GEMM wrappers pass only exact dense layouts in place
+ * (`_tf32_dense_2d_layout`, aten_fast.py:4457-4467) and leave the rest to MAX's matmul. */
+int tmb_pad_rows(void* out, const void* in, int64_t rows, int64_t row_len, int64_t in_pitch,
+                 int64_t out_pitch, int itemsize, void* stream);
+
 /* Plain device copy kernel (16-byte vectors, grid-stride) — the bandwidth yardstick the
  * benchmark and the counter calibration use. No reference counterpart. */
 int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* stream);

@@ -164,26 +164,32 @@ def test_relayout_rules_on_the_host():
     assert ok
     # an odd contraction length (a vocabulary as K): both operands padded with zeros to 64 | K
     a, b = torch.randn(16, 1001).to(bf), torch.randn(1001, 24).to(bf)
-    ok, (a2, b2, la, lb, k) = prep(a, b)
-    assert not ok and k == 1024 and tuple(a2.shape) == (16, 1024) and tuple(b2.shape) == (1024, 24)
+    ok, (a2, b2, la, lb, k, rows) = prep(a, b)
+    assert not ok and k == 1024 and rows == 16 and tuple(a2.shape) == (16, 1024) and tuple(b2.shape) == (1024, 24)
     assert la == (0, 1024) and lb == (0, 24)
     assert torch.equal(a2[:, :1001], a) and not a2[:, 1001:].any() and not b2[1001:].any()
     assert hip_ops._mfma_layouts_ok(a2, b2, la, lb, 16, 24, k, False)
-    # the weight-gradient form with an odd M: A becomes row-major, B stays
+    # the weight-gradient form with an odd M keeps its form: the stored [K, M] rows get zero
+    # columns up to 8 | M, B stays, and the launch computes the few extra rows
     a, b = torch.randn(512, 1001).to(bf).t(), torch.randn(512, 96).to(bf)
-    ok, (a2, b2, la, lb, k) = prep(a, b)
-    assert not ok and a2.is_contiguous() and torch.equal(a2, a) and b2 is b and k == 512
+    ok, (a2, b2, la, lb, k, rows) = prep(a, b)
+    assert not ok and rows == 1008 and la == (1, 1008) and tuple(a2.shape) == (1008, 512) and b2 is b
+    assert torch.equal(a2[:1001], a) and not a2[1001:].any() and k == 512
+    assert hip_ops._mfma_layouts_ok(a2, b2, la, lb, rows, 96, k, False)
+    # ... but not with 64 or fewer columns (no weight-gradient kernel there): row-major A
+    ok, (a2, b2, la, lb, k, rows) = prep(torch.randn(512, 1001).to(bf).t(), torch.randn(512, 64).to(bf))
+    assert not ok and la == (0, 512) and rows == 1001
     # ... and the same form when it is eligible is left alone
     ok, _ = prep(torch.randn(512, 1024).to(bf).t(), torch.randn(512, 96).to(bf))
     assert ok
     # a narrow product behind a transposed A (attention's dV = P^T dO)
-    ok, (a2, b2, la, lb, k) = prep(torch.randn(3, 256, 128).to(bf).transpose(1, 2), torch.randn(3, 256, 64).to(bf))
-    assert not ok and la == (0, 256) and b2.shape == (3, 256, 64)
+    ok, (a2, b2, la, lb, k, rows) = prep(torch.randn(3, 256, 128).to(bf).transpose(1, 2), torch.randn(3, 256, 64).to(bf))
+    assert not ok and la == (0, 256) and b2.shape == (3, 256, 64) and rows == 128
     # N-major B with an odd pitch becomes K-major; float32 counts in vectors of four
     a, b = torch.randn(32, 64).to(bf), torch.randn(64, 77).to(bf)
-    ok, (a2, b2, la, lb, k) = prep(a, b)
+    ok, (a2, b2, la, lb, k, rows) = prep(a, b)
     assert not ok and lb == (1, 64) and torch.equal(b2, b)
     ok, _ = prep(torch.zeros(8, 36), torch.zeros(36, 20))
     assert ok
-    ok, (a2, b2, la, lb, k) = prep(torch.randn(8, 50), torch.randn(50, 20))
+    ok, (a2, b2, la, lb, k, rows) = prep(torch.randn(8, 50), torch.randn(50, 20))
     assert not ok and k == 64 and la == (0, 64)

@@ -626,3 +626,24 @@ def test_large_products_with_awkward_layouts_match_float64(case):
     assert np.abs(as64(got) - want).max() <= tol * scale
     ref = oracle.gemm(av.cpu(), bv.cpu())
     assert np.abs(as64(got) - as64(ref)).max() <= tol * scale
+
+
+def test_pad_rows_kernel_matches_a_plain_copy():
+    """Every alignment class of the source (odd pitches, odd offsets), 2- and 4-byte elements,
+    3-D inputs with a constant row pitch; the padding is exact zeros."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+    for dtype, shape, size in ((torch.bfloat16, (37, 1001), 1024), (torch.float16, (5, 9, 77), 80),
+                               (torch.float32, (64, 50), 64), (torch.bfloat16, (3, 8), 8),
+                               (torch.bfloat16, (129, 7), 64)):
+        x = seeded(shape, seed=51, dtype=dtype).cuda()
+        got = hip_ops._pad_last(x, size)
+        assert got.is_contiguous() and got.shape[-1] == size
+        assert torch.equal(got[..., : shape[-1]], x) and not got[..., shape[-1]:].any()
+        # a view that starts at an odd element and has an odd pitch
+        view = x[..., 1:]
+        got = hip_ops._pad_last(view, size)
+        assert torch.equal(got[..., : shape[-1] - 1], view) and not got[..., shape[-1] - 1:].any()
+    # a transposed source is not row-major: PyTorch-ROCm's strided copy takes it
+    x = seeded((40, 24), seed=52, dtype=torch.bfloat16).cuda().t()
+    got = hip_ops._pad_last(x, 48)
+    assert torch.equal(got[:, :40], x) and not got[:, 40:].any()

@@ -115,7 +115,74 @@ int launch_cat2(void* out, const void* a, const void* b, int64_t rows, int64_t a
   return check_launch();
 }
 
+// out[r, :] = in[r, :row_units] followed by zeros up to the output pitch, for rows whose source
+// pitch or start is only element-aligned (UNIT = the element: 2 or 4 bytes): what the matrix-core
+// kernels need when an operand's rows are not whole 16-byte vectors (a 50257-wide vocabulary as
+// the contraction or the transposed dimension). One thread writes one aligned 16-byte vector of
+// the output from one (possibly unaligned) 16-byte load; global memory takes unaligned vector
+// accesses on this target.
+template <typename UNIT, typename IDX>
+__global__ __launch_bounds__(256) void pad_rows_kernel(uint4* __restrict__ out,
+                                                       const UNIT* __restrict__ in, IDX total,
+                                                       IDX out_vecs, IDX row_units,
+                                                       int64_t in_pitch_units) {
+  constexpr int PER = 16 / static_cast<int>(sizeof(UNIT));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef u32x4 __attribute__((aligned(2))) u32x4_unaligned;  // element alignment is all the source has
+  const IDX i = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  const IDX row = i / out_vecs, v = i - row * out_vecs;
+  const IDX first = v * PER;
+  const UNIT* src = in + static_cast<int64_t>(row) * in_pitch_units + first;
+  u32x4 val = {0u, 0u, 0u, 0u};
+  if (first + PER <= row_units) {
+    val = *reinterpret_cast<const u32x4_unaligned*>(src);
+  } else if (first < row_units) {
+    UNIT piece[PER];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) piece[e] = first + e < row_units ? src[e] : UNIT{0};
+    __builtin_memcpy(&val, piece, 16);
+  }
+  __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(out) + i);
+}
+
+template <typename UNIT>
+int launch_pad_rows(void* out, const void* in, int64_t rows, int64_t row_units,
+                    int64_t in_pitch_units, int64_t out_pitch_units, hipStream_t s) {
+  constexpr int PER = 16 / static_cast<int>(sizeof(UNIT));
+  const int64_t out_vecs = out_pitch_units / PER;
+  const int64_t total = rows * out_vecs;
+  const int64_t blocks = (total + 255) / 256;
+  if (blocks >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(blocks));
+  if (total < (int64_t{1} << 32) && row_units < (int64_t{1} << 32)) {
+    pad_rows_kernel<UNIT, uint32_t><<<grid, dim3(256), 0, s>>>(
+        static_cast<uint4*>(out), static_cast<const UNIT*>(in), static_cast<uint32_t>(total),
+        static_cast<uint32_t>(out_vecs), static_cast<uint32_t>(row_units), in_pitch_units);
+  } else {
+    pad_rows_kernel<UNIT, uint64_t><<<grid, dim3(256), 0, s>>>(
+        static_cast<uint4*>(out), static_cast<const UNIT*>(in), static_cast<uint64_t>(total),
+        static_cast<uint64_t>(out_vecs), static_cast<uint64_t>(row_units), in_pitch_units);
+  }
+  return check_launch();
+}
+
 }  // namespace tmb
+
+extern "C" int tmb_pad_rows(void* out, const void* in, int64_t rows, int64_t row_len,
+                            int64_t in_pitch, int64_t out_pitch, int itemsize, void* stream) {
+  if (rows < 0 || row_len < 0 || in_pitch < 0 || out_pitch < row_len) return TMB_ERR_INVALID_ARGUMENT;
+  if (itemsize != 2 && itemsize != 4) return TMB_ERR_UNSUPPORTED;
+  if (rows == 0 || out_pitch == 0) return TMB_OK;
+  if (!out || (row_len && !in)) return TMB_ERR_INVALID_ARGUMENT;
+  if ((out_pitch * itemsize) % 16 != 0 || !tmb::aligned16(out) ||
+      (reinterpret_cast<uintptr_t>(in) % static_cast<uintptr_t>(itemsize)) != 0)
+    return TMB_ERR_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return itemsize == 2
+             ? tmb::launch_pad_rows<uint16_t>(out, in, rows, row_len, in_pitch, out_pitch, s)
+             : tmb::launch_pad_rows<uint32_t>(out, in, rows, row_len, in_pitch, out_pitch, s);
+}
 
 extern "C" int tmb_cat2_rows(void* out, const void* a, const void* b, int64_t rows,
                              int64_t a_row_bytes, int64_t b_row_bytes, void* stream) {

@@ -52,6 +52,7 @@ SIGNATURES = {
     "tmb_layer_norm_backward_rows": (_ci, [_vp] * 8 + [_i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
     "tmb_cat2_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "tmb_pad_rows": (_ci, [_vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp]),
 }
 
 _lib = None

@@ -101,11 +101,34 @@ _RELAYOUT_MIN_WORK = 1 << 26
 
 
 def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
-    """`x` with its last dimension zero-padded to `size`, contiguous (one copy, one small fill)."""
+    """`x` with its last dimension zero-padded to `size`, contiguous. Row-major sources go
+    through the row-padding kernel (copy speed whatever the source alignment); anything else is
+    copied by PyTorch-ROCm's strided copy."""
     out = torch.empty(tuple(x.shape[:-1]) + (size,), dtype=x.dtype, device=x.device)
-    out[..., : x.shape[-1]].copy_(x)
-    if size > x.shape[-1]:
-        out[..., x.shape[-1]:].zero_()
+    cols = x.shape[-1]
+    if out.numel() == 0:
+        return out
+    flat = x.is_cuda and x.dim() >= 2 and x.stride(-1) == 1 and x.element_size() in (2, 4) and \
+        (size * x.element_size()) % 16 == 0 and cols > 0
+    if flat:
+        # rows must be evenly spaced: [.., rows, cols] with a constant pitch over the leading dims
+        pitch = x.stride(-2)
+        rows = 1
+        for d in range(x.dim() - 2, -1, -1):
+            if x.shape[d] != 1 and x.stride(d) != pitch * rows:
+                flat = False
+                break
+            rows *= x.shape[d]
+    if flat:
+        rc = _ek.lib().tmb_pad_rows(out.data_ptr(), x.data_ptr(), rows, cols, pitch, size,
+                                    x.element_size(), _stream())
+        if rc == 0:
+            return out
+        if rc != _ek.ERR_UNSUPPORTED:
+            _check("tmb_pad_rows", rc)
+    out[..., :cols].copy_(x)
+    if size > cols:
+        out[..., cols:].zero_()
     return out
 
 
@@ -126,14 +149,26 @@ def _mfma_layouts_ok(a, b, la, lb, m, n, k, batched, plain_epilogue=True) -> boo
     return k % 8 == 0
 
 
-def _relayout_for_mfma(a, b, la, lb, m, n, k, batched):
-    """Re-lays the operands of a large product so that the matrix-core kernels take it: a
-    transposed A the weight-gradient kernel cannot read becomes row-major, a contraction length
-    or pitch that is not whole 16-byte vectors (a 50257-wide vocabulary as K) is zero-padded, B
-    becomes K-major where its own pitch is the obstacle. Returns (a, b, la, lb, k)."""
+def _relayout_for_mfma(a, b, la, lb, m, n, k, batched, plain=True):
+    """Re-lays the operands of a large product so that the matrix-core kernels take it. A
+    contraction length or pitch that is not whole 16-byte vectors (a 50257-wide vocabulary as K)
+    is zero-padded; B becomes K-major where its own pitch is the obstacle; a transposed A with an
+    odd M in the weight-gradient form keeps its form and gets zero columns (the product then has
+    a few extra rows, which the caller drops); any other transposed A becomes row-major.
+    `plain`: no epilogue and no residual. Returns (a, b, la, lb, k, rows of the launch)."""
     unit = 16 // a.element_size()
     if la[0]:
-        a = a.contiguous()                      # [.., M, K] row-major
+        b_fits = lb[1] % unit == 0 and b.data_ptr() % 16 == 0
+        if a.element_size() == 2:
+            keep_form = plain and not batched and b_fits and not lb[0] and k % 32 == 0 \
+                and k >= 256 and n % 8 == 0 and n > 64
+        else:
+            keep_form = not batched and b_fits and (k if lb[0] else n) % 4 == 0
+        if keep_form:
+            mp = (m + unit - 1) // unit * unit
+            stored = _pad_last(a.transpose(-1, -2), mp)          # [K, mp], zero columns
+            return stored.transpose(-1, -2), b, (1, mp), lb, k, mp
+        a = a.contiguous()                      # [.., M, K] row-major (a transposing copy)
     kp = k if k % unit == 0 else (k + 63) // 64 * 64
     if a.shape[-1] != kp or a.stride(-2) % unit or a.data_ptr() % 16 or not a.is_contiguous():
         a = _pad_last(a, kp)
@@ -149,7 +184,7 @@ def _relayout_for_mfma(a, b, la, lb, m, n, k, batched):
             b = grown
     elif not k_major_ok:
         b = _pad_last(bt, kp).transpose(-1, -2)  # K-major, padded along K
-    return a, b, _matrix_layout(a), _matrix_layout(b), kp
+    return a, b, _matrix_layout(a), _matrix_layout(b), kp, m
 
 
 _I64X3 = ctypes.c_int64 * 3
@@ -237,9 +272,11 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
     if lb is None or (batched and batch > 1 and b.stride(0) < 0):
         b = b.contiguous()
         lb = (0, max(n, 1))
+    m_given = m
     if batch * m * n * k >= _RELAYOUT_MIN_WORK and not _mfma_layouts_ok(
             a, b, la, lb, m, n, k, batched, epilogue == _ek.EPI_NONE):
-        a, b, la, lb, k = _relayout_for_mfma(a, b, la, lb, m, n, k, batched)
+        a, b, la, lb, k, m = _relayout_for_mfma(a, b, la, lb, m, n, k, batched,
+                                                epilogue == _ek.EPI_NONE and residual is None)
     out_shape = (batch, m, n) if batched else (m, n)
     if residual is not None and (residual.dtype not in (a.dtype, torch.float32)
                                  or tuple(residual.shape) != out_shape):
@@ -300,14 +337,14 @@ def gemm(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
             batch, m, n, k, la[1], lb[1], n, 0, 0, m * n, la[0], lb[0], code_of(a.dtype), epi_flags,
             ws.data_ptr(), ws_bytes, _stream())
         _check("tmb_gemm_ws", rc)
-        return out
+        return out if m == m_given else out[:m_given]  # rows of a padded M are dropped (a view)
     rc = lib.tmb_gemm(
         out.data_ptr(), a.data_ptr(), b.data_ptr(), None if bias is None else bias.data_ptr(),
         batch, m, n, k, la[1], lb[1], n,
         a.stride(0) if batched else 0, b.stride(0) if batched else 0, m * n,
         la[0], lb[0], code_of(a.dtype), epi_flags, _stream())
     _check("tmb_gemm", rc)
-    return out
+    return out if m == m_given else out[:m_given]
 
 
 # ---------------------------------------------------------------------------
