@@ -446,9 +446,58 @@ def _partitioned_training_graphs(model, idx, targets, partition_fn):
     return graphs, [p.grad.clone() for p in model.parameters()]
 
 
-def test_training_partition_recomputes_attention_scores_and_forward_fuses():
+def _host_attention_pieces(monkeypatch):
+    """The op-by-op route of the two fused training steps, on PyTorch's own CPU kernels."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    monkeypatch.setattr(compiler, "_attention_fused_ok", lambda *a: False)
+    # (the matchers key on the registry entries being the built-in ones: replace both sides)
+    softmax = lambda x, d, h: torch.softmax(x, d)  # noqa: E731
+    for op, name, fn in ((aten.bmm, "_BUILTIN_BMM", torch.bmm), (aten._softmax, "_BUILTIN_SOFTMAX", softmax)):
+        monkeypatch.setitem(MAPPING_TORCH_ATEN_TO_MOJO, op, fn)
+        monkeypatch.setattr(compiler, name, fn)
+    monkeypatch.setattr(compiler, "_causal_q_len", lambda *a: -1)
+    monkeypatch.setattr(hip_ops, "softmax_backward",
+                        lambda g, o, d, log: aten._softmax_backward_data(g, o, d, o.dtype))
+
+
+def test_training_partition_replaces_attention_forward_and_backward(monkeypatch):
+    """A 16-bit attention chain and its backward nodes become the two fused steps: the forward
+    graph hands over q, k, v, the output and the log-sum-exp, nothing of size [tokens, tokens]
+    exists in either graph, and (on the op-by-op route, which runs on this host) the gradients are
+    those of PyTorch's own split."""
     from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
     from torch._functorch.partitioners import default_partition
+
+    _host_attention_pieces(monkeypatch)
+    idx, targets = seeded_tokens(2, 8, seed=0), seeded_tokens(2, 8, seed=1)
+    make = lambda: build_gpt2_small(seed=0, n_layer=2).bfloat16()  # noqa: E731
+    plain, want = _partitioned_training_graphs(make(), idx, targets, default_partition)
+    (fw, bw), got = _partitioned_training_graphs(make(), idx, targets,
+                                                 compiler.attention_recompute_partition)
+    for g, w in zip(got, want):
+        scale = w.float().abs().max().item() + 1e-12
+        assert (g.float() - w.float()).abs().max().item() <= 3e-2 * scale  # bf16, other op order
+    count = lambda gm, target: sum(1 for n in gm.graph.nodes if n.target is target)  # noqa: E731
+    assert count(fw, compiler.attention_train_forward) == 2
+    assert count(bw, compiler.attention_train_backward) == 2
+    for gm in (fw, bw):
+        assert count(gm, aten.bmm.default) == 0 and count(gm, aten._softmax.default) == 0
+        assert count(gm, aten._softmax_backward_data.default) == 0
+        for n in gm.graph.nodes:
+            val = n.meta.get("val")
+            if isinstance(val, torch.Tensor) and val.dim() >= 3:
+                assert tuple(val.shape[-2:]) != (8, 8), n.name
+    assert count(plain[1], aten.bmm.default) == 8  # PyTorch's split: four per block
+
+
+def test_training_partition_recomputes_attention_scores_and_forward_fuses(monkeypatch):
+    """Where the backward nodes of a chain cannot be replaced, the chain is tagged for
+    recomputation instead."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch._functorch.partitioners import default_partition
+
+    monkeypatch.setattr(compiler, "_fuse_attention_backward", lambda *a: False)
 
     idx, targets = seeded_tokens(2, 8, seed=0), seeded_tokens(2, 8, seed=1)
     make = lambda: build_gpt2_small(seed=0, n_layer=2).bfloat16()  # noqa: E731

@@ -48,38 +48,53 @@ def gpt2_training_step_gradients_match_cpu():
     assert grew == set(watched), f"not every backward twin ran: {grew}"
 
 
-def training_forward_runs_the_fused_attention_kernel():
-    """The training partitioner recomputes the attention scores in backward, so the forward graph
-    of a bf16 training step runs one fused attention per block; a float32 graph, which the
-    16-bit kernel does not take, is split as PyTorch would. Either way the gradients match float64
-    autograd of the same weights."""
+def training_graph_runs_the_fused_attention_forward_and_backward():
+    """A bf16 training graph runs one fused attention forward and one fused attention backward
+    per block (the partitioner replaces the chain and its backward nodes); a float32 graph, which
+    the 16-bit kernels do not take, is split as PyTorch would. With a mask buffer that is not
+    causal the same two steps run op by op. In every case the gradients match float64 autograd of
+    the same weights."""
     from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
     from torch_mojo_backend import mojo_backend
     from torch_mojo_backend.eager_kernels import hip_ops
 
-    calls = []
-    real = hip_ops.attention
+    calls = {"fwd": 0, "bwd": 0}
+    real_f, real_b = hip_ops.attention, hip_ops.attention_backward
 
-    def counted(*a, **k):
-        calls.append(a[0].dtype)
-        return real(*a, **k)
+    def fwd(*a, **k):
+        calls["fwd"] += 1
+        return real_f(*a, **k)
 
-    hip_ops.attention = counted
+    def bwd(*a, **k):
+        calls["bwd"] += 1
+        return real_b(*a, **k)
+
+    hip_ops.attention, hip_ops.attention_backward = fwd, bwd
     idx, targets = seeded_tokens(2, 64, seed=0), seeded_tokens(2, 64, seed=1)
-    ref = build_gpt2_small(seed=0, n_layer=2).double()
-    _loss(ref, idx, targets).backward()
-    for dtype, bound in ((torch.float32, 2e-4), (torch.bfloat16, 6e-2)):
-        calls.clear()
+
+    def punch_mask(model):
+        for name, buf in model.named_buffers():
+            if name.endswith("bias") and buf.dim() == 4:
+                buf[..., 5, 40:50] = 1  # query 5 also sees ten later keys: not causal any more
+
+    for dtype, bound, causal in ((torch.float32, 2e-4, True), (torch.bfloat16, 6e-2, True),
+                                 (torch.bfloat16, 6e-2, False)):
+        ref = build_gpt2_small(seed=0, n_layer=2).double()
         model = build_gpt2_small(seed=0, n_layer=2).to(dtype).cuda()
+        if not causal:
+            punch_mask(ref)
+            punch_mask(model)
+        _loss(ref, idx, targets).backward()
+        calls["fwd"] = calls["bwd"] = 0
         loss = _loss(torch.compile(model, backend=mojo_backend), idx.cuda(), targets.cuda())
-        expected = [dtype, dtype] if dtype is torch.bfloat16 else []
-        assert calls == expected, calls
+        fused = 2 if (dtype is torch.bfloat16 and causal) else 0
+        assert calls == {"fwd": fused, "bwd": 0}, (dtype, causal, calls)
         loss.backward()
-        assert calls == expected, "backward must not run the forward kernel again"
+        assert calls == {"fwd": fused, "bwd": fused}, (dtype, causal, calls)
         for (name, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
             scale = q.grad.abs().max().item() + 1e-12
             err = (p.grad.double().cpu() - q.grad).abs().max().item()
-            assert err <= bound * scale, (dtype, name, err / scale)
+            assert err <= bound * scale, (dtype, causal, name, err / scale)
         torch._dynamo.reset()
 
 

@@ -486,14 +486,16 @@ def attention_backward_supported(dout: torch.Tensor, q: torch.Tensor, k: torch.T
 
 def attention_backward(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                        out: torch.Tensor, lse: torch.Tensor, scale: float, causal: bool,
-                       packed: bool = False):
+                       packed: bool = False, grad_strides=None):
     """(dq, dk, dv) of `attention`: `out` and `dout` are [batch, heads, q_len, 64] views (the
     transposed view of what `attention` returned, and the gradient in the same layout), `lse` what
     `attention(..., return_lse=True)` returned. Each gradient is laid out as
     `torch.empty_like` of its input (what ATen's fused attention backward returns); with `packed`
     and q_len == kv_len the three are [batch, heads, tokens, 64] views of one
     [batch, tokens, 3, heads, 64] buffer, so the gradient of a packed q/k/v projection needs no
-    concatenation."""
+    concatenation. `grad_strides`: three stride tuples (or None) for dq, dk, dv where a caller
+    needs particular layouts; a layout the kernels cannot write (head_dim not contiguous, strides
+    not multiples of 4) is ignored and the default used."""
     require_hip(dout, q, k, v, out, lse)
     if not (scale > 0.0 and math.isfinite(scale)):
         raise ValueError(f"attention_backward: scale must be positive and finite, got {scale}")
@@ -505,7 +507,15 @@ def attention_backward(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: 
         buf = torch.empty((b, t, 3, h, d), dtype=q.dtype, device=q.device)
         dq, dk, dv = (buf[:, :, i].transpose(1, 2) for i in range(3))
     else:
-        dq, dk, dv = _gradient_like(q), _gradient_like(k), _gradient_like(v)
+        grads = []
+        for x, want in zip((q, k, v), grad_strides or (None, None, None)):
+            if want is not None and len(want) == 4 and want[3] == 1 and \
+                    all(st % 4 == 0 and st >= 0 for st in want[:3]):
+                grads.append(torch.empty_strided(tuple(x.shape), tuple(want), dtype=x.dtype,
+                                                 device=x.device))
+            else:
+                grads.append(_gradient_like(x))
+        dq, dk, dv = grads
     lib = _ek.lib()
     workspace = torch.empty(max(int(lib.tmb_attention_bwd_workspace_bytes(b, h, t)), 16),
                             dtype=torch.uint8, device=q.device)

@@ -764,6 +764,87 @@ def _fused_attention(q, k, v, scale, root, slices):
     return ctx.transpose(1, 2).clone(memory_format=torch.contiguous_format)
 
 
+def _attention_fused_ok(q, k, v, scale, root, slices) -> bool:
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    return scale > 0 and hip_ops.attention_supported(q, k, v) and \
+        _causal_q_len(root, slices, (q.shape[2], k.shape[2])) == q.shape[2]
+
+
+def _attention_probabilities(q, k, scale, root, slices):
+    """softmax(masked_fill(q k^T * scale, mask == 0, -inf)) as [batch, heads, t, s], op by op."""
+    b, h, t, d = q.shape
+    s_len = k.shape[2]
+    flat = lambda x: x.expand(x.shape).clone(memory_format=torch.contiguous_format).view(  # noqa: E731
+        b * h, x.shape[2], x.shape[3])
+    scores = _BUILTIN_BMM(flat(q), flat(k.transpose(-2, -1))).view(b, h, t, s_len)
+    return _fused_masked_softmax(scores, scale, root, slices, -1), flat
+
+
+def attention_train_forward(q, k, v, scale, root, slices):
+    """The attention chain of a training graph as one step: (out [batch, tokens, heads, head_dim]
+    contiguous, float32 log-sum-exp [batch, heads, tokens]). The fused kernel takes the call when
+    the mask buffer is causal and the operands are 16-bit heads of 64; otherwise the chain runs
+    op by op and the log-sum-exp stays unwritten (the backward step then takes the same route:
+    both ask the same question about the same operands)."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    b, h, t, d = q.shape
+    if _attention_fused_ok(q, k, v, scale, root, slices):
+        return hip_ops.attention(q, k, v, scale, True, return_lse=True)
+    probs, flat = _attention_probabilities(q, k, scale, root, slices)
+    ctx = _BUILTIN_BMM(probs.view(b * h, t, k.shape[2]), flat(v)).view(b, h, t, d)
+    return (ctx.transpose(1, 2).clone(memory_format=torch.contiguous_format),
+            torch.empty((b, h, t), dtype=torch.float32, device=q.device))
+
+
+def _in_layout(x, layout):
+    """`x` ([batch, heads, tokens, head_dim]) in the layout the rest of a backward graph was
+    traced with: None = token-major ([batch, tokens, heads, head_dim] contiguous underneath), a
+    stride tuple = exactly those strides."""
+    if layout is None:
+        want = (x.shape[1] * x.shape[2] * x.shape[3], x.shape[3], x.shape[1] * x.shape[3], 1)
+    else:
+        want = tuple(layout)
+    if tuple(x.stride()) == want:
+        return x
+    fixed = torch.empty_strided(tuple(x.shape), want, dtype=x.dtype, device=x.device)
+    fixed.copy_(x)
+    return fixed
+
+
+def attention_train_backward(grad_out, q, k, v, out, lse, scale, root, slices, layouts):
+    """(dq, dk, dv), each [batch, heads, tokens, head_dim], from the gradient of
+    attention_train_forward's `out` (same [batch, tokens, heads, head_dim] layout). `layouts`:
+    per gradient, the strides the consumers in the graph were traced with, or None where the
+    token-major layout the kernels write by themselves serves those consumers as well."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    b, h, t, d = q.shape
+    s_len = k.shape[2]
+    if _attention_fused_ok(q, k, v, scale, root, slices):
+        g = grad_out if grad_out.stride(3) == 1 and grad_out.data_ptr() % 16 == 0 and \
+            all(st % 8 == 0 for st in grad_out.stride()[:3]) else grad_out.contiguous()
+        grads = hip_ops.attention_backward(g.transpose(1, 2), q, k, v, out.transpose(1, 2), lse,
+                                           scale, True, grad_strides=layouts)
+        return tuple(_in_layout(x, lay) if lay is not None else x for x, lay in zip(grads, layouts))
+    # op by op from the recomputed probabilities: masked positions hold p = 0, so dS is 0 there
+    probs, flat = _attention_probabilities(q, k, scale, root, slices)
+    p3 = probs.view(b * h, t, s_len)
+    do3 = flat(grad_out.transpose(1, 2))
+    dv = _BUILTIN_BMM(p3.transpose(1, 2), do3)
+    dp = _BUILTIN_BMM(do3, flat(v).transpose(1, 2))
+    ds = hip_ops.softmax_backward(dp, p3, -1, False) * scale
+    dq = _BUILTIN_BMM(ds, flat(k))
+    dk = _BUILTIN_BMM(ds.transpose(1, 2), flat(q))
+    grads = (dq.view(b, h, t, d), dk.view(b, h, s_len, d), dv.view(b, h, s_len, d))
+    return tuple(_in_layout(x, lay) for x, lay in zip(grads, layouts))
+
+
+# the two steps above appear as call_function targets in rewritten training graphs
+MAPPING_TORCH_ATEN_TO_MOJO[attention_train_forward] = attention_train_forward
+MAPPING_TORCH_ATEN_TO_MOJO[attention_train_backward] = attention_train_backward
+
 _BUILTIN_ADDMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.addmm]
 _BUILTIN_BMM = MAPPING_TORCH_ATEN_TO_MOJO[aten.bmm]
 _BUILTIN_ADD = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.add)
@@ -968,21 +1049,13 @@ def boxed_func(*args, **kwargs):
     return make_boxed_func(BaseMaxCompiler(*args, **kwargs).__call__)
 
 
-def _tag_attention_for_recompute(joint_module: torch.fx.GraphModule, num_fwd_outputs: int) -> list:
-    """Marks, in a joint forward + backward graph, every node that the fused attention step
-    would stand for in the forward graph as "recompute in the backward graph": attention
-    probabilities, scores, the mask comparison and the flattened operand copies are then not
-    saved for backward, the forward graph keeps the single-user chain the attention rewrite
-    needs, and the backward graph rebuilds the probabilities from q, k and the mask buffer
-    (fused masked softmax) before the usual softmax / bmm backward ops. Returns the tagged
-    nodes. The forward half is matched on a copy of the graph cut at the forward outputs, with
-    the same matchers the forward compile uses, so a chain is tagged only if it will fuse."""
+def _match_forward_attention(joint_module: torch.fx.GraphModule, num_fwd_outputs: int):
+    """The attention chains the forward rewrite would fuse, found on a copy of the joint graph
+    cut at the forward outputs with the matchers the forward compile uses. Yields, in joint-graph
+    nodes: (final clone node, chain nodes, q, k, v, scale, mask root, slices)."""
     import torch.utils._pytree as pytree
-    from torch.utils.checkpoint import CheckpointPolicy
 
     graph = joint_module.graph
-    if any(n.op == "call_function" and n.is_impure(impure_random=False) for n in graph.nodes):
-        return []  # the partitioner refuses recompute tags next to impure ops
     forward = torch.fx.Graph()  # node names carry over: they are how twins are found below
     leaves = pytree.arg_tree_leaves(forward.graph_copy(graph, {}))
     forward.output(tuple(leaves[:num_fwd_outputs]))
@@ -990,14 +1063,136 @@ def _tag_attention_for_recompute(joint_module: torch.fx.GraphModule, num_fwd_out
     rewrites = _GraphFactory._fuse_masked_softmax(forward)
     absorbed = _GraphFactory._fuse_attention(rewrites)
     by_name = {n.name: n for n in graph.nodes}
+    found = []
+    for final, chain in absorbed.items():
+        _, q, k, v, scale, root, slices = rewrites[final]
+        val = q.meta["val"]
+        if val.dtype not in (torch.bfloat16, torch.float16) or val.shape[-1] != 64:
+            continue  # the kernels take 16-bit heads of 64: elsewhere nothing is gained
+        twins = [by_name.get(n.name) for n in (final, q, k, v, root)]
+        if any(n is None for n in twins):
+            continue
+        found.append((twins[0], [by_name[n.name] for n in chain if n.name in by_name],
+                      twins[1], twins[2], twins[3], scale, twins[4], slices))
+    return found
+
+
+def _fuse_attention_backward(joint_module: torch.fx.GraphModule, match) -> bool:
+    """Replaces one matched attention chain AND its backward nodes in a joint graph by the two
+    steps attention_train_forward / attention_train_backward. The backward nodes are those
+    autograd recorded for the chain's ops (same sequence number, tagged as backward); the
+    rewrite only happens when they form one region with a single incoming gradient (that of the
+    chain's output) and exactly three results, consumed by the backward nodes of q, k and v.
+    Returns False, with the graph untouched, otherwise."""
+    final, chain, q, k, v, scale, root, slices = match
+    graph = joint_module.graph
+    seqs = {n.meta["seq_nr"] for n in [final, *chain] if "seq_nr" in n.meta}
+    if not seqs or any("seq_nr" not in n.meta for n in (q, k, v)):
+        return False
+    region = [n for n in graph.nodes if n.op == "call_function"
+              and n.meta.get("partitioner_tag") == "is_backward" and n.meta.get("seq_nr") in seqs]
+    if not region:
+        return False
+    inside = set(region)
+    gradients, results = [], []
+    for n in region:
+        for inp in n.all_input_nodes:
+            if inp not in inside and inp not in gradients and (
+                    inp.meta.get("partitioner_tag") == "is_backward"
+                    or (inp.op == "placeholder" and "tangents" in str(inp.target))):
+                gradients.append(inp)
+        if any(u not in inside for u in n.users):
+            results.append(n)
+    if len(gradients) != 1 or len(results) != 3:
+        return False
+    grad_final = gradients[0]
+    fval, gval = final.meta.get("val"), grad_final.meta.get("val")
+    if fval is None or gval is None or tuple(gval.shape) != tuple(fval.shape):
+        return False
+    # which result is whose gradient: its consumers differentiate the op that produced q, k or v
+    owner = {}
+    for r in results:
+        consumer_seqs = {u.meta.get("seq_nr") for u in r.users if u not in inside}
+        for name, src in (("q", q), ("k", k), ("v", v)):
+            if consumer_seqs == {src.meta["seq_nr"]}:
+                if name in owner:
+                    return False
+                owner[name] = r
+    if len(owner) != 3 or len({id(r) for r in owner.values()}) != 3:
+        return False
+    for name, src in (("q", q), ("k", k), ("v", v)):
+        rv = owner[name].meta.get("val")
+        if rv is None or tuple(rv.shape) != tuple(src.meta["val"].shape):
+            return False
+
+    def layout_for(result):
+        """None (token-major serves) when every consumer transposes tokens and heads back and then
+        only copies or reshapes; otherwise the strides the graph was traced with."""
+        def token_major_ok(node):
+            if node.target is not aten.transpose.int or {x % 4 for x in node.args[1:3]} != {1, 2}:
+                return False
+            return all(u.target in (aten.clone.default, aten.view.default, aten._unsafe_view.default,
+                                    aten.reshape.default) for u in node.users)
+        consumers = [u for u in result.users if u not in inside]
+        if consumers and all(token_major_ok(u) for u in consumers):
+            return None
+        strides = result.meta["val"].stride()
+        return tuple(int(x) for x in strides) if all(isinstance(x, int) for x in strides) else None
+
+    layouts = tuple(layout_for(owner[name]) for name in "qkv")
+    qv = q.meta["val"]
+    b, h, t, d = qv.shape
+    with qv.fake_mode:
+        out_val = torch.empty((b, t, h, d), dtype=qv.dtype, device=qv.device)
+        lse_val = torch.empty((b, h, t), dtype=torch.float32, device=qv.device)
+
+    def tagged(node, val, tag, like):
+        node.meta["val"] = val
+        node.meta["partitioner_tag"] = tag
+        for key in ("seq_nr", "stack_trace", "nn_module_stack", "fwd_nn_module_stack"):
+            if key in like.meta:
+                node.meta[key] = like.meta[key]
+        return node
+
+    with graph.inserting_before(final):
+        fwd = tagged(graph.call_function(attention_train_forward, (q, k, v, scale, root, slices)),
+                     (out_val, lse_val), "is_forward", final)
+        out = tagged(graph.call_function(operator.getitem, (fwd, 0)), out_val, "is_forward", final)
+        lse = tagged(graph.call_function(operator.getitem, (fwd, 1)), lse_val, "is_forward", final)
+    first_result = min(results, key=lambda n: list(graph.nodes).index(n))
+    with graph.inserting_before(first_result):
+        vals = tuple(owner[name].meta["val"] for name in "qkv")
+        bwd = tagged(graph.call_function(attention_train_backward,
+                                         (grad_final, q, k, v, out, lse, scale, root, slices,
+                                          layouts)),
+                     vals, "is_backward", first_result)
+        grads = [tagged(graph.call_function(operator.getitem, (bwd, i)), vals[i], "is_backward",
+                        first_result) for i in range(3)]
+    final.replace_all_uses_with(out)
+    for i, name in enumerate("qkv"):
+        owner[name].replace_all_uses_with(grads[i], delete_user_cb=lambda u: u not in inside)
+    graph.eliminate_dead_code()
+    joint_module.recompile()
+    return True
+
+
+def _tag_attention_for_recompute(joint_module: torch.fx.GraphModule, num_fwd_outputs: int) -> list:
+    """Marks, in a joint forward + backward graph, every node that the fused attention step
+    would stand for in the forward graph as "recompute in the backward graph": attention
+    probabilities, scores, the mask comparison and the flattened operand copies are then not
+    saved for backward, the forward graph keeps the single-user chain the attention rewrite
+    needs, and the backward graph rebuilds the probabilities from q, k and the mask buffer
+    (fused masked softmax) before the usual softmax / bmm backward ops. Returns the tagged
+    nodes. A chain is tagged only if it will fuse (see _match_forward_attention)."""
+    from torch.utils.checkpoint import CheckpointPolicy
+
+    graph = joint_module.graph
+    if any(n.op == "call_function" and n.is_impure(impure_random=False) for n in graph.nodes):
+        return []  # the partitioner refuses recompute tags next to impure ops
     tagged = []
-    for region, (final, chain) in enumerate(absorbed.items(), start=1):
-        q = rewrites[final][1].meta["val"]
-        if q.dtype not in (torch.bfloat16, torch.float16) or q.shape[-1] != 64:
-            continue  # the kernel takes 16-bit heads of 64: elsewhere recomputing buys nothing
-        for twin in chain:
-            node = by_name.get(twin.name)
-            if node is None or node.op != "call_function":
+    for region, match in enumerate(_match_forward_attention(joint_module, num_fwd_outputs), start=1):
+        for node in match[1]:
+            if node.op != "call_function":
                 continue
             node.meta["recompute"] = CheckpointPolicy.MUST_RECOMPUTE
             node.meta["ac_graph_id"] = region
@@ -1016,13 +1211,19 @@ def attention_recompute_partition(joint_module, joint_inputs, *, num_fwd_outputs
     """The partitioner of a training graph: PyTorch's default split (what is between the forward
     inputs and outputs is the forward graph, everything it computed is available to backward;
     the reference passes no partitioner and gets the same, compiler.py:573-577), after the
-    attention score chains were tagged for recomputation so that the forward graph runs the
-    fused attention kernel and saves q, k, v instead of the [heads, tokens, tokens] matrices."""
+    attention chains were dealt with: a chain whose backward nodes form one clean region is
+    replaced, forward and backward, by the two fused steps (the forward saves q, k, v, its output
+    and the log-sum-exp; nothing of size [heads, tokens, tokens] exists in either graph); any
+    other chain the forward rewrite would fuse is tagged for recomputation, so that the forward
+    graph still runs the fused kernel and the backward graph rebuilds the probabilities."""
     from torch._functorch.partitioners import default_partition
 
     if _fusion_enabled() and _attention_fusion_enabled():
         try:
-            _tag_attention_for_recompute(joint_module, num_fwd_outputs)
+            matches = _match_forward_attention(joint_module, num_fwd_outputs)
+            fused = sum(1 for match in matches if _fuse_attention_backward(joint_module, match))
+            if fused < len(matches):
+                _tag_attention_for_recompute(joint_module, num_fwd_outputs)
         except Exception as exc:  # noqa: BLE001 - the untagged split is always valid
             for node in joint_module.graph.nodes:
                 if node.meta.get("recompute") is not None and "ac_graph_id" in node.meta:
