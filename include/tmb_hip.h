@@ -94,6 +94,18 @@ int tmb_layer_norm_rows(void* out, float* mean, float* rstd, const void* x, cons
                         const void* beta, int64_t rows, int64_t cols, double eps, int in_dtype,
                         int dtype, void* stream);
 
+/* Reduction over the LEADING dimension of a row-major [rows, cols] matrix: out[c] = op_r in[r, c]
+ * (SUM, MEAN = sum / rows, AMAX with NaN propagation), floats only, fp32 accumulation, one cast.
+ * The bias gradient of a linear layer and every sum(x, dim=0): the input is read once in row
+ * order, row slabs are reduced into float32 partial rows in the workspace
+ * (tmb_reduce_cols_workspace_bytes) and added slab by slab in a fixed order. rows == 0 returns
+ * TMB_ERR_UNSUPPORTED (the identity of an empty reduction is the caller's rule).
+ * Replaces the permute + contiguous copy into [kept, reduced] order (op_utils/__init__.mojo:651-720)
+ * that precedes SumSpec/MeanSpec/AmaxSpec (reduction_ops.mojo:1094-1184) for such dims. */
+size_t tmb_reduce_cols_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+int tmb_reduce_cols(void* out, const void* in, int64_t rows, int64_t cols, int op, int dtype,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
 /* Bytes of device workspace `tmb_reduce_rows` / `tmb_argmax_rows` need for a shape (may be 0). */
 size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dtype);
 

@@ -173,3 +173,70 @@ def test_argmax_dim_none_keepdim_and_nan():
     assert torch.equal(ops.argmax(_dev(x), 2, False).cpu(), torch.argmax(x, dim=2))
     all_equal = torch.zeros(3, 70000)
     assert torch.equal(ops.argmax(_dev(all_equal), 1, False).cpu(), torch.zeros(3, dtype=torch.int64))
+
+
+# ---- reductions over the leading dimension (bias gradients, sum(x, dim=0)) ---------------------
+# (rows, cols): one slab and many, whole vectors and ragged widths, the bias-gradient shapes of
+# GPT-2 (tokens x 768 / 2304 / 3072), a width of one, more columns than rows
+COLS_SHAPES = [(16, 1024), (17, 1031), (4096, 768), (16384, 2304), (2048, 3072), (100000, 8),
+               (50000, 1), (33, 50257), (30000, 5)]
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", COLS_SHAPES)
+def test_sum_mean_amax_over_the_leading_dimension(shape, dtype):
+    x = seeded(shape, seed=shape[0] % 991, dtype=dtype)
+    assert x.numel() >= _ops()._COLS_KERNEL_MIN_ELEMENTS
+    xd, x64 = _dev(x), as64(x)
+    bound = cf.sum_error_bound(x64.T, axis=-1)
+    s = _ops().reduce(xd, [0], False, _ek().SUM)
+    assert s.dtype == dtype and tuple(s.shape) == (shape[1],)
+    assert_close64(s, x64.sum(0), extra_abs=bound, what=f"sum {shape}")
+    m = _ops().reduce(xd, [0], True, _ek().MEAN)
+    assert tuple(m.shape) == (1, shape[1])
+    assert_close64(m[0], x64.mean(0), extra_abs=bound / shape[0], what=f"mean {shape}")
+    a = _ops().reduce(xd, [0], False, _ek().AMAX)
+    assert np.array_equal(as64(a), x64.max(0)), "amax must be exact"
+    # the C restatement works on rows: hand it the transposed matrix
+    ref = oracle.reduce_rows(x.t().contiguous(), oracle.SUM)
+    assert_close64(s, as64(ref), extra_abs=2 * bound, rounded_want=True, what="sum vs C oracle")
+    # same call, same bits (fixed order of additions)
+    assert torch.equal(s, _ops().reduce(xd, [0], False, _ek().SUM))
+
+
+def test_leading_dimension_reductions_of_higher_rank_nan_and_views():
+    x = seeded((12, 50, 40, 16), seed=7)
+    for dims in ([0], [0, 1], [0, 1, 2]):
+        got = _ops().reduce(_dev(x), dims, False, _ek().SUM)
+        assert_close64(got, as64(x).sum(tuple(dims)), extra_abs=cf.sum_error_bound(
+            np.moveaxis(as64(x), dims, [-1 - i for i in range(len(dims))]).reshape(*x.shape[len(dims):], -1), axis=-1))
+        assert tuple(_ops().reduce(_dev(x), dims, True, _ek().AMAX).shape) == tuple(
+            1 if d in dims else x.shape[d] for d in range(4))
+    y = seeded((5000, 24), seed=8)
+    y[1234, 7] = float("nan")
+    y[4000, 3] = float("inf")
+    a = _ops().reduce(_dev(y), [0], False, _ek().AMAX).cpu()
+    assert torch.isnan(a[7]) and a[3] == float("inf") and not torch.isnan(a[[0, 1, 2]]).any()
+    # a view that is not contiguous, and an integer tensor, keep the transposing route
+    z = _dev(seeded((300, 128), seed=9))
+    assert_close64(_ops().reduce(z[:, ::2], [0], False, _ek().SUM), as64(z.cpu())[:, ::2].sum(0), atol=1e-3)
+    i = torch.arange(40000, dtype=torch.int64).reshape(2000, 20)
+    assert torch.equal(_ops().reduce(_dev(i), [0], False, _ek().SUM).cpu(), i.sum(0))
+
+
+def test_reduce_cols_entry_point_checks_its_workspace():
+    ek = _ek()
+    L = ek.lib()
+    x = _dev(seeded((4096, 768), seed=1))
+    out = torch.empty(768, device="cuda")
+    need = L.tmb_reduce_cols_workspace_bytes(4096, 768, ek.F32)
+    assert need >= 768 * 4
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, ek.SUM, ek.F32, ws.data_ptr(), need - 1, st) == -3
+    assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, ek.SUM, ek.F32, None, 0, st) == -3
+    assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 0, 768, ek.SUM, ek.F32, None, 0, st) == -2
+    assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, 7, ek.F32, ws.data_ptr(), need, st) == -1
+    assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, ek.SUM, ek.I64, ws.data_ptr(), need, st) == -2
+    assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, ek.SUM, ek.F32, ws.data_ptr(), need, st) == 0
+    assert_close64(out, as64(x.cpu()).sum(0), atol=2e-3)

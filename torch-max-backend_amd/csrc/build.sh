@@ -6,7 +6,7 @@ set -e
 here="$(cd "$(dirname "$0")" && pwd)"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Wno-inline-asm -Xclang -target-feature -Xclang -packed-fp32-ops"
-units="softmax layer_norm reduce gemm attention attention_bwd backward misc"
+units="softmax layer_norm reduce reduce_cols gemm attention attention_bwd backward misc"
 objs=""
 pids=""
 for f in $units; do

@@ -52,6 +52,8 @@ SIGNATURES = {
     "tmb_layer_norm_backward_rows": (_ci, [_vp] * 8 + [_i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
     "tmb_cat2_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "tmb_reduce_cols_workspace_bytes": (_sz, [_i64, _i64, _ci]),
+    "tmb_reduce_cols": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
     "tmb_pad_rows": (_ci, [_vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp]),
 }
 

@@ -707,12 +707,34 @@ def _workspace(rows: int, cols: int, code: int, device) -> Tuple[Optional[torch.
     return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
 
 
+# Below this many elements the transposing route costs the same few microseconds.
+_COLS_KERNEL_MIN_ELEMENTS = 1 << 14
+
+
 def reduce(x: torch.Tensor, dims: Sequence[int], keepdim: bool, op: int) -> torch.Tensor:
     """sum / mean / amax over `dims` (already normalised, sorted, unique, non-empty unless
     x is 0-d). Output dtype = input dtype."""
     require_hip(x)
     code = code_of(x.dtype)
     rank = x.dim()
+    dims = list(dims)
+    # The leading dims of a contiguous float tensor (the bias gradient of a linear layer,
+    # sum(x, dim=0)): reduced in place by the column kernel instead of transposing first.
+    lead = len(dims)
+    if 0 < lead < rank and dims == list(range(lead)) and x.dtype in FLOAT_DTYPES \
+            and x.is_contiguous() and x.numel() >= _COLS_KERNEL_MIN_ELEMENTS:
+        n_rows = math.prod(x.shape[:lead])
+        n_cols = math.prod(x.shape[lead:])
+        if 0 < n_rows < (1 << 40) and n_cols > 0:
+            lib = _ek.lib()
+            out = torch.empty(tuple(x.shape[lead:]), dtype=x.dtype, device=x.device)
+            nbytes = int(lib.tmb_reduce_cols_workspace_bytes(n_rows, n_cols, code))
+            ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+            rc = lib.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), n_rows, n_cols, op, code,
+                                     ws.data_ptr(), nbytes, _stream())
+            if rc != _ek.ERR_UNSUPPORTED:
+                _check("tmb_reduce_cols", rc)
+                return out.reshape([1] * lead + list(x.shape[lead:])) if keepdim else out
     moved, rows, cols, kept_shape = _reduce_geometry(x, dims)
     if cols == 0 or rows == 0:
         raise ValueError("reduce: empty reduction has no kernel; the caller decides its value")
