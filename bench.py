@@ -438,6 +438,16 @@ def main() -> int:
                                                              op, code, ws.data_ptr(), ws_bytes, stream),
                         nbytes + es)
             assert torch.equal(out_all.reshape(()), hip_ops.reduce(bufs[(39 + 8) % len(bufs)], [0, 1], False, ek.AMAX))
+            # the same matrices summed over their leading dimension (the bias gradient of a linear
+            # layer): out[c] = sum_r x[r, c]
+            out_cols = torch.empty(cols, dtype=dtype, device=dev)
+            cws_bytes = lib.tmb_reduce_cols_workspace_bytes(rows, cols, code)
+            cws = torch.empty(max(cws_bytes, 16), dtype=torch.uint8, device=dev)
+            hbm_row(f"sum_{dn}_cols_{rows}x{cols}", len(bufs),
+                    lambda i: lib.tmb_reduce_cols(out_cols.data_ptr(), in_ptrs[i], rows, cols, ek.SUM, code,
+                                                  cws.data_ptr(), cws_bytes, stream),
+                    nbytes + cols * es)
+            assert torch.allclose(out_cols.float(), bufs[(39 + 8) % len(bufs)].float().sum(0), rtol=2e-2, atol=2.0)
             del bufs
         rows, cols = 512, 50257
         bufs = rotating(lambda i: gen((rows, cols), 40 + i, torch.float32), rows * cols * 4)
@@ -574,6 +584,7 @@ def main() -> int:
         from torch_mojo_backend import mojo_backend
 
         B, T = 16, 1024
+        torch._dynamo.reset()  # its own static graph, whatever batch sizes ran before
         model = build_gpt2_small(seed=0).to(torch.bfloat16).to(dev)
         idx, targets = seeded_tokens(B, T, seed=0).to(dev), seeded_tokens(B, T, seed=1).to(dev)
 

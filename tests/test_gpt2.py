@@ -95,6 +95,31 @@ def test_gpt2_small_bf16_logits_vs_fp32_oracle():
     assert torch.equal(nxt.cpu(), torch.argmax(logits[:, -1, :], dim=-1).cpu())
 
 
+def test_gpt2_small_bf16_second_batch_size_runs_the_symbolic_graph():
+    """A compiled module called with a second batch size is retraced with a symbolic batch
+    dimension: the plans made at build time then hold symbols where the first graph held numbers,
+    and every step has to take its sizes from the tensors it is handed. Both sizes, and the first
+    one again, give the logits of the graph compiled for that size alone."""
+    from torch_mojo_backend import mojo_backend
+
+    gpu_model = build_gpt2_small(seed=0).to(torch.bfloat16).to("cuda")
+    torch._dynamo.reset()
+    compiled = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)
+    got = {}
+    with torch.no_grad():
+        for batch in (2, 3, 2):
+            idx = seeded_tokens(batch, 128, seed=batch).to("cuda")
+            got[batch] = (idx, compiled(idx)[0])
+    for batch, (idx, logits) in got.items():
+        torch._dynamo.reset()
+        alone = torch.compile(gpu_model, backend=mojo_backend, fullgraph=True)
+        with torch.no_grad():
+            want = alone(idx)[0]
+        assert logits.shape == (batch, 128, 50257)
+        assert (logits.float() - want.float()).abs().max().item() <= 2e-2
+    torch._dynamo.reset()
+
+
 def test_gpt2_small_bf16_bit_identical_mode_matches_the_vendor_pipeline(monkeypatch):
     """TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED=1: every tensor of the graph is rounded where the
     unfused kernels would have stored it; the logit error is then that of any bf16 pipeline."""

@@ -715,8 +715,11 @@ def _fused_addmm_residual(bias, mat1, mat2, residual, out_shape, out_dtype, *,
                           round_like_unfused=False):
     """add(view(addmm(bias, mat1, mat2), out_shape), residual). ``residual`` arrives in the
     graph's dtype or, from a widened producer, in float32; ``out_dtype`` is None (the graph's
-    dtype) or float32 (this step's consumers all read float32)."""
+    dtype) or float32 (this step's consumers all read float32). The residual has the result's
+    shape, which is read from it at run time (the planned `out_shape` holds symbols in a graph
+    with dynamic sizes)."""
     n = mat2.shape[-1]
+    out_shape = tuple(residual.shape)
     if isinstance(mat1, torch.Tensor) and mat1.is_cuda and bias.dim() == 1 and bias.shape[0] == n \
             and bias.dtype == mat1.dtype and residual.dtype in (mat1.dtype, torch.float32):
         return aten_functions.addmm_residual(bias, mat1, mat2, residual, out_dtype,
