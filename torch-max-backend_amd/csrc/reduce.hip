@@ -385,7 +385,11 @@ __device__ __forceinline__ void scan_one(V& best, int& best_off, V x, int off) {
   best_off = take ? off : best_off;
 }
 
-template <typename T, int NT>
+// U 16-byte loads per lane are requested before the first of them is compared; a batch that
+// reaches past the end of the range is cut short lane by lane, so there is no one-load-at-a-time
+// remainder loop (a row of 50257 floats over 1024 lanes is 12.3 vectors per lane: two batches of
+// seven instead of three of four plus one).
+template <typename T, int NT, int U = 4>
 __device__ __forceinline__ Best<typename ArgTraits<T>::val_t> argmax_range(const T* __restrict__ p,
                                                                            int64_t n, int tid,
                                                                            int64_t base) {
@@ -399,21 +403,18 @@ __device__ __forceinline__ Best<typename ArgTraits<T>::val_t> argmax_range(const
   if (tid < head) scan_one(best, off, ArgTraits<T>::conv(p[tid]), tid);
   const T* body = p + head;
   const int nvec = static_cast<int>((n - head) / EPV);
-  int i = tid;
-  for (; i + 3 * NT < nvec; i += 4 * NT) {  // four 16-byte loads in flight per lane
-    Vec16<T> v[4];
+  for (int i = tid; i < nvec; i += U * NT) {
+    Vec16<T> v[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = load_vec16_stream(body + static_cast<int64_t>(i + u * NT) * EPV);
+    for (int u = 0; u < U; ++u)
+      if (i + u * NT < nvec) v[u] = load_vec16_stream(body + static_cast<int64_t>(i + u * NT) * EPV);
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < U; ++u)
+      if (i + u * NT < nvec) {
 #pragma unroll
-      for (int e = 0; e < EPV; ++e)
-        scan_one(best, off, ArgTraits<T>::conv(v[u].v[e]), head + (i + u * NT) * EPV + e);
-  }
-  for (; i < nvec; i += NT) {
-    const Vec16<T> v0 = load_vec16_stream(body + static_cast<int64_t>(i) * EPV);
-#pragma unroll
-    for (int e = 0; e < EPV; ++e) scan_one(best, off, ArgTraits<T>::conv(v0.v[e]), head + i * EPV + e);
+        for (int e = 0; e < EPV; ++e)
+          scan_one(best, off, ArgTraits<T>::conv(v[u].v[e]), head + (i + u * NT) * EPV + e);
+      }
   }
   const int tail = head + nvec * EPV;
   if (tail + tid < n) scan_one(best, off, ArgTraits<T>::conv(p[tail + tid]), tail + tid);
@@ -438,7 +439,7 @@ struct alignas(16) BestSlot {
   V val;
 };
 
-template <typename T, int BLK>
+template <typename T, int BLK, int U = 4>
 __global__ __launch_bounds__(BLK) void argmax_chunk_kernel(int64_t* __restrict__ out,
                                                            void* __restrict__ ws,
                                                            const T* __restrict__ in, int64_t rows,
@@ -453,7 +454,7 @@ __global__ __launch_bounds__(BLK) void argmax_chunk_kernel(int64_t* __restrict__
   const int64_t c0 = static_cast<int64_t>(split) * chunk;
   int64_t n = cols - c0;
   if (n > chunk) n = chunk;
-  Best<V> b = argmax_range<T, BLK>(in + row * cols + c0, n, threadIdx.x, c0);
+  Best<V> b = argmax_range<T, BLK, U>(in + row * cols + c0, n, threadIdx.x, c0);
   b = wave_best(b);
   const int wave = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) slot[wave] = BestSlot<V>{b.idx, b.val};
@@ -503,7 +504,7 @@ static int launch_argmax(int64_t* out, const void* in_, int64_t rows, int64_t co
   // the same work per thread in a single launch (the second stage alone costs 4-5 us).
   if (plan.splits > 1 && plan.splits <= 4 && rows >= 256 && rows < (int64_t{1} << 31) &&
       cols < (int64_t{1} << 30)) {
-    argmax_chunk_kernel<T, 1024><<<dim3(static_cast<unsigned>(rows)), dim3(1024), 0, stream>>>(
+    argmax_chunk_kernel<T, 1024, 7><<<dim3(static_cast<unsigned>(rows)), dim3(1024), 0, stream>>>(
         out, ws, in, rows, cols, 1, cols);
     return check_launch();
   }
