@@ -120,6 +120,31 @@ def test_gpt2_small_bf16_second_batch_size_runs_the_symbolic_graph():
     torch._dynamo.reset()
 
 
+@pytest.mark.parametrize("dynamic", [None, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_two_layer_gpt2_with_changing_batch_and_sequence_length(dtype, dynamic):
+    """One compiled module, seven (batch, sequence) shapes in a row, with the shapes left to
+    dynamo (static first, symbolic after the first change) and declared dynamic from the start:
+    every fused step and the attention rewrite take their sizes from the tensors at run time.
+    Reference: the same module in PyTorch-ROCm eager (same dtype), float32 to 1e-4, bf16 to the
+    spread two bf16 pipelines show on this model."""
+    from torch_mojo_backend import mojo_backend
+
+    model = build_gpt2_small(seed=0, n_layer=2).to(dtype).to("cuda")
+    torch._dynamo.reset()
+    compiled = torch.compile(model, backend=mojo_backend, dynamic=dynamic)
+    for batch, seq in ((2, 128), (3, 128), (3, 256), (1, 64), (4, 100), (2, 1), (5, 77)):
+        idx = seeded_tokens(batch, seq, seed=1000 * batch + seq).to("cuda")
+        with torch.no_grad():
+            got, nxt = compiled(idx)
+            want, _ = model(idx)
+        assert got.shape == (batch, seq, 50257) and got.dtype == dtype
+        err = (got.float() - want.float()).abs().max().item()
+        assert err <= (1e-4 if dtype == torch.float32 else 4e-2), (batch, seq, err)
+        assert torch.equal(nxt, torch.argmax(got[:, -1, :], dim=-1))
+    torch._dynamo.reset()
+
+
 def test_gpt2_small_bf16_bit_identical_mode_matches_the_vendor_pipeline(monkeypatch):
     """TORCH_MOJO_BACKEND_ROUND_LIKE_UNFUSED=1: every tensor of the graph is rounded where the
     unfused kernels would have stored it; the logit error is then that of any bf16 pipeline."""

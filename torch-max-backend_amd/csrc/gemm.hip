@@ -123,8 +123,12 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
     if (g.k % 64 == 0) {
       const int64_t t256 = tiles(256, 256);
       const int64_t rounds = (t256 + 255) / 256;
-      if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9)
-        return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI>(g, batch, stream);
+      if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9) {
+        // (the 16x16x32 MFMA wins where the launch is limited by power, i.e. at long K)
+        if (g.k >= 4096)
+          return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
+        return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, false>(g, batch, stream);
+      }
       if (tiles(256, 128) >= 512)
         return launch_ring<T, 256, 128, 64, 4, 2, 3, B_KMAJOR, EPI>(g, batch, stream);
     }
@@ -248,12 +252,13 @@ static int launch_splitk(const GemmArgs& g, const SplitKPlan& plan, int trans_a,
   part.splits = plan.splits;
   int rc;
   if (plan.tile == 256) {
+    // (a split's run of K is short: the 32x32x16 MFMA, as for short unsplit products)
     if (trans_a)
-      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, true, true>(part, plan.splits, stream);
+      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, true, true, false>(part, plan.splits, stream);
     else if (trans_b)
-      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, true, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, true, TMB_EPI_NONE, false, true, false>(part, plan.splits, stream);
     else
-      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, false, true>(part, plan.splits, stream);
+      rc = launch_ring<T, 256, 256, 64, 2, 4, 2, false, TMB_EPI_NONE, false, true, false>(part, plan.splits, stream);
   } else if (trans_a) {
     rc = launch_ring<T, 128, 128, 32, 2, 2, 4, false, TMB_EPI_NONE, true, true>(part, plan.splits, stream);
   } else if (trans_b) {

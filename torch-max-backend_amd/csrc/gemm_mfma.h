@@ -60,6 +60,30 @@ struct Mfma<f16_t> {
   }
 };
 
+// v_mfma_f32_16x16x32: a lane holds row (lane % 16) and eight consecutive k starting at
+// 8 * (lane / 16) of each operand; of the 16 x 16 result it holds column (lane % 16) and rows
+// 4 * (lane / 16) + {0..3}. Per multiply-add it reads and writes half as many accumulator
+// registers as the 32x32x16 form and draws measurably less power: a loop of nothing but MFMAs on
+// random bf16 operands sustains 2.02 PFLOP/s against 1.79 PFLOP/s, the clock being set by the
+// power the matrix pipes draw.
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4v_t;
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<bf16_t> {
+  static __device__ __forceinline__ f32x4v_t run(u32x4_t a, u32x4_t b, f32x4v_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma16<f16_t> {
+  static __device__ __forceinline__ f32x4v_t run(u32x4_t a, u32x4_t b, f32x4v_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+};
+
 constexpr int kBK = 64;  // K extent of one LDS stage (64 x 2 bytes = one 128-byte line)
 constexpr int kLineBytes = 128;
 
@@ -448,6 +472,79 @@ __device__ __forceinline__ void store_wave_tile(f32x16_t (&acc)[TM][TN], lds_byt
   }
 }
 
+// The same for accumulators of 16x16 tiles (operand-swapped v_mfma_f32_16x16x32: a lane holds
+// row lane % 16 and columns 4 * (lane / 16) + {0..3} of a tile): AM x AN tiles, two tile rows per
+// 32-row band. The band layouts and the flush are shared with the 32x32 form.
+template <typename T, int EPI, int AM, int AN, bool STREAM>
+__device__ __forceinline__ void store_wave_tile16_impl(f32x4v_t (&acc)[AM][AN], lds_byte_t* band,
+                                                  void* __restrict__ Cv, int64_t ldc, int64_t row0,
+                                                  int64_t col0, int64_t M, int64_t N,
+                                                  const T* __restrict__ bias,
+                                                  const EpilogueArgs& ep, int lane) {
+  constexpr int WN = AN * 16;
+  static_assert(AM % 2 == 0, "whole 32-row bands");
+  float bias_f[AN][4];
+#pragma unroll
+  for (int j = 0; j < AN; ++j) {
+    const u32x2_t b4 = load_bias4<T>(bias, col0 + j * 16 + 4 * (lane >> 4), N);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bias_f[j][e] = unpack_elem<T>(b4, e);
+  }
+  if constexpr (EPI == TMB_EPI_NONE) {
+    if (ep.wide()) {  // wave-uniform
+      constexpr int PITCH = BandLayoutF32<WN>::PITCH;
+      lds_byte_t* mine = band + (lane & 15) * PITCH + 16 * (lane >> 4);
+#pragma unroll
+      for (int b = 0; b < AM / 2; ++b) {
+        if (row0 + b * 32 >= M) break;  // wave-uniform
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int j = 0; j < AN; ++j) {
+            const f32x4v_t& a = acc[2 * b + h][j];
+            const f32x4_lds_t v = {a[0] + bias_f[j][0], a[1] + bias_f[j][1], a[2] + bias_f[j][2],
+                                   a[3] + bias_f[j][3]};
+            *(lds_f32x4_t*)(mine + h * 16 * PITCH + j * 64) = v;
+          }
+        flush_band_wide<T, WN, STREAM>(band, Cv, ldc, row0 + b * 32, col0, M, N, ep, lane);
+      }
+      return;
+    }
+  }
+  constexpr int PITCH = BandLayout<WN>::PITCH;
+  lds_byte_t* mine = band + (lane & 15) * PITCH + 8 * (lane >> 4);
+  T* __restrict__ C = static_cast<T*>(Cv);
+  const T* __restrict__ R = static_cast<const T*>(ep.residual);
+#pragma unroll
+  for (int b = 0; b < AM / 2; ++b) {
+    if (row0 + b * 32 >= M) break;  // wave-uniform
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < AN; ++j) {
+        const f32x4v_t& a = acc[2 * b + h][j];
+        u32x2_t packed;
+        packed[0] = finish2<T, EPI>(a[0] + bias_f[j][0], a[1] + bias_f[j][1], ep.twice);
+        packed[1] = finish2<T, EPI>(a[2] + bias_f[j][2], a[3] + bias_f[j][3], ep.twice);
+        *(lds_u32x2_t*)(mine + h * 16 * PITCH + j * 32) = packed;
+      }
+    flush_band<T, WN, STREAM>(band, C, ldc, row0 + b * 32, col0, M, N, R, ep.ldr, lane);
+  }
+}
+
+template <typename T, int EPI, int AM, int AN>
+__device__ __forceinline__ void store_wave_tile16(f32x4v_t (&acc)[AM][AN], lds_byte_t* band,
+                                                  void* __restrict__ C, int64_t ldc, int64_t row0,
+                                                  int64_t col0, int64_t M, int64_t N,
+                                                  const T* __restrict__ bias, bool stream,
+                                                  const EpilogueArgs& ep, int lane) {
+  if (stream) {
+    store_wave_tile16_impl<T, EPI, AM, AN, true>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane);
+  } else {
+    store_wave_tile16_impl<T, EPI, AM, AN, false>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane);
+  }
+}
+
 // The batch entry's epilogue description out of the launch arguments.
 template <typename T>
 __device__ __forceinline__ EpilogueArgs epilogue_args(const GemmArgs& g, int64_t batch) {
@@ -489,6 +586,31 @@ __device__ __forceinline__ void store_wave_tile_f32(f32x16_t (&acc)[TM][TN], flo
             if (col + e < N) dst[e] = acc[i][j][4 * q + e];
         }
       }
+  }
+}
+
+// The same for 16x16 accumulator tiles: lanes l, l+16, l+32, l+48 write 64 contiguous bytes.
+template <int AM, int AN>
+__device__ __forceinline__ void store_wave_tile16_f32(f32x4v_t (&acc)[AM][AN], float* __restrict__ P,
+                                                      int64_t ldp, int64_t row0, int64_t col0,
+                                                      int64_t M, int64_t N, int lane) {
+#pragma unroll
+  for (int i = 0; i < AM; ++i) {
+    const int64_t row = row0 + i * 16 + (lane & 15);
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < AN; ++j) {
+      const int64_t col = col0 + j * 16 + 4 * (lane >> 4);
+      float* dst = P + row * ldp + col;
+      if (col + 4 <= N) {
+        f32x4_unaligned_t v = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+        *reinterpret_cast<f32x4_unaligned_t*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < N) dst[e] = acc[i][j][e];
+      }
+    }
   }
 }
 

@@ -20,7 +20,9 @@
 // ds_read_b64_tr_b16: sixteen lanes read a 4(k) x 16(n) block as 8-byte row pieces and get it
 // back transposed (lane = n, four consecutive k), which is the MFMA operand layout, so no
 // shuffle or repacking is spent on the transpose. Its 16-byte chunks are XOR-swizzled with
-// 4*(k%4), which spreads the four k-rows of such a block over distinct banks.
+// 4*(k%4), which spreads the four k-rows of such a block over distinct banks, and with
+// 2*((k/8)%2), which does the same for two groups of 16 lanes that read blocks eight k apart
+// (the 16-row fragments of v_mfma_f32_16x16x32).
 //
 // The ring is unrolled by hand (stage indices are compile-time), so every fragment read is a
 // per-lane base register plus an immediate offset.
@@ -82,17 +84,27 @@ constexpr bool kRingPersistent = ring_waves_per_simd(BM, BN, BK, WAVES, R) <= 2;
 // product dy^T x); it is then staged and read exactly like N-major B.
 // OUT_F32: a split-K launch: the batch index is the split, the accumulators are stored as fp32
 // partials (no bias, no epilogue, no cast).
+// MI16_: multiply with v_mfma_f32_16x16x32 (64-deep stages only).
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
-          bool A_MMAJOR = false, bool OUT_F32 = false>
+          bool A_MMAJOR = false, bool OUT_F32 = false, bool MI16_ = (BK == 64)>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
                              ring_waves_per_simd(BM, BN, BK, WAVES_M* WAVES_N, R))
 void gemm_ring_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  constexpr int TM = WM / 32, TN = WN / 32;
+  // 64-deep stages can be multiplied with v_mfma_f32_16x16x32 (two k-steps of 32 per stage; a
+  // stage of 32 would be a single k-step and the fragment double buffer would change parity from
+  // stage to stage). Long products are limited by the power the chip may draw, and this form
+  // draws less per multiply-add: +3-6 % at K >= 4096. Short products (K = 768) are not, and lose
+  // 3-10 % to its doubled instruction count; the launcher picks per shape.
+  static_assert(!MI16_ || BK == 64, "16x16x32 needs 64-deep stages");
+  constexpr bool MI16 = MI16_;
+  constexpr int FRAG = MI16 ? 16 : 32;                // rows of an operand fragment
+  constexpr int TM = WM / FRAG, TN = WN / FRAG;       // result tiles per wave
   constexpr int LINE = BK * 2;         // bytes of one row of a K-major operand per stage
-  constexpr int KSTEPS = BK / 16;      // MFMA k-steps per stage
+  constexpr int KSTEPS = BK / (MI16 ? 32 : 16);       // MFMA k-steps per stage
+  constexpr int KCHUNKS = MI16 ? 4 : 2;               // 16-byte chunks of a row per k-step
   constexpr int LPR = LINE / 16;       // lanes (16-byte chunks) per row of a load
   constexpr int RPG = 1024 / LINE;     // rows per 1 KiB load
   constexpr int A_BYTES = BM * LINE, B_BYTES = BN * LINE;
@@ -149,7 +161,7 @@ void gemm_ring_kernel(GemmArgs g) {
       // stage bytes [group*1024 + 16*lane] = k-row (BM*2 bytes each), swizzled 16-byte slot
       const int at = (wave * A_GROUPS + j) * 1024 + lane * 16;
       const int krow = at / (BM * 2);
-      const int chunk = ((at % (BM * 2)) >> 4) ^ ((krow & 3) << 2);
+      const int chunk = ((at % (BM * 2)) >> 4) ^ ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1);
       int64_t col = m0 + chunk * 8;
       col = col < M ? col : m0;  // rows past the edge: any valid address, never stored
       a_off[j] = static_cast<uint32_t>((krow * g.lda + col) * 2);
@@ -167,7 +179,7 @@ void gemm_ring_kernel(GemmArgs g) {
       // stage bytes [group*1024 + 16*lane] = k-row (BN*2 bytes each), swizzled 16-byte slot
       const int at = (wave * B_GROUPS + j) * 1024 + lane * 16;
       const int krow = at / (BN * 2);
-      const int chunk = ((at % (BN * 2)) >> 4) ^ ((krow & 3) << 2);
+      const int chunk = ((at % (BN * 2)) >> 4) ^ ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1);
       int64_t col = n0 + chunk * 8;
       col = col < N ? col : n0;  // columns past the edge: any valid address, never stored
       b_off[j] = static_cast<uint32_t>((krow * g.ldb + col) * 2);
@@ -218,17 +230,19 @@ void gemm_ring_kernel(GemmArgs g) {
     fetch_b(stage_off, k0);
   };
 
-  f32x16_t acc[TM][TN];
+  using acc_t = std::conditional_t<MI16, f32x4v_t, f32x16_t>;
+  acc_t acc[TM][TN];
 
   // Fragment addresses as LDS byte offsets inside a stage: one per-lane register per k-step
   // (the XOR swizzle is not additive in the k chunk) and, for N-major B, per 32-column tile;
   // the 32-row tile index (and the k-step of N-major B) is an immediate offset of the ds_read.
-  const int frag_row = lane & 31, frag_half = lane >> 5;
+  // a fragment is FRAG rows; lane -> (row, which eight k of the k-step)
+  const int frag_row = lane & (FRAG - 1), frag_half = lane / FRAG;
   const int frag_swz = ring_swizzle<LINE>(frag_row);
   int a_lane[KSTEPS], b_lane[KSTEPS];
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
-    const int slot16 = ((ks * 2 + frag_half) ^ frag_swz) << 4;
+    const int slot16 = ((ks * KCHUNKS + frag_half) ^ frag_swz) << 4;
     a_lane[ks] = (wm * WM + frag_row) * LINE + slot16;
     b_lane[ks] = A_BYTES + (wn * WN + frag_row) * LINE + slot16;
   }
@@ -237,22 +251,25 @@ void gemm_ring_kernel(GemmArgs g) {
   // and lanes 32..63 the upper eight k of the MFMA step.
   int bt_lane[TN];
   if constexpr (!B_KMAJOR) {
-    const int j16 = lane & 15, q = j16 >> 2, nsub = (lane >> 4) & 1;
-    const int krow = frag_half * 8 + q;  // + 16*ks + 4*r, which leave krow % 4 == q
+    // (16-row fragments: all four groups of 16 lanes read the same 16 columns, eight k apart)
+    const int j16 = lane & 15, q = j16 >> 2, nsub = MI16 ? 0 : (lane >> 4) & 1;
+    const int krow = frag_half * 8 + q;  // + k-step and + 4, which leave krow % 4 == q
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int ncol = wn * WN + j * 32 + nsub * 16 + (j16 & 3) * 4;
-      bt_lane[j] = A_BYTES + krow * (BN * 2) + (((ncol >> 3) ^ (q << 2)) << 4) + (ncol & 7) * 2;
+      const int ncol = wn * WN + j * FRAG + nsub * 16 + (j16 & 3) * 4;
+      bt_lane[j] = A_BYTES + krow * (BN * 2) + (((ncol >> 3) ^ (q << 2) ^ ((frag_half & 1) << 1)) << 4) +
+                   (ncol & 7) * 2;
     }
   }
   int at_lane[TM];
   if constexpr (A_MMAJOR) {
-    const int j16 = lane & 15, q = j16 >> 2, msub = (lane >> 4) & 1;
+    const int j16 = lane & 15, q = j16 >> 2, msub = MI16 ? 0 : (lane >> 4) & 1;
     const int krow = frag_half * 8 + q;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int mcol = wm * WM + i * 32 + msub * 16 + (j16 & 3) * 4;
-      at_lane[i] = krow * (BM * 2) + (((mcol >> 3) ^ (q << 2)) << 4) + (mcol & 7) * 2;
+      const int mcol = wm * WM + i * FRAG + msub * 16 + (j16 & 3) * 4;
+      at_lane[i] = krow * (BM * 2) + (((mcol >> 3) ^ (q << 2) ^ ((frag_half & 1) << 1)) << 4) +
+                   (mcol & 7) * 2;
     }
   }
   typedef __attribute__((address_space(3))) u32x4_t lds_u32x4_t;
@@ -266,9 +283,9 @@ void gemm_ring_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       if constexpr (!A_MMAJOR) {
-        af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (32 * LINE));
+        af[s][i] = *(const lds_u32x4_t*)(stage + a_lane[ks] + i * (FRAG * LINE));
       } else {
-        lds_u8* src = stage + at_lane[i] + ks * 16 * (BM * 2);
+        lds_u8* src = stage + at_lane[i] + ks * (MI16 ? 32 : 16) * (BM * 2);
         const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
         const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src + 4 * (BM * 2)));
         typedef short i16x8_t __attribute__((ext_vector_type(8)));
@@ -279,9 +296,9 @@ void gemm_ring_kernel(GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if constexpr (B_KMAJOR) {
-        bf[s][j] = *(const lds_u32x4_t*)(stage_b + b_lane[ks] + j * (32 * LINE));
+        bf[s][j] = *(const lds_u32x4_t*)(stage_b + b_lane[ks] + j * (FRAG * LINE));
       } else {
-        lds_u8* src = stage_b + bt_lane[j] + ks * 16 * (BN * 2);
+        lds_u8* src = stage_b + bt_lane[j] + ks * (MI16 ? 32 : 16) * (BN * 2);
         const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src));
         const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(src + 4 * (BN * 2)));
         typedef short i16x8_t __attribute__((ext_vector_type(8)));
@@ -293,12 +310,22 @@ void gemm_ring_kernel(GemmArgs g) {
   auto load_frags = [&](uint32_t stage_off, int ks, int s) {
     load_frags2(stage_off, stage_off, ks, s);
   };
-  auto mfma_step = [&](int s) {
+  // tile rows [i0, i1) of the k-step whose fragments sit in slot s
+  auto mfma_rows = [&](int s, int i0, int i1) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = i0; i < i1; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[s][j], af[s][i], acc[i][j]);
+      for (int j = 0; j < TN; ++j) {
+        if constexpr (MI16) acc[i][j] = Mfma16<T>::run(bf[s][j], af[s][i], acc[i][j]);
+        else acc[i][j] = Mfma<T>::run(bf[s][j], af[s][i], acc[i][j]);
+      }
   };
+  auto mfma_step = [&](int s) { mfma_rows(s, 0, TM); };
+  // The barrier that ends a stage sits before the last k-step's MFMAs, which cover the LDS
+  // latency of the next stage's first fragments. With two k-steps per stage that would be the
+  // middle of the stage, and the stage requested at its start would have to land in half of
+  // it: half of the last k-step is therefore issued before the barrier.
+  constexpr int EARLY = MI16 ? TM / 2 : 0;
 
   // Ring position as a byte offset that lives in an SGPR (every wave computes the same value).
   auto next_stage = [](uint32_t off) {
@@ -323,11 +350,15 @@ void gemm_ring_kernel(GemmArgs g) {
       mfma_step(ks & 1);
       __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (EARLY > 0) {
+      mfma_rows((KSTEPS - 1) & 1, 0, EARLY);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     wait_vm_lgkm0<INFLIGHT * PER_STAGE>();
     __builtin_amdgcn_s_barrier();
     load_frags(nxt, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_step((KSTEPS - 1) & 1);
+    mfma_rows((KSTEPS - 1) & 1, EARLY, TM);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -358,7 +389,7 @@ void gemm_ring_kernel(GemmArgs g) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+        for (int e = 0; e < (MI16 ? 4 : 16); ++e) acc[i][j][e] = 0.0f;
   }
   if constexpr (SPLIT_RING) {
     // A buffer i at i * A_BYTES, B buffer j at 2 * A_BYTES + j * B_BYTES (offsets below leave out
@@ -401,11 +432,15 @@ void gemm_ring_kernel(GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
       });
       // A of the next stage is older than B of the one after it: only the latter may be pending
+      if constexpr (EARLY > 0) {
+        mfma_rows((KSTEPS - 1) & 1, 0, EARLY);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       wait_vm_lgkm0<ISSUE_B ? B_GROUPS : 0>();
       __builtin_amdgcn_s_barrier();
       load_frags2(a_n, b_n, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      mfma_step((KSTEPS - 1) & 1);
+      mfma_rows((KSTEPS - 1) & 1, EARLY, TM);
       __builtin_amdgcn_sched_barrier(0);
       a_cur = a_n;
       b_cur = b_n;
@@ -462,7 +497,8 @@ void gemm_ring_kernel(GemmArgs g) {
 
   if constexpr (OUT_F32) {
     float* P = static_cast<float*>(g.c) + batch * g.stride_c;
-    store_wave_tile_f32<TM, TN>(acc, P, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, lane);
+    if constexpr (MI16) store_wave_tile16_f32<TM, TN>(acc, P, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, lane);
+    else store_wave_tile_f32<TM, TN>(acc, P, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, lane);
     return;
   }
   const T* __restrict__ bias = static_cast<const T*>(g.bias);
@@ -474,8 +510,13 @@ void gemm_ring_kernel(GemmArgs g) {
                      wave * (ep.wide() ? BandLayoutF32<WN>::BYTES : BandLayout<WN>::BYTES);
   void* Cout = g.out_f32 ? static_cast<void*>(static_cast<float*>(g.c) + batch * g.stride_c)
                          : static_cast<void*>(C);
-  store_wave_tile<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                  g.stream_c != 0, ep, lane);
+  if constexpr (MI16) {
+    store_wave_tile16<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
+                                      g.stream_c != 0, ep, lane);
+  } else {
+    store_wave_tile<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
+                                    g.stream_c != 0, ep, lane);
+  }
   };
   // Configurations compiled for four waves per SIMD have no registers to spare for the loop
   // state; their second resident workgroup already overlaps the tile boundaries.
@@ -492,7 +533,7 @@ void gemm_ring_kernel(GemmArgs g) {
 }
 
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
-          bool A_MMAJOR = false, bool OUT_F32 = false>
+          bool A_MMAJOR = false, bool OUT_F32 = false, bool MI16_ = (BK == 64)>
 static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) {
   GemmArgs g = base;
   g.tiles_m = static_cast<int>((g.m + BM - 1) / BM);
@@ -514,7 +555,7 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
                                                                                        : resident;
   // four start phases 5 us apart when every workgroup walks several tiles of a streamed output
   g.stagger_ticks = (g.stream_c && !OUT_F32 && grid_x == resident && tiles >= 4 * resident) ? 500 : 0;
-  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR, OUT_F32>
+  gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR, OUT_F32, MI16_>
       <<<dim3(static_cast<unsigned>(grid_x), static_cast<unsigned>(batch)),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();
