@@ -416,6 +416,21 @@ void gemm_ring_kernel(GemmArgs g) {
       fetch_a(a_n, (t + 1) * BK);
       const uint32_t b_t = b_next(b_n);
       const unsigned char* bk2 = b_base + (t + 2) * BK * b_kstep;
+      if constexpr (MI16) {
+        // two k-steps of TM tile rows: B's loads go out between pairs of tile rows of the first
+        // (+2-3 % over issuing them with A's; spreading A's loads as well costs 2-3 %: they are
+        // needed at this step's barrier and want every cycle of it)
+        static_assert(B_GROUPS <= TM / 2, "one B load per pair of tile rows");
+        load_frags2(a_cur, b_cur, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<TM / 2>([&](auto r_tag) {
+          constexpr int r = decltype(r_tag)::value;
+          mfma_rows(0, 2 * r, 2 * r + 2);
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (ISSUE_B && r < B_GROUPS) dma16(b_m0 + b_t + r * 1024, b_off[r], bk2);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      } else {
       if constexpr (ISSUE_B) {
         dma16(b_m0 + b_t, b_off[0], bk2);
 #pragma unroll
@@ -431,6 +446,7 @@ void gemm_ring_kernel(GemmArgs g) {
         mfma_step(ks & 1);
         __builtin_amdgcn_sched_barrier(0);
       });
+      }
       // A of the next stage is older than B of the one after it: only the latter may be pending
       if constexpr (EARLY > 0) {
         mfma_rows((KSTEPS - 1) & 1, 0, EARLY);
