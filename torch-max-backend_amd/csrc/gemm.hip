@@ -124,8 +124,10 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
       const int64_t t256 = tiles(256, 256);
       const int64_t rounds = (t256 + 255) / 256;
       if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9) {
-        // (the 16x16x32 MFMA wins where the launch is limited by power, i.e. at long K)
-        if (g.k >= 4096)
+        // (the 16x16x32 MFMA: +3-6 % at long K, +2-4 % at K = 768 .. 3072; a short-K product
+        // whose output streams to memory, as the 50257-wide vocabulary projection, loses 4 %)
+        const bool streamed = g.m * g.n * batch * 2 >= (int64_t{256} << 20);
+        if (g.k >= 4096 || !streamed)
           return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
         return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, false>(g, batch, stream);
       }

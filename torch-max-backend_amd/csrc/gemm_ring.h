@@ -95,9 +95,10 @@ void gemm_ring_kernel(GemmArgs g) {
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   // 64-deep stages can be multiplied with v_mfma_f32_16x16x32 (two k-steps of 32 per stage; a
   // stage of 32 would be a single k-step and the fragment double buffer would change parity from
-  // stage to stage). Long products are limited by the power the chip may draw, and this form
-  // draws less per multiply-add: +3-6 % at K >= 4096. Short products (K = 768) are not, and lose
-  // 3-10 % to its doubled instruction count; the launcher picks per shape.
+  // stage to stage). Products of this size are limited by the power the chip may draw, and this
+  // form draws less per multiply-add: +3-8 % at K >= 4096, +2-4 % at K = 768 .. 3072; the
+  // launcher keeps the 32x32x16 form where it measured faster (short K with a streamed output,
+  // split-K partials).
   static_assert(!MI16_ || BK == 64, "16x16x32 needs 64-deep stages");
   constexpr bool MI16 = MI16_;
   constexpr int FRAG = MI16 ? 16 : 32;                // rows of an operand fragment
