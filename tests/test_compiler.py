@@ -489,6 +489,8 @@ def test_training_partition_replaces_attention_forward_and_backward(monkeypatch)
             if isinstance(val, torch.Tensor) and val.dim() >= 3:
                 assert tuple(val.shape[-2:]) != (8, 8), n.name
     assert count(plain[1], aten.bmm.default) == 8  # PyTorch's split: four per block
+    # the gradient of the packed q/k/v projection comes out of the backward step as one tensor
+    assert count(plain[1], aten.cat.default) == 2 and count(bw, aten.cat.default) == 0
 
 
 def test_training_partition_recomputes_attention_scores_and_forward_fuses(monkeypatch):

@@ -820,14 +820,25 @@ def attention_train_backward(grad_out, q, k, v, out, lse, scale, root, slices, l
     """(dq, dk, dv), each [batch, heads, tokens, head_dim], from the gradient of
     attention_train_forward's `out` (same [batch, tokens, heads, head_dim] layout). `layouts`:
     per gradient, the strides the consumers in the graph were traced with, or None where the
-    token-major layout the kernels write by themselves serves those consumers as well."""
+    token-major layout the kernels write by themselves serves those consumers as well; or the
+    string "packed": the three are views of one [batch, tokens, 3 * heads * head_dim] tensor,
+    returned as a fourth result, which is what the graph's concatenation of the three (the
+    backward of the split of a packed q/k/v projection) would have produced."""
     from torch_mojo_backend.eager_kernels import hip_ops
 
     b, h, t, d = q.shape
     s_len = k.shape[2]
+    packed = isinstance(layouts, str)
     if _attention_fused_ok(q, k, v, scale, root, slices):
         g = grad_out if grad_out.stride(3) == 1 and grad_out.data_ptr() % 16 == 0 and \
             all(st % 8 == 0 for st in grad_out.stride()[:3]) else grad_out.contiguous()
+        if packed:
+            dq, dk, dv = hip_ops.attention_backward(g.transpose(1, 2), q, k, v,
+                                                    out.transpose(1, 2), lse, scale, True,
+                                                    packed=True)
+            # dq is buf[:, :, 0].transpose(1, 2) of the [b, t, 3, h, d] buffer
+            whole = dq.as_strided((b, t, 3 * h * d), (3 * t * h * d, 3 * h * d, 1))
+            return dq, dk, dv, whole
         grads = hip_ops.attention_backward(g.transpose(1, 2), q, k, v, out.transpose(1, 2), lse,
                                            scale, True, grad_strides=layouts)
         return tuple(_in_layout(x, lay) if lay is not None else x for x, lay in zip(grads, layouts))
@@ -841,6 +852,12 @@ def attention_train_backward(grad_out, q, k, v, out, lse, scale, root, slices, l
     dq = _BUILTIN_BMM(ds, flat(k))
     dk = _BUILTIN_BMM(ds.transpose(1, 2), flat(q))
     grads = (dq.view(b, h, t, d), dk.view(b, h, s_len, d), dv.view(b, h, s_len, d))
+    if packed:
+        buf = torch.empty((b, t, 3, h, d), dtype=q.dtype, device=q.device)
+        for i, x in enumerate(grads):
+            buf[:, :, i].copy_(x.transpose(1, 2))
+        views = tuple(buf[:, :, i].transpose(1, 2) for i in range(3))
+        return (*views, buf.view(b, t, 3 * h * d))
     return tuple(_in_layout(x, lay) for x, lay in zip(grads, layouts))
 
 
@@ -1174,9 +1191,59 @@ def _fuse_attention_backward(joint_module: torch.fx.GraphModule, match) -> bool:
     final.replace_all_uses_with(out)
     for i, name in enumerate("qkv"):
         owner[name].replace_all_uses_with(grads[i], delete_user_cb=lambda u: u not in inside)
+    cat = _packed_gradient_cat(grads, (b, t, h * d))
+    if cat is not None:
+        # the three gradients are only ever concatenated: written into one buffer instead
+        bwd.args = (*bwd.args[:-1], "packed")
+        bwd.meta["val"] = (*vals, cat.meta["val"])
+        with graph.inserting_after(grads[-1]):
+            whole = tagged(graph.call_function(operator.getitem, (bwd, 3)), cat.meta["val"],
+                           "is_backward", first_result)
+        cat.replace_all_uses_with(whole)
     graph.eliminate_dead_code()
     joint_module.recompile()
     return True
+
+
+def _packed_gradient_cat(grads, flat_shape):
+    """The aten.cat node that joins dq, dk and dv (in this order, along the last dimension, each
+    as [batch, tokens, heads * head_dim]) when that is all the graph does with them: each goes
+    through transpose(1, 2) and copies / reshapes that every node of has a single user. None
+    otherwise."""
+    ends = []
+    for g in grads:
+        users = list(g.users)
+        if len(users) != 1 or users[0].target is not aten.transpose.int or \
+                {x % 4 for x in users[0].args[1:3]} != {1, 2}:
+            return None
+        node = users[0]
+        while True:
+            users = list(node.users)
+            if len(users) != 1:
+                return None
+            nxt = users[0]
+            if nxt.target in (aten.clone.default, aten.view.default, aten._unsafe_view.default,
+                              aten.reshape.default):
+                node = nxt
+                continue
+            if nxt.target is aten.cat.default:
+                ends.append((node, nxt))
+                break
+            return None
+    cat = ends[0][1]
+    if any(c is not cat for _, c in ends):
+        return None
+    dim = cat.args[1] if len(cat.args) > 1 else cat.kwargs.get("dim", 0)
+    if list(cat.args[0]) != [e for e, _ in ends] or not isinstance(dim, int) or dim % 3 != 2:
+        return None
+    for e, _ in ends:
+        val = e.meta.get("val")
+        if val is None or tuple(val.shape) != tuple(flat_shape):
+            return None
+    cval = cat.meta.get("val")
+    if cval is None or cval.dim() != 3 or not cval.is_contiguous():
+        return None
+    return cat
 
 
 def _tag_attention_for_recompute(joint_module: torch.fx.GraphModule, num_fwd_outputs: int) -> list:
