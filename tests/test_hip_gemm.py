@@ -87,6 +87,30 @@ def test_mm_fp32(mnk):
     assert_close64(got, want, extra_abs=bound, what=f"mm fp32 {mnk}")
 
 
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", [(4096, 4096, 4096), (7000, 7096, 4096), (4000, 4104, 4096),
+                                 (2100, 3000, 768)])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_addmm_half_long_k_ragged_tiles(mnk, dtype, trans_b):
+    """Products that run on the 64-deep ring configurations with the 16x16x32 MFMA (256x256x64 and
+    256x128x64), in both storage types, with whole and with ragged edge tiles: rows sampled from
+    the first, the last and the interior tiles against float64, every column."""
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(7)
+    a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
+    b = torch.randn(k, n, generator=g, device="cuda").to(dtype)
+    if trans_b:
+        b = b.t().contiguous().t()
+    bias = torch.randn(n, generator=g, device="cuda").to(dtype)
+    got = _ops().gemm(a, b, bias)
+    rows = torch.cat([torch.arange(0, 40), torch.arange(m - 40, m),
+                      torch.randperm(m, generator=torch.Generator().manual_seed(2))[:48]]).to("cuda")
+    want = (a[rows].cpu().double() @ b.cpu().double() + bias.cpu().double()).numpy()
+    assert rel_frobenius(got[rows], want) <= 1e-2
+    assert_close64(got[rows], want, rtol=2e-5, atol=2e-3, what=f"rows of {mnk} {dtype}")
+    assert torch.equal(got, _ops().gemm(a, b, bias))
+
+
 @pytest.mark.parametrize("mnk", [(4096, 4096, 4096), (8192, 8192, 8192)])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_addmm_bf16_large_sampled_rows(mnk, trans_b):
@@ -391,6 +415,27 @@ def test_mm_transposed_a(mnk, dtype):
     # every element, not just the norm: fp32 accumulation + one rounding to the storage type
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     assert np.abs(as64(got) - want).max() <= ulp * np.abs(want).max() + 1e-3
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", [(16392, 768, 2048), (8200, 3072, 1024)])
+def test_mm_transposed_a_many_tiles(mnk, dtype):
+    """Enough 256 x 256 tiles for the unsplit 64-deep ring with both operands staged k-outer
+    (the vocabulary projection's weight gradient): sampled rows, every column, against float64;
+    the last tile row is ragged."""
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a_km = torch.randn(k, m, generator=g, device="cuda").to(dtype)
+    b = torch.randn(k, n, generator=g, device="cuda").to(dtype)
+    got = _ops().gemm(a_km.t(), b)
+    assert got.dtype == dtype and tuple(got.shape) == (m, n)
+    rows = torch.cat([torch.arange(0, 33), torch.arange(m - 33, m),
+                      torch.randperm(m, generator=torch.Generator().manual_seed(3))[:40]]).to("cuda")
+    want = (a_km[:, rows].cpu().double().t() @ b.cpu().double()).numpy()
+    assert rel_frobenius(got[rows], want) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert np.abs(as64(got[rows]) - want).max() <= ulp * np.abs(want).max() + 1e-3
+    assert torch.equal(got, _ops().gemm(a_km.t(), b))
 
 
 def test_mm_transposed_a_batched_and_strided():
