@@ -293,6 +293,20 @@ def main() -> int:
             row["cpu_note"] = t[2]
         sweep[name] = row
 
+    def with_copy(name, nbuf, ptrs, nbytes):
+        """Beside a row-wise kernel's row: tmb_copy_bytes over the same buffers (the same bytes
+        read and written by a kernel that does nothing else), timed in the same run."""
+        state = {"i": 0}
+
+        def step():
+            o, x = ptrs[state["i"] % nbuf]
+            lib.tmb_copy_bytes(o, x, nbytes, stream)
+            state["i"] += 1
+
+        _, ms = timed(step, 40, 8)
+        sweep[name]["copy_us_same_bytes"] = round(ms * 1e3, 2)
+        sweep[name]["vs_copy"] = round(ms * 1e3 / sweep[name]["us"], 3)
+
     if want in ("all", "attn"):
         # attention of the GPT-2 workload (B=32, H=12, T=1024, head_dim 64, bf16), q/k/v as the
         # strided thirds of the packed projection, exactly as the compiled graph hands them over
@@ -382,6 +396,7 @@ def main() -> int:
                         2 * nbytes, steps=20 if nbytes > 3e9 else 40, cpu_fn=cpu_softmax)
                 # spot-check the raw launch against the tensor-level op
                 assert torch.equal(outs[0], hip_ops.softmax(bufs[0], -1))
+                with_copy(f"softmax_{dn}_{rows}x{cols}", len(bufs), ptrs, nbytes)
                 del bufs, outs
             for (rows, cols) in ((32768, 768), (16384, 4096)):
                 nbytes = rows * cols * es
@@ -406,6 +421,7 @@ def main() -> int:
                                                           rows, cols, 1e-5, code, code, stream),
                         2 * nbytes + 2 * cols * es + 2 * rows * 4, cpu_fn=cpu_ln)
                 assert torch.equal(outs[0], hip_ops.layer_norm(bufs[0], [cols], g_, b_, 1e-5)[0])
+                with_copy(f"layer_norm_{dn}_{rows}x{cols}", len(bufs), ptrs, nbytes)
                 del bufs, outs
 
     if want in ("all", "reduce"):
