@@ -534,6 +534,45 @@ def test_training_partition_recomputes_attention_scores_and_forward_fuses(monkey
     assert sum(1 for p in bw_rewrites.values() if p is not None and p[0] == "softmax") == 2
 
 
+def test_training_partition_packs_gradients_only_for_a_packed_projection(monkeypatch):
+    """Separate q, k and v projections: the backward step is still put in, but there is no
+    concatenation of its three results to replace, so they come back as three tensors; the
+    gradients are those of PyTorch's own split."""
+    from demo_scripts.gpt2 import seeded_tokens
+    from torch._functorch.partitioners import default_partition
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            torch.manual_seed(0)
+            self.emb = torch.nn.Embedding(64, 128)
+            self.q, self.k, self.v = (torch.nn.Linear(128, 128) for _ in range(3))
+            self.head = torch.nn.Linear(128, 64)
+            self.register_buffer("mask", torch.tril(torch.ones(8, 8)).view(1, 1, 8, 8))
+
+        def forward(self, idx):
+            x = self.emb(idx)
+            b, t, c = x.shape
+            q, k, v = (m(x).view(b, t, 2, 64).transpose(1, 2) for m in (self.q, self.k, self.v))
+            att = (q @ k.transpose(-2, -1)) * 0.125
+            att = torch.softmax(att.masked_fill(self.mask[:, :, :t, :t] == 0, float("-inf")), dim=-1)
+            y = (att @ v).transpose(1, 2).contiguous().view(b, t, c)
+            return self.head(y), None
+
+    _host_attention_pieces(monkeypatch)
+    idx, targets = seeded_tokens(2, 8, seed=0) % 64, seeded_tokens(2, 8, seed=1) % 64
+    make = lambda: Block().bfloat16()  # noqa: E731
+    _, want = _partitioned_training_graphs(make(), idx, targets, default_partition)
+    (fw, bw), got = _partitioned_training_graphs(make(), idx, targets,
+                                                 compiler.attention_recompute_partition)
+    for g, w in zip(got, want):
+        scale = w.float().abs().max().item() + 1e-12
+        assert (g.float() - w.float()).abs().max().item() <= 3e-2 * scale
+    steps = [n for n in bw.graph.nodes if n.target is compiler.attention_train_backward]
+    assert len(steps) == 1 and not isinstance(steps[0].args[-1], str)
+    assert {u.args[1] for u in steps[0].users} == {0, 1, 2}
+
+
 def test_training_partition_leaves_graphs_without_attention_alone():
     from torch._functorch.partitioners import default_partition
 
