@@ -134,8 +134,17 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
       if (tiles(256, 128) >= 512)
         return launch_ring<T, 256, 128, 64, 4, 2, 3, B_KMAJOR, EPI>(g, batch, stream);
     }
-    if (g.k % 32 == 0 && tiles(128, 128) >= 32)
+    if (g.k % 32 == 0 && tiles(128, 128) >= 32) {
+      // (16x16x32 MFMA, one k-step per 32-deep stage: +5-7 % for K-major B once the launch has
+      // a few rounds of tiles; level or behind for small launches and for N-major B, whose
+      // fragments need twice the LDS instructions; the 32-deep configurations that run four
+      // waves per SIMD have no registers for its fragments at all)
+      if constexpr (B_KMAJOR) {
+        if (tiles(128, 128) >= 512)
+          return launch_ring<T, 128, 128, 32, 2, 2, 4, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
+      }
       return launch_ring<T, 128, 128, 32, 2, 2, 4, B_KMAJOR, EPI>(g, batch, stream);
+    }
   }
   // Register-staged kernel for the rest (short K, K not a multiple of 32, ragged N-major N).
   if (g.n <= 64) return launch_mfma<T, 256, 64, 4, 1, B_KMAJOR, EPI>(g, batch, stream);

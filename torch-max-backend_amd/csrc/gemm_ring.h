@@ -99,7 +99,8 @@ void gemm_ring_kernel(GemmArgs g) {
   // form draws less per multiply-add: +3-8 % at K >= 4096, +2-4 % at K = 768 .. 3072; the
   // launcher keeps the 32x32x16 form where it measured faster (short K with a streamed output,
   // split-K partials).
-  static_assert(!MI16_ || BK == 64, "16x16x32 needs 64-deep stages");
+  static_assert(!MI16_ || BK == 64 || !(R == 2 && BM == 256 && BN == 256),
+                "the split ring is 64 deep");
   constexpr bool MI16 = MI16_;
   constexpr int FRAG = MI16 ? 16 : 32;                // rows of an operand fragment
   constexpr int TM = WM / FRAG, TN = WN / FRAG;       // result tiles per wave
@@ -339,27 +340,32 @@ void gemm_ring_kernel(GemmArgs g) {
   // for. sched_barrier(0): nothing is scheduled across. Left alone, the scheduler sinks each
   // fragment load to just before its MFMA and reuses one register for all of them, which puts
   // the LDS latency back on the critical path.
+  // P: the fragment slot the stage's first k-step sits in. With an even number of k-steps per
+  // stage it is always 0; a 32-deep stage multiplied with 16x16x32 is a single k-step, so the
+  // slot alternates from stage to stage and the loops below run the steps in pairs.
   auto step = [&](uint32_t cur, uint32_t nxt, uint32_t pre, int64_t k_pre, auto issue_tag,
-                  auto inflight_tag) {
+                  auto inflight_tag, auto parity_tag) {
     constexpr bool ISSUE = decltype(issue_tag)::value;
     constexpr int INFLIGHT = decltype(inflight_tag)::value;
+    constexpr int P = decltype(parity_tag)::value;
     if constexpr (ISSUE) fetch_stage(pre, k_pre);
     static_for<KSTEPS - 1>([&](auto ks_tag) {
       constexpr int ks = decltype(ks_tag)::value;
-      load_frags(cur, ks + 1, (ks + 1) & 1);
+      load_frags(cur, ks + 1, (P + ks + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);
-      mfma_step(ks & 1);
+      mfma_step((P + ks) & 1);
       __builtin_amdgcn_sched_barrier(0);
     });
+    constexpr int LAST = (P + KSTEPS - 1) & 1;
     if constexpr (EARLY > 0) {
-      mfma_rows((KSTEPS - 1) & 1, 0, EARLY);
+      mfma_rows(LAST, 0, EARLY);
       __builtin_amdgcn_sched_barrier(0);
     }
     wait_vm_lgkm0<INFLIGHT * PER_STAGE>();
     __builtin_amdgcn_s_barrier();
-    load_frags(nxt, 0, 0);
+    load_frags(nxt, 0, (P + KSTEPS) & 1);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_rows((KSTEPS - 1) & 1, EARLY, TM);
+    mfma_rows(LAST, EARLY, TM);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -487,29 +493,52 @@ void gemm_ring_kernel(GemmArgs g) {
   load_frags(0, 0, 0);
   uint32_t cur = 0, pre = (R - 1) * STAGE_BYTES;
   // main part: every step also requests tile t+R-1
-#pragma unroll 1
-  for (int64_t t = 0; t + (R - 1) < k_tiles; ++t) {
+  auto main_step = [&](int64_t t, auto parity_tag) {
     const uint32_t nxt = next_stage(cur);
     step(cur, nxt, pre, (t + (R - 1)) * BK, std::true_type{},
-         std::integral_constant<int, R - 2>{});
+         std::integral_constant<int, R - 2>{}, parity_tag);
     pre = cur;
     cur = nxt;
-  }
+  };
   // the last R-1 tiles are already in flight or resident; the in-flight count runs down
-  static_for<R - 2>([&](auto s) {
-    const uint32_t nxt = next_stage(cur);
-    step(cur, nxt, pre, 0, std::false_type{}, std::integral_constant<int, R - 3 - decltype(s)::value>{});
-    pre = cur;
-    cur = nxt;
-  });
-  static_for<KSTEPS - 1>([&](auto ks_tag) {
-    constexpr int ks = decltype(ks_tag)::value;
-    load_frags(cur, ks + 1, (ks + 1) & 1);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_step(ks & 1);
-    __builtin_amdgcn_sched_barrier(0);
-  });
-  mfma_step((KSTEPS - 1) & 1);
+  auto finish = [&](auto parity_tag) {
+    constexpr int P0 = decltype(parity_tag)::value;
+    static_for<R - 2>([&](auto s) {
+      constexpr int P = (P0 + decltype(s)::value * KSTEPS) & 1;
+      const uint32_t nxt = next_stage(cur);
+      step(cur, nxt, pre, 0, std::false_type{},
+           std::integral_constant<int, R - 3 - decltype(s)::value>{}, std::integral_constant<int, P>{});
+      pre = cur;
+      cur = nxt;
+    });
+    constexpr int P = (P0 + (R - 2) * KSTEPS) & 1;
+    static_for<KSTEPS - 1>([&](auto ks_tag) {
+      constexpr int ks = decltype(ks_tag)::value;
+      load_frags(cur, ks + 1, (P + ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step((P + ks) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    mfma_step((P + KSTEPS - 1) & 1);
+  };
+  if constexpr (KSTEPS % 2 == 0) {
+#pragma unroll 1
+    for (int64_t t = 0; t + (R - 1) < k_tiles; ++t) main_step(t, std::integral_constant<int, 0>{});
+    finish(std::integral_constant<int, 0>{});
+  } else {
+    int64_t t = 0;
+#pragma unroll 1
+    for (; t + R < k_tiles; t += 2) {
+      main_step(t, std::integral_constant<int, 0>{});
+      main_step(t + 1, std::integral_constant<int, 1>{});
+    }
+    if (t + (R - 1) < k_tiles) {  // wave-uniform
+      main_step(t, std::integral_constant<int, 0>{});
+      finish(std::integral_constant<int, 1>{});
+    } else {
+      finish(std::integral_constant<int, 0>{});
+    }
+  }
   }  // whole-stage ring
 
   if constexpr (OUT_F32) {
