@@ -539,7 +539,9 @@ def main() -> int:
         for name, fn, fl in (
                 ("linear_backward_dgrad_bf16_32768x768x3072", lambda: hip_ops.gemm(dy, wt), 2.0 * rows_ * in_f * out_f),
                 ("linear_backward_wgrad_bf16_3072x768x32768", lambda: hip_ops.gemm(dy.t(), xin), 2.0 * rows_ * in_f * out_f)):
-            _, ms = timed(fn, 30, 8)
+            # (long enough for the clock to settle: the first launches after the memory-bound
+            # rows above run 20-30 % slower than the steady state)
+            _, ms = timed(fn, 80, 40)
             sweep[name] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(fl / ms / 1e9, 2),
                            "frac_mfma": round(fl / ms / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4)}
         del dy, xin, wt

@@ -112,8 +112,9 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
     // Short K: the prologue and epilogue of a tile weigh as much as its main loop, so rings that
     // leave room for two workgroups per CU (72 KB of LDS each) win by overlapping them.
     if (g.k % 32 == 0) {
+      // (with the 16x16x32 MFMA and one fragment slot: four waves per SIMD, +2-4 %)
       if (!B_KMAJOR && g.k < 4096 && tiles(128, 256) >= 256)
-        return launch_ring<T, 128, 256, 32, 2, 4, 3, B_KMAJOR, EPI>(g, batch, stream);
+        return launch_ring<T, 128, 256, 32, 2, 4, 3, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
       // (with at least three rounds of 256 x 256 tiles the big tile's reuse wins again:
       // 32768 x 2304 x 768 runs in 118-127 us there against 136-144 us here)
       if (B_KMAJOR && g.k <= 1024 && g.n <= 2304 && tiles(256, 128) >= 512 &&

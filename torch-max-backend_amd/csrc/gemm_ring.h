@@ -328,6 +328,11 @@ void gemm_ring_kernel(GemmArgs g) {
   // middle of the stage, and the stage requested at its start would have to land in half of
   // it: half of the last k-step is therefore issued before the barrier.
   constexpr int EARLY = MI16 ? TM / 2 : 0;
+  // Four waves per SIMD leave a wave 128 registers, which the accumulators and two slots of
+  // 16-row fragments exceed: such a configuration keeps one slot (the other waves of the SIMD
+  // cover the LDS latency after the barrier).
+  constexpr bool SINGLE_SLOT =
+      MI16 && KSTEPS == 1 && ring_waves_per_simd(BM, BN, BK, WAVES_M * WAVES_N, R) >= 4;
 
   // Ring position as a byte offset that lives in an SGPR (every wave computes the same value).
   auto next_stage = [](uint32_t off) {
@@ -349,6 +354,15 @@ void gemm_ring_kernel(GemmArgs g) {
     constexpr int INFLIGHT = decltype(inflight_tag)::value;
     constexpr int P = decltype(parity_tag)::value;
     if constexpr (ISSUE) fetch_stage(pre, k_pre);
+    if constexpr (SINGLE_SLOT) {
+      mfma_step(0);
+      __builtin_amdgcn_sched_barrier(0);
+      wait_vm_lgkm0<INFLIGHT * PER_STAGE>();
+      __builtin_amdgcn_s_barrier();
+      load_frags(nxt, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
     static_for<KSTEPS - 1>([&](auto ks_tag) {
       constexpr int ks = decltype(ks_tag)::value;
       load_frags(cur, ks + 1, (P + ks + 1) & 1);
@@ -511,7 +525,7 @@ void gemm_ring_kernel(GemmArgs g) {
       pre = cur;
       cur = nxt;
     });
-    constexpr int P = (P0 + (R - 2) * KSTEPS) & 1;
+    constexpr int P = SINGLE_SLOT ? 0 : (P0 + (R - 2) * KSTEPS) & 1;
     static_for<KSTEPS - 1>([&](auto ks_tag) {
       constexpr int ks = decltype(ks_tag)::value;
       load_frags(cur, ks + 1, (P + ks + 1) & 1);
@@ -521,7 +535,7 @@ void gemm_ring_kernel(GemmArgs g) {
     });
     mfma_step((P + KSTEPS - 1) & 1);
   };
-  if constexpr (KSTEPS % 2 == 0) {
+  if constexpr (KSTEPS % 2 == 0 || SINGLE_SLOT) {
 #pragma unroll 1
     for (int64_t t = 0; t + (R - 1) < k_tiles; ++t) main_step(t, std::integral_constant<int, 0>{});
     finish(std::integral_constant<int, 0>{});
