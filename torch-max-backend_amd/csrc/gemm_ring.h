@@ -84,7 +84,7 @@ constexpr bool kRingPersistent = ring_waves_per_simd(BM, BN, BK, WAVES, R) <= 2;
 // product dy^T x); it is then staged and read exactly like N-major B.
 // OUT_F32: a split-K launch: the batch index is the split, the accumulators are stored as fp32
 // partials (no bias, no epilogue, no cast).
-// MI16_: multiply with v_mfma_f32_16x16x32 (64-deep stages only).
+// MI16_: multiply with v_mfma_f32_16x16x32 instead of v_mfma_f32_32x32x16.
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int R, bool B_KMAJOR, int EPI,
           bool A_MMAJOR = false, bool OUT_F32 = false, bool MI16_ = (BK == 64)>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
@@ -93,12 +93,12 @@ void gemm_ring_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  // 64-deep stages can be multiplied with v_mfma_f32_16x16x32 (two k-steps of 32 per stage; a
-  // stage of 32 would be a single k-step and the fragment double buffer would change parity from
-  // stage to stage). Products of this size are limited by the power the chip may draw, and this
-  // form draws less per multiply-add: +3-8 % at K >= 4096, +2-4 % at K = 768 .. 3072; the
-  // launcher keeps the 32x32x16 form where it measured faster (short K with a streamed output,
-  // split-K partials).
+  // v_mfma_f32_16x16x32 takes k-steps of 32: two per 64-deep stage, one per 32-deep stage (the
+  // fragment slots then alternate from stage to stage, or there is only one, see below). Large
+  // products are limited by the power the chip may draw, and this form draws less per
+  // multiply-add: +3-8 % at K >= 4096, +2-4 % at K = 768 .. 3072; the launcher keeps the
+  // 32x32x16 form where it measured faster (short K with a streamed output, split-K partials,
+  // small launches, N-major B on the 128 x 128 x 32 tile).
   static_assert(!MI16_ || BK == 64 || !(R == 2 && BM == 256 && BN == 256),
                 "the split ring is 64 deep");
   constexpr bool MI16 = MI16_;
