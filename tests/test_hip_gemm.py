@@ -89,12 +89,17 @@ def test_mm_fp32(mnk):
 
 @pytest.mark.parametrize("dtype", HALF)
 @pytest.mark.parametrize("mnk", [(4096, 4096, 4096), (7000, 7096, 4096), (4000, 4104, 4096),
-                                 (2100, 3000, 768)])
+                                 (2100, 3000, 768),
+                                 # 32-deep stages as single k-steps: alternating fragment slots with an
+                                 # odd and an even number of steps, and the one-slot configuration
+                                 (2048, 4096, 2048), (2048, 4096, 1056), (2000, 4104, 1056),
+                                 (5000, 9000, 1024)])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_addmm_half_long_k_ragged_tiles(mnk, dtype, trans_b):
-    """Products that run on the 64-deep ring configurations with the 16x16x32 MFMA (256x256x64 and
-    256x128x64), in both storage types, with whole and with ragged edge tiles: rows sampled from
-    the first, the last and the interior tiles against float64, every column."""
+    """Products that run on the ring configurations with the 16x16x32 MFMA (256x256x64, 256x128x64,
+    128x128x32 with K-major B, 128x256x32 with N-major B), in both storage types, with whole and
+    with ragged edge tiles: rows sampled from the first, the last and the interior tiles against
+    float64, every column."""
     m, n, k = mnk
     g = torch.Generator(device="cuda").manual_seed(7)
     a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
