@@ -93,12 +93,15 @@ def test_mm_fp32(mnk):
                                  # 32-deep stages as single k-steps: alternating fragment slots with an
                                  # odd and an even number of steps, and the one-slot configuration
                                  (2048, 4096, 2048), (2048, 4096, 1056), (2000, 4104, 1056),
-                                 (5000, 9000, 1024)])
+                                 (5000, 9000, 1024),
+                                 # one partial round of 256 x 256 tiles; 256 x 128 tiles with 32-deep
+                                 # stages (K-major B, K an odd multiple of 32)
+                                 (3000, 3400, 2048), (16500, 1000, 992)])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_addmm_half_long_k_ragged_tiles(mnk, dtype, trans_b):
     """Products that run on the ring configurations with the 16x16x32 MFMA (256x256x64, 256x128x64,
-    128x128x32 with K-major B, 128x256x32 with N-major B), in both storage types, with whole and
-    with ragged edge tiles: rows sampled from the first, the last and the interior tiles against
+    128x128x32 with K-major B, 128x256x32 with N-major B) and on their 32x32x16 neighbours in the
+    tile choice, in both storage types, with whole and with ragged edge tiles: rows sampled from the first, the last and the interior tiles against
     float64, every column."""
     m, n, k = mnk
     g = torch.Generator(device="cuda").manual_seed(7)

@@ -109,20 +109,26 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
   // the idle tail. N-major B is staged in whole 16-byte column chunks, so N must be a multiple
   // of 8 there (nothing past column N-1 is ever read).
   if (g.k >= 256 && g.n > 64 && (B_KMAJOR || g.n % 8 == 0)) {
+    const int64_t t256 = tiles(256, 256);
+    // One partial round of 256 x 256 tiles (at least 144 of the 256 CUs busy) still beats smaller
+    // tiles in several rounds: 16384 x 768 x 3072 runs in 66-72 us so, against 76-88 us with the
+    // best smaller tile. (The 16x16x32 MFMA helps there from K = 2048 on and for K-major B only.)
+    if (g.k % 64 == 0 && t256 >= 144 && t256 <= 256 && t256 * 10 < 256 * 9) {
+      if (B_KMAJOR && g.k >= 2048)
+        return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
+      return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, false>(g, batch, stream);
+    }
     // Short K: the prologue and epilogue of a tile weigh as much as its main loop, so rings that
     // leave room for two workgroups per CU (72 KB of LDS each) win by overlapping them.
     if (g.k % 32 == 0) {
       // (with the 16x16x32 MFMA and one fragment slot: four waves per SIMD, +2-4 %)
       if (!B_KMAJOR && g.k < 4096 && tiles(128, 256) >= 256)
         return launch_ring<T, 128, 256, 32, 2, 4, 3, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
-      // (with at least three rounds of 256 x 256 tiles the big tile's reuse wins again:
-      // 32768 x 2304 x 768 runs in 118-127 us there against 136-144 us here)
-      if (B_KMAJOR && g.k <= 1024 && g.n <= 2304 && tiles(256, 128) >= 512 &&
-          !(g.k % 64 == 0 && tiles(256, 256) >= 768))
+      // (K not a multiple of 64 only: the 64-deep form of this tile below is 5-10 % faster)
+      if (B_KMAJOR && g.k % 64 != 0 && g.k <= 1024 && g.n <= 2304 && tiles(256, 128) >= 512)
         return launch_ring<T, 256, 128, 32, 4, 2, 3, B_KMAJOR, EPI>(g, batch, stream);
     }
     if (g.k % 64 == 0) {
-      const int64_t t256 = tiles(256, 256);
       const int64_t rounds = (t256 + 255) / 256;
       if (t256 >= 768 || t256 * 10 >= rounds * 256 * 9) {
         // (the 16x16x32 MFMA: +3-6 % at long K, +2-4 % at K = 768 .. 3072; a short-K product
@@ -132,7 +138,9 @@ static int mfma_pick_tile(const GemmArgs& g, int64_t batch, hipStream_t stream) 
           return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, true>(g, batch, stream);
         return launch_ring<T, 256, 256, 64, 2, 4, 2, B_KMAJOR, EPI, false, false, false>(g, batch, stream);
       }
-      if (tiles(256, 128) >= 512)
+      // (from three quarters of a round on: 8192 x 768 x 3072 runs in 39-42 us here against
+      // 50-55 us with 128 x 128 tiles)
+      if (tiles(256, 128) >= 192)
         return launch_ring<T, 256, 128, 64, 4, 2, 3, B_KMAJOR, EPI>(g, batch, stream);
     }
     if (g.k % 32 == 0 && tiles(128, 128) >= 32) {
