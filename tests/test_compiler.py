@@ -271,6 +271,59 @@ def test_intermediates_are_released_after_their_last_use():
     assert program.steps[-1].out not in released
 
 
+def test_padded_copies_are_shared_only_inside_a_graph_run(monkeypatch):
+    """The padded copy of a large operand is kept for the next product only while the run-scoped
+    dictionary exists: same memory, shape, strides and width give the same copy; anything else,
+    and every call outside a run, makes a new one."""
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    monkeypatch.setattr(hip_ops, "_PAD_REUSE_MIN_BYTES", 1 << 10)
+    x = torch.randn(64, 33)
+    a, b = hip_ops._pad_last(x, 40), hip_ops._pad_last(x, 40)
+    assert a is not b and torch.equal(a, b) and a.shape == (64, 40)
+    assert torch.equal(a[:, :33], x) and bool((a[:, 33:] == 0).all())
+    monkeypatch.setattr(hip_ops, "_PAD_REUSE", {})
+    a = hip_ops._pad_last(x, 40)
+    assert hip_ops._pad_last(x.t().t(), 40) is a          # another view of the same rows
+    assert hip_ops._pad_last(x[:32], 40) is not a         # other shape
+    assert hip_ops._pad_last(x, 40) is not a              # one entry: the narrower view replaced it
+    c = hip_ops._pad_last(x, 48)
+    assert c.shape == (64, 48) and hip_ops._pad_last(x, 48) is c
+    small = torch.randn(4, 33)
+    assert hip_ops._pad_last(small, 40) is not hip_ops._pad_last(small, 40)
+    (kept_source, kept_copy), = hip_ops._PAD_REUSE.values()
+    assert kept_source is x and kept_copy is c
+
+
+def test_graph_runs_share_padded_copies_unless_a_node_writes_in_place(cpu_hot_ops):
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    seen = []
+
+    def spy(a, b):
+        seen.append(hip_ops._PAD_REUSE)
+        return torch.mm(a, b)
+
+    MAPPING_TORCH_ATEN_TO_MOJO[aten.mm] = spy  # (the fixture restores the entry)
+    x, w = torch.randn(4, 6), torch.randn(6, 6)
+    pure = make_fx(lambda x, w: torch.mm(torch.mm(x, w), w))(x, w)
+    run = compiler.BaseMaxCompiler(pure, [x, w])
+    assert run.pad_reuse_module is hip_ops
+    out, = run(x, w)
+    assert torch.allclose(out, x @ w @ w)
+    assert seen == [{}, {}] and seen[0] is seen[1] and hip_ops._PAD_REUSE is None
+    one = make_fx(lambda x, w: torch.mm(x, w))(x, w)
+    assert compiler.BaseMaxCompiler(one, [x, w]).pad_reuse_module is None
+
+    def writes(x, w):
+        y = torch.mm(x, w)
+        torch.add(y, 1.0, out=y)
+        return torch.mm(y, w)
+
+    assert compiler.BaseMaxCompiler(make_fx(writes)(x, w), [x, w]).pad_reuse_module is None
+
+
 class _Attn(torch.nn.Module):
     """Score pipeline of a decoder block, as demo_scripts/gpt2.py writes it."""
 

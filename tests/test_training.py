@@ -13,7 +13,8 @@ pytestmark = pytest.mark.gpu
 CHECKS = ["gpt2_training_step_gradients_match_cpu", "training_graph_runs_the_fused_attention_forward_and_backward",
           "sdpa_training_graph_runs_the_fused_forward_and_backward",
           "one_sgd_step_lowers_the_loss",
-          "log_softmax_and_linear_backward_in_a_compiled_graph"]
+          "log_softmax_and_linear_backward_in_a_compiled_graph",
+          "vocabulary_projection_backward_pads_its_gradient_once"]
 
 
 @pytest.mark.parametrize("check", CHECKS)

@@ -189,6 +189,48 @@ def log_softmax_and_linear_backward_in_a_compiled_graph():
         torch.testing.assert_close(got.cpu(), ref, rtol=1e-4, atol=1e-5)
 
 
+def vocabulary_projection_backward_pads_its_gradient_once():
+    """Both products of a 50257-wide projection's backward pass (the input gradient contracts
+    over the vocabulary, the weight gradient has it as its transposed dimension) need the incoming
+    gradient in rows of whole 16-byte vectors: one padded copy serves both, and the gradients
+    still match float64 on the host."""
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    torch.manual_seed(0)
+    rows, hidden, vocab = 1024, 256, 50257
+    w = (torch.randn(vocab, hidden) * 0.05).bfloat16()
+    x = torch.randn(rows, hidden).bfloat16()
+    g = (torch.randn(rows, vocab) * 0.1).bfloat16()
+
+    def fn(inp, weight, grad):
+        return ((inp @ weight.t()) * grad).sum()
+
+    copies = []
+    plain_copy = hip_ops._pad_last_copy
+
+    def counting(t, size):
+        if t.numel() * t.element_size() >= hip_ops._PAD_REUSE_MIN_BYTES:
+            copies.append((tuple(t.shape), size))
+        return plain_copy(t, size)
+
+    hip_ops._pad_last_copy = counting
+    try:
+        xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+        torch.compile(fn, backend=mojo_backend)(xd, wd, g.cuda()).backward()
+        torch.cuda.synchronize()
+    finally:
+        hip_ops._pad_last_copy = plain_copy
+    assert copies == [((rows, vocab), 50304)], copies
+    assert hip_ops._PAD_REUSE is None
+    want_dx = g.double() @ w.double()
+    want_dw = g.double().t() @ x.double()
+    for got, want in ((xd.grad, want_dx), (wd.grad, want_dw)):
+        assert got.shape == want.shape and got.is_contiguous()
+        err = (got.cpu().double() - want).norm() / want.norm()
+        assert err < 4e-3, err
+
+
 if __name__ == "__main__":
     import os
 

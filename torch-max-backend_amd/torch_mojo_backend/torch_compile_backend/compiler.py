@@ -964,6 +964,17 @@ class BaseMaxCompiler:
             self.run_device = torch.device("cuda", index)
         self.program = _GraphFactory(self.run_device, example_inputs).create_graph(gm.graph)
         self.num_slots = len(self.program.slots)
+        # A graph with at least two matrix products and no in-place node may share padded copies
+        # of large operands between its products (hip_ops._PAD_REUSE says what that saves).
+        products = (torch.ops.aten.mm.default, torch.ops.aten.addmm.default,
+                    torch.ops.aten.bmm.default)
+        targets = [n.target for n in gm.graph.nodes if n.op == "call_function"]
+        self.pad_reuse_module = None
+        if sum(t in products for t in targets) >= 2 and \
+                not any(getattr(getattr(t, "_schema", None), "is_mutable", False) for t in targets):
+            from torch_mojo_backend.eager_kernels import hip_ops
+
+            self.pad_reuse_module = hip_ops
         if profiling_enabled():
             elapsed = dt.timedelta(microseconds=(time.time_ns() - start) / 1000)
             print(f"Building the step program in {elapsed}")
@@ -993,6 +1004,28 @@ class BaseMaxCompiler:
         for slot, value in program.constants:
             env[slot] = value
         check = debug_graph()
+        pads = self.pad_reuse_module
+        if pads is not None:
+            pads_before, pads._PAD_REUSE = pads._PAD_REUSE, {}
+            try:
+                self._run_steps(program, env, check)
+            finally:
+                pads._PAD_REUSE = pads_before
+        else:
+            self._run_steps(program, env, check)
+        result = _materialize(program.output_template, env)
+        if profiling_enabled():
+            elapsed = dt.timedelta(microseconds=(time.time_ns() - start) / 1000)
+            print(f"Enqueueing the graph in {elapsed}")
+        if isinstance(result, tuple):
+            result = list(result)
+        elif not isinstance(result, list):
+            result = [result]
+        if run_device is not None:
+            result = [self._to_home(r) for r in result]
+        return [int(r) if isinstance(r, torch.SymInt) else r for r in result]
+
+    def _run_steps(self, program, env, check) -> None:
         for step in program.steps:
             a = _materialize(step.args, env) if step.dynamic_args else step.args
             kw = _materialize(step.kwargs, env) if step.dynamic_kwargs else step.kwargs
@@ -1015,17 +1048,6 @@ class BaseMaxCompiler:
             env[step.out] = out
             for slot in step.release:
                 env[slot] = None
-        result = _materialize(program.output_template, env)
-        if profiling_enabled():
-            elapsed = dt.timedelta(microseconds=(time.time_ns() - start) / 1000)
-            print(f"Enqueueing the graph in {elapsed}")
-        if isinstance(result, tuple):
-            result = list(result)
-        elif not isinstance(result, list):
-            result = [result]
-        if run_device is not None:
-            result = [self._to_home(r) for r in result]
-        return [int(r) if isinstance(r, torch.SymInt) else r for r in result]
 
     def _to_home(self, value):
         """A result back where the graph's tensors live: adopted as a mojo wrapper (zero-copy,
