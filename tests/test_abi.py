@@ -170,10 +170,11 @@ def test_relayout_rules_on_the_host():
     assert torch.equal(a2[:, :1001], a) and not a2[:, 1001:].any() and not b2[1001:].any()
     assert hip_ops._mfma_layouts_ok(a2, b2, la, lb, 16, 24, k, False)
     # the weight-gradient form with an odd M keeps its form: the stored [K, M] rows get zero
-    # columns up to 8 | M, B stays, and the launch computes the few extra rows
+    # columns up to 64 | M (the width an odd contraction length gets, so that one padded copy can
+    # serve both), B stays, and the launch computes the few extra rows
     a, b = torch.randn(512, 1001).to(bf).t(), torch.randn(512, 96).to(bf)
     ok, (a2, b2, la, lb, k, rows) = prep(a, b)
-    assert not ok and rows == 1008 and la == (1, 1008) and tuple(a2.shape) == (1008, 512) and b2 is b
+    assert not ok and rows == 1024 and la == (1, 1024) and tuple(a2.shape) == (1024, 512) and b2 is b
     assert torch.equal(a2[:1001], a) and not a2[1001:].any() and k == 512
     assert hip_ops._mfma_layouts_ok(a2, b2, la, lb, rows, 96, k, False)
     # ... but not with 64 or fewer columns (no weight-gradient kernel there): row-major A
