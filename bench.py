@@ -398,6 +398,17 @@ def main() -> int:
                 assert torch.equal(outs[0], hip_ops.softmax(bufs[0], -1))
                 with_copy(f"softmax_{dn}_{rows}x{cols}", len(bufs), ptrs, nbytes)
                 del bufs, outs
+            # log-softmax over GPT-2's vocabulary: the pitch is odd, no row but the first starts on
+            # a 16-byte boundary
+            rows, cols = 16384, 50257
+            nbytes = rows * cols * es
+            bufs = [gen((rows, cols), 20, dtype, scale=4.0)]
+            outs = [torch.empty_like(bufs[0])]
+            hbm_row(f"log_softmax_{dn}_{rows}x{cols}", 1,
+                    lambda i: lib.tmb_softmax_rows(outs[0].data_ptr(), bufs[0].data_ptr(), rows, cols,
+                                                   code, code, 1, stream), 2 * nbytes, steps=20)
+            assert torch.equal(outs[0], hip_ops.softmax(bufs[0], -1, log=True))
+            del bufs, outs
             for (rows, cols) in ((32768, 768), (16384, 4096)):
                 nbytes = rows * cols * es
                 g_ = gen((cols,), 1, dtype, scale=0.1, shift=1.0)
@@ -513,6 +524,17 @@ def main() -> int:
                                                             ys[i].data_ptr(), rows, cols, code, 0, stream),
                     3 * nb)
             del ys, gs, outs
+            # log-softmax backward over GPT-2's vocabulary (odd pitch)
+            rows, cols = 16384, 50257
+            nb = rows * cols * es
+            ys = [torch.log_softmax(gen((rows, cols), 75, torch.float32), -1).to(dtype)]
+            gs = [gen((rows, cols), 85, dtype)]
+            outs = [torch.empty_like(ys[0])]
+            hbm_row(f"log_softmax_backward_{dn}_{rows}x{cols}", 1,
+                    lambda i: lib.tmb_softmax_backward_rows(outs[0].data_ptr(), gs[0].data_ptr(),
+                                                            ys[0].data_ptr(), rows, cols, code, 1, stream),
+                    3 * nb, steps=20)
+            del ys, gs, outs
             # layer norm backward (all three outputs)
             for (rows, cols) in ((32768, 768), (16384, 4096)):
                 nb = rows * cols * es
@@ -619,6 +641,23 @@ def main() -> int:
         loss_c = train_step(compiled).item()
         compile_s = time.perf_counter() - t0
         wall, _ = timed(lambda: train_step(compiled), 5, 2)
+
+        # the same step with the loss inside the compiled graph (log-softmax forward and backward
+        # over the vocabulary then run on this library's kernels too)
+        def loss_of(i_, t_):
+            logits, _ = model(i_)
+            return F.cross_entropy(logits.view(-1, logits.shape[-1]), t_.view(-1))
+
+        def train_step_whole(fn):
+            loss = fn(idx, targets)
+            loss.backward()
+            for p_ in model.parameters():
+                p_.grad = None
+            return loss
+
+        compiled_loss = torch.compile(loss_of, backend=mojo_backend)
+        loss_w = train_step_whole(compiled_loss).item()
+        wall_w, _ = timed(lambda: train_step_whole(compiled_loss), 5, 2)
         loss_e = train_step(model).item()
         wall_e, _ = timed(lambda: train_step(model), 5, 2)
         # forward FLOPs of the projections and attention; backward = 2x
@@ -626,6 +665,7 @@ def main() -> int:
         sweep[f"gpt2_small_train_step_bf16_B{B}_T{T}"] = {
             "tokens/s": round(B * T / (wall * 1e-3), 1), "ms_per_step": round(wall, 3),
             "TFLOP/s_over_whole_step": round(3 * fwd_flops / (wall * 1e-3) / 1e12, 2),
+            "ms_per_step_loss_in_graph": round(wall_w, 3), "loss_in_graph": round(loss_w, 4),
             "pytorch_rocm_eager_ms_per_step": round(wall_e, 3), "compile_s": round(compile_s, 2),
             "loss": round(loss_c, 4), "pytorch_rocm_eager_loss": round(loss_e, 4),
             "batch": B, "seq": T, "dtype": "bf16",

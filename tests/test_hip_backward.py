@@ -52,7 +52,9 @@ def test_gelu_backward_limits():
 
 
 # ---- softmax / log-softmax ----------------------------------------------------------------------
-SOFTMAX_SHAPES = [(1, 1), (3, 5), (33, 257), (64, 1024), (17, 4096), (5, 8192), (4, 50257), (2, 70000)]
+SOFTMAX_SHAPES = [(1, 1), (3, 5), (33, 257), (64, 1024), (17, 4096), (5, 8192), (4, 50257), (2, 70000),
+                  # long ragged rows: one 1024-thread workgroup per row with unaligned vectors
+                  (37, 4099), (5, 16389), (6, 30001), (3, 65535), (130, 50257)]
 
 
 @pytest.mark.parametrize("dtype", FLOATS)
@@ -74,6 +76,25 @@ def test_softmax_backward_rows(shape, dtype, log):
     assert np.abs(as64(got) - want).max() <= bound
     ref = oracle.softmax_backward_rows(g, fwd, log)
     assert np.abs(as64(got) - as64(ref)).max() <= 2 * bound
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_backward_long_rows_at_an_odd_address(dtype, log):
+    """The saved output starts one element past a 16-byte boundary, the gradient does not: the
+    long-row kernel with unaligned vector accesses."""
+    rows, cols = 5, 8200
+    x = seeded((rows, cols), seed=5, dtype=torch.float32) * 2
+    fwd = (torch.log_softmax if log else torch.softmax)(x, -1).to(dtype)
+    g = seeded((rows, cols), seed=6, dtype=dtype)
+    buf = torch.zeros(rows * cols + 1, dtype=dtype, device="cuda")
+    saved = buf[1:].view(rows, cols)
+    saved.copy_(fwd)
+    assert saved.data_ptr() % 16 != 0
+    got = _ops().softmax_backward(g.cuda(), saved, -1, log)
+    ref = oracle.softmax_backward_rows(g, fwd, log)
+    bound = TOL[dtype] * (np.abs(as64(ref)).max() + 1.0) + cols * 2.0 ** -24 * 16.0
+    assert np.abs(as64(got) - as64(ref)).max() <= bound
 
 
 def test_softmax_backward_invariants_and_dims():

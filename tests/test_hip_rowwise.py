@@ -27,7 +27,10 @@ def _ops():
 # fallback (unaligned widths, beyond-register widths) and the GPT-2 / benchmark shapes.
 SOFTMAX_SHAPES = [(7, 1), (5, 8), (33, 257), (64, 64), (19, 128), (300, 768), (130, 1024),
                   (67, 2048), (35, 4096), (9, 8192), (5, 16384), (3, 32768), (2, 40000),
-                  (4, 50257), (3, 70000)]
+                  (4, 50257), (3, 70000),
+                  # long ragged rows (one 1024-thread workgroup per row, unaligned vectors): each
+                  # vector count per lane, tails of 1 .. 7 elements, the widest row it takes
+                  (37, 4099), (5, 16389), (6, 30001), (3, 65535), (130, 50257)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -48,11 +51,29 @@ def test_softmax_matches_oracle(shape, dtype, log):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_softmax_half_to_float(dtype):
-    x = seeded((37, 1024), seed=3, scale=4.0, dtype=dtype)
+@pytest.mark.parametrize("shape", [(37, 1024), (9, 50257)])
+def test_softmax_half_to_float(dtype, shape):
+    x = seeded(shape, seed=3, scale=4.0, dtype=dtype)
     got = _ops().softmax(_dev(x), -1, half_to_float=True)
     assert got.dtype == torch.float32
     assert_close64(got, cf.softmax(as64(x)), what="half_to_float")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_long_rows_at_an_odd_address(dtype, log):
+    """Whole vectors per row, but the tensor starts one element past a 16-byte boundary (a slice
+    of a larger buffer): the unaligned long-row kernel, with nothing written outside the rows."""
+    rows, cols = 6, 8192
+    x = seeded((rows, cols), seed=11, scale=4.0, dtype=dtype)
+    buf = torch.zeros(rows * cols + 1, dtype=dtype, device="cuda")
+    view = buf[1:].view(rows, cols)
+    view.copy_(x)
+    assert view.data_ptr() % 16 != 0
+    got = _ops().softmax(view, -1, log=log)
+    want = (cf.log_softmax if log else cf.softmax)(as64(x))
+    assert_close64(got, want, what=f"odd address log={log} {dtype}")
+    assert float(buf[0]) == 0.0 and torch.equal(view.cpu(), x)
 
 
 @pytest.mark.parametrize("dim", [0, 1, 2, -1, -2])

@@ -138,6 +138,128 @@ __global__ __launch_bounds__(BLOCK) void softmax_backward_regs_kernel(T* __restr
   }
 }
 
+// Long rows of any width at any element alignment (the gradient of a [rows, 50257] log-softmax):
+// one 1024-thread workgroup per row, both operands held in registers in their storage type (a
+// lane's share of a 16-bit row of 65536 columns is 2 x 32 registers); every element is read once
+// and written once. PEEL: the three rows sit at the same offset from a 16-byte boundary, the
+// vectors start at the first boundary inside the row and every vector access is aligned; the
+// elements in front of the first vector and after the last one are held one each by the first
+// lanes of wave 0. Without PEEL the vectors start with the row and the accesses are unaligned.
+template <typename T, int VPL, bool LOG, bool PEEL>
+__global__ __launch_bounds__(1024) void softmax_backward_long_rows_kernel(
+    T* __restrict__ gin, const T* __restrict__ gout, const T* __restrict__ y, int cols) {
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int WAVES = 16;
+  __shared__ float slot[WAVES];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * cols;
+  const T* gsrc = gout + base;
+  const T* ysrc = y + base;
+  T* dst = gin + base;
+  int head = 0;
+  if constexpr (PEEL) {
+    const int off = static_cast<int>((reinterpret_cast<uintptr_t>(gsrc) & 15u) / sizeof(T));
+    head = off ? EPV - off : 0;
+  }
+  const int nvec = (cols - head) / EPV;
+  const int tail_from = head + nvec * EPV;
+  int edge = -1;
+  if (wave == 0 && lane < 8 && lane < head) edge = lane;
+  if (wave == 0 && lane >= 8 && lane < 16 && tail_from + lane - 8 < cols) edge = tail_from + lane - 8;
+
+  // LATE_Y (sixteen vectors per lane: fp32 rows beyond 32768 columns): the row sum of the log form
+  // needs the gradient only, so the saved output is fetched after the reduction, vector by vector
+  constexpr bool LATE_Y = VPL > 8;
+  static_assert(!LATE_Y || LOG, "the plain form needs both operands for its row sum");
+  Vec16<T> gv[VPL], yv[LATE_Y ? 1 : VPL];
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WAVES + wave) * kWave + lane;
+    const unsigned at = static_cast<unsigned>(head + (vi < nvec ? vi : 0) * EPV);
+    if constexpr (PEEL) {
+      gv[v] = load_vec16_stream(gsrc + at);
+      if constexpr (!LATE_Y) yv[v] = load_vec16_stream(ysrc + at);
+    } else {
+      gv[v] = load_vec16_unaligned(gsrc + at);
+      if constexpr (!LATE_Y) yv[v] = load_vec16_unaligned(ysrc + at);
+    }
+  }
+  float gt = 0.0f, yt = 0.0f;
+  if (edge >= 0) {
+    gt = to_f32(gsrc[edge]);
+    yt = to_f32(ysrc[edge]);
+  }
+  float s = LOG ? gt : gt * yt;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WAVES + wave) * kWave + lane;
+    float part = 0.0f;
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      if constexpr (LOG) {
+        part += to_f32(gv[v].v[e]);
+      } else {
+        part += to_f32(gv[v].v[e]) * to_f32(yv[v].v[e]);
+      }
+    }
+    s += vi < nvec ? part : 0.0f;  // an empty slot holds a copy of vector 0
+  }
+  s = wave_sum(s);
+  s = group_reduce(s, slot, wave, 0, WAVES, SumOp{});
+  constexpr int CHUNK = LATE_Y ? 2 : VPL;  // vectors of the saved output in flight at a time
+#pragma unroll
+  for (int v0 = 0; v0 < VPL; v0 += CHUNK) {
+    Vec16<T> late[CHUNK];
+    if constexpr (LATE_Y) {
+#pragma unroll
+      for (int c = 0; c < CHUNK; ++c) {
+        const int vi = ((v0 + c) * WAVES + wave) * kWave + lane;
+        const unsigned at = static_cast<unsigned>(head + (vi < nvec ? vi : 0) * EPV);
+        if constexpr (PEEL) {
+          late[c] = load_vec16_stream(ysrc + at);
+        } else {
+          late[c] = load_vec16_unaligned(ysrc + at);
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNK; ++c) {
+      const int v = v0 + c;
+      const int vi = (v * WAVES + wave) * kWave + lane;
+      float r[EPV];
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float g = to_f32(gv[v].v[e]);
+        const float o = to_f32(LATE_Y ? late[c].v[e] : yv[LATE_Y ? 0 : v].v[e]);
+        r[e] = LOG ? g - exp_for<T>(o) * s : o * (g - s);
+      }
+      if (vi < nvec) {
+        T* at = dst + static_cast<unsigned>(head + vi * EPV);
+        if constexpr (PEEL) {
+          store_converted<T, EPV>(at, r);
+        } else {
+          store_converted_unaligned<T, EPV>(at, r);
+        }
+      }
+    }
+  }
+  if (edge >= 0) dst[edge] = from_f32<T>(LOG ? gt - exp_for<T>(yt) * s : yt * (gt - s));
+}
+
+template <typename T, int VPL, bool LOG>
+static int launch_softmax_backward_long_rows(T* gin, const T* gout, const T* y, int64_t rows,
+                                             int64_t cols, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(rows)), block(1024);
+  const int c = static_cast<int>(cols);
+  const uintptr_t a = reinterpret_cast<uintptr_t>(gin) & 15u;
+  if (a == (reinterpret_cast<uintptr_t>(gout) & 15u) && a == (reinterpret_cast<uintptr_t>(y) & 15u)) {
+    softmax_backward_long_rows_kernel<T, VPL, LOG, true><<<grid, block, 0, stream>>>(gin, gout, y, c);
+  } else {
+    softmax_backward_long_rows_kernel<T, VPL, LOG, false><<<grid, block, 0, stream>>>(gin, gout, y, c);
+  }
+  return check_launch();
+}
+
 // Any width / alignment: one workgroup per row, the row is read twice (the second time from L2).
 template <typename T, bool LOG>
 __global__ __launch_bounds__(256) void softmax_backward_generic_kernel(T* __restrict__ gin,
@@ -191,6 +313,22 @@ static int softmax_backward_dispatch(void* gin_, const void* gout_, const void* 
     TMB_SB(16, 4, 1024)
   }
 #undef TMB_SB
+  // ragged or unaligned rows long enough to occupy a 1024-thread workgroup (eight 16-bit vector
+  // pairs per lane plus the products of the plain softmax form do not fit the 128 registers of
+  // such a workgroup: that form stops at four)
+  const int64_t max_vec = 1024 * ((!LOG && sizeof(T) == 2) ? 4 : 8);
+  if (cols >= 4096 && cols / EPV <= max_vec && rows < (int64_t{1} << 31)) {
+    if (cols / EPV <= 1024 * 2)
+      return launch_softmax_backward_long_rows<T, 2, LOG>(gin, gout, y, rows, cols, stream);
+    if (cols / EPV <= 1024 * 4)
+      return launch_softmax_backward_long_rows<T, 4, LOG>(gin, gout, y, rows, cols, stream);
+    if constexpr (LOG || sizeof(T) != 2)
+      return launch_softmax_backward_long_rows<T, 8, LOG>(gin, gout, y, rows, cols, stream);
+  }
+  if constexpr (LOG && sizeof(T) == 4) {  // fp32 rows of up to 65536 columns (a vocabulary)
+    if (cols >= 4096 && cols / EPV <= 1024 * 16 && rows < (int64_t{1} << 31))
+      return launch_softmax_backward_long_rows<T, 16, LOG>(gin, gout, y, rows, cols, stream);
+  }
   const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
   softmax_backward_generic_kernel<T, LOG>
       <<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(gin, gout, y, rows, cols);

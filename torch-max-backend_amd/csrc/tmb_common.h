@@ -58,6 +58,44 @@ __device__ __forceinline__ void store_vec16_stream(T* p, const Vec16<T>& v) {
   __builtin_nontemporal_store(__builtin_bit_cast(raw16_t, v), reinterpret_cast<raw16_t*>(p));
 }
 
+// The same 16 bytes at an address that is only element-aligned (rows of an odd pitch, as in a
+// [rows, 50257] tensor): global memory takes unaligned vector accesses on this target, and one
+// 16-byte access per lane beats 16 / sizeof(T) element accesses by far.
+typedef raw16_t __attribute__((aligned(2))) raw16_a2_t;
+typedef raw16_t __attribute__((aligned(4))) raw16_a4_t;
+template <typename T>
+__device__ __forceinline__ Vec16<T> load_vec16_unaligned(const T* p) {
+  if constexpr (sizeof(T) == 2) {
+    const raw16_t r = *reinterpret_cast<const raw16_a2_t*>(p);
+    return __builtin_bit_cast(Vec16<T>, r);
+  } else {
+    const raw16_t r = *reinterpret_cast<const raw16_a4_t*>(p);
+    return __builtin_bit_cast(Vec16<T>, r);
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store_vec16_unaligned(T* p, const Vec16<T>& v) {
+  if constexpr (sizeof(T) == 2) {
+    *reinterpret_cast<raw16_a2_t*>(p) = __builtin_bit_cast(raw16_t, v);
+  } else {
+    *reinterpret_cast<raw16_a4_t*>(p) = __builtin_bit_cast(raw16_t, v);
+  }
+}
+// N fp32 values as TOut elements at an element-aligned address (several 16-byte stores when TOut
+// is wider than the type N was counted in).
+template <typename TOut, int N>
+__device__ __forceinline__ void store_converted_unaligned(TOut* p, const float (&x)[N]) {
+  constexpr int OUT_PER_VEC = 16 / sizeof(TOut);
+  static_assert(N % OUT_PER_VEC == 0, "vector width mismatch");
+#pragma unroll
+  for (int c = 0; c < N / OUT_PER_VEC; ++c) {
+    Vec16<TOut> o;
+#pragma unroll
+    for (int e = 0; e < OUT_PER_VEC; ++e) o.v[e] = from_f32<TOut>(x[c * OUT_PER_VEC + e]);
+    store_vec16_unaligned(p + c * OUT_PER_VEC, o);
+  }
+}
+
 // Stores N = 16/sizeof(TIn) fp32 values as TOut elements. When TOut is wider
 // than TIn (half_to_float softmax) this issues several 16-byte stores.
 template <typename TOut, int N, bool STREAM = false>
