@@ -282,17 +282,22 @@ def test_padded_copies_are_shared_only_inside_a_graph_run(monkeypatch):
     a, b = hip_ops._pad_last(x, 40), hip_ops._pad_last(x, 40)
     assert a is not b and torch.equal(a, b) and a.shape == (64, 40)
     assert torch.equal(a[:, :33], x) and bool((a[:, 33:] == 0).all())
-    monkeypatch.setattr(hip_ops, "_PAD_REUSE", {})
-    a = hip_ops._pad_last(x, 40)
-    assert hip_ops._pad_last(x.t().t(), 40) is a          # another view of the same rows
-    assert hip_ops._pad_last(x[:32], 40) is not a         # other shape
-    assert hip_ops._pad_last(x, 40) is not a              # one entry: the narrower view replaced it
-    c = hip_ops._pad_last(x, 48)
-    assert c.shape == (64, 48) and hip_ops._pad_last(x, 48) is c
-    small = torch.randn(4, 33)
-    assert hip_ops._pad_last(small, 40) is not hip_ops._pad_last(small, 40)
-    (kept_source, kept_copy), = hip_ops._PAD_REUSE.values()
-    assert kept_source is x and kept_copy is c
+    before = hip_ops.pad_reuse_begin()
+    assert before is None
+    try:
+        a = hip_ops._pad_last(x, 40)
+        assert hip_ops._pad_last(x.t().t(), 40) is a          # another view of the same rows
+        assert hip_ops._pad_last(x[:32], 40) is not a         # other shape
+        assert hip_ops._pad_last(x, 40) is not a              # one entry: the narrower view replaced it
+        c = hip_ops._pad_last(x, 48)
+        assert c.shape == (64, 48) and hip_ops._pad_last(x, 48) is c
+        small = torch.randn(4, 33)
+        assert hip_ops._pad_last(small, 40) is not hip_ops._pad_last(small, 40)
+        (kept_source, kept_copy), = hip_ops.pad_reuse_active().values()
+        assert kept_source is x and kept_copy is c
+    finally:
+        hip_ops.pad_reuse_end(before)
+    assert hip_ops.pad_reuse_active() is None
 
 
 def test_graph_runs_share_padded_copies_unless_a_node_writes_in_place(cpu_hot_ops):
@@ -302,7 +307,7 @@ def test_graph_runs_share_padded_copies_unless_a_node_writes_in_place(cpu_hot_op
     seen = []
 
     def spy(a, b):
-        seen.append(hip_ops._PAD_REUSE)
+        seen.append(hip_ops.pad_reuse_active())
         return torch.mm(a, b)
 
     MAPPING_TORCH_ATEN_TO_MOJO[aten.mm] = spy  # (the fixture restores the entry)
@@ -312,7 +317,7 @@ def test_graph_runs_share_padded_copies_unless_a_node_writes_in_place(cpu_hot_op
     assert run.pad_reuse_module is hip_ops
     out, = run(x, w)
     assert torch.allclose(out, x @ w @ w)
-    assert seen == [{}, {}] and seen[0] is seen[1] and hip_ops._PAD_REUSE is None
+    assert seen == [{}, {}] and seen[0] is seen[1] and hip_ops.pad_reuse_active() is None
     one = make_fx(lambda x, w: torch.mm(x, w))(x, w)
     assert compiler.BaseMaxCompiler(one, [x, w]).pad_reuse_module is None
 

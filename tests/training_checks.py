@@ -222,7 +222,7 @@ def vocabulary_projection_backward_pads_its_gradient_once():
     finally:
         hip_ops._pad_last_copy = plain_copy
     assert copies == [((rows, vocab), 50304)], copies
-    assert hip_ops._PAD_REUSE is None
+    assert hip_ops.pad_reuse_active() is None
     want_dx = g.double() @ w.double()
     want_dw = g.double().t() @ x.double()
     for got, want in ((xd.grad, want_dx), (wd.grad, want_dw)):

@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import threading
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -105,16 +106,32 @@ _RELAYOUT_MIN_WORK = 1 << 26
 # vocabulary projection needs its incoming gradient padded twice, as A of the input gradient and
 # as A^T of the weight gradient (0.5 ms per copy at 16384 rows). The entry holds the source tensor,
 # so its memory cannot be handed to another tensor while the entry lives; outside such a run the
-# dictionary is None and nothing is kept.
-_PAD_REUSE: Optional[dict] = None
+# dictionary is None and nothing is kept. The dictionary belongs to the thread that runs the graph
+# (a backward graph may run on PyTorch's autograd thread while the main thread goes on).
+_PAD_STATE = threading.local()
 _PAD_REUSE_MIN_BYTES = 64 << 20
+
+
+def pad_reuse_begin() -> Optional[dict]:
+    """Starts keeping padded copies on this thread; returns what `pad_reuse_end` must get back."""
+    before = getattr(_PAD_STATE, "reuse", None)
+    _PAD_STATE.reuse = {}
+    return before
+
+
+def pad_reuse_end(before: Optional[dict]) -> None:
+    _PAD_STATE.reuse = before
+
+
+def pad_reuse_active() -> Optional[dict]:
+    return getattr(_PAD_STATE, "reuse", None)
 
 
 def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
     """`x` with its last dimension zero-padded to `size`, contiguous. Row-major sources go
     through the row-padding kernel (copy speed whatever the source alignment); anything else is
     copied by PyTorch-ROCm's strided copy."""
-    reuse, key = _PAD_REUSE, None
+    reuse, key = getattr(_PAD_STATE, "reuse", None), None
     if reuse is not None and x.numel() * x.element_size() >= _PAD_REUSE_MIN_BYTES:
         key = (x.data_ptr(), tuple(x.shape), x.stride(), x.dtype, size)
         kept = reuse.get(key)

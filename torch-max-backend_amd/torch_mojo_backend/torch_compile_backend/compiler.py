@@ -965,7 +965,7 @@ class BaseMaxCompiler:
         self.program = _GraphFactory(self.run_device, example_inputs).create_graph(gm.graph)
         self.num_slots = len(self.program.slots)
         # A graph with at least two matrix products and no in-place node may share padded copies
-        # of large operands between its products (hip_ops._PAD_REUSE says what that saves).
+        # of large operands between its products (hip_ops._pad_last says what that saves).
         products = (torch.ops.aten.mm.default, torch.ops.aten.addmm.default,
                     torch.ops.aten.bmm.default)
         targets = [n.target for n in gm.graph.nodes if n.op == "call_function"]
@@ -1006,11 +1006,11 @@ class BaseMaxCompiler:
         check = debug_graph()
         pads = self.pad_reuse_module
         if pads is not None:
-            pads_before, pads._PAD_REUSE = pads._PAD_REUSE, {}
+            pads_before = pads.pad_reuse_begin()
             try:
                 self._run_steps(program, env, check)
             finally:
-                pads._PAD_REUSE = pads_before
+                pads.pad_reuse_end(pads_before)
         else:
             self._run_steps(program, env, check)
         result = _materialize(program.output_template, env)
