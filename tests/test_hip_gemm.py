@@ -96,7 +96,7 @@ def test_mm_fp32(mnk):
                                  (5000, 9000, 1024),
                                  # one partial round of 256 x 256 tiles; 256 x 128 tiles with 32-deep
                                  # stages (K-major B, K an odd multiple of 32)
-                                 (3000, 3400, 2048), (16500, 1000, 992)])
+                                 (3000, 3400, 2048), (3000, 3400, 8192), (16500, 1000, 992)])
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_addmm_half_long_k_ragged_tiles(mnk, dtype, trans_b):
     """Products that run on the ring configurations with the 16x16x32 MFMA (256x256x64, 256x128x64,
