@@ -426,11 +426,14 @@ def test_mm_transposed_a(mnk, dtype):
 
 
 @pytest.mark.parametrize("dtype", HALF)
-@pytest.mark.parametrize("mnk", [(16392, 768, 2048), (8200, 3072, 1024)])
+@pytest.mark.parametrize("mnk", [(16392, 768, 2048), (8200, 3072, 1024),
+                                 # a last round of 256 x 256 tiles that would be mostly empty:
+                                 # 128 x 256 tiles, even and odd numbers of 32-deep stages
+                                 (24008, 768, 2048), (24008, 776, 1056)])
 def test_mm_transposed_a_many_tiles(mnk, dtype):
-    """Enough 256 x 256 tiles for the unsplit 64-deep ring with both operands staged k-outer
-    (the vocabulary projection's weight gradient): sampled rows, every column, against float64;
-    the last tile row is ragged."""
+    """Enough tiles for the unsplit rings with both operands staged k-outer (the vocabulary
+    projection's weight gradient): sampled rows, every column, against float64; the last tile
+    row is ragged."""
     m, n, k = mnk
     g = torch.Generator(device="cuda").manual_seed(11)
     a_km = torch.randn(k, m, generator=g, device="cuda").to(dtype)
