@@ -753,7 +753,21 @@ __global__ __launch_bounds__(1024) void layer_norm_param_final_kernel(
   const int64_t col = static_cast<int64_t>(blockIdx.x) * 32 + tx;
   float sg = 0.0f, sb = 0.0f;
   if (col < cols) {
-    for (int64_t s = ty; s < slabs; s += 32) {
+    int64_t s = ty;
+    for (; s + 96 < slabs; s += 128) {  // eight loads in flight, added in slab order
+      float vg[4], vb[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        vg[u] = partial[((s + 32 * u) * 2 + 0) * cols + col];
+        vb[u] = partial[((s + 32 * u) * 2 + 1) * cols + col];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        sg += vg[u];
+        sb += vb[u];
+      }
+    }
+    for (; s < slabs; s += 32) {
       sg += partial[(s * 2 + 0) * cols + col];
       sb += partial[(s * 2 + 1) * cols + col];
     }
