@@ -257,6 +257,33 @@ def main() -> int:
         for (m, n, k) in ((128, 768, 768), (1024, 3072, 768), (1024, 768, 3072), (4096, 4096, 4096)):
             gemm_row(f"addmm_bf16_{m}x{n}x{k}", m, n, k)
         gemm_row("bmm_bf16_48x1024x64x1024", 1024, 1024, 64, batch=48)
+        # GPT-2 small's projections at 32768 tokens (weights stored [out, in]: K-major B)
+        for (m, n, k) in ((32768, 2304, 768), (32768, 3072, 768), (32768, 768, 3072), (32768, 768, 768)):
+            gemm_row(f"linear_bf16_{m}x{n}x{k}", m, n, k, trans_b=True, steps=30)
+        # the vocabulary projection, alone and behind other work (four 8192^3 products evict its
+        # weight from the Infinity Cache, as the rest of a model does): the difference of the
+        # pair's time and the other work's
+        for m in (16384, 32768):
+            xv, wv = gen((m, 768), 6, torch.bfloat16), gen((50257, 768), 7, torch.bfloat16, scale=0.02)
+            other = gen((8192, 8192), 8, torch.bfloat16)
+            _, alone = timed(lambda: hip_ops.gemm(xv, wv.t()), 10, 5)
+
+            def evict():
+                for _ in range(4):
+                    hip_ops.gemm(other, other)
+
+            def pair():
+                evict()
+                return hip_ops.gemm(xv, wv.t())
+
+            _, both = timed(pair, 6, 2)
+            _, rest = timed(evict, 6, 2)
+            fl = 2.0 * m * 50257 * 768
+            sweep[f"linear_bf16_{m}x50257x768"] = {
+                "us": round(alone * 1e3, 1), "TFLOP/s": round(fl / alone / 1e9, 1),
+                "us_behind_other_work": round((both - rest) * 1e3, 1),
+                "frac_mfma": round(fl / alone / 1e9 / PEAK_BF16_DENSE_TFLOPS, 4)}
+            del xv, wv, other
         # fp32 storage: true fp32 products on the matrix cores (peak 157.3 TFLOP/s)
         gemm_row("addmm_fp32_4096x4096x4096", 4096, 4096, 4096, steps=20, dtype=torch.float32)
         gemm_row("addmm_fp32_128x3072x768", 128, 3072, 768, dtype=torch.float32)
