@@ -124,9 +124,15 @@ int tmb_reduce_rows(void* out, const void* in, int64_t rows, int64_t cols, int o
  * TMB_REDUCE_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
  * ends) instead of a caller's workspace. Allocates and frees nothing. Shapes whose
  * tmb_reduce_workspace_bytes exceeds the array are refused with TMB_ERR_SCRATCH_LIMIT before
- * anything is enqueued (a split reduction has at most rows + 8192 partials of 16 bytes, and only
- * for rows < 4096, so every shape that fits the device's memory fits). The first call on a device
- * looks the array's address up (hipGetSymbolAddress); make that call outside graph capture.
+ * anything is enqueued. A split reduction has at most rows + 8192 partials of 16 bytes, and only
+ * for rows < 4096, unless a row is longer than 2^30 elements: such rows are cut into chunks of
+ * 2^30 whatever the row count, and thousands of them exceed the array (4000 rows of 6 * 2^30
+ * elements need 4000 * 6 * 16 bytes). The stream must belong to the calling thread's current
+ * device (checked: TMB_ERR_INVALID_ARGUMENT otherwise), whose copy of the array is used. The first
+ * call on a device looks the array's address up (hipGetSymbolAddress); make that call outside
+ * graph capture. A HIP runtime failure of that lookup, of the device queries or of a launch is
+ * returned as the positive hipError_t value, as from every other entry point; the library's own
+ * codes (tmb_status) are negative.
  * All calls on one GPU share the array: calls that overlap there (two streams, two threads)
  * race; calls on one stream are ordered and safe. Nothing in it needs clearing between calls:
  * the first stage writes every partial the second stage reads.

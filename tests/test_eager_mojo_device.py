@@ -302,33 +302,84 @@ def test_mojo_backend_over_mojo_tensors_returns_zero_copy_wrappers():
 
 
 @gpu
-def test_mojo_backend_over_host_tensors_copies_in_and_out():
+def test_mojo_backend_over_host_tensors_copies_in_and_out(monkeypatch):
     """The workload's CPU-resident configuration: a float32 GPT-2-shaped module that lives on the
     host, compiled with mojo_backend. There is no CPU kernel path: parameters and inputs cross to
-    the HIP device (parameters once, cached), results come back as host tensors."""
+    the HIP device at every call, results come back as host tensors. Every kind of write to a
+    host parameter is seen by the next call, as with the reference's aliasing import of host
+    buffers (torch_compile_backend/compiler.py:535-566): in place, through `.data`, through the
+    numpy view. The fused attention step still runs (the causal verdict is taken on the host
+    buffer while the graph is built and travels with each device copy)."""
     from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
     from torch_mojo_backend import mojo_backend
     from torch_mojo_backend.torch_compile_backend import compiler
 
+    monkeypatch.delenv("TORCH_MOJO_BACKEND_CACHE_HOST_PARAMETERS", raising=False)
     model = build_gpt2_small(seed=0, n_layer=2)
     idx = seeded_tokens(1, 128, seed=0)
+    fused = []
+    real = compiler.aten_functions.hip_ops.softmax_scaled
+    monkeypatch.setattr(compiler.aten_functions.hip_ops, "softmax_scaled",
+                        lambda *a, **kw: (fused.append(1), real(*a, **kw))[1])
     with torch.no_grad():
         want_logits, want_next = model(idx)
         compiled = torch.compile(model, backend=mojo_backend, fullgraph=True)
-        logits, nxt = compiled(idx)
         made = compiler._DEVICE_COPIES["made"]
+        logits, nxt = compiled(idx)
         logits2, _ = compiled(idx)
     assert logits.device.type == "cpu" and nxt.device.type == "cpu"
     torch.testing.assert_close(logits, want_logits, rtol=1e-4, atol=1e-4)
     assert torch.equal(nxt, torch.argmax(logits[:, -1, :], dim=-1))
-    assert made > 0 and compiler._DEVICE_COPIES["made"] == made       # parameters crossed once
+    assert compiler._DEVICE_COPIES["made"] == made                    # nothing is kept
     assert torch.equal(logits, logits2)
-    # an in-place update of a host parameter is seen by the next call
+    assert len(fused) == 4                                            # two layers, two calls
     with torch.no_grad():
-        model.transformer.ln_f.bias.add_(1.0)
+        model.transformer.ln_f.bias.add_(1.0)                         # bumps the version counter
         logits3, _ = compiled(idx)
         want3, _ = model(idx)
-    torch.testing.assert_close(logits3, want3, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(logits3, want3, rtol=1e-4, atol=1e-4)
+        model.transformer.h[0].mlp.c_fc.weight.data.mul_(0.5)         # does not
+        logits4, _ = compiled(idx)
+        want4, _ = model(idx)
+        assert not torch.allclose(want4, want3, atol=1e-3)
+        torch.testing.assert_close(logits4, want4, rtol=1e-4, atol=1e-4)
+        model.transformer.ln_f.weight.detach().numpy()[:] *= 2.0      # nor does numpy
+        logits5, _ = compiled(idx)
+        want5, _ = model(idx)
+        torch.testing.assert_close(logits5, want5, rtol=1e-4, atol=1e-4)
+
+
+@gpu
+def test_kept_parameter_copies_are_opt_in_and_can_be_dropped(monkeypatch):
+    """TORCH_MOJO_BACKEND_CACHE_HOST_PARAMETERS=1: parameters cross once and are reused while
+    data pointer and version counter stand; a write the counter misses needs
+    `invalidate_device_copies`."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    monkeypatch.setenv("TORCH_MOJO_BACKEND_CACHE_HOST_PARAMETERS", "1")
+    model = build_gpt2_small(seed=0, n_layer=1)
+    idx = seeded_tokens(1, 64, seed=0)
+    with torch.no_grad():
+        compiled = torch.compile(model, backend=mojo_backend, fullgraph=True)
+        before = dict(compiler._DEVICE_COPIES)
+        compiled(idx)
+        made = compiler._DEVICE_COPIES["made"] - before["made"]
+        compiled(idx)
+        assert made > 0 and compiler._DEVICE_COPIES["made"] - before["made"] == made
+        assert compiler._DEVICE_COPIES["reused"] - before["reused"] >= made
+        model.transformer.ln_f.bias.add_(1.0)                         # seen: the counter moved
+        got, _ = compiled(idx)
+        want, _ = model(idx)
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+        model.transformer.ln_f.weight.data.mul_(2.0)                  # not seen ...
+        stale, _ = compiled(idx)
+        want, _ = model(idx)
+        assert not torch.allclose(stale, want, atol=1e-3)
+        assert compiler.invalidate_device_copies(model) >= made       # ... until dropped
+        got, _ = compiled(idx)
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
 
 
 def test_out_of_memory_launch_status_becomes_torch_out_of_memory_error(monkeypatch):

@@ -170,7 +170,8 @@ def test_gpt2_small_bf16_bit_identical_mode_matches_the_vendor_pipeline(monkeypa
 def test_gpt2_small_bf16_full_size_graph_routes_every_hot_op():
     """The benchmark configuration itself (B=32, T=1024, bf16): every GEMM, layer norm, the
     attention and the argmax run on the HIP kernels (call counts of the mapping functions and of
-    the fused steps), the argmax is exact on the graph's own logits, and rows sampled from the
+    the fused steps), the argmax is exact on the graph's own logits, batch rows 0 and 31 are within
+    2e-2 (max-abs) of the float32 CPU model run on those rows alone, and rows sampled from the
     logits equal those of the same graph without the attention rewrite up to the reordered
     storage roundings."""
     from torch_mojo_backend import mojo_backend
@@ -221,6 +222,24 @@ def test_gpt2_small_bf16_full_size_graph_routes_every_hot_op():
     assert counts["attention"] == 12 and counts["layer_norm"] == 25
     assert counts["argmax"] == 1 and counts["embedding"] == 2
     assert torch.equal(nxt, torch.argmax(logits[:, -1, :].float(), dim=-1))
+    # The tolerance the workload states, at the workload's own sequence length: batch rows are
+    # independent, so the float32 CPU model (bf16-rounded weights) run on single rows of the batch
+    # is the reference for those rows of the B = 32 graph (the reference's harness compares whole
+    # outputs with the CPU run of the same module, torch_mojo_backend/testing.py:186-229).
+    ref_model = build_gpt2_small(seed=0).to(torch.bfloat16).to(torch.float32)
+    worst = 0.0
+    for b in (0, 31):
+        with torch.no_grad():
+            want, want_next = ref_model(idx[b:b + 1].cpu())
+        err = (logits[b].float().cpu() - want[0]).abs()
+        print(f"B=32 T=1024 batch row {b}: max-abs logit error vs the float32 model "
+              f"{err.max().item():.4f} (mean {err.mean().item():.5f})")
+        worst = max(worst, err.max().item())
+        assert err.mean().item() <= 3e-3
+        top2 = want[0, -1].topk(2).values
+        if (top2[0] - top2[1]).item() > 4e-2:
+            assert nxt[b].item() == want_next[0].item()
+    assert worst <= 2e-2
     rows = [(0, 0), (0, 1023), (7, 511), (31, 0), (31, 1023)]
     picked = torch.stack([logits[b, t] for b, t in rows]).float()
     del logits
@@ -316,6 +335,39 @@ def test_causal_verdict_follows_the_buffer_not_its_address():
     big = torch.tril(torch.ones(1, 1, 128, 128, device="cuda"))
     assert compiler._causal_q_len(big, ((2, 0, 64, 1), (3, 0, 64, 1)), x) == 64
     assert compiler._causal_q_len(big, ((2, 0, 64, 1), (3, 1, 65, 1)), x) == 0
+
+
+def test_a_running_step_never_compares_mask_values(monkeypatch):
+    """check=False is how every step of a running graph asks: the answer comes from verdicts
+    taken while the graph was built (exact slices, or any slice from the origin of a buffer
+    that is causal as a whole: the sizes of a graph with dynamic shapes), and a buffer without
+    a valid verdict (never seen, or edited since) gives 0 = run the unfused ops. No comparison,
+    hence no synchronisation, on that path."""
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    mask = torch.tril(torch.ones(1, 1, 128, 128, device="cuda"))
+    x = (64, 64)
+    origin = ((2, 0, 64, 1), (3, 0, 64, 1))
+    assert compiler._causal_q_len(mask, origin, x, check=False) == 0      # never seen
+    compiler._take_causal_verdict(mask, None, None)                        # build time
+    monkeypatch.setattr(compiler, "_is_causal", lambda *a: pytest.fail("values compared in a step"))
+    assert compiler._causal_q_len(mask, origin, x, check=False) == 64
+    assert compiler._causal_q_len(mask, ((2, 0, 2 ** 63 - 1, 1), (3, 0, 2 ** 63 - 1, 1)), (128, 128),
+                                  check=False) == 128
+    assert compiler._causal_q_len(mask, ((2, 0, 96, 1), (3, 0, 96, 1)), (96, 96), check=False) == 96
+    assert compiler._causal_q_len(mask, ((2, 0, 64, 1), (3, 1, 65, 1)), x, check=False) == 0
+    assert compiler._causal_q_len(mask, ((2, 0, 64, 2), (3, 0, 64, 1)), (32, 64), check=False) == 0
+    assert compiler._causal_q_len(mask, origin, (64, 32), check=False) == 0  # sizes do not match
+    mask[0, 0, 3, 40] = 1.0                                                 # edited: verdict void
+    assert compiler._causal_q_len(mask, origin, x, check=False) == 0
+    # a host buffer's verdict travels with each device copy made for a call
+    monkeypatch.undo()
+    host = torch.tril(torch.ones(1, 1, 32, 32))
+    compiler._take_causal_verdict(host, ((2, 0, 16, 1), (3, 0, 16, 1)), (16, 16))
+    copy = compiler._on_device(host, torch.device("cuda", 0))
+    monkeypatch.setattr(compiler, "_is_causal", lambda *a: pytest.fail("values compared in a step"))
+    assert compiler._causal_q_len(copy, ((2, 0, 16, 1), (3, 0, 16, 1)), (16, 16), check=False) == 16
+    assert compiler._causal_q_len(copy, ((2, 0, 8, 1), (3, 0, 8, 1)), (8, 8), check=False) == 8
 
 
 def test_attention_fusion_stays_within_the_storage_rounding(monkeypatch):

@@ -11,6 +11,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 CHECKS = ["gpt2_training_step_gradients_match_cpu", "training_graph_runs_the_fused_attention_forward_and_backward",
+          "attention_backward_follows_the_route_the_forward_took",
           "sdpa_training_graph_runs_the_fused_forward_and_backward",
           "one_sgd_step_lowers_the_loss",
           "log_softmax_and_linear_backward_in_a_compiled_graph",

@@ -98,6 +98,62 @@ def training_graph_runs_the_fused_attention_forward_and_backward():
         torch._dynamo.reset()
 
 
+def attention_backward_follows_the_route_the_forward_took():
+    """The mask buffer edited between forward and backward: the backward step takes the route the
+    forward recorded in its log-sum-exp (all values: fused; no elements: op by op) and never
+    asks about the buffer again. Fused forward + punched mask -> fused backward with the causal
+    gradients; op-by-op forward + repaired mask -> op-by-op backward, finite gradients."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    calls = {"fwd": 0, "bwd": 0}
+    real_f, real_b = hip_ops.attention, hip_ops.attention_backward
+
+    def fwd(*a, **k):
+        calls["fwd"] += 1
+        return real_f(*a, **k)
+
+    def bwd(*a, **k):
+        calls["bwd"] += 1
+        return real_b(*a, **k)
+
+    hip_ops.attention, hip_ops.attention_backward = fwd, bwd
+    idx, targets = seeded_tokens(2, 64, seed=0), seeded_tokens(2, 64, seed=1)
+
+    def masks(model):
+        return [b for n, b in model.named_buffers() if n.endswith("bias") and b.dim() == 4]
+
+    ref = build_gpt2_small(seed=0, n_layer=2).double()
+    _loss(ref, idx, targets).backward()
+    model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).cuda()
+    loss = _loss(torch.compile(model, backend=mojo_backend), idx.cuda(), targets.cuda())
+    assert calls == {"fwd": 2, "bwd": 0}
+    for buf in masks(model):           # through .data: autograd's version check does not see it
+        buf.data[..., 5, 40:50] = 1
+    loss.backward()
+    assert calls == {"fwd": 2, "bwd": 2}
+    for (name, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        scale = q.grad.abs().max().item() + 1e-12
+        err = (p.grad.double().cpu() - q.grad).abs().max().item()
+        assert err <= 6e-2 * scale, (name, err / scale)
+    torch._dynamo.reset()
+
+    calls["fwd"] = calls["bwd"] = 0
+    model = build_gpt2_small(seed=0, n_layer=2).to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        for buf in masks(model):
+            buf[..., 5, 40:50] = 1
+    loss = _loss(torch.compile(model, backend=mojo_backend), idx.cuda(), targets.cuda())
+    assert calls == {"fwd": 0, "bwd": 0}
+    for buf in masks(model):
+        buf.data[..., 5, 40:50] = 0
+    loss.backward()
+    assert calls == {"fwd": 0, "bwd": 0}
+    assert all(torch.isfinite(p.grad).all().item() for p in model.parameters())
+    torch._dynamo.reset()
+
+
 def sdpa_training_graph_runs_the_fused_forward_and_backward():
     """F.scaled_dot_product_attention on bf16 tensors reaches a training graph as
     aten::_scaled_dot_product_flash_attention and its backward op: both run on the fused kernels

@@ -574,21 +574,33 @@ namespace tmb {
 constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mutex;
 static void* g_scratch_ptr[kMaxDevices] = {};
+static int g_scratch_rc[kMaxDevices] = {};   // a failed lookup is remembered, not retried
 
-// Device address of `scratch` on the current device, looked up once per device.
-static int static_scratch(void** ptr) {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
+// Device address of `scratch` on the device `stream` belongs to (the current device for the
+// null stream), looked up once per device with that device current.
+static int static_scratch(hipStream_t stream, void** ptr) {
+  int current = -1;
+  hipError_t e = hipGetDevice(&current);
   if (e != hipSuccess) return static_cast<int>(e);
+  int dev = current;
+  if (stream != nullptr) {
+    hipDevice_t of_stream = 0;
+    e = hipStreamGetDevice(stream, &of_stream);
+    if (e != hipSuccess) return static_cast<int>(e);
+    dev = static_cast<int>(of_stream);
+  }
   if (dev < 0 || dev >= kMaxDevices) return TMB_ERR_UNSUPPORTED;
+  // Kernels are launched on the current device: a stream of another one cannot take them.
+  if (dev != current) return TMB_ERR_INVALID_ARGUMENT;
   std::lock_guard<std::mutex> guard(g_scratch_mutex);
-  if (g_scratch_ptr[dev] == nullptr) {
+  if (g_scratch_ptr[dev] == nullptr && g_scratch_rc[dev] == 0) {
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) return static_cast<int>(e);
-    if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
-    g_scratch_ptr[dev] = p;
+    if (e != hipSuccess) g_scratch_rc[dev] = static_cast<int>(e);
+    else if (p == nullptr) g_scratch_rc[dev] = static_cast<int>(hipErrorInvalidSymbol);
+    else g_scratch_ptr[dev] = p;
   }
+  if (g_scratch_rc[dev] != 0) return g_scratch_rc[dev];
   *ptr = g_scratch_ptr[dev];
   return TMB_OK;
 }
@@ -603,7 +615,7 @@ extern "C" int tmb_reduce_rows_static(void* out, const void* in, int64_t rows, i
   if (need == 0) return tmb_reduce_rows(out, in, rows, cols, op, dtype, nullptr, 0, stream);
   if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;
   void* ws = nullptr;
-  const int rc = tmb::static_scratch(&ws);
+  const int rc = tmb::static_scratch(static_cast<hipStream_t>(stream), &ws);
   if (rc != TMB_OK) return rc;
   // Every partial the second stage reads is written by the first stage of the same call, so
   // nothing in the array has to start at zero.

@@ -34,3 +34,13 @@ def round_like_unfused() -> bool:
     unfused one. Off by default: a fused epilogue stays in float32 up to its one cast, and a
     16-bit graph keeps its residual stream in float32 between the blocks."""
     return _flag("ROUND_LIKE_UNFUSED")
+
+
+def cache_host_parameters() -> bool:
+    """Graphs over host tensors: keep the device copy of each ``nn.Parameter`` between calls
+    (revalidated by data pointer and version counter). Off by default, because writes that
+    bypass the version counter (``p.data.mul_()``, writes through ``p.numpy()``) would keep the
+    stale copy in use; with the switch off every call uploads what the host tensors hold at that
+    moment, as the reference's aliasing buffer import sees them
+    (torch_compile_backend/compiler.py:535-566)."""
+    return _flag("CACHE_HOST_PARAMETERS")

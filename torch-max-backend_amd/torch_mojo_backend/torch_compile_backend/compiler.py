@@ -46,8 +46,8 @@ from torch_mojo_backend.aten_functions import (
     DECOMPOSITION_TABLE,
     MAPPING_TORCH_ATEN_TO_MOJO,
 )
-from torch_mojo_backend.flags import (debug_graph, profiling_enabled, round_like_unfused,
-                                      verbose_enabled)
+from torch_mojo_backend.flags import (cache_host_parameters, debug_graph, profiling_enabled,
+                                      round_like_unfused, verbose_enabled)
 from torch_mojo_backend.torch_compile_backend.utils import get_accelerators, get_error_message
 
 __all__ = ["mojo_backend", "MojoCompilerError", "MAPPING_TORCH_ATEN_TO_MOJO", "get_accelerators",
@@ -502,17 +502,27 @@ class _GraphFactory:
                 plans[user] = ("wide_ln", val.dtype)
 
     def _prewarm_causal_verdicts(self, graph: torch.fx.Graph, plans: dict) -> None:
-        """The fused softmax / attention steps ask whether their mask buffer is causal, which
-        costs one device synchronisation per buffer. Where the buffer's values are known while
-        the program is built (module attributes, real example inputs) the question is answered
-        here, so that no step of a running graph synchronises for it."""
+        """The fused softmax / attention steps ask whether their mask buffer is causal. The
+        question is answered here, while the program is built, for every buffer whose values are
+        at hand (module attributes; graph inputs, for which dynamo's real example tensors stand
+        in where the compiler itself was handed fake ones), so that no step of a running graph
+        compares values or synchronises for it. A buffer that only shows up at run time runs the
+        unfused ops. Host buffers get their verdict on the host tensor; it travels with each
+        device copy (`_on_device`)."""
         from torch._subclasses.fake_tensor import FakeTensor
 
         placeholders = [n for n in graph.nodes if n.op == "placeholder"]
-        for node, plan in plans.items():
+        examples = _real_examples_for(placeholders, self.example_inputs)
+        asked = dict(plans)
+        for node in graph.nodes:   # the fused forward step of a training graph asks as well
+            if node.op == "call_function" and node.target is attention_train_forward:
+                asked[node] = ("attention",) + tuple(node.args)
+        for node, plan in asked.items():
             if plan is None or plan[0] not in ("softmax", "attention"):
                 continue
             root, slices = (plan[3], plan[4]) if plan[0] == "softmax" else (plan[5], plan[6])
+            if not isinstance(root, torch.fx.Node):
+                continue
             value = None
             if root.op == "get_attr":
                 value = graph.owning_module
@@ -520,12 +530,12 @@ class _GraphFactory:
                     value = getattr(value, part, None)
             elif root.op == "placeholder" and root in placeholders:
                 pos = placeholders.index(root)
-                if pos < len(self.example_inputs):
-                    value = self.example_inputs[pos]
+                if pos < len(examples):
+                    value = examples[pos]
             if not isinstance(value, torch.Tensor) or isinstance(value, FakeTensor):
                 continue
-            if self.run_device is not None:
-                value = _on_device(value, self.run_device)
+            if value.device.type == "mojo":
+                value = value._holder
             scores = (plan[1] if plan[0] == "softmax" else None)
             val = scores.meta.get("val") if scores is not None else None
             if plan[0] == "attention":
@@ -533,11 +543,14 @@ class _GraphFactory:
                 shape = None if q is None or k is None else (q.shape[2], k.shape[2])
             else:
                 shape = None if val is None or val.dim() < 2 else tuple(val.shape[-2:])
-            if shape is None or not all(isinstance(d, int) for d in shape):
-                continue
+            if shape is not None and not all(isinstance(d, int) for d in shape):
+                shape = None     # symbolic sizes: the verdict about the whole buffer serves them
+            if shape is not None and not all(isinstance(v, (int, type(None)))
+                                             for piece in slices for v in piece):
+                shape = None
             try:
-                _causal_q_len(value, slices, shape)
-            except Exception:  # noqa: BLE001 - the step asks again at run time
+                _take_causal_verdict(value, slices if shape is not None else None, shape)
+            except Exception:  # noqa: BLE001 - without a verdict the step runs its ops unfused
                 pass
 
     def create_graph(self, graph: torch.fx.Graph):
@@ -583,8 +596,8 @@ class _GraphFactory:
                 value = owner
                 for part in node.target.split("."):
                     value = getattr(value, part)
-                if self.run_device is not None and isinstance(value, torch.Tensor):
-                    value = _on_device(value, self.run_device)
+                # a host or mojo tensor stays what it is here and crosses to the device at each
+                # call (`BaseMaxCompiler.__call__`), so later writes to it are seen
                 self.constants.append((self.slots[node.name], value))
             elif node.op == "call_function":
                 key, fn = self.resolve(idx, node)
@@ -656,17 +669,89 @@ def _fused_addmm_gelu(input, mat1, mat2, *, approximate="none", round_like_unfus
     return _BUILTIN_GELU(_BUILTIN_ADDMM(input, mat1, mat2), approximate=approximate)
 
 
-# The verdict about a mask buffer rides on the buffer tensor itself as an attribute
-# (version counter, slices and shapes, verdict); verdict = query length if the sliced buffer is a
-# causal mask (nonzero exactly where column <= row), else 0. Checking costs one device sync, once
-# per buffer object and shape (at graph build time where the values are known by then). The
-# attribute dies with the tensor, so a new tensor that reuses the address of a dead one starts
-# without a verdict; the version counter catches in-place edits of the buffer.
+# The verdict about a mask buffer rides on the buffer tensor itself as an attribute: the version
+# counter and layout it was taken at, one verdict per (slices, score shape) asked about (the query
+# length if the sliced buffer is a causal mask, i.e. nonzero exactly where column <= row, else 0)
+# and one about the whole buffer ("its last two dimensions are such a mask, everything in front has
+# size 1": then so is every slice of them that starts at 0 with step 1, whatever sizes a graph
+# with dynamic shapes asks for later). Taking a verdict compares values, which on a device buffer
+# costs a synchronisation: it happens while the step program is built, never in a running step.
+# A step that meets a buffer without a valid verdict (first seen at run time, or edited in place
+# since: the version counter differs) runs its ops unfused. The attribute dies with the tensor,
+# so a new tensor that reuses the address of a dead one starts without a verdict.
 _CAUSAL_ATTR = "_tmb_causal_verdict"
 
 
-def _causal_q_len(root: torch.Tensor, slices: tuple, x) -> int:
-    """`x`: the score tensor, or just its last two sizes (q_len, kv_len)."""
+def _verdict_key(root: torch.Tensor) -> tuple:
+    return (tuple(root.shape), tuple(root.stride()), root.dtype, root.data_ptr())
+
+
+def _verdict_entry(root: torch.Tensor):
+    entry = getattr(root, _CAUSAL_ATTR, None)
+    if entry is not None and entry[0] == root._version and entry[1] == _verdict_key(root):
+        return entry
+    return None
+
+
+def _is_causal(block: torch.Tensor, q: int, cols: int) -> bool:
+    # real arithmetic on a real tensor, also while a graph is being compiled under fake tensors
+    from torch.utils._python_dispatch import _disable_current_modes
+
+    with _disable_current_modes():
+        keep = torch.ones(q, cols, dtype=torch.bool, device=block.device).tril()
+        return bool(torch.equal(block.reshape(q, cols) != 0, keep))
+
+
+def _take_causal_verdict(root: torch.Tensor, slices: Optional[tuple], x_shape: Optional[tuple]) -> int:
+    """Compares values (a synchronisation for a device buffer) and stores what it finds on the
+    tensor. With `slices` / `x_shape` None only the verdict about the whole buffer is taken."""
+    entry = _verdict_entry(root)
+    if entry is None:
+        whole = root.dim() >= 2 and root.numel() == root.shape[-2] * root.shape[-1] and \
+            root.numel() > 0 and _is_causal(root, root.shape[-2], root.shape[-1])
+        entry = (root._version, _verdict_key(root), {}, whole)
+        try:
+            setattr(root, _CAUSAL_ATTR, entry)
+        except (AttributeError, RuntimeError):
+            pass
+    if slices is None or x_shape is None:
+        return 0
+    ask = (slices, tuple(x_shape))
+    if ask not in entry[2]:
+        from torch.utils._python_dispatch import _disable_current_modes
+
+        with _disable_current_modes():
+            sub = root
+            for dim, start, end, step in slices:
+                sub = sub[(slice(None),) * (dim % sub.dim()) + (slice(start, end, step),)]
+            q, cols = ask[1]
+            verdict = 0
+            if sub.dim() >= 2 and tuple(sub.shape[-2:]) == (q, cols) and sub.numel() == q * cols \
+                    and q * cols > 0 and _is_causal(sub, q, cols):
+                verdict = q
+        entry[2][ask] = verdict
+    return entry[2][ask]
+
+
+def _sliced_from_origin(root: torch.Tensor, slices: tuple) -> Optional[tuple]:
+    """Sizes of the last two dimensions after `slices`, if every slice starts at 0 with step 1
+    (arithmetic on sizes only); None otherwise."""
+    shape = list(root.shape)
+    for dim, start, end, step in slices:
+        dim = dim % len(shape)
+        if start not in (0, None) or step not in (1, None):
+            return None
+        size = shape[dim]
+        if end is not None:
+            end = int(end)
+            size = max(0, min(size, end if end >= 0 else size + end))
+        shape[dim] = size
+    return tuple(shape[-2:])
+
+
+def _causal_q_len(root: torch.Tensor, slices: tuple, x, check: bool = True) -> int:
+    """`x`: the score tensor, or just its last two sizes (q_len, kv_len). With `check` False (every
+    call from a running step) the answer comes from verdicts taken earlier or is 0."""
     if isinstance(x, torch.Tensor):
         if not (x.is_cuda and x.dim() >= 2):
             return 0
@@ -675,24 +760,30 @@ def _causal_q_len(root: torch.Tensor, slices: tuple, x) -> int:
         x_shape = tuple(x)
     if not (isinstance(root, torch.Tensor) and root.is_cuda):
         return 0
-    what = (tuple(root.shape), tuple(root.stride()), root.dtype, root.data_ptr(), slices, x_shape)
-    entry = getattr(root, _CAUSAL_ATTR, None)
-    if entry is not None and entry[0] == root._version and entry[1] == what:
-        return entry[2]
-    sub = root
-    for dim, start, end, step in slices:
-        sub = sub[(slice(None),) * (dim % sub.dim()) + (slice(start, end, step),)]
-    q, cols = x_shape
-    verdict = 0
-    if sub.dim() >= 2 and tuple(sub.shape[-2:]) == (q, cols) and sub.numel() == q * cols:
-        keep = torch.ones(q, cols, dtype=torch.bool, device=sub.device).tril()
-        if bool(torch.equal(sub.reshape(q, cols) != 0, keep)):
-            verdict = q
+    x_shape = tuple(int(d) for d in x_shape)
+    if check:
+        return _take_causal_verdict(root, slices, x_shape)
+    entry = _verdict_entry(root)
+    if entry is None:
+        return 0
+    known = entry[2].get((slices, x_shape))
+    if known is not None:
+        return known
+    if entry[3] and _sliced_from_origin(root, slices) == x_shape:
+        return x_shape[0]
+    return 0
+
+
+def _carry_causal_verdict(source: torch.Tensor, copy: torch.Tensor) -> None:
+    """A verdict taken on a host buffer holds for the device copy made of it just now."""
+    entry = _verdict_entry(source)
+    if entry is None or tuple(copy.shape) != tuple(source.shape) or \
+            tuple(copy.stride()) != tuple(source.stride()):
+        return
     try:
-        setattr(root, _CAUSAL_ATTR, (root._version, what, verdict))
+        setattr(copy, _CAUSAL_ATTR, (copy._version, _verdict_key(copy), entry[2], entry[3]))
     except (AttributeError, RuntimeError):
         pass
-    return verdict
 
 
 def _fused_masked_softmax(x, scale, root, slices, dim):
@@ -700,7 +791,7 @@ def _fused_masked_softmax(x, scale, root, slices, dim):
     from torch_mojo_backend.eager_kernels import hip_ops
 
     if isinstance(x, torch.Tensor) and x.is_cuda and x.dtype in hip_ops.FLOAT_DTYPES:
-        q_len = _causal_q_len(root, slices, x)
+        q_len = _causal_q_len(root, slices, x, check=False)
         if q_len:
             # round_scaled: same bits as the separate mul kernel would have handed on
             return hip_ops.softmax_scaled(x, scale, causal_q_len=q_len, round_scaled=True)
@@ -756,7 +847,7 @@ def _fused_attention(q, k, v, scale, root, slices):
     b, h, t, d = q.shape
     s_len = k.shape[2]
     if scale > 0 and hip_ops.attention_supported(q, k, v) and \
-            _causal_q_len(root, slices, (t, s_len)) == t:
+            _causal_q_len(root, slices, (t, s_len), check=False) == t:
         return hip_ops.attention(q, k, v, scale, True)
     # the unfused chain, op by op as the graph had it
     flat = lambda x: x.expand(x.shape).clone(memory_format=torch.contiguous_format).view(  # noqa: E731
@@ -771,7 +862,7 @@ def _attention_fused_ok(q, k, v, scale, root, slices) -> bool:
     from torch_mojo_backend.eager_kernels import hip_ops
 
     return scale > 0 and hip_ops.attention_supported(q, k, v) and \
-        _causal_q_len(root, slices, (q.shape[2], k.shape[2])) == q.shape[2]
+        _causal_q_len(root, slices, (q.shape[2], k.shape[2]), check=False) == q.shape[2]
 
 
 def _attention_probabilities(q, k, scale, root, slices):
@@ -788,8 +879,9 @@ def attention_train_forward(q, k, v, scale, root, slices):
     """The attention chain of a training graph as one step: (out [batch, tokens, heads, head_dim]
     contiguous, float32 log-sum-exp [batch, heads, tokens]). The fused kernel takes the call when
     the mask buffer is causal and the operands are 16-bit heads of 64; otherwise the chain runs
-    op by op and the log-sum-exp stays unwritten (the backward step then takes the same route:
-    both ask the same question about the same operands)."""
+    op by op and the log-sum-exp comes back with no elements, which is how the backward step
+    knows the route the forward took (it never asks about the mask buffer again: the buffer may
+    have changed in between)."""
     from torch_mojo_backend.eager_kernels import hip_ops
 
     b, h, t, d = q.shape
@@ -798,7 +890,7 @@ def attention_train_forward(q, k, v, scale, root, slices):
     probs, flat = _attention_probabilities(q, k, scale, root, slices)
     ctx = _BUILTIN_BMM(probs.view(b * h, t, k.shape[2]), flat(v)).view(b, h, t, d)
     return (ctx.transpose(1, 2).clone(memory_format=torch.contiguous_format),
-            torch.empty((b, h, t), dtype=torch.float32, device=q.device))
+            torch.empty((0,), dtype=torch.float32, device=q.device))
 
 
 def _in_layout(x, layout):
@@ -829,7 +921,8 @@ def attention_train_backward(grad_out, q, k, v, out, lse, scale, root, slices, l
     b, h, t, d = q.shape
     s_len = k.shape[2]
     packed = isinstance(layouts, str)
-    if _attention_fused_ok(q, k, v, scale, root, slices):
+    # a log-sum-exp of b*h*t values means the forward ran the fused kernel: its backward matches
+    if lse.numel() == b * h * t and lse.numel() > 0:
         g = grad_out if grad_out.stride(3) == 1 and grad_out.data_ptr() % 16 == 0 and \
             all(st % 8 == 0 for st in grad_out.stride()[:3]) else grad_out.contiguous()
         if packed:
@@ -903,36 +996,90 @@ def _graph_home(gm: torch.fx.GraphModule, example_inputs: list) -> str:
     return "cpu"
 
 
-# Parameters of a module that lives on the host are the same tensor objects on every call: they
-# cross PCIe once, not once per call (the reference caches its imported buffers per tensor object
-# as well, :535-566). The copy rides on the host tensor itself (an attribute: it dies with the
-# tensor, and no weak reference gets in the way of torch.utils.swap_tensors); the version counter
-# catches in-place updates, the data pointer a swapped storage.
+# A graph over host tensors uploads what they hold at every call: the reference imports host
+# buffers by aliasing them (:535-566), so any write to a parameter or input is seen by the next
+# call, including writes that leave the version counter alone (`p.data.mul_()`, writes through
+# `p.numpy()`). With TORCH_MOJO_BACKEND_CACHE_HOST_PARAMETERS=1 the copy of an nn.Parameter is kept
+# on the host tensor itself (an attribute: it dies with the tensor, and no weak reference gets in
+# the way of torch.utils.swap_tensors) and reused while data pointer and version counter stand;
+# `invalidate_device_copies` drops such copies after a write the counter does not see.
 _COPY_ATTR = "_tmb_device_copy"
 _DEVICE_COPIES = {"made": 0, "reused": 0}   # counters, for tests and diagnostics
 
 
 def _on_device(t: torch.Tensor, device: torch.device) -> torch.Tensor:
     """`t` as a HIP tensor: mojo wrappers hand over their holder (zero-copy), host tensors are
-    copied (parameters and large tensors keep their copy), HIP tensors pass through."""
+    copied (at every call, unless parameter copies are kept, see above), HIP tensors pass
+    through. A causal-mask verdict taken on the host tensor travels with the copy."""
     kind = t.device.type
     if kind == "cuda":
         return t
     if kind == "mojo":
         return t._holder
-    entry = getattr(t, _COPY_ATTR, None)
-    if entry is not None and entry[0] == t.data_ptr() and entry[1] == t._version \
-            and entry[2].device == device:
-        _DEVICE_COPIES["reused"] += 1
-        return entry[2]
+    keep = isinstance(t, torch.nn.Parameter) and cache_host_parameters()
+    if keep:
+        entry = getattr(t, _COPY_ATTR, None)
+        if entry is not None and entry[0] == t.data_ptr() and entry[1] == t._version \
+                and entry[2].device == device:
+            _DEVICE_COPIES["reused"] += 1
+            return entry[2]
     copy = t.detach().to(device)
-    if isinstance(t, torch.nn.Parameter) or t.numel() >= 4096:
+    if keep:
         try:
             setattr(t, _COPY_ATTR, (t.data_ptr(), t._version, copy))
             _DEVICE_COPIES["made"] += 1
         except (AttributeError, RuntimeError):
             pass
+    _carry_causal_verdict(t, copy)
     return copy
+
+
+def invalidate_device_copies(*owners) -> int:
+    """Drops the kept device copies of the given host tensors, or of every parameter and buffer
+    of the given modules; returns how many were dropped. For use after a write that the version
+    counter does not record while TORCH_MOJO_BACKEND_CACHE_HOST_PARAMETERS=1."""
+    dropped = 0
+    for owner in owners:
+        tensors = [owner] if isinstance(owner, torch.Tensor) else \
+            list(owner.parameters()) + list(owner.buffers())
+        for t in tensors:
+            if getattr(t, _COPY_ATTR, None) is not None:
+                delattr(t, _COPY_ATTR)
+                dropped += 1
+    return dropped
+
+
+# aot_autograd hands its compilers fake tensors; the tensors dynamo called the backend with are
+# real. `mojo_backend` leaves them here while aot_autograd runs, for build-time questions about
+# values (is this buffer a causal mask?).
+_REAL_EXAMPLE_INPUTS: List[Any] = []
+
+
+def _real_examples_for(placeholders: list, example_inputs: list) -> list:
+    """Per placeholder, a tensor with real values or None: the compiler's own example input if it
+    is real, else dynamo's tensor at the same position, provided the graph has exactly dynamo's
+    inputs and that tensor has the placeholder's shape, dtype and device (aot_autograd keeps the
+    order of a forward graph's inputs; anything that does not line up is left out)."""
+    from torch._subclasses.fake_tensor import FakeTensor
+
+    out: list = []
+    real = _REAL_EXAMPLE_INPUTS[-1] if _REAL_EXAMPLE_INPUTS else None
+    lined_up = real is not None and len(real) == len(placeholders)
+    for pos, node in enumerate(placeholders):
+        value = example_inputs[pos] if pos < len(example_inputs) else None
+        if isinstance(value, torch.Tensor) and not isinstance(value, FakeTensor):
+            out.append(value)
+            continue
+        cand = real[pos] if lined_up else None
+        meta = node.meta.get("val")
+        if isinstance(cand, torch.Tensor) and not isinstance(cand, FakeTensor) and \
+                isinstance(meta, torch.Tensor) and cand.dtype == meta.dtype and \
+                cand.device == meta.device and all(isinstance(d, int) for d in meta.shape) and \
+                tuple(cand.shape) == tuple(meta.shape):
+            out.append(cand)
+        else:
+            out.append(None)
+    return out
 
 
 def _hip_available() -> bool:
@@ -1001,8 +1148,12 @@ class BaseMaxCompiler:
         else:
             for slot, value in zip(program.input_slots, args):
                 env[slot] = _on_device(value, run_device) if isinstance(value, torch.Tensor) else value
-        for slot, value in program.constants:
-            env[slot] = value
+        if run_device is None:
+            for slot, value in program.constants:
+                env[slot] = value
+        else:
+            for slot, value in program.constants:
+                env[slot] = _on_device(value, run_device) if isinstance(value, torch.Tensor) else value
         check = debug_graph()
         pads = self.pad_reuse_module
         if pads is not None:
@@ -1327,10 +1478,14 @@ def attention_recompute_partition(joint_module, joint_inputs, *, num_fwd_outputs
 
 class mojo_backend:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs: list):
-        self.func_to_execute = aot_autograd(
-            fw_compiler=boxed_func, partition_fn=attention_recompute_partition,
-            decompositions=DECOMPOSITION_TABLE
-        )(gm, example_inputs)
+        _REAL_EXAMPLE_INPUTS.append(list(example_inputs))
+        try:
+            self.func_to_execute = aot_autograd(
+                fw_compiler=boxed_func, partition_fn=attention_recompute_partition,
+                decompositions=DECOMPOSITION_TABLE
+            )(gm, example_inputs)
+        finally:
+            _REAL_EXAMPLE_INPUTS.pop()
 
     def __call__(self, *args) -> list:
         result = self.func_to_execute(*args)
