@@ -334,6 +334,20 @@ def main() -> int:
         sweep[name]["copy_us_same_bytes"] = round(ms * 1e3, 2)
         sweep[name]["vs_copy"] = round(ms * 1e3 / sweep[name]["us"], 3)
 
+    def with_read(name, nbuf, in_ptrs, nbytes):
+        """Beside a reduction's row: tmb_read_bytes over the same buffers (the same bytes read by
+        a kernel that keeps nothing), timed in the same run."""
+        state = {"i": 0}
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+        def step():
+            lib.tmb_read_bytes(in_ptrs[state["i"] % nbuf], nbytes, sink.data_ptr(), stream)
+            state["i"] += 1
+
+        _, ms = timed(step, 40, 8)
+        sweep[name]["read_us_same_bytes"] = round(ms * 1e3, 2)
+        sweep[name]["vs_read"] = round(ms * 1e3 / sweep[name]["us"], 3)
+
     if want in ("all", "attn"):
         # attention of the GPT-2 workload (B=32, H=12, T=1024, head_dim 64, bf16), q/k/v as the
         # strided thirds of the packed projection, exactly as the compiled graph hands them over
@@ -507,7 +521,7 @@ def main() -> int:
         bufs = rotating(lambda i: gen((rows, cols), 40 + i, torch.float32), rows * cols * 4)
         in_ptrs = [x_.data_ptr() for x_ in bufs]
         out_idx = torch.empty(rows, dtype=torch.int64, device=dev)
-        ws_bytes = lib.tmb_reduce_workspace_bytes(rows, cols, ek.F32)
+        ws_bytes = lib.tmb_argmax_workspace_bytes(rows, cols, ek.F32)
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
 
         def cpu_argmax():
@@ -520,6 +534,7 @@ def main() -> int:
                                               ws.data_ptr(), ws_bytes, stream),
                 rows * cols * 4 + rows * 8, steps=100, cpu_fn=cpu_argmax)
         assert torch.equal(out_idx, torch.argmax(bufs[(99 + 8) % len(bufs)], dim=1))
+        with_read(f"argmax_fp32_{rows}x{cols}", len(bufs), in_ptrs, rows * cols * 4)
         del bufs
 
     # ------------------------------------------------------------------ backward twins

@@ -106,8 +106,10 @@ size_t tmb_reduce_cols_workspace_bytes(int64_t rows, int64_t cols, int dtype);
 int tmb_reduce_cols(void* out, const void* in, int64_t rows, int64_t cols, int op, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes of device workspace `tmb_reduce_rows` / `tmb_argmax_rows` need for a shape (may be 0). */
+/* Bytes of device workspace `tmb_reduce_rows` needs for a shape (may be 0). */
 size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+/* The same for `tmb_argmax_rows`, whose rows are cut into smaller pieces (may be 0). */
+size_t tmb_argmax_workspace_bytes(int64_t rows, int64_t cols, int dtype);
 
 /* Row reduction of [rows, cols] (cols contiguous) to [rows]; a full reduction is rows == 1.
  * Floats accumulate in fp32 and are cast once (F32/F16/BF16); I64 sums and I64/I32 maxima use
@@ -144,7 +146,9 @@ int tmb_reduce_rows_static(void* out, const void* in, int64_t rows, int64_t cols
 
 /* First-occurrence argmax of every row of [rows, cols] to int64 [rows]; NaN counts as the
  * maximum (first NaN wins), otherwise greater value wins and equal values keep the lower index
- * at every stage of the tree. `dtype` in {F32,F16,BF16,I64,I32}.
+ * at every stage of the tree. `dtype` in {F32,F16,BF16,I64,I32}. Long rows are cut into pieces
+ * whose (value, index) partials (16 bytes each, tmb_argmax_workspace_bytes in total) a second
+ * launch combines in column order.
  * Replaces nn_ops.mojo:1424-1522 (`_argmax_rows`) behind ArgmaxSpec (nn_ops.mojo:2599-2653). */
 int tmb_argmax_rows(int64_t* out, const void* in, int64_t rows, int64_t cols, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream);
@@ -329,6 +333,12 @@ int tmb_pad_rows(void* out, const void* in, int64_t rows, int64_t row_len, int64
 /* Plain device copy kernel (16-byte vectors, grid-stride) — the bandwidth yardstick the
  * benchmark and the counter calibration use. No reference counterpart. */
 int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* stream);
+
+/* The read-only yardstick beside it: reads `bytes` (whole 16-byte vectors of them) once and
+ * writes nothing (`sink`, at least 4 bytes of device memory, is written only if a 16 KiB piece
+ * folds to one particular bit pattern). What a reduction over the same bytes is measured
+ * against. No reference counterpart. */
+int tmb_read_bytes(const void* in, size_t bytes, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -160,6 +160,99 @@ def test_argmax_shapes(shape):
     assert torch.equal(got, oracle.argmax_rows(x))
 
 
+# Rows of at least 2048 floating-point columns are cut into work units of 256 lanes, one 16-byte
+# vector at a time per lane; the cases below sit on every seam of that scheme: unit boundaries,
+# elements in front of / behind the whole vectors of a unit (odd pitches), units with a single
+# vector per lane and with seven, rows of exactly one unit, storage offsets.
+VEC_SHAPES = [(3, 2048), (5, 2049), (7, 4099), (2, 7168), (2, 7169), (4, 7233), (33, 14336), (9, 14337),
+              (512, 50257), (32, 50257), (1, 50257), (2048, 6151), (1, 1 << 20), (3, (1 << 21) + 5)]
+
+
+def _argmax_adversarial(shape, dtype, seed):
+    rows, cols = shape
+    x = seeded(shape, seed=seed).to(dtype)
+    g = torch.Generator().manual_seed(seed + 7)
+    pick = lambda n: torch.randint(0, cols, (n,), generator=g).tolist()   # noqa: E731
+    top = float(x.float().max()) + 1
+    for r in range(rows):
+        kind = r % 16
+        if kind == 0:      # tie between two random columns
+            a = pick(2)
+            x[r, a] = top
+        elif kind == 1:    # maximum in the first / last column
+            x[r, 0] = top
+        elif kind == 2:
+            x[r, cols - 1] = top
+        elif kind == 3:    # two NaN: the first wins, whatever else the row holds
+            a = pick(2)
+            x[r, a] = float("nan")
+            x[r, pick(1)] = float("inf")
+        elif kind == 4:    # the whole row equal
+            x[r] = 0.75
+        elif kind == 5:    # all -inf
+            x[r] = float("-inf")
+        elif kind == 6:    # -inf everywhere but one finite value
+            x[r] = float("-inf")
+            x[r, pick(1)] = -3.0
+        elif kind == 7:    # +inf twice, and a -inf (the sum check fires without any NaN)
+            a = pick(3)
+            x[r, a[:2]] = float("inf")
+            x[r, a[2]] = float("-inf")
+        elif kind == 8:    # zeros of both signs tie
+            x[r] = -0.0
+            x[r, pick(1)] = 0.0
+        elif kind == 9:    # NaN in the last column only
+            x[r, cols - 1] = float("nan")
+        elif kind == 10:   # a tie that straddles a unit boundary (units are multiples of 64 wide)
+            j = min(cols - 1, (cols // 2) // 64 * 64)
+            x[r, max(j - 1, 0)] = top
+            x[r, j] = top
+        elif kind == 11:   # negative NaN (sign bit set), as 0/0 produces on the host
+            x[r, pick(1)] = -float("nan")
+    return x
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", VEC_SHAPES)
+def test_argmax_vector_units_are_bit_exact(shape, dtype):
+    x = _argmax_adversarial(shape, dtype, seed=shape[1] % 977)
+    want = torch.argmax(x, dim=1)
+    got = _ops().argmax(_dev(x), 1, False).cpu()
+    bad = (got != want).nonzero().flatten().tolist()
+    assert not bad, f"{shape} {dtype}: rows {bad[:8]} got {got[bad[:8]].tolist()} want {want[bad[:8]].tolist()}"
+    if shape[0] * shape[1] <= 1 << 22:
+        assert torch.equal(got, oracle.argmax_rows(x))
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+def test_argmax_rows_that_start_anywhere(dtype):
+    """A view whose rows start 1 .. 9 elements into 16-byte vectors (storage offset, odd pitch)."""
+    base = seeded((6, 9001), seed=5).to(dtype)
+    for offset in (1, 2, 3, 5, 9):
+        flat = torch.zeros(6 * 9001 + offset, dtype=dtype)
+        flat[offset:] = base.reshape(-1)
+        dev = _dev(flat)[offset:].view(6, 9001)
+        assert dev.data_ptr() % 16 != 0 or offset * base.element_size() % 16 == 0
+        assert torch.equal(_ops().argmax(dev, 1, False).cpu(), torch.argmax(base, dim=1))
+
+
+def test_argmax_workspace_is_what_the_entry_point_asks_for():
+    ek = _ek()
+    L = ek.lib()
+    need = L.tmb_argmax_workspace_bytes(512, 50257, ek.F32)
+    assert need == 512 * 8 * 16                       # eight units per row, 16 bytes each
+    assert L.tmb_argmax_workspace_bytes(512, 50257, ek.I64) == L.tmb_reduce_workspace_bytes(512, 50257, ek.I64)
+    assert L.tmb_argmax_workspace_bytes(4096, 4096, ek.F32) == 0        # one unit per row
+    assert L.tmb_argmax_workspace_bytes(0, 4096, ek.F32) == 0
+    x = _dev(seeded((512, 50257), seed=1))
+    out = torch.empty(512, dtype=torch.int64, device=x.device)
+    small = torch.empty(need - 16, dtype=torch.uint8, device=x.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 512, 50257, ek.F32, small.data_ptr(),
+                             need - 16, stream) == ek.ERR_WORKSPACE
+    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 512, 50257, ek.F32, None, 0, stream) == ek.ERR_WORKSPACE
+
+
 def test_argmax_dim_none_keepdim_and_nan():
     x = seeded((7, 9, 11), seed=8)
     ops = _ops()

@@ -33,7 +33,11 @@ __device__ __forceinline__ float lanes_sum(float v) {
 //
 // The grid is persistent: about 16 waves per CU, each group walking rows with the grid's
 // stride, gamma and beta fetched once per lane (kept packed in their storage type) instead of
-// once per row. The input may be wider than the output (fp32 rows normalised into a 16-bit
+// once per row. A group's next row is requested right after the current row's stores; asking
+// for it earlier (as soon as the current row is unpacked into fp32 registers) was measured on
+// every geometry and changes nothing where the stores are non-temporal, except 4096-column fp32
+// rows, which lose 4 % (88 -> 92 us): the other waves of the CU already cover the latency.
+// The input may be wider than the output (fp32 rows normalised into a 16-bit
 // tensor: the residual stream of a 16-bit model kept in fp32); gamma and beta have the output's
 // type.
 template <typename TIn, typename TOut, int G, int VPL, bool STREAM, int BLOCK>
@@ -47,7 +51,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_rows_kernel(
   constexpr int SUB = G > 64 ? 64 : G;
   static_assert(BLOCK % G == 0 && GPB >= 1, "workgroup holds whole row groups");
   static_assert(sizeof(TOut) <= sizeof(TIn), "the output is never wider than the input");
-  __shared__ float slot[2][BLOCK / kWave];
+  __shared__ float slot[2][2][BLOCK / kWave];  // [row parity][statistic][wave]
 
   const int tid = threadIdx.x;
   const int g = tid / G, l = tid % G;
@@ -85,6 +89,10 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_rows_kernel(
   load_row(gid, raw);
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = it * total + gid;
+    // Rows alternate between two sets of LDS slots: a wave that writes a slot for row it + 2 has
+    // passed both barriers of row it + 1, which every wave reaches only after its last read of
+    // row it's slots. Two barriers per row instead of three.
+    float(&meet)[2][BLOCK / kWave] = slot[it & 1];
     float x[VPL][EPV];
     float s = 0.0f;
 #pragma unroll
@@ -98,11 +106,11 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_rows_kernel(
     }
     s = lanes_sum<SUB>(s);
     if constexpr (WPR > 1) {
-      if ((tid & 63) == 0) slot[0][wave] = s;
+      if ((tid & 63) == 0) meet[0][wave] = s;
       __syncthreads();
-      s = slot[0][g * WPR];
+      s = meet[0][g * WPR];
 #pragma unroll
-      for (int w = 1; w < WPR; ++w) s += slot[0][g * WPR + w];
+      for (int w = 1; w < WPR; ++w) s += meet[0][g * WPR + w];
     }
     float mean = s / n;
     float q = 0.0f;
@@ -118,11 +126,11 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_rows_kernel(
     }
     q = lanes_sum<SUB>(q);
     if constexpr (WPR > 1) {
-      if ((tid & 63) == 0) slot[1][wave] = q;
+      if ((tid & 63) == 0) meet[1][wave] = q;
       __syncthreads();
-      q = slot[1][g * WPR];
+      q = meet[1][g * WPR];
 #pragma unroll
-      for (int w = 1; w < WPR; ++w) q += slot[1][g * WPR + w];
+      for (int w = 1; w < WPR; ++w) q += meet[1][g * WPR + w];
     }
     const float var = q / n;
     const float rstd = 1.0f / sqrtf(var + eps);
@@ -162,7 +170,6 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_rows_kernel(
       }
     }
     if (it + 1 < iters) load_row(row + total, raw);
-    if constexpr (WPR > 1) __syncthreads();  // the slots are written again for the next row
   }
 }
 
@@ -220,8 +227,11 @@ static int launch_ln(TOut* out, float* mean, float* rstd, const TIn* x, const TO
     const int64_t walk = (max_grid + grid - 1) / grid;
     grid = (max_grid + walk - 1) / walk;
   }
+  // Non-temporal stores once input and output together are larger than the L2s (8 x 4 MB):
+  // measured 4-5 % faster on 100 ... 200 MB passes ([32768, 768] bf16: 20.3 -> 19.4 us,
+  // fp32: 37.0 -> 35.4 us), 10 % where the output alone is 134 MB.
   const bool stream_hint =
-      rows * cols * static_cast<int64_t>(sizeof(TIn) + sizeof(TOut)) >= (int64_t{256} << 20);
+      rows * cols * static_cast<int64_t>(sizeof(TIn) + sizeof(TOut)) >= (int64_t{64} << 20);
   const dim3 grid3(static_cast<unsigned>(grid)), block(BLOCK);
   const int c = static_cast<int>(cols);
   if (stream_hint)

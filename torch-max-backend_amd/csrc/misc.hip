@@ -232,6 +232,37 @@ extern "C" int tmb_gelu(void* out, const void* in, int64_t numel, int dtype, int
   }
 }
 
+namespace tmb {
+// The read half of copy_kernel: every block reads one contiguous 16 KiB piece and keeps nothing.
+// The loads stay alive through a store that only happens when the piece folds to one particular
+// 32-bit pattern.
+__global__ __launch_bounds__(256) void read_kernel(const uint4* __restrict__ in, size_t nvec,
+                                                   uint32_t* __restrict__ sink) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4* src = reinterpret_cast<const u32x4*>(in);
+  const size_t base = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  u32x4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    v[u] = __builtin_nontemporal_load(src + (base + u * 256 < nvec ? base + u * 256 : 0));
+  const u32x4 x = v[0] ^ v[1] ^ v[2] ^ v[3];
+  if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u && x[0] == 0x7f4a7c15u) sink[0] = x[1];
+}
+}  // namespace tmb
+
+extern "C" int tmb_read_bytes(const void* in, size_t bytes, void* sink, void* stream) {
+  if (bytes < 16) return TMB_OK;
+  if (in == nullptr || sink == nullptr) return TMB_ERR_INVALID_ARGUMENT;
+  if (!tmb::aligned16(in)) return TMB_ERR_UNSUPPORTED;
+  const size_t nvec = bytes / 16;
+  const size_t blocks = (nvec + 1023) / 1024;
+  if (blocks >= (size_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  tmb::read_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream)>>>(static_cast<const uint4*>(in), nvec,
+                                                         static_cast<uint32_t*>(sink));
+  return tmb::check_launch();
+}
+
 extern "C" int tmb_copy_bytes(void* out, const void* in, size_t bytes, void* stream) {
   if (bytes == 0) return TMB_OK;
   if (out == nullptr || in == nullptr) return TMB_ERR_INVALID_ARGUMENT;

@@ -495,10 +495,243 @@ __global__ __launch_bounds__(kFinalBlock) void argmax_final_kernel(int64_t* __re
   }
 }
 
+// ---------------------------------------------------------------------------
+// Argmax of floating-point rows, a vector at a time.
+//
+// The scan above spends six to seven instructions on every element (three compares, two
+// selects and their mask arithmetic), and a wave64 instruction occupies its SIMD for four
+// cycles: 25 M elements are 4-5 us of vector ALU time on the whole chip, next to 15 us of memory
+// time. Here a lane looks at one 16-byte vector at a time: the vector's maximum (v_max3),
+// one strict compare with the lane's maximum so far, and on "greater" the lane keeps that vector
+// (raw) and its number. Strict "greater" keeps the first vector that reached the lane's maximum,
+// and the first element equal to the maximum inside the kept vector is the lane's first
+// occurrence. v_max ignores NaN, so a float sum of everything the lane saw runs beside it: it is
+// NaN exactly when the lane saw a NaN or infinities of both signs, and then the whole workgroup
+// redoes its range with the exact scan (first NaN wins), reading it again. Half the instructions
+// per element, nothing kept in registers but one vector.
+//
+// Work units are small (256 lanes, at most seven vectors each, about 28 KB): measured on
+// [512, 50257] fp32, eight units per row plus the combining launch take 20 us where one
+// 1024-lane workgroup per row took 23 (the units alone 17; a plain read of the same bytes 15.7).
+// ---------------------------------------------------------------------------
+constexpr int kArgBlock = 256;
+constexpr int kArgMaxVectors = 7;  // per lane
+
+template <typename T>
+struct LaneBest {
+  float m;
+  Vec16<T> kept;
+  int u;
+  float sum;
+};
+
+template <typename T>
+__device__ __forceinline__ void lane_step(LaneBest<T>& t, const Vec16<T>& x, int u) {
+  constexpr int EPV = Vec16<T>::N;
+  float f[EPV];
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) f[e] = to_f32(x.v[e]);
+  float m = __builtin_fmaxf(f[0], f[1]);
+  float s = f[0] + f[1];
+#pragma unroll
+  for (int e = 2; e < EPV; e += 2) {
+    m = __builtin_fmaxf(__builtin_fmaxf(m, f[e]), f[e + 1]);
+    s += f[e] + f[e + 1];
+  }
+  const bool take = m > t.m;
+  t.m = take ? m : t.m;
+  const raw16_t xr = __builtin_bit_cast(raw16_t, x), kr = __builtin_bit_cast(raw16_t, t.kept);
+  raw16_t nr;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) nr[w] = take ? xr[w] : kr[w];
+  t.kept = __builtin_bit_cast(Vec16<T>, nr);
+  t.u = take ? u : t.u;
+  t.sum += s;
+}
+
+__device__ __forceinline__ int wave_min_i32(int v) {
+  v = min(v, dpp_i32<kDppQuadXor1>(v));
+  v = min(v, dpp_i32<kDppQuadXor2>(v));
+  v = min(v, dpp_i32<kDppRowHalfMirror>(v));
+  v = min(v, dpp_i32<kDppRowMirror>(v));
+  v = min(v, __shfl_xor(v, 16, kWave));
+  return min(v, __shfl_xor(v, 32, kWave));
+}
+
+// One workgroup per (row, split): columns [split * chunk, min(cols, (split + 1) * chunk)) of the
+// row, chunk <= kArgBlock * U vectors. splits == 1 writes the row's index, otherwise a
+// (value, index) partial for argmax_final_kernel.
+template <typename T, int U>
+__global__ __launch_bounds__(kArgBlock) void argmax_vec_kernel(int64_t* __restrict__ out,
+                                                               void* __restrict__ ws,
+                                                               const T* __restrict__ in,
+                                                               int64_t cols, int splits, int chunk) {
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int WAVES = kArgBlock / kWave;
+  constexpr int kNone = 0x7fffffff;
+  __shared__ float smax[WAVES];
+  __shared__ int sflag[WAVES];
+  __shared__ int soff[WAVES];
+  __shared__ BestSlot<float> sbest[WAVES];
+  const int tid = threadIdx.x, wave = tid >> 6;
+  const int64_t item = blockIdx.x;
+  const int64_t row = item / splits;
+  const int split = static_cast<int>(item - row * splits);
+  const int64_t c0 = static_cast<int64_t>(split) * chunk;
+  const T* p = in + row * cols + c0;
+  int n = static_cast<int>(cols - c0 < chunk ? cols - c0 : chunk);
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+  int head = static_cast<int>(((16u - (addr & 15u)) & 15u) / sizeof(T));
+  if (head > n) head = n;
+  const T* body = p + head;
+  const int nvec = (n - head) / EPV;
+  const int tail = head + nvec * EPV;
+  // up to EPV - 1 elements in front of the first and behind the last whole vector: one each for
+  // the first lanes. Lanes without one (and vector slots past the end, below) read element 0 /
+  // vector 0 again instead of branching: a copy can equal the maximum but never raise it, and a
+  // lane that kept a copy is recognised by its vector number.
+  const bool has_head = tid < head, has_tail = tail + tid < n;
+  const float hv = to_f32(__builtin_nontemporal_load(p + (has_head ? tid : 0)));
+  const float tv = to_f32(__builtin_nontemporal_load(p + (has_tail ? tail + tid : 0)));
+  Vec16<T> v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint32_t at = static_cast<uint32_t>(tid + u * kArgBlock);
+    v[u] = load_vec16_stream(body + static_cast<size_t>(at < static_cast<uint32_t>(nvec) ? at : 0u) * EPV);
+  }
+  const float ninf = -__builtin_inff();
+  LaneBest<T> t;
+  t.m = ninf;
+  t.kept = v[0];
+  t.u = -1;
+  t.sum = 0.0f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) lane_step(t, v[u], u);
+
+  // the lane's candidate, in ascending index order: head element, kept vector, tail element
+  float m = ninf;
+  int off = kNone;
+  if (tid < nvec) {
+    // u < 0: nothing exceeded -inf, so every element seen is -inf (or NaN: caught below) and the
+    // first of them is element 0 of the lane's first vector
+    const int u = t.u < 0 ? 0 : t.u;
+    const int vi = tid + u * kArgBlock;
+    if (vi < nvec) {
+      int e = EPV - 1;
+#pragma unroll
+      for (int k = EPV - 2; k >= 0; --k) e = to_f32(t.kept.v[k]) == t.m ? k : e;
+      if (t.u < 0) e = 0;
+      m = t.m;
+      off = head + vi * EPV + e;
+    }
+    // vi >= nvec: a copy of vector 0 exceeded everything this lane owns, so lane 0 holds a
+    // greater value and this lane cannot win
+  }
+  if (has_head && (off == kNone || !(m > hv))) { m = hv; off = tid; }
+  if (has_tail && (off == kNone || tv > m)) { m = tv; off = tail + tid; }
+  const float sum = t.sum + hv + tv;
+  const float wm = wave_reduce(m, MaxOp{});
+  const int wf = __any(sum != sum) ? 1 : 0;
+  if ((tid & 63) == 0) { smax[wave] = wm; sflag[wave] = wf; }
+  __syncthreads();
+  float M = smax[0];
+  int flag = sflag[0];
+#pragma unroll
+  for (int w = 1; w < WAVES; ++w) { M = __builtin_fmaxf(M, smax[w]); flag |= sflag[w]; }
+  if (flag == 0) {
+    off = (off != kNone && m == M) ? off : kNone;
+    off = wave_min_i32(off);
+    if ((tid & 63) == 0) soff[wave] = off;
+    __syncthreads();
+    if (tid == 0) {
+      int first = soff[0];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) first = min(first, soff[w]);
+      if (splits == 1) {
+        out[row] = first;
+      } else {
+        static_cast<BestSlot<float>*>(ws)[item] = BestSlot<float>{c0 + first, M};
+      }
+    }
+  } else {
+    Best<float> b = argmax_range<T, kArgBlock, 4>(p, n, tid, c0);
+    b = wave_best(b);
+    if ((tid & 63) == 0) sbest[wave] = BestSlot<float>{b.idx, b.val};
+    __syncthreads();
+    if (tid == 0) {
+      Best<float> r{sbest[0].val, sbest[0].idx};
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) r = best_combine(r, Best<float>{sbest[w].val, sbest[w].idx});
+      if (splits == 1) {
+        out[row] = r.idx;
+      } else {
+        static_cast<BestSlot<float>*>(ws)[item] = BestSlot<float>{r.idx, r.val};
+      }
+    }
+  }
+}
+
+// How a floating-point argmax is cut into work units: a pure function of the shape. Rows
+// shorter than kArgVecMinCols elements stay with the kernels above.
+constexpr int64_t kArgVecMinCols = 2048;
+struct ArgPlan {
+  int splits;
+  int chunk;    // elements
+  int vectors;  // per lane, upper bound
+};
+static bool argmax_vec_plan(int64_t rows, int64_t cols, int elem_size, ArgPlan* plan) {
+  if (rows <= 0 || cols < kArgVecMinCols || cols >= (int64_t{1} << 31) - 4096) return false;
+  const int64_t epv = 16 / elem_size;
+  const int64_t nvec = cols / epv;
+  const int64_t unit_max = static_cast<int64_t>(kArgBlock) * kArgMaxVectors;  // vectors
+  int64_t splits = (nvec + unit_max - 1) / unit_max;
+  // few rows: more, smaller units (down to one vector per lane) until about eight per CU exist
+  int64_t wanted = (2048 + rows - 1) / rows;
+  const int64_t finest = nvec / kArgBlock;
+  if (wanted > finest) wanted = finest;
+  if (splits < wanted) splits = wanted;
+  if (splits < 1) splits = 1;
+  int64_t chunk;
+  for (;; ++splits) {
+    chunk = ((cols + splits - 1) / splits + 63) / 64 * 64;
+    // a unit may start up to epv - 1 elements before its first whole vector
+    if (chunk / epv <= unit_max) break;
+  }
+  splits = (cols + chunk - 1) / chunk;
+  if (rows * splits >= (int64_t{1} << 31)) return false;
+  plan->splits = static_cast<int>(splits);
+  plan->chunk = static_cast<int>(chunk);
+  plan->vectors = static_cast<int>((chunk / epv + kArgBlock - 1) / kArgBlock);
+  return true;
+}
+
+template <typename T>
+static int launch_argmax_vec(int64_t* out, const T* in, int64_t rows, int64_t cols, const ArgPlan& plan,
+                             void* ws, size_t ws_bytes, hipStream_t stream) {
+  const int64_t items = rows * plan.splits;
+  if (plan.splits > 1 && (ws == nullptr || ws_bytes < static_cast<size_t>(items) * 16)) return TMB_ERR_WORKSPACE;
+  const dim3 grid(static_cast<unsigned>(items)), block(kArgBlock);
+#define TMB_ARG(U) argmax_vec_kernel<T, U><<<grid, block, 0, stream>>>(out, ws, in, cols, plan.splits, plan.chunk)
+  if (plan.vectors <= 1) TMB_ARG(1);
+  else if (plan.vectors <= 2) TMB_ARG(2);
+  else if (plan.vectors <= 4) TMB_ARG(4);
+  else TMB_ARG(kArgMaxVectors);
+#undef TMB_ARG
+  int rc = check_launch();
+  if (rc != 0 || plan.splits == 1) return rc;
+  argmax_final_kernel<T, 64><<<dim3(static_cast<unsigned>(rows)), dim3(64), 0, stream>>>(out, ws, rows, plan.splits);
+  return check_launch();
+}
+
 template <typename T>
 static int launch_argmax(int64_t* out, const void* in_, int64_t rows, int64_t cols, void* ws,
                          size_t ws_bytes, hipStream_t stream) {
   const T* in = static_cast<const T*>(in_);
+  if constexpr (__is_same(typename ArgTraits<T>::val_t, float)) {
+    ArgPlan vec;
+    if (argmax_vec_plan(rows, cols, static_cast<int>(sizeof(T)), &vec))
+      return launch_argmax_vec<T>(out, in, rows, cols, vec, ws, ws_bytes, stream);
+  }
   const SplitPlan plan = plan_splits(rows, cols);
   // At least one row per CU and only a few chunks per row: one 1024-thread workgroup per row does
   // the same work per thread in a single launch (the second stage alone costs 4-5 us).
@@ -535,6 +768,15 @@ extern "C" size_t tmb_reduce_workspace_bytes(int64_t rows, int64_t cols, int dty
   const tmb::SplitPlan plan = tmb::plan_splits(rows, cols);
   if (plan.splits == 1) return 0;
   return static_cast<size_t>(rows) * static_cast<size_t>(plan.splits) * 16;
+}
+
+extern "C" size_t tmb_argmax_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
+  if (rows <= 0 || cols <= 0) return 0;
+  const int elem = dtype == TMB_F32 ? 4 : (dtype == TMB_F16 || dtype == TMB_BF16 ? 2 : 0);
+  tmb::ArgPlan plan;
+  if (elem != 0 && tmb::argmax_vec_plan(rows, cols, elem, &plan))
+    return plan.splits == 1 ? 0 : static_cast<size_t>(rows) * static_cast<size_t>(plan.splits) * 16;
+  return tmb_reduce_workspace_bytes(rows, cols, dtype);
 }
 
 extern "C" int tmb_reduce_rows(void* out, const void* in, int64_t rows, int64_t cols, int op,

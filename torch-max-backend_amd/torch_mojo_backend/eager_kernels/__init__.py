@@ -20,7 +20,7 @@ F32, F16, BF16, I64, I32 = 0, 1, 2, 3, 4
 SUM, MEAN, AMAX = 0, 1, 2
 EPI_NONE, EPI_GELU_TANH, EPI_GELU_ERF = 0, 1, 2
 EPI_ROUND_LIKE_UNFUSED = 0x100  # flag: fused steps round where separate kernels would store
-ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED = -1, -2  # tmb_status values of include/tmb_hip.h
+ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_SCRATCH_LIMIT = -1, -2, -3, -4  # tmb_status (include/tmb_hip.h)
 
 # Every symbol include/tmb_hip.h declares, with its ctypes signature.
 _i64, _vp, _ci, _sz, _dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_double
@@ -32,6 +32,7 @@ SIGNATURES = {
     "tmb_softmax_rows_scaled": (_ci, [_vp, _vp, _i64, _i64, _ci, _flt, _ci, _i64, _vp]),
     "tmb_layer_norm_rows": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _dbl, _ci, _ci, _vp]),
     "tmb_reduce_workspace_bytes": (_sz, [_i64, _i64, _ci]),
+    "tmb_argmax_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_reduce_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),
     "tmb_reduce_rows_static": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp]),
     "tmb_argmax_rows": (_ci, [_vp, _vp, _i64, _i64, _ci, _vp, _sz, _vp]),
@@ -51,6 +52,7 @@ SIGNATURES = {
     "tmb_layer_norm_backward_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_layer_norm_backward_rows": (_ci, [_vp] * 8 + [_i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
+    "tmb_read_bytes": (_ci, [_vp, _sz, _vp, _vp]),
     "tmb_cat2_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "tmb_reduce_cols_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_reduce_cols": (_ci, [_vp, _vp, _i64, _i64, _ci, _ci, _vp, _sz, _vp]),

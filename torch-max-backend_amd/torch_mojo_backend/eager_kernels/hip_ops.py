@@ -743,8 +743,9 @@ def _reduce_geometry(x: torch.Tensor, dims: Sequence[int]):
     return moved, rows, cols, [x.shape[d] for d in kept]
 
 
-def _workspace(rows: int, cols: int, code: int, device) -> Tuple[Optional[torch.Tensor], int]:
-    nbytes = _ek.lib().tmb_reduce_workspace_bytes(rows, cols, code)
+def _workspace(rows: int, cols: int, code: int, device, argmax: bool = False) -> Tuple[Optional[torch.Tensor], int]:
+    lib = _ek.lib()
+    nbytes = (lib.tmb_argmax_workspace_bytes if argmax else lib.tmb_reduce_workspace_bytes)(rows, cols, code)
     if nbytes == 0:
         return None, 0
     return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
@@ -803,7 +804,7 @@ def argmax(x: torch.Tensor, dim: Optional[int], keepdim: bool) -> torch.Tensor:
         dims = [dim % rank] if rank else []
     moved, rows, cols, kept_shape = _reduce_geometry(x, dims)
     out = torch.empty(kept_shape, dtype=torch.int64, device=x.device)
-    ws, ws_bytes = _workspace(rows, cols, code, x.device)
+    ws, ws_bytes = _workspace(rows, cols, code, x.device, argmax=True)
     rc = _ek.lib().tmb_argmax_rows(out.data_ptr(), moved.data_ptr(), rows, cols, code,
                                    None if ws is None else ws.data_ptr(), ws_bytes, _stream())
     _check("tmb_argmax_rows", rc)
