@@ -129,6 +129,17 @@ def main() -> int:
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return wall, start.elapsed_time(end) / steps
 
+    def settle(fn, seconds=0.03):
+        """Untimed launches for `seconds` of wall time in front of a timed region: the first
+        launches after a pause (input generation, a CPU leg) run at whatever clock the idle chip
+        was left at, 10-15 % slower on the 100 us products, and the yardstick beside a row would
+        otherwise be measured on a warmer chip than the row itself."""
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(8):
+                fn()
+            sync()
+
     def cpu_time(fn, iters=3, warmup=1):
         for _ in range(warmup):
             fn()
@@ -233,11 +244,14 @@ def main() -> int:
             x = gen((m, k), 3, dtype)
             w = gen((n, k), 4, dtype).t() if trans_b else gen((k, n), 4, dtype)
             bs = gen((n,), 5, dtype)
+        settle(lambda: hip_ops.gemm(x, w, bs))
         _, ms = timed(lambda: hip_ops.gemm(x, w, bs), steps, 10)
         # yardstick, not part of the product: PyTorch-ROCm's own library GEMM on the same tensors
         if batch:
+            settle(lambda: torch.bmm(x, w))
             _, yard = timed(lambda: torch.bmm(x, w), max(steps // 2, 5), 5)
         else:
+            settle(lambda: torch.addmm(bs, x, w))
             _, yard = timed(lambda: torch.addmm(bs, x, w), max(steps // 2, 5), 5)
         bt = batch or 1
         size = x.element_size()

@@ -234,22 +234,155 @@ __global__ __launch_bounds__(1024) void softmax_long_rows_kernel(TOut* __restric
   if (edge >= 0) dst[edge] = from_f32<TOut>(LOG ? xt - lg : xt * inv);
 }
 
+// The same row kernel for rows that fit 64 registers per lane, so that two 1024-thread
+// workgroups share a CU and one row's stores run under the other's loads (the kernel above, with
+// 64 .. 128 registers, leaves a CU to one row at a time: 0.61-0.63 of the memory peak on
+// 16384 x 50257). 16-bit rows stay in their storage type (four registers per vector) and are
+// converted again in each of the three passes, with the exponential taken twice (one multiply and
+// one v_exp_f32 each for a 16-bit result). fp32 rows (transformed in place) would need 8 or 13
+// vectors per lane, which spills: they stay with the kernel above.
+template <typename TIn, typename TOut, int VPL, bool LOG, bool PEEL, bool STREAM>
+__global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* __restrict__ out,
+                                                                         const TIn* __restrict__ in,
+                                                                         int cols) {
+  constexpr int EPV = Vec16<TIn>::N;
+  constexpr int WAVES = 16;
+  constexpr bool IN_PLACE = sizeof(TIn) == 4;
+  static_assert(!PEEL || sizeof(TIn) == sizeof(TOut), "one offset for both rows");
+  static_assert(VPL * 4 <= 32, "the row must leave room for the rest in 64 registers");
+  __shared__ float slot[WAVES];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const float neg_inf = -__builtin_inff();
+  const TIn* src = in + static_cast<int64_t>(blockIdx.x) * cols;
+  TOut* dst = out + static_cast<int64_t>(blockIdx.x) * cols;
+  int head = 0;
+  if constexpr (PEEL) {
+    const int off = static_cast<int>((reinterpret_cast<uintptr_t>(src) & 15u) / sizeof(TIn));
+    head = off ? EPV - off : 0;
+  }
+  const int nvec = (cols - head) / EPV;
+  const int tail_from = head + nvec * EPV;
+  int edge = -1;
+  if (wave == 0 && lane < 8 && lane < head) edge = lane;
+  if (wave == 0 && lane >= 8 && lane < 16 && tail_from + lane - 8 < cols) edge = tail_from + lane - 8;
+
+  // vector slots past the end of the row hold -inf in every element: exp gives 0, nothing is
+  // stored from them. Addresses are a uniform row base plus a 32-bit byte offset per lane.
+  const char* src_b = reinterpret_cast<const char*>(src + head);
+  char* dst_b = reinterpret_cast<char*>(dst + head);
+  const uint32_t lane_vec = static_cast<uint32_t>(wave * kWave + lane);
+  Vec16<TIn> raw[VPL];
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const uint32_t vi = lane_vec + v * (WAVES * kWave);
+    const bool ok = vi < static_cast<uint32_t>(nvec);
+    const TIn* at = reinterpret_cast<const TIn*>(src_b + (ok ? vi : 0u) * 16u);
+    Vec16<TIn> t;
+    if constexpr (PEEL) {
+      t = load_vec16_stream(at);
+    } else {
+      t = load_vec16_unaligned(at);
+    }
+    const raw16_t all_neg_inf = sizeof(TIn) == 4 ? raw16_t{0xff800000u, 0xff800000u, 0xff800000u, 0xff800000u}
+                                : (__is_same(TIn, bf16_t) ? raw16_t{0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u}
+                                                          : raw16_t{0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u});
+    raw[v] = ok ? t : __builtin_bit_cast(Vec16<TIn>, all_neg_inf);
+  }
+  float xt = neg_inf;
+  if (edge >= 0) xt = to_f32(src[edge]);
+  // 16-bit rows: the compiler must not carry the converted values from one pass to the next
+  // (that is the register budget this kernel exists to avoid), so the raw vectors are made
+  // opaque between the passes
+  auto forget = [&]() {
+    if constexpr (!IN_PLACE) {
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) {
+        raw16_t r = __builtin_bit_cast(raw16_t, raw[v]);
+        asm volatile("" : "+v"(r));
+        raw[v] = __builtin_bit_cast(Vec16<TIn>, r);
+      }
+    }
+  };
+
+  float m = xt;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) m = fmaxf(m, to_f32(raw[v].v[e]));
+  m = wave_max(m);
+  m = group_reduce(m, slot, wave, 0, WAVES, MaxOp{});
+  forget();
+
+  const float ext = exp_for<TOut>(xt - m);
+  xt = LOG ? xt - m : ext;
+  float s = ext;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      const float d = to_f32(raw[v].v[e]) - m;
+      const float ex = exp_for<TOut>(d);
+      if constexpr (IN_PLACE) raw[v].v[e] = LOG ? d : ex;
+      s += ex;
+    }
+  s = wave_sum(s);
+  s = group_reduce(s, slot, wave, 0, WAVES, SumOp{});
+  const float lg = logf(s), inv = 1.0f / s;
+  forget();
+
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const uint32_t vi = lane_vec + v * (WAVES * kWave);
+    float y[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      if constexpr (IN_PLACE) {
+        y[e] = LOG ? to_f32(raw[v].v[e]) - lg : to_f32(raw[v].v[e]) * inv;
+      } else {
+        const float d = to_f32(raw[v].v[e]) - m;
+        y[e] = LOG ? d - lg : exp_for<TOut>(d) * inv;
+      }
+    }
+    if (vi < static_cast<uint32_t>(nvec)) {
+      TOut* at = reinterpret_cast<TOut*>(dst_b + static_cast<size_t>(vi) * (EPV * sizeof(TOut)));
+      if constexpr (PEEL) {
+        store_converted<TOut, EPV, STREAM>(at, y);
+      } else {
+        store_converted_unaligned<TOut, EPV>(at, y);
+      }
+    }
+  }
+  if (edge >= 0) dst[edge] = from_f32<TOut>(LOG ? xt - lg : xt * inv);
+}
+
 template <typename TIn, typename TOut, int VPL, bool LOG>
 static int launch_long_rows(TOut* out, const TIn* in, int64_t rows, int64_t cols,
                             hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(rows)), block(1024);
   const int c = static_cast<int>(cols);
+  // rows that fit 52 registers per lane take the kernel that shares a CU between two rows
+  // (16-bit rows only: fp32 rows of 8 or 13 vectors per lane do not fit 64 registers and spill)
+  constexpr bool LEAN = sizeof(TIn) == 2 && VPL > 4;
+#define TMB_LONG(PEEL, STREAM)                                                                        \
+  do {                                                                                                \
+    if constexpr (LEAN)                                                                               \
+      softmax_long_rows_lean_kernel<TIn, TOut, VPL, LOG, PEEL, STREAM><<<grid, block, 0, stream>>>(out, in, c); \
+    else                                                                                              \
+      softmax_long_rows_kernel<TIn, TOut, VPL, LOG, PEEL, STREAM><<<grid, block, 0, stream>>>(out, in, c);      \
+  } while (0)
   if constexpr (sizeof(TIn) == sizeof(TOut)) {
     if ((reinterpret_cast<uintptr_t>(in) & 15u) == (reinterpret_cast<uintptr_t>(out) & 15u)) {
       if (rows * cols * static_cast<int64_t>(sizeof(TIn) + sizeof(TOut)) >= (int64_t{256} << 20)) {
-        softmax_long_rows_kernel<TIn, TOut, VPL, LOG, true, true><<<grid, block, 0, stream>>>(out, in, c);
+        TMB_LONG(true, true);
       } else {
-        softmax_long_rows_kernel<TIn, TOut, VPL, LOG, true, false><<<grid, block, 0, stream>>>(out, in, c);
+        TMB_LONG(true, false);
       }
       return check_launch();
     }
   }
-  softmax_long_rows_kernel<TIn, TOut, VPL, LOG, false, false><<<grid, block, 0, stream>>>(out, in, c);
+  TMB_LONG(false, false);
+#undef TMB_LONG
   return check_launch();
 }
 
@@ -328,7 +461,13 @@ static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols
     // better the loads and stores of different waves interleave; one or two vectors per lane and
     // more waves per row beat one wave per row by 8-12 %.
     if (nvec <= 64) return launch_regs<TIn, TOut, LOG, SCALED, 1, 1, 256>(out, in, rows, cols, sc, stream);
-    if (nvec <= 128) return launch_regs<TIn, TOut, LOG, SCALED, 2, 1, 256>(out, in, rows, cols, sc, stream);
+    if (nvec <= 128) {
+      // 16-bit rows of 1024 columns: one wave per row with two vectors per lane (no LDS, no
+      // barrier) measured 63 us against 66-69 us for two waves per row on [98304, 1024] bf16
+      if constexpr (sizeof(TIn) == 2)
+        return launch_regs<TIn, TOut, LOG, SCALED, 1, 2, 256>(out, in, rows, cols, sc, stream);
+      return launch_regs<TIn, TOut, LOG, SCALED, 2, 1, 256>(out, in, rows, cols, sc, stream);
+    }
     if (nvec <= 256) return launch_regs<TIn, TOut, LOG, SCALED, 2, 2, 256>(out, in, rows, cols, sc, stream);
     if (nvec <= 512) return launch_regs<TIn, TOut, LOG, SCALED, 4, 2, 256>(out, in, rows, cols, sc, stream);
     if (nvec <= 1024) return launch_regs<TIn, TOut, LOG, SCALED, 8, 2, 512>(out, in, rows, cols, sc, stream);
@@ -345,7 +484,12 @@ static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols
     if (cols >= 4096 && cols / EPV <= 1024 * MAXV && rows < (int64_t{1} << 31)) {
       if (cols / EPV <= 1024 * 2) return launch_long_rows<TIn, TOut, 2, LOG>(out, in, rows, cols, stream);
       if (cols / EPV <= 1024 * 4) return launch_long_rows<TIn, TOut, 4, LOG>(out, in, rows, cols, stream);
-      return launch_long_rows<TIn, TOut, MAXV, LOG>(out, in, rows, cols, stream);
+      if constexpr (MAXV == 8) {  // 16-bit rows: up to 65536 columns in 32 registers
+        if (cols / EPV <= 1024 * 7) return launch_long_rows<TIn, TOut, 7, LOG>(out, in, rows, cols, stream);
+        return launch_long_rows<TIn, TOut, 8, LOG>(out, in, rows, cols, stream);
+      } else {
+        return launch_long_rows<TIn, TOut, MAXV, LOG>(out, in, rows, cols, stream);
+      }
     }
   }
   const int64_t blocks = rows < 65536 * 16 ? rows : 65536 * 16;
