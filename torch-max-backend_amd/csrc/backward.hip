@@ -45,6 +45,7 @@ __global__ __launch_bounds__(256) void gelu_backward_kernel(T* __restrict__ out,
                                                             const T* __restrict__ in,
                                                             int64_t numel, int64_t nvec) {
   constexpr int EPV = Vec16<T>::N;
+  const bool stream = numel * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid < nvec) {
     const Vec16<T> xv = load_vec16_stream(in + tid * EPV);
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(256) void gelu_backward_kernel(T* __restrict__ out,
       const float x = to_f32(xv.v[e]), g = to_f32(gv.v[e]);
       y[e] = TANH ? gelu_grad_tanh(x, g) : gelu_grad_erf(x, g);
     }
-    store_converted<T, EPV>(out + tid * EPV, y);
+    store_converted_hinted<T, EPV>(out + tid * EPV, y, stream);
   }
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t i = nvec * EPV + tid; i < numel; i += stride) {
@@ -92,6 +93,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_backward_regs_kernel(T* __restr
                                                                       const T* __restrict__ y,
                                                                       int64_t rows, int cols) {
   constexpr int EPV = Vec16<T>::N;
+  const bool stream = rows * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WAVES = BLOCK / kWave;
   constexpr int GROUPS = WAVES / WPR;
   __shared__ float slot[WAVES];
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_backward_regs_kernel(T* __restr
 #pragma unroll
     for (int e = 0; e < EPV; ++e)
       r[e] = LOG ? g[v][e] - exp_for<T>(o[v][e]) * s : o[v][e] * (g[v][e] - s);
-    if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r);
+    if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r, stream);
   }
 }
 
@@ -149,6 +151,7 @@ template <typename T, int VPL, bool LOG, bool PEEL>
 __global__ __launch_bounds__(1024) void softmax_backward_long_rows_kernel(
     T* __restrict__ gin, const T* __restrict__ gout, const T* __restrict__ y, int cols) {
   constexpr int EPV = Vec16<T>::N;
+  const bool stream = static_cast<int64_t>(gridDim.x) * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WAVES = 16;
   __shared__ float slot[WAVES];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -236,7 +239,7 @@ __global__ __launch_bounds__(1024) void softmax_backward_long_rows_kernel(
       if (vi < nvec) {
         T* at = dst + static_cast<unsigned>(head + vi * EPV);
         if constexpr (PEEL) {
-          store_converted<T, EPV>(at, r);
+          store_converted_hinted<T, EPV>(at, r, stream);
         } else {
           store_converted_unaligned<T, EPV>(at, r);
         }
@@ -344,6 +347,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
     const float* __restrict__ mean, const float* __restrict__ rstd, const T* __restrict__ gamma,
     int64_t rows, int cols) {
   constexpr int EPV = Vec16<T>::N;
+  const bool stream = rows * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WAVES = BLOCK / kWave;
   constexpr int GROUPS = WAVES / WPR;
   __shared__ float slot[WAVES];
@@ -391,7 +395,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
     float r[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; ++e) r[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
-    if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r);
+    if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r, stream);
   }
 }
 
@@ -405,6 +409,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
     const T* __restrict__ x, const float* __restrict__ mean, const float* __restrict__ rstd,
     const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk) {
   constexpr int EPV = Vec16<T>::N;
+  const bool stream = rows * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WAVES = BLOCK / kWave;
   constexpr int GROUPS = WAVES / WPR;
   __shared__ float slot[WAVES];
@@ -472,7 +477,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
         float r[EPV];
 #pragma unroll
         for (int e = 0; e < EPV; ++e) r[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
-        if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r);
+        if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r, stream);
       }
     }
   }
@@ -499,6 +504,7 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
     const T* __restrict__ x, const float* __restrict__ mean, const float* __restrict__ rstd,
     const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk) {
   constexpr int EPV = Vec16<T>::N;
+  const bool stream = rows * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WIDTH = VPL * kWave * EPV;  // columns a wave covers
   __shared__ float sums[4][2][WIDTH];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -568,7 +574,7 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
           float out[EPV];
 #pragma unroll
           for (int e = 0; e < EPV; ++e) out[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
-          if (vi < nvec) store_converted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, out);
+          if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, out, stream);
         }
       }
     }

@@ -11,6 +11,7 @@ __global__ __launch_bounds__(256) void gelu_kernel(T* __restrict__ out, const T*
   constexpr int EPV = Vec16<T>::N;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const bool stream = numel * static_cast<int64_t>(2 * sizeof(T)) >= kStreamStoreBytes;
   for (int64_t i = tid; i < nvec; i += stride) {
     const Vec16<T> v = load_vec16_stream(in + i * EPV);  // read once
     float y[EPV];
@@ -19,7 +20,7 @@ __global__ __launch_bounds__(256) void gelu_kernel(T* __restrict__ out, const T*
       const float x = to_f32(v.v[e]);
       y[e] = TANH ? gelu_tanh_f32(x) : gelu_erf_f32(x);
     }
-    store_converted<T, EPV>(out + i * EPV, y);
+    store_converted_hinted<T, EPV>(out + i * EPV, y, stream);
   }
   for (int64_t i = nvec * EPV + tid; i < numel; i += stride) {
     const float x = to_f32(in[i]);
