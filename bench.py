@@ -311,6 +311,10 @@ def main() -> int:
     stream = torch.cuda.current_stream().cuda_stream
 
     def rotating(make, bytes_per_buffer):
+        # fresh segments for every row's buffers: blocks carved out of segments that earlier rows
+        # left behind measured up to 12 % slower on the same kernel (layer norm bf16 [16384, 4096]:
+        # 47 us with --only rows, 53 us behind the GEMM and attention rows)
+        torch.cuda.empty_cache()
         n = max(2, math.ceil(768e6 / max(bytes_per_buffer, 1)) + 1)
         n = min(n, 16)
         return [make(i) for i in range(n)]
@@ -324,6 +328,7 @@ def main() -> int:
                 raise RuntimeError(f"{name}: launch failed with {ek.status_string(rc)}")
             state["i"] += 1
 
+        settle(step)
         _, ms = timed(step, steps, 8)
         gbs = bytes_algo / ms / 1e6
         row = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
@@ -333,6 +338,7 @@ def main() -> int:
             row["cpu_GB/s"] = round(t[1] / t[0] / 1e9, 3)
             row["cpu_note"] = t[2]
         sweep[name] = row
+        return (state["i"] - 1) % nbuf   # the buffer the last launch worked on
 
     def with_copy(name, nbuf, ptrs, nbytes):
         """Beside a row-wise kernel's row: tmb_copy_bytes over the same buffers (the same bytes
@@ -344,6 +350,7 @@ def main() -> int:
             lib.tmb_copy_bytes(o, x, nbytes, stream)
             state["i"] += 1
 
+        settle(step)
         _, ms = timed(step, 40, 8)
         sweep[name]["copy_us_same_bytes"] = round(ms * 1e3, 2)
         sweep[name]["vs_copy"] = round(ms * 1e3 / sweep[name]["us"], 3)
@@ -358,6 +365,7 @@ def main() -> int:
             lib.tmb_read_bytes(in_ptrs[state["i"] % nbuf], nbytes, sink.data_ptr(), stream)
             state["i"] += 1
 
+        settle(step)
         _, ms = timed(step, 40, 8)
         sweep[name]["read_us_same_bytes"] = round(ms * 1e3, 2)
         sweep[name]["vs_read"] = round(ms * 1e3 / sweep[name]["us"], 3)
@@ -515,21 +523,21 @@ def main() -> int:
                         lambda i, op=op: lib.tmb_reduce_rows(out_rows.data_ptr(), in_ptrs[i], rows, cols, op,
                                                              code, None, 0, stream),
                         nbytes + rows * es, cpu_fn=cpu_red)
-                hbm_row(f"{opname}_{dn}_all_{rows}x{cols}", len(bufs),
-                        lambda i, op=op: lib.tmb_reduce_rows(out_all.data_ptr(), in_ptrs[i], 1, rows * cols,
-                                                             op, code, ws.data_ptr(), ws_bytes, stream),
-                        nbytes + es)
-            assert torch.equal(out_all.reshape(()), hip_ops.reduce(bufs[(39 + 8) % len(bufs)], [0, 1], False, ek.AMAX))
+                last = hbm_row(f"{opname}_{dn}_all_{rows}x{cols}", len(bufs),
+                               lambda i, op=op: lib.tmb_reduce_rows(out_all.data_ptr(), in_ptrs[i], 1, rows * cols,
+                                                                    op, code, ws.data_ptr(), ws_bytes, stream),
+                               nbytes + es)
+            assert torch.equal(out_all.reshape(()), hip_ops.reduce(bufs[last], [0, 1], False, ek.AMAX))
             # the same matrices summed over their leading dimension (the bias gradient of a linear
             # layer): out[c] = sum_r x[r, c]
             out_cols = torch.empty(cols, dtype=dtype, device=dev)
             cws_bytes = lib.tmb_reduce_cols_workspace_bytes(rows, cols, code)
             cws = torch.empty(max(cws_bytes, 16), dtype=torch.uint8, device=dev)
-            hbm_row(f"sum_{dn}_cols_{rows}x{cols}", len(bufs),
-                    lambda i: lib.tmb_reduce_cols(out_cols.data_ptr(), in_ptrs[i], rows, cols, ek.SUM, code,
-                                                  cws.data_ptr(), cws_bytes, stream),
-                    nbytes + cols * es)
-            assert torch.allclose(out_cols.float(), bufs[(39 + 8) % len(bufs)].float().sum(0), rtol=2e-2, atol=2.0)
+            last = hbm_row(f"sum_{dn}_cols_{rows}x{cols}", len(bufs),
+                           lambda i: lib.tmb_reduce_cols(out_cols.data_ptr(), in_ptrs[i], rows, cols, ek.SUM, code,
+                                                         cws.data_ptr(), cws_bytes, stream),
+                           nbytes + cols * es)
+            assert torch.allclose(out_cols.float(), bufs[last].float().sum(0), rtol=2e-2, atol=2.0)
             del bufs
         rows, cols = 512, 50257
         bufs = rotating(lambda i: gen((rows, cols), 40 + i, torch.float32), rows * cols * 4)
@@ -543,11 +551,11 @@ def main() -> int:
             t = cpu_time(lambda: oracle.argmax_rows(xh), iters=3, warmup=1)
             return t, rows * cols * 4, f"all {rows} rows, C oracle, {cpu_threads} threads"
 
-        hbm_row(f"argmax_fp32_{rows}x{cols}", len(bufs),
-                lambda i: lib.tmb_argmax_rows(out_idx.data_ptr(), in_ptrs[i], rows, cols, ek.F32,
-                                              ws.data_ptr(), ws_bytes, stream),
-                rows * cols * 4 + rows * 8, steps=100, cpu_fn=cpu_argmax)
-        assert torch.equal(out_idx, torch.argmax(bufs[(99 + 8) % len(bufs)], dim=1))
+        last = hbm_row(f"argmax_fp32_{rows}x{cols}", len(bufs),
+                       lambda i: lib.tmb_argmax_rows(out_idx.data_ptr(), in_ptrs[i], rows, cols, ek.F32,
+                                                     ws.data_ptr(), ws_bytes, stream),
+                       rows * cols * 4 + rows * 8, steps=100, cpu_fn=cpu_argmax)
+        assert torch.equal(out_idx, torch.argmax(bufs[last], dim=1))
         with_read(f"argmax_fp32_{rows}x{cols}", len(bufs), in_ptrs, rows * cols * 4)
         del bufs
 
