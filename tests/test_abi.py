@@ -139,6 +139,24 @@ def test_missing_library_raises(monkeypatch, tmp_path):
         ek.lib()
 
 
+def test_library_path_can_name_another_build(tmp_path):
+    """TORCH_MOJO_BACKEND_HIP_LIBRARY points the loader at another build of the library (a
+    diagnostic variant); a path that does not exist fails as loudly as the default one."""
+    import subprocess
+    import sys
+
+    bogus = str(tmp_path / "libtmb_hip_diag9.so")
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from torch_mojo_backend import eager_kernels as ek\n"
+            "assert ek.LIBRARY_PATH == %r, ek.LIBRARY_PATH\n"
+            "try:\n    ek.lib()\nexcept ek.HipLibraryMissing as e:\n    print('missing:', e)\n"
+            % (os.path.join(ROOT, "torch-max-backend_amd"), bogus))
+    env = dict(os.environ, TORCH_MOJO_BACKEND_HIP_LIBRARY=bogus)
+    done = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert "missing:" in done.stdout and "libtmb_hip_diag9.so" in done.stdout
+
+
 def test_product_never_imports_the_oracle():
     pkg = os.path.join(ROOT, "torch-max-backend_amd")
     for dirpath, _, files in os.walk(pkg):

@@ -333,3 +333,20 @@ def test_reduce_cols_entry_point_checks_its_workspace():
     assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, ek.SUM, ek.I64, ws.data_ptr(), need, st) == -2
     assert L.tmb_reduce_cols(out.data_ptr(), x.data_ptr(), 4096, 768, ek.SUM, ek.F32, ws.data_ptr(), need, st) == 0
     assert_close64(out, as64(x.cpu()).sum(0), atol=2e-3)
+
+
+def test_read_only_yardstick_reads_and_writes_nothing():
+    """tmb_read_bytes: the bandwidth yardstick beside the reductions. It must leave its sink
+    alone on ordinary data and refuse what it cannot read as 16-byte vectors."""
+    ek = _ek()
+    L = ek.lib()
+    x = _dev(seeded((1024, 1031), seed=3))
+    sink = torch.full((4,), 12345, dtype=torch.int32, device=x.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.tmb_read_bytes(x.data_ptr(), x.numel() * 4, sink.data_ptr(), stream) == 0
+    assert L.tmb_read_bytes(x.data_ptr(), 8, sink.data_ptr(), stream) == 0          # less than a vector
+    torch.cuda.synchronize()
+    assert sink.cpu().tolist() == [12345] * 4
+    assert L.tmb_read_bytes(None, 1024, sink.data_ptr(), stream) == ek.ERR_INVALID_ARGUMENT
+    assert L.tmb_read_bytes(x.data_ptr(), 1024, None, stream) == ek.ERR_INVALID_ARGUMENT
+    assert L.tmb_read_bytes(x.data_ptr() + 4, 1024, sink.data_ptr(), stream) == ek.ERR_UNSUPPORTED

@@ -33,6 +33,14 @@
 
 #include "gemm_mfma.h"
 
+// Diagnostic builds of the ring kernels (`sh build.sh -DTMB_GEMM_DIAG=n`, results are wrong by
+// construction): what a launch takes without one of its parts. 1: no epilogue (one dword per
+// lane keeps the products alive); 2: no operand fetch (the DMA is skipped: whatever LDS holds is
+// multiplied); 3: every tile fetches the operands of tile (0, 0) (all L2 hits); 4: 1 and 2.
+#ifndef TMB_GEMM_DIAG
+#define TMB_GEMM_DIAG 0
+#endif
+
 namespace tmb {
 
 typedef __attribute__((address_space(3))) void lds_void_t;
@@ -205,6 +213,7 @@ void gemm_ring_kernel(GemmArgs g) {
   const uint32_t a_m0 = ring_lds + wave_s * (A_GROUPS * 1024);
   const uint32_t b_m0 = ring_lds + A_BYTES + wave_s * (B_GROUPS * 1024);
   auto dma16 = [](uint32_t m0, uint32_t voff, const unsigned char* sbase) {
+    if constexpr (TMB_GEMM_DIAG == 2 || TMB_GEMM_DIAG == 4) return;
     if constexpr (SPLIT_RING) {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1"
                    :
@@ -402,9 +411,11 @@ void gemm_ring_kernel(GemmArgs g) {
   {
     int tile_m, tile_n;
     tile_of_block(static_cast<int>(pid), g.tiles_m, g.tiles_n, tile_m, tile_n);
+    m0 = TMB_GEMM_DIAG == 3 ? 0 : static_cast<int64_t>(tile_m) * BM;
+    n0 = TMB_GEMM_DIAG == 3 ? 0 : static_cast<int64_t>(tile_n) * BN;
+    plan_tile_loads();
     m0 = static_cast<int64_t>(tile_m) * BM;
     n0 = static_cast<int64_t>(tile_n) * BN;
-    plan_tile_loads();
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -570,7 +581,14 @@ void gemm_ring_kernel(GemmArgs g) {
                      wave * (ep.wide() ? BandLayoutF32<WN>::BYTES : BandLayout<WN>::BYTES);
   void* Cout = g.out_f32 ? static_cast<void*>(static_cast<float*>(g.c) + batch * g.stride_c)
                          : static_cast<void*>(C);
-  if constexpr (MI16) {
+  if constexpr (TMB_GEMM_DIAG == 1 || TMB_GEMM_DIAG == 4) {
+    float keep = 0.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) keep += acc[i][j][0] + acc[i][j][3];
+    static_cast<float*>(Cout)[wave * 64 + lane] = keep;
+  } else if constexpr (MI16) {
     store_wave_tile16<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
                                       g.stream_c != 0, ep, lane);
   } else {

@@ -14,7 +14,9 @@ import ctypes
 import os
 
 _CSRC = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", "csrc"))
-LIBRARY_PATH = os.path.join(_CSRC, "libtmb_hip.so")
+# TORCH_MOJO_BACKEND_HIP_LIBRARY names another build of the library (a diagnostic variant made with
+# `TMB_VARIANT=... sh build.sh ...`); unset, the library beside the sources is loaded.
+LIBRARY_PATH = os.environ.get("TORCH_MOJO_BACKEND_HIP_LIBRARY") or os.path.join(_CSRC, "libtmb_hip.so")
 
 F32, F16, BF16, I64, I32 = 0, 1, 2, 3, 4
 SUM, MEAN, AMAX = 0, 1, 2
