@@ -354,6 +354,49 @@ def test_residual_epilogue_in_float32_one_cast(mnk, dtype, resid_f32, out_f32):
         assert e_once <= e_twice
 
 
+# A float32 residual stream over whole tiles, every element checked: the residual of a wave tile is
+# requested as a whole before its bands are staged. Shapes: one tile per workgroup, two and three
+# tiles per workgroup, short K, and (below) a batch.
+STREAM_TILES = [(8192, 1024, 768), (16384, 768, 768), (32768, 768, 768), (16384, 768, 3072), (32768, 768, 192),
+                (32768, 1536, 128), (65536, 256, 256)]
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", STREAM_TILES)
+def test_float32_residual_stream_over_whole_tiles(mnk, dtype):
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(29)
+    a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
+    w = (torch.randn(n, k, generator=g, device="cuda") * 0.1).to(dtype)
+    bias = torch.randn(n, generator=g, device="cuda").to(dtype)
+    res = torch.randn(m, n, generator=g, device="cuda") * 3
+    out = _ops().gemm(a, w.t(), bias, residual=res, out_dtype=torch.float32)
+    # every element, against float64
+    exact = a.double() @ w.double().t() + bias.double()
+    bound = k * 2.0 ** -24 * (a.double().abs() @ w.double().abs().t())
+    err = (out.double() - (exact + res.double())).abs()
+    limit = bound + 1e-6 + 1e-6 * (exact + res.double()).abs()
+    worst = (err - limit).max().item()
+    assert worst <= 0, f"{mnk} {dtype}: {worst} over the bound at {torch.nonzero(err > limit)[:4].tolist()}"
+    # and the same bits for a residual whose rows do not start on 16-byte boundaries
+    wide = torch.zeros(m, n + 1, device="cuda")
+    wide[:, :n] = res
+    assert torch.equal(out, _ops().gemm(a, w.t(), bias, residual=wide[:, :n], out_dtype=torch.float32))
+    # again into a used buffer: nothing of an earlier launch may survive
+    again = _ops().gemm(a, w.t(), bias, residual=res, out_dtype=torch.float32)
+    assert torch.equal(out, again)
+
+
+def test_float32_residual_stream_batched():
+    g = torch.Generator(device="cuda").manual_seed(30)
+    a = torch.randn(3, 8192, 320, generator=g, device="cuda").bfloat16()
+    b = (torch.randn(3, 384, 320, generator=g, device="cuda") * 0.1).bfloat16()
+    res = torch.randn(3, 8192, 384, generator=g, device="cuda")
+    out = _ops().gemm(a, b.transpose(1, 2), residual=res, out_dtype=torch.float32)
+    want = torch.bmm(a.double(), b.double().transpose(1, 2)) + res.double()
+    torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-4)
+
+
 def test_float32_stream_rejects_the_bit_identical_mode_and_composes_with_layer_norm():
     g = torch.Generator(device="cuda").manual_seed(24)
     a = torch.randn(512, 768, generator=g, device="cuda").bfloat16()

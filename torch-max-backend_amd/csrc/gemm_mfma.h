@@ -329,10 +329,57 @@ typedef f32x4_g_t __attribute__((aligned(4))) f32x4_g_unaligned_t;
 
 // Writes the staged fp32 band (32 x WN) to C: a lane takes 8 columns of a row, adds the residual
 // (8 x T or 8 x fp32) in fp32 and stores 8 x T (one 16-byte store) or 8 x fp32.
-template <typename T, int WN, bool STREAM>
+// The 8 fp32 residual values a lane adds to one row of a band in flush_band_wide (zeros past
+// the edges of C).
+__device__ __forceinline__ void load_residual8(const EpilogueArgs& ep, int64_t row, int64_t col,
+                                               int64_t M, int64_t N, float (&out)[8]) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = 0.0f;
+  if (row >= M || col >= N) return;
+  const float* rsrc = static_cast<const float*>(ep.residual) + row * ep.ldr + col;
+  if (col + 8 <= N) {
+    const f32x4_g_t r0 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc);
+    const f32x4_g_t r1 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      out[e] = r0[e];
+      out[4 + e] = r1[e];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (col + e < N) out[e] = rsrc[e];
+  }
+}
+
+// The fp32 residual of a whole wave tile of 16x16 accumulators (AM x AN tiles), held in
+// registers from before the tile's main loop: 8 values per lane, pass and band. Only for wave
+// tiles where that is at most 64 registers per lane.
+template <int AM, int AN>
+struct ResidualTile {
+  static constexpr int WN = AN * 16;
+  static constexpr int LPR = WN / 8, RPP = 64 / LPR, PASSES = 32 / RPP, BANDS = AM / 2;
+  static constexpr bool FITS = BANDS * PASSES * 8 <= 64;
+  float v[FITS ? BANDS : 1][FITS ? PASSES : 1][8];
+  __device__ __forceinline__ void request(const EpilogueArgs& ep, int64_t row0, int64_t col0, int64_t M,
+                                          int64_t N, int lane) {
+    if constexpr (FITS) {
+#pragma unroll
+      for (int b = 0; b < BANDS; ++b)
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+          load_residual8(ep, row0 + b * 32 + p * RPP + lane / LPR, col0 + (lane % LPR) * 8, M, N, v[b][p]);
+    }
+  }
+};
+
+// PRE: an fp32 residual was requested by the caller long before (`pre`, one load_residual8 per
+// pass: ResidualTile), so no pass waits for memory.
+template <typename T, int WN, bool STREAM, bool PRE = false>
 __device__ __forceinline__ void flush_band_wide(const lds_byte_t* band, void* __restrict__ Cv,
                                                 int64_t ldc, int64_t row0, int64_t col0, int64_t M,
-                                                int64_t N, const EpilogueArgs& ep, int lane) {
+                                                int64_t N, const EpilogueArgs& ep, int lane,
+                                                const float (*pre)[8] = nullptr) {
   constexpr int PITCH = BandLayoutF32<WN>::PITCH;
   constexpr int LPR = WN / 8;    // lanes per row
   constexpr int RPP = 64 / LPR;  // rows per pass
@@ -346,7 +393,10 @@ __device__ __forceinline__ void flush_band_wide(const lds_byte_t* band, void* __
     const int64_t row = row0 + r, col = col0 + c;
     if (row >= M || col >= N) continue;
     const bool whole = col + 8 <= N;
-    if (ep.resid_f32) {
+    if (PRE && ep.resid_f32) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += pre[p][e];
+    } else if (ep.resid_f32) {
       const float* rsrc = static_cast<const float*>(ep.residual) + row * ep.ldr + col;
       if (whole) {
         const f32x4_g_t r0 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc);
@@ -480,7 +530,8 @@ __device__ __forceinline__ void store_wave_tile16_impl(f32x4v_t (&acc)[AM][AN], 
                                                   void* __restrict__ Cv, int64_t ldc, int64_t row0,
                                                   int64_t col0, int64_t M, int64_t N,
                                                   const T* __restrict__ bias,
-                                                  const EpilogueArgs& ep, int lane) {
+                                                  const EpilogueArgs& ep, int lane,
+                                                  const ResidualTile<AM, AN>* pre) {
   constexpr int WN = AN * 16;
   static_assert(AM % 2 == 0, "whole 32-row bands");
   float bias_f[AN][4];
@@ -494,6 +545,7 @@ __device__ __forceinline__ void store_wave_tile16_impl(f32x4v_t (&acc)[AM][AN], 
     if (ep.wide()) {  // wave-uniform
       constexpr int PITCH = BandLayoutF32<WN>::PITCH;
       lds_byte_t* mine = band + (lane & 15) * PITCH + 16 * (lane >> 4);
+      constexpr bool PRE = ResidualTile<AM, AN>::FITS;  // then `pre` holds an fp32 residual
 #pragma unroll
       for (int b = 0; b < AM / 2; ++b) {
         if (row0 + b * 32 >= M) break;  // wave-uniform
@@ -506,7 +558,8 @@ __device__ __forceinline__ void store_wave_tile16_impl(f32x4v_t (&acc)[AM][AN], 
                                    a[3] + bias_f[j][3]};
             *(lds_f32x4_t*)(mine + h * 16 * PITCH + j * 64) = v;
           }
-        flush_band_wide<T, WN, STREAM>(band, Cv, ldc, row0 + b * 32, col0, M, N, ep, lane);
+        flush_band_wide<T, WN, STREAM, PRE>(band, Cv, ldc, row0 + b * 32, col0, M, N, ep, lane,
+                                            pre->v[PRE ? b : 0]);
       }
       return;
     }
@@ -537,11 +590,12 @@ __device__ __forceinline__ void store_wave_tile16(f32x4v_t (&acc)[AM][AN], lds_b
                                                   void* __restrict__ C, int64_t ldc, int64_t row0,
                                                   int64_t col0, int64_t M, int64_t N,
                                                   const T* __restrict__ bias, bool stream,
-                                                  const EpilogueArgs& ep, int lane) {
+                                                  const EpilogueArgs& ep, int lane,
+                                                  const ResidualTile<AM, AN>* pre) {
   if (stream) {
-    store_wave_tile16_impl<T, EPI, AM, AN, true>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane);
+    store_wave_tile16_impl<T, EPI, AM, AN, true>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane, pre);
   } else {
-    store_wave_tile16_impl<T, EPI, AM, AN, false>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane);
+    store_wave_tile16_impl<T, EPI, AM, AN, false>(acc, band, C, ldc, row0, col0, M, N, bias, ep, lane, pre);
   }
 }
 

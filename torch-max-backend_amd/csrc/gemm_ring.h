@@ -407,6 +407,18 @@ void gemm_ring_kernel(GemmArgs g) {
   // tile would. The stores of a tile drain while the next tile's operands are already being
   // fetched and multiplied.
   const int64_t total_tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
+  const EpilogueArgs ep = epilogue_args<T>(g, batch);
+  // An fp32 residual is requested as a whole in front of the epilogue's first band where the
+  // wave's share fits 64 registers: one wait for memory per wave tile instead of one per pass
+  // (32768 x 768 x 768 with an fp32 residual stream: 81 -> 72 us). Such a launch stays a
+  // sequence of phases in which either the matrix pipes or memory work, on all CUs at once
+  // (43 us of the one, 19 us of residual reads, 15 us of stores). Two ways of mixing them were
+  // measured and dropped: start offsets between workgroups add their own length, and a finished
+  // tile held in registers, leaving two stores per step under the next tile's loads while the
+  // next residual is requested early, is no faster (74 us): loads and stores retire in order, so
+  // the waits for the operands then wait for the stores as well.
+  ResidualTile<MI16 ? TM : 2, MI16 ? TN : 1> resid;
+  constexpr bool RESID_EARLY = MI16 && !OUT_F32 && EPI == TMB_EPI_NONE && decltype(resid)::FITS;
   auto run_tile = [&](int64_t pid) {
   {
     int tile_m, tile_n;
@@ -576,7 +588,9 @@ void gemm_ring_kernel(GemmArgs g) {
   __syncthreads();  // every wave is done with the ring: reuse it for the output
   static_assert(NW * BandLayout<WN>::BYTES <= RING_BYTES, "band staging");
   static_assert(NW * BandLayoutF32<WN>::BYTES <= RING_BYTES, "fp32 band staging");
-  const EpilogueArgs ep = epilogue_args<T>(g, batch);
+  if constexpr (RESID_EARLY) {
+    if (ep.wide() && ep.resid_f32) resid.request(ep, m0 + wm * WM, n0 + wn * WN, M, N, lane);  // wave-uniform
+  }
   lds_byte_t* band = (lds_byte_t*)ring +
                      wave * (ep.wide() ? BandLayoutF32<WN>::BYTES : BandLayout<WN>::BYTES);
   void* Cout = g.out_f32 ? static_cast<void*>(static_cast<float*>(g.c) + batch * g.stride_c)
@@ -590,7 +604,7 @@ void gemm_ring_kernel(GemmArgs g) {
     static_cast<float*>(Cout)[wave * 64 + lane] = keep;
   } else if constexpr (MI16) {
     store_wave_tile16<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
-                                      g.stream_c != 0, ep, lane);
+                                      g.stream_c != 0, ep, lane, &resid);
   } else {
     store_wave_tile<T, EPI, TM, TN>(acc, band, Cout, g.ldc, m0 + wm * WM, n0 + wn * WN, M, N, bias,
                                     g.stream_c != 0, ep, lane);
