@@ -329,57 +329,48 @@ typedef f32x4_g_t __attribute__((aligned(4))) f32x4_g_unaligned_t;
 
 // Writes the staged fp32 band (32 x WN) to C: a lane takes 8 columns of a row, adds the residual
 // (8 x T or 8 x fp32) in fp32 and stores 8 x T (one 16-byte store) or 8 x fp32.
-// The 8 fp32 residual values a lane adds to one row of a band in flush_band_wide (zeros past
-// the edges of C).
-__device__ __forceinline__ void load_residual8(const EpilogueArgs& ep, int64_t row, int64_t col,
-                                               int64_t M, int64_t N, float (&out)[8]) {
-#pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = 0.0f;
-  if (row >= M || col >= N) return;
-  const float* rsrc = static_cast<const float*>(ep.residual) + row * ep.ldr + col;
-  if (col + 8 <= N) {
-    const f32x4_g_t r0 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc);
-    const f32x4_g_t r1 = *reinterpret_cast<const f32x4_g_unaligned_t*>(rsrc + 4);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      out[e] = r0[e];
-      out[4 + e] = r1[e];
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      if (col + e < N) out[e] = rsrc[e];
-  }
-}
-
 // The fp32 residual of a whole wave tile of 16x16 accumulators (AM x AN tiles), held in
-// registers from before the tile's main loop: 8 values per lane, pass and band. Only for wave
-// tiles where that is at most 64 registers per lane.
+// registers: 8 values per lane, pass and band of flush_band_wide. Only for wave tiles where that
+// is at most 64 registers per lane, and only when N is a multiple of 8 (a lane's eight columns
+// are then inside C or outside as a whole). The loads carry no conditions: lanes outside C read
+// a valid address whose value is never used, so nothing but the loads' latency stands between
+// the request and the next instruction.
 template <int AM, int AN>
 struct ResidualTile {
   static constexpr int WN = AN * 16;
   static constexpr int LPR = WN / 8, RPP = 64 / LPR, PASSES = 32 / RPP, BANDS = AM / 2;
   static constexpr bool FITS = BANDS * PASSES * 8 <= 64;
-  float v[FITS ? BANDS : 1][FITS ? PASSES : 1][8];
+  f32x4_g_t v[FITS ? BANDS : 1][FITS ? PASSES : 1][2];
+  bool loaded = false;  // wave-uniform
   __device__ __forceinline__ void request(const EpilogueArgs& ep, int64_t row0, int64_t col0, int64_t M,
                                           int64_t N, int lane) {
     if constexpr (FITS) {
+      loaded = ep.wide() && ep.resid_f32 && N % 8 == 0;
+      if (!loaded) return;
+      int64_t col = col0 + (lane % LPR) * 8;
+      col = col < N ? col : 0;
+      const float* base = static_cast<const float*>(ep.residual) + col;
 #pragma unroll
       for (int b = 0; b < BANDS; ++b)
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p)
-          load_residual8(ep, row0 + b * 32 + p * RPP + lane / LPR, col0 + (lane % LPR) * 8, M, N, v[b][p]);
+        for (int p = 0; p < PASSES; ++p) {
+          int64_t row = row0 + b * 32 + p * RPP + lane / LPR;
+          row = row < M ? row : M - 1;
+          const float* src = base + row * ep.ldr;
+          v[b][p][0] = *reinterpret_cast<const f32x4_g_unaligned_t*>(src);
+          v[b][p][1] = *reinterpret_cast<const f32x4_g_unaligned_t*>(src + 4);
+        }
     }
   }
 };
 
-// PRE: an fp32 residual was requested by the caller long before (`pre`, one load_residual8 per
-// pass: ResidualTile), so no pass waits for memory.
+// PRE and pre != nullptr: the fp32 residual was requested by the caller before (`pre`: this
+// band of a ResidualTile), so no pass waits for memory.
 template <typename T, int WN, bool STREAM, bool PRE = false>
 __device__ __forceinline__ void flush_band_wide(const lds_byte_t* band, void* __restrict__ Cv,
                                                 int64_t ldc, int64_t row0, int64_t col0, int64_t M,
                                                 int64_t N, const EpilogueArgs& ep, int lane,
-                                                const float (*pre)[8] = nullptr) {
+                                                const f32x4_g_t (*pre)[2] = nullptr) {
   constexpr int PITCH = BandLayoutF32<WN>::PITCH;
   constexpr int LPR = WN / 8;    // lanes per row
   constexpr int RPP = 64 / LPR;  // rows per pass
@@ -393,9 +384,12 @@ __device__ __forceinline__ void flush_band_wide(const lds_byte_t* band, void* __
     const int64_t row = row0 + r, col = col0 + c;
     if (row >= M || col >= N) continue;
     const bool whole = col + 8 <= N;
-    if (PRE && ep.resid_f32) {
+    if (PRE && pre != nullptr) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] += pre[p][e];
+      for (int e = 0; e < 4; ++e) {
+        v[e] += pre[p][0][e];
+        v[4 + e] += pre[p][1][e];
+      }
     } else if (ep.resid_f32) {
       const float* rsrc = static_cast<const float*>(ep.residual) + row * ep.ldr + col;
       if (whole) {
@@ -559,7 +553,7 @@ __device__ __forceinline__ void store_wave_tile16_impl(f32x4v_t (&acc)[AM][AN], 
             *(lds_f32x4_t*)(mine + h * 16 * PITCH + j * 64) = v;
           }
         flush_band_wide<T, WN, STREAM, PRE>(band, Cv, ldc, row0 + b * 32, col0, M, N, ep, lane,
-                                            pre->v[PRE ? b : 0]);
+                                            pre->loaded ? pre->v[PRE ? b : 0] : nullptr);
       }
       return;
     }
