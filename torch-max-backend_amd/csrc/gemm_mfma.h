@@ -119,18 +119,18 @@ struct GemmArgs {
   // fp32-partial launches (split-K): blockIdx.y is the split; split z of `splits` multiplies the
   // K stages [stages * z / splits, stages * (z + 1) / splits) and stores partial z (0: not split)
   int splits = 0;
+  // a split launch whose workgroups all run at once: the (split, tile) pairs, split-major, are
+  // dealt to the 8 XCDs in runs of this many, so that an XCD works on tiles of one or two splits
+  // and their operand slices are fetched into its L2 once (0: blockIdx.y is the split)
+  int xcd_chunk = 0;
 };
 
 // Maps the launch-order workgroup id to a tile so that each XCD (workgroups are dealt to the
 // 8 XCDs round-robin) works on a contiguous run of tiles, walked in column-major groups of
 // `kGroupM` tile rows.
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int kXcds = 8;
+// (tile_of_index: the walk itself, from a position in it)
+__device__ __forceinline__ void tile_of_index(int tile, int tiles_m, int tiles_n, int& tm, int& tn) {
   constexpr int kGroupM = 8;
-  const int total = tiles_m * tiles_n;
-  const int q = total / kXcds, r = total % kXcds;
-  const int xcd = pid % kXcds, idx = pid / kXcds;
-  const int tile = xcd * q + (xcd < r ? xcd : r) + idx;
   const int per_group = kGroupM * tiles_n;
   const int group = tile / per_group;
   const int first_m = group * kGroupM;
@@ -138,6 +138,13 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   const int in_group = tile - group * per_group;
   tm = first_m + in_group % gsz;
   tn = in_group / gsz;
+}
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  constexpr int kXcds = 8;
+  const int total = tiles_m * tiles_n;
+  const int q = total / kXcds, r = total % kXcds;
+  const int xcd = pid % kXcds, idx = pid / kXcds;
+  tile_of_index(xcd * q + (xcd < r ? xcd : r) + idx, tiles_m, tiles_n, tm, tn);
 }
 
 // Epilogue. A lane of the (operand-swapped) MFMA result holds, for row lane%32 of a 32x32 tile,

@@ -146,7 +146,17 @@ void gemm_ring_kernel(GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   int64_t m0 = 0, n0 = 0;  // origin of the tile being worked on (set per tile below)
-  const int64_t batch = blockIdx.y;
+  int64_t batch = blockIdx.y;
+  int64_t only_tile = -1;  // >= 0: this workgroup's one tile, as a position in the walk of tiles
+  if constexpr (OUT_F32) {
+    if (g.xcd_chunk > 0) {
+      const uint32_t pair = (blockIdx.x % 8) * static_cast<uint32_t>(g.xcd_chunk) + blockIdx.x / 8;
+      const uint32_t tiles = static_cast<uint32_t>(g.tiles_m) * static_cast<uint32_t>(g.tiles_n);
+      if (pair >= tiles * static_cast<uint32_t>(g.splits)) return;  // (the whole workgroup, before any barrier)
+      batch = __builtin_amdgcn_readfirstlane(static_cast<int>(pair / tiles));
+      only_tile = __builtin_amdgcn_readfirstlane(static_cast<int>(pair % tiles));
+    }
+  }
   const int64_t M = g.m, N = g.n;
   T* __restrict__ C = static_cast<T*>(g.c) + batch * g.stride_c;
   const unsigned char* a_base =
@@ -423,7 +433,8 @@ void gemm_ring_kernel(GemmArgs g) {
   auto run_tile = [&](int64_t pid) {
   {
     int tile_m, tile_n;
-    tile_of_block(static_cast<int>(pid), g.tiles_m, g.tiles_n, tile_m, tile_n);
+    if (only_tile >= 0) tile_of_index(static_cast<int>(pid), g.tiles_m, g.tiles_n, tile_m, tile_n);
+    else tile_of_block(static_cast<int>(pid), g.tiles_m, g.tiles_n, tile_m, tile_n);
     m0 = TMB_GEMM_DIAG == 3 ? 0 : static_cast<int64_t>(tile_m) * BM;
     n0 = TMB_GEMM_DIAG == 3 ? 0 : static_cast<int64_t>(tile_n) * BN;
     plan_tile_loads();
@@ -611,14 +622,17 @@ void gemm_ring_kernel(GemmArgs g) {
   };
   // Configurations compiled for four waves per SIMD have no registers to spare for the loop
   // state; their second resident workgroup already overlaps the tile boundaries.
+  // (one call site for run_tile: called from two, it is no longer inlined)
   if constexpr (kRingPersistent<BM, BN, BK, WAVES_M * WAVES_N, R>) {
+    const int64_t stride = only_tile >= 0 ? total_tiles : static_cast<int64_t>(gridDim.x);
 #pragma unroll 1
-    for (int64_t pid = blockIdx.x; pid < total_tiles; pid += gridDim.x) {
+    for (int64_t pid = only_tile >= 0 ? only_tile : static_cast<int64_t>(blockIdx.x); pid < total_tiles;
+         pid += stride) {
       run_tile(pid);
       __syncthreads();  // the staging bands overlay the ring: all read back before the next fetch
     }
   } else {
-    run_tile(blockIdx.x);
+    run_tile(only_tile >= 0 ? only_tile : static_cast<int64_t>(blockIdx.x));
   }
 #endif
 }
@@ -678,8 +692,19 @@ static int launch_ring(const GemmArgs& base, int64_t batch, hipStream_t stream) 
   // four start phases 5 us apart when every workgroup walks several tiles of a streamed output
   g.stagger_ticks = (g.stream_c && !OUT_F32 && grid_x == resident && tiles >= 4 * resident) ? 500 : 0;
   if (grid_x == resident && tiles >= 4 * resident) warm_b_for_streamed_output(g, batch, B_KMAJOR, stream);
+  unsigned grid_y = static_cast<unsigned>(batch);
+  int64_t grid_x_launch = grid_x;
+  if constexpr (OUT_F32) {
+    // (3072 x 768 x 32768 in 7 splits of 36 tiles: 559 -> 258 MB fetched past the L2s, 170 -> 162 us
+    // with the reduction; 768 x 768 x 32768: 71 -> 59 us)
+    if (g.splits > 0 && batch == g.splits && fits) {
+      g.xcd_chunk = static_cast<int>((tiles * batch + 7) / 8);
+      grid_x_launch = int64_t{8} * g.xcd_chunk;
+      grid_y = 1;
+    }
+  }
   gemm_ring_kernel<T, BM, BN, BK, WAVES_M, WAVES_N, R, B_KMAJOR, EPI, A_MMAJOR, OUT_F32, MI16_>
-      <<<dim3(static_cast<unsigned>(grid_x), static_cast<unsigned>(batch)),
+      <<<dim3(static_cast<unsigned>(grid_x_launch), grid_y),
          dim3(WAVES_M * WAVES_N * 64), 0, stream>>>(g);
   return check_launch();
 }
