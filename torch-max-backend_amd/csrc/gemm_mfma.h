@@ -546,7 +546,7 @@ __device__ __forceinline__ void store_wave_tile16_impl(f32x4v_t (&acc)[AM][AN], 
     if (ep.wide()) {  // wave-uniform
       constexpr int PITCH = BandLayoutF32<WN>::PITCH;
       lds_byte_t* mine = band + (lane & 15) * PITCH + 16 * (lane >> 4);
-      constexpr bool PRE = ResidualTile<AM, AN>::FITS;  // then `pre` holds an fp32 residual
+      constexpr bool PRE = ResidualTile<AM, AN>::FITS;  // then `pre` may hold an fp32 residual
 #pragma unroll
       for (int b = 0; b < AM / 2; ++b) {
         if (row0 + b * 32 >= M) break;  // wave-uniform

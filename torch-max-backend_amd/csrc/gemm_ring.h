@@ -429,7 +429,9 @@ void gemm_ring_kernel(GemmArgs g) {
   // the waits for the operands then wait for the stores as well. Requesting the residual in front
   // of the tile's operand loads instead of here changes nothing either (72.9 us).
   ResidualTile<MI16 ? TM : 2, MI16 ? TN : 1> resid;
-  constexpr bool RESID_EARLY = MI16 && !OUT_F32 && EPI == TMB_EPI_NONE && decltype(resid)::FITS;
+  // (only where 64 more registers are to be had: one workgroup of eight waves per CU)
+  constexpr bool RESID_EARLY = MI16 && !OUT_F32 && EPI == TMB_EPI_NONE && decltype(resid)::FITS &&
+                               BM == 256 && BN == 128 && BK == 64 && NW == 8;
   auto run_tile = [&](int64_t pid) {
   {
     int tile_m, tile_n;
