@@ -397,6 +397,30 @@ def test_float32_residual_stream_batched():
     torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-4)
 
 
+# A product without bias whose output streams to memory (256 MB and more) runs persistent
+# workgroups that request the next tile's operands before they store the finished one. Whole
+# tiles only, tiles cut by both edges, and a row count that leaves some workgroups a tile short.
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("mnk", [(8192, 16384, 768), (8192, 50257, 768), (8100, 16648, 320), (16384, 8192, 128)])
+def test_streamed_product_without_bias(mnk, dtype):
+    m, n, k = mnk
+    g = torch.Generator(device="cuda").manual_seed(31)
+    a = torch.randn(m, k, generator=g, device="cuda").to(dtype)
+    w = (torch.randn(n, k, generator=g, device="cuda") * 0.1).to(dtype)
+    out = _ops().gemm(a, w.t())
+    assert tuple(out.shape) == (m, n) and out.dtype == dtype
+    for lo in range(0, m, 2048):  # every element, in slabs of rows
+        hi = min(m, lo + 2048)
+        exact = a[lo:hi].double() @ w.double().t()
+        bound = k * 2.0 ** -24 * (a[lo:hi].double().abs() @ w.double().abs().t())
+        err = (out[lo:hi].double() - exact).abs()
+        ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        limit = bound + ulp * exact.abs() + 1e-6
+        worst = (err - limit).max().item()
+        assert worst <= 0, f"{mnk} {dtype} rows {lo}..{hi}: {worst} over the bound"
+    assert torch.equal(out, _ops().gemm(a, w.t()))
+
+
 def test_float32_stream_rejects_the_bit_identical_mode_and_composes_with_layer_norm():
     g = torch.Generator(device="cuda").manual_seed(24)
     a = torch.randn(512, 768, generator=g, device="cuda").bfloat16()
