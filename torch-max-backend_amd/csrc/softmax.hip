@@ -240,16 +240,25 @@ __global__ __launch_bounds__(1024) void softmax_long_rows_kernel(TOut* __restric
 // 16384 x 50257). 16-bit rows stay in their storage type (four registers per vector) and are
 // converted again in each of the three passes, with the exponential taken twice (one multiply and
 // one v_exp_f32 each for a 16-bit result). fp32 rows (transformed in place) would need 8 or 13
-// vectors per lane, which spills: they stay with the kernel above.
-template <typename TIn, typename TOut, int VPL, bool LOG, bool PEEL, bool STREAM>
-__global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* __restrict__ out,
-                                                                         const TIn* __restrict__ in,
-                                                                         int cols) {
+// vectors per lane there, which spills: they run in 512-thread workgroups (below).
+// BLOCK = 512: fp32 rows, transformed in place in up to 100 registers per lane: two workgroups
+// of eight waves share a CU at 128 registers each, where the kernel above runs one of sixteen.
+// HELD < VPL: only the first HELD vectors of a lane stay in registers; the others (a fifth of a
+// 50257-wide fp32 row) are read again in each pass, from the L2 they were fetched into (two rows
+// per CU leave 64 x 40 KB of such vectors per XCD). The arithmetic per element is the same either
+// way.
+template <typename TIn, typename TOut, int VPL, bool LOG, bool PEEL, bool STREAM, int BLOCK = 1024,
+          int HELD = VPL>
+__global__ __launch_bounds__(BLOCK, BLOCK == 1024 ? 8 : 4) void softmax_long_rows_lean_kernel(
+    TOut* __restrict__ out, const TIn* __restrict__ in, int cols) {
   constexpr int EPV = Vec16<TIn>::N;
-  constexpr int WAVES = 16;
+  constexpr int WAVES = BLOCK / kWave;
   constexpr bool IN_PLACE = sizeof(TIn) == 4;
   static_assert(!PEEL || sizeof(TIn) == sizeof(TOut), "one offset for both rows");
-  static_assert(VPL * 4 <= 32, "the row must leave room for the rest in 64 registers");
+  static_assert(BLOCK == 1024 || BLOCK == 512, "two workgroups per CU either way");
+  static_assert(HELD * 4 <= (BLOCK == 1024 ? 32 : 84),
+                "the row must leave room for the rest in 64 (128) registers");
+  static_assert(HELD == VPL || sizeof(TIn) == 4, "rows are read again in the in-place form only");
   __shared__ float slot[WAVES];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -272,23 +281,26 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
   const char* src_b = reinterpret_cast<const char*>(src + head);
   char* dst_b = reinterpret_cast<char*>(dst + head);
   const uint32_t lane_vec = static_cast<uint32_t>(wave * kWave + lane);
-  Vec16<TIn> raw[VPL];
-#pragma unroll
-  for (int v = 0; v < VPL; ++v) {
+  Vec16<TIn> raw[HELD];
+  // vector v of the lane, -inf in every element past the end of the row; `again`: a vector that
+  // is not held (plain loads: it is wanted from the L2 twice more)
+  auto fetch = [&](int v, bool again) {
     const uint32_t vi = lane_vec + v * (WAVES * kWave);
     const bool ok = vi < static_cast<uint32_t>(nvec);
     const TIn* at = reinterpret_cast<const TIn*>(src_b + (ok ? vi : 0u) * 16u);
     Vec16<TIn> t;
     if constexpr (PEEL) {
-      t = load_vec16_stream(at);
+      t = again ? load_vec16(at) : load_vec16_stream(at);
     } else {
       t = load_vec16_unaligned(at);
     }
     const raw16_t all_neg_inf = sizeof(TIn) == 4 ? raw16_t{0xff800000u, 0xff800000u, 0xff800000u, 0xff800000u}
                                 : (__is_same(TIn, bf16_t) ? raw16_t{0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u}
                                                           : raw16_t{0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u});
-    raw[v] = ok ? t : __builtin_bit_cast(Vec16<TIn>, all_neg_inf);
-  }
+    return ok ? t : __builtin_bit_cast(Vec16<TIn>, all_neg_inf);
+  };
+#pragma unroll
+  for (int v = 0; v < HELD; ++v) raw[v] = fetch(v, false);
   float xt = neg_inf;
   if (edge >= 0) xt = to_f32(src[edge]);
   // 16-bit rows: the compiler must not carry the converted values from one pass to the next
@@ -297,7 +309,7 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
   auto forget = [&]() {
     if constexpr (!IN_PLACE) {
 #pragma unroll
-      for (int v = 0; v < VPL; ++v) {
+      for (int v = 0; v < HELD; ++v) {
         raw16_t r = __builtin_bit_cast(raw16_t, raw[v]);
         asm volatile("" : "+v"(r));
         raw[v] = __builtin_bit_cast(Vec16<TIn>, r);
@@ -307,7 +319,16 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
 
   float m = xt;
 #pragma unroll
-  for (int v = 0; v < VPL; ++v)
+  for (int v = HELD; v < VPL; v += 2) {  // (two at a time, behind the loads of the held ones)
+    __builtin_amdgcn_sched_barrier(0);
+    const Vec16<TIn> t0 = fetch(v, true);
+    const Vec16<TIn> t1 = fetch(v + 1 < VPL ? v + 1 : v, true);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) m = fmaxf(m, fmaxf(to_f32(t0.v[e]), to_f32(t1.v[e])));
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int v = 0; v < HELD; ++v)
 #pragma unroll
     for (int e = 0; e < EPV; ++e) m = fmaxf(m, to_f32(raw[v].v[e]));
   m = wave_max(m);
@@ -318,7 +339,7 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
   xt = LOG ? xt - m : ext;
   float s = ext;
 #pragma unroll
-  for (int v = 0; v < VPL; ++v)
+  for (int v = 0; v < HELD; ++v) {
 #pragma unroll
     for (int e = 0; e < EPV; ++e) {
       const float d = to_f32(raw[v].v[e]) - m;
@@ -326,6 +347,21 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
       if constexpr (IN_PLACE) raw[v].v[e] = LOG ? d : ex;
       s += ex;
     }
+    if constexpr (BLOCK == 512) __builtin_amdgcn_sched_barrier(0);  // (one vector's temporaries at a time)
+  }
+  // (in the order of the held form: the sum is the same; two vectors in flight at a time)
+#pragma unroll
+  for (int v = HELD; v < VPL; v += 2) {
+    const Vec16<TIn> t0 = fetch(v, true);
+    const Vec16<TIn> t1 = fetch(v + 1 < VPL ? v + 1 : v, true);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) s += exp_for<TOut>(to_f32(t0.v[e]) - m);
+    if (v + 1 < VPL) {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) s += exp_for<TOut>(to_f32(t1.v[e]) - m);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   s = wave_sum(s);
   s = group_reduce(s, slot, wave, 0, WAVES, SumOp{});
   const float lg = logf(s), inv = 1.0f / s;
@@ -335,9 +371,14 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
   for (int v = 0; v < VPL; ++v) {
     const uint32_t vi = lane_vec + v * (WAVES * kWave);
     float y[EPV];
+    Vec16<TIn> t;
+    if (v >= HELD) t = fetch(v, true);  // (compile-time: the loop is unrolled)
 #pragma unroll
     for (int e = 0; e < EPV; ++e) {
-      if constexpr (IN_PLACE) {
+      if (v >= HELD) {
+        const float d = to_f32(t.v[e]) - m;
+        y[e] = LOG ? d - lg : exp_for<TOut>(d) * inv;
+      } else if constexpr (IN_PLACE) {
         y[e] = LOG ? to_f32(raw[v].v[e]) - lg : to_f32(raw[v].v[e]) * inv;
       } else {
         const float d = to_f32(raw[v].v[e]) - m;
@@ -345,29 +386,34 @@ __global__ __launch_bounds__(1024, 8) void softmax_long_rows_lean_kernel(TOut* _
       }
     }
     if (vi < static_cast<uint32_t>(nvec)) {
-      TOut* at = reinterpret_cast<TOut*>(dst_b + static_cast<size_t>(vi) * (EPV * sizeof(TOut)));
+      // (a uniform base per vector plus one lane offset for all of them: an offset per vector
+      // would be kept in a register each from the loads on)
+      TOut* at = reinterpret_cast<TOut*>(dst_b + static_cast<size_t>(v) * (WAVES * kWave * EPV * sizeof(TOut)) +
+                                         lane_vec * static_cast<uint32_t>(EPV * sizeof(TOut)));
       if constexpr (PEEL) {
         store_converted<TOut, EPV, STREAM>(at, y);
       } else {
         store_converted_unaligned<TOut, EPV>(at, y);
       }
     }
+    if constexpr (BLOCK == 512) __builtin_amdgcn_sched_barrier(0);
   }
   if (edge >= 0) dst[edge] = from_f32<TOut>(LOG ? xt - lg : xt * inv);
 }
 
-template <typename TIn, typename TOut, int VPL, bool LOG>
+template <typename TIn, typename TOut, int VPL, bool LOG, int BLOCK = 1024, int HELD = VPL>
 static int launch_long_rows(TOut* out, const TIn* in, int64_t rows, int64_t cols,
                             hipStream_t stream) {
-  const dim3 grid(static_cast<unsigned>(rows)), block(1024);
+  const dim3 grid(static_cast<unsigned>(rows)), block(BLOCK);
   const int c = static_cast<int>(cols);
   // rows that fit 52 registers per lane take the kernel that shares a CU between two rows
-  // (16-bit rows only: fp32 rows of 8 or 13 vectors per lane do not fit 64 registers and spill)
-  constexpr bool LEAN = sizeof(TIn) == 2 && VPL > 4;
+  // (16-bit rows in 1024-thread workgroups; fp32 rows, which would spill there, in 512-thread
+  // workgroups with twice the registers)
+  constexpr bool LEAN = (sizeof(TIn) == 2 && VPL > 4) || BLOCK == 512;
 #define TMB_LONG(PEEL, STREAM)                                                                        \
   do {                                                                                                \
     if constexpr (LEAN)                                                                               \
-      softmax_long_rows_lean_kernel<TIn, TOut, VPL, LOG, PEEL, STREAM><<<grid, block, 0, stream>>>(out, in, c); \
+      softmax_long_rows_lean_kernel<TIn, TOut, VPL, LOG, PEEL, STREAM, BLOCK, HELD><<<grid, block, 0, stream>>>(out, in, c); \
     else                                                                                              \
       softmax_long_rows_kernel<TIn, TOut, VPL, LOG, PEEL, STREAM><<<grid, block, 0, stream>>>(out, in, c);      \
   } while (0)
@@ -488,6 +534,11 @@ static int softmax_dispatch(TOut* out, const TIn* in, int64_t rows, int64_t cols
         if (cols / EPV <= 1024 * 7) return launch_long_rows<TIn, TOut, 7, LOG>(out, in, rows, cols, stream);
         return launch_long_rows<TIn, TOut, 8, LOG>(out, in, rows, cols, stream);
       } else {
+        if constexpr (sizeof(TIn) == 4) {
+          // (16384 x 50257 log-softmax: 1.30 -> 1.26 ms)
+          if (cols / EPV <= 512 * 13) return launch_long_rows<TIn, TOut, 13, LOG, 512>(out, in, rows, cols, stream);
+          if (cols / EPV <= 512 * 25) return launch_long_rows<TIn, TOut, 25, LOG, 512, (LOG ? 17 : 15)>(out, in, rows, cols, stream);
+        }
         return launch_long_rows<TIn, TOut, MAXV, LOG>(out, in, rows, cols, stream);
       }
     }
