@@ -165,7 +165,7 @@ def test_argmax_shapes(shape):
 # elements in front of / behind the whole vectors of a unit (odd pitches), units with a single
 # vector per lane and with seven, rows of exactly one unit, storage offsets.
 VEC_SHAPES = [(3, 2048), (5, 2049), (7, 4099), (2, 7168), (2, 7169), (4, 7233), (33, 14336), (9, 14337),
-              (512, 50257), (32, 50257), (1, 50257), (2048, 6151), (1, 1 << 20), (3, (1 << 21) + 5)]
+              (512, 50257), (300, 57344), (257, 57347), (256, 2048), (260, 28673), (32, 50257), (1, 50257), (2048, 6151), (1, 1 << 20), (3, (1 << 21) + 5)]
 
 
 def _argmax_adversarial(shape, dtype, seed):
@@ -239,18 +239,26 @@ def test_argmax_rows_that_start_anywhere(dtype):
 def test_argmax_workspace_is_what_the_entry_point_asks_for():
     ek = _ek()
     L = ek.lib()
-    need = L.tmb_argmax_workspace_bytes(512, 50257, ek.F32)
-    assert need == 512 * 8 * 16                       # eight units per row, 16 bytes each
+    stream = torch.cuda.current_stream().cuda_stream
+    # at least a row per CU of fp32 rows that a workgroup holds: whole rows, one launch, no workspace
+    assert L.tmb_argmax_workspace_bytes(512, 50257, ek.F32) == 0
+    x = _dev(seeded((512, 50257), seed=1))
+    out = torch.empty(512, dtype=torch.int64, device=x.device)
+    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 512, 50257, ek.F32, None, 0, stream) == 0
+    assert torch.equal(out.cpu(), torch.argmax(x.cpu(), dim=1))
+    # fewer rows: units of a row and a combining launch, 16 bytes per unit
+    need = L.tmb_argmax_workspace_bytes(128, 50257, ek.F32)
+    assert need > 0 and need % (128 * 16) == 0
     assert L.tmb_argmax_workspace_bytes(512, 50257, ek.I64) == L.tmb_reduce_workspace_bytes(512, 50257, ek.I64)
     assert L.tmb_argmax_workspace_bytes(4096, 4096, ek.F32) == 0        # one unit per row
     assert L.tmb_argmax_workspace_bytes(0, 4096, ek.F32) == 0
-    x = _dev(seeded((512, 50257), seed=1))
-    out = torch.empty(512, dtype=torch.int64, device=x.device)
     small = torch.empty(need - 16, dtype=torch.uint8, device=x.device)
-    stream = torch.cuda.current_stream().cuda_stream
-    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 512, 50257, ek.F32, small.data_ptr(),
+    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 128, 50257, ek.F32, small.data_ptr(),
                              need - 16, stream) == ek.ERR_WORKSPACE
-    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 512, 50257, ek.F32, None, 0, stream) == ek.ERR_WORKSPACE
+    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 128, 50257, ek.F32, None, 0, stream) == ek.ERR_WORKSPACE
+    full = torch.empty(need, dtype=torch.uint8, device=x.device)
+    assert L.tmb_argmax_rows(out.data_ptr(), x.data_ptr(), 128, 50257, ek.F32, full.data_ptr(), need, stream) == 0
+    assert torch.equal(out[:128].cpu(), torch.argmax(x[:128].cpu(), dim=1))
 
 
 def test_argmax_dim_none_keepdim_and_nan():
