@@ -296,6 +296,21 @@ int tmb_gelu_backward(void* grad_in, const void* grad_out, const void* in, int64
 int tmb_softmax_backward_rows(void* grad_in, const void* grad_out, const void* out, int64_t rows,
                               int64_t cols, int dtype, int log_mode, void* stream);
 
+/* The gradient a cross-entropy loss sends to the logits, from the saved log-probabilities
+ * logp [rows, cols] (row pitch ldi) and the int64 targets [rows]: the dense NLL gradient (-w at a
+ * row's target unless that is ignore_index or no class; w = grad_out / total_weight for
+ * reduction 1 = mean, grad_out for 2 = sum, grad_out[row] for 0 = none; grad_out and total_weight
+ * are device scalars of the tensor type) sent through the log-softmax backward,
+ * dx = g - exp(logp) * rowsum(g), without g being stored. dx has a row pitch of its own
+ * (ldo >= cols, a whole number of 16-byte vectors, dx 16-byte aligned); columns cols .. ldo-1 are
+ * set to zero, so a consumer that needs rows of whole vectors can take dx as it is.
+ * Replaces NllLossBackwardF32 (eager_kernels/aten_fast.py:3450-3497, loss_ops.mojo:234-311)
+ * followed by `_log_softmax_backward_data` (aten_functions.py:788-833). */
+int tmb_nll_log_softmax_backward_rows(void* dx, const void* logp, const int64_t* target,
+                                      const void* grad_out, const void* total_weight, int64_t rows,
+                                      int64_t cols, int64_t ldi, int64_t ldo, int reduction,
+                                      int64_t ignore_index, int dtype, void* stream);
+
 /* Layer-norm backward over contiguous [rows, cols] from the saved fp32 statistics:
  *   grad_in    = rstd * (g dy - mean_row(g dy) - xhat * mean_row(g dy xhat)),  xhat = (x - mean) rstd
  *   grad_gamma = sum over rows of dy * xhat,   grad_beta = sum over rows of dy

@@ -89,6 +89,7 @@ def lib() -> ctypes.CDLL:
         L.orc_gather_rows.restype = ci
         L.orc_softmax_backward.argtypes = [vp, vp, vp, i64, i64, ci, ci]
         L.orc_layer_norm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, vp]
+        L.orc_nll_log_softmax_backward.argtypes = [vp, vp, vp, vp, vp, i64, i64, ci, i64, ci, vp]
         for f in (L.orc_gelu_backward, L.orc_softmax_backward, L.orc_layer_norm_backward):
             f.restype = ci
         L.orc_convert_to_f32.argtypes = [vp, vp, i64, ci]
@@ -324,6 +325,23 @@ def softmax_backward_rows(grad: torch.Tensor, out: torch.Tensor, log: bool) -> t
         _check(lib().orc_softmax_backward(res.data_ptr(), grad.data_ptr(), out.data_ptr(),
                                           out.shape[0], out.shape[1], _code(out.dtype), int(log)),
                "softmax_backward")
+    return res
+
+
+def nll_log_softmax_backward(grad_out: torch.Tensor, logp: torch.Tensor, target: torch.Tensor,
+                             total_weight: torch.Tensor, reduction: int, ignore_index: int) -> torch.Tensor:
+    """What ``nll_loss_backward`` followed by ``_log_softmax_backward_data`` hands to the logits
+    (reference: eager_kernels/loss_ops.mojo:234-311, aten_functions.py:788-833)."""
+    grad_out, logp, target = _cpu(grad_out).to(logp.dtype), _cpu(logp), _cpu(target)
+    total_weight = _cpu(total_weight).to(logp.dtype)
+    assert logp.dim() == 2 and target.dtype == torch.int64 and target.shape == (logp.shape[0],)
+    res = torch.empty_like(logp)
+    scratch = torch.empty_like(logp)
+    if logp.numel():
+        _check(lib().orc_nll_log_softmax_backward(
+            res.data_ptr(), logp.data_ptr(), target.data_ptr(), grad_out.contiguous().data_ptr(),
+            total_weight.contiguous().data_ptr(), logp.shape[0], logp.shape[1], int(reduction),
+            int(ignore_index), _code(logp.dtype), scratch.data_ptr()), "nll_log_softmax_backward")
     return res
 
 

@@ -35,6 +35,8 @@
  *                           row_len + i % row_len]); out-of-range indices read the nearest row
  *   orc_softmax_backward    ../aten_functions.py:788-833 (grad - exp(out) * sum(grad)) and its
  *                           softmax twin out * (grad - sum(grad * out))
+ *   orc_nll_log_softmax_backward  loss_ops.mojo:234-311 (dense NLL gradient) followed by
+ *                           orc_softmax_backward's log form
  *   orc_layer_norm_backward aten_fast.py:2797-2913 (LayerNormBackwardF32: grad_input from the
  *                           saved mean / rstd, grad_weight = sum dy*xhat, grad_bias = sum dy)
  *
@@ -496,6 +498,28 @@ int orc_softmax_backward(void* gin, const void* gout, const void* y, int64_t row
     }
   }
   return 0;
+}
+
+/* The dense gradient of the negative log-likelihood loss with respect to the log-probabilities
+ * (loss_ops.mojo:234-311: scale = grad_output / total_weight for the mean, grad_output for the
+ * sum, grad_output[row] without reduction; -scale at a row's target when that is a class and not
+ * ignore_index, 0 elsewhere), stored in the tensor type, and the log-softmax backward of it
+ * (orc_softmax_backward): what a cross-entropy loss sends back to the logits. reduction: 0 none,
+ * 1 mean, 2 sum (ATen's codes). scratch: rows * cols elements of the tensor type. */
+int orc_nll_log_softmax_backward(void* dx, const void* logp, const int64_t* target,
+                                 const void* grad_out, const void* total_weight, int64_t rows,
+                                 int64_t cols, int reduction, int64_t ignore_index, int dtype,
+                                 void* scratch) {
+  float scale = 0.0f;
+  if (reduction == 1) scale = load_f(grad_out, 0, dtype) / load_f(total_weight, 0, dtype);
+  else if (reduction == 2) scale = load_f(grad_out, 0, dtype);
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t t = target[r];
+    const int valid = t != ignore_index && t >= 0 && t < cols;
+    const float g = valid ? -(reduction == 0 ? load_f(grad_out, r, dtype) : scale) : 0.0f;
+    for (int64_t j = 0; j < cols; ++j) store_f(scratch, r * cols + j, dtype, (valid && j == t) ? g : 0.0f);
+  }
+  return orc_softmax_backward(dx, scratch, logp, rows, cols, dtype, 1);
 }
 
 /* dgamma / dbeta are accumulated row after row in fp32 (any of the outputs may be NULL). */

@@ -118,6 +118,107 @@ def test_softmax_backward_invariants_and_dims():
         torch.testing.assert_close(got, xr.grad, rtol=1e-5, atol=1e-6)
 
 
+# ---- cross-entropy: NLL backward + log-softmax backward in one pass ------------------------------
+LOSS_SHAPES = [(1, 5), (7, 64), (33, 1000), (64, 4104), (19, 50257), (300, 257), (5, 8200)]
+
+
+def _loss_case(shape, dtype, seed):
+    rows, cols = shape
+    x = seeded(shape, seed=seed, dtype=torch.float32) * 3
+    logp = torch.log_softmax(x, -1).to(dtype)
+    g = torch.Generator().manual_seed(seed + 1)
+    target = torch.randint(0, cols, (rows,), generator=g)
+    target[::5] = -100                       # ignored rows
+    if rows > 2:
+        target[1], target[2] = 0, cols - 1   # first and last class
+    return logp, target
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", LOSS_SHAPES)
+@pytest.mark.parametrize("reduction", [0, 1, 2])
+def test_nll_log_softmax_backward(shape, dtype, reduction):
+    rows, cols = shape
+    logp, target = _loss_case(shape, dtype, seed=13)
+    valid = int((target != -100).sum())
+    total_weight = torch.tensor(float(max(valid, 1)), dtype=dtype)
+    grad_out = (seeded((rows,), seed=15).abs() + 0.5).to(dtype) if reduction == 0 \
+        else torch.tensor(0.75, dtype=dtype)
+    got = _ops().nll_log_softmax_backward(grad_out.cuda(), logp.cuda(), target.cuda(),
+                                          total_weight.cuda(), reduction, -100)
+    assert got.dtype == dtype and tuple(got.shape) == shape
+    # float64 closed form: w * (softmax - onehot), zero rows where the target is ignored
+    p = np.exp(as64(logp))
+    w = as64(grad_out) if reduction == 0 else np.full(rows, float(grad_out))
+    if reduction == 1:
+        w = w / float(total_weight)
+    onehot = np.zeros(shape)
+    keep = (target != -100).numpy()
+    onehot[np.arange(rows)[keep], target.numpy()[keep]] = 1.0
+    want = (w * keep)[:, None] * (p - onehot)
+    bound = 2 * TOL[dtype] * (np.abs(want).max() + np.abs(w).max())
+    assert np.abs(as64(got) - want).max() <= bound
+    # the C restatement of the reference's two kernels
+    ref = oracle.nll_log_softmax_backward(grad_out, logp, target, total_weight, reduction, -100)
+    assert np.abs(as64(got) - as64(ref)).max() <= bound
+    # and, bit for bit, the two kernels this pass stands for
+    dense = torch.ops.aten.nll_loss_backward(grad_out.cuda(), logp.cuda(), target.cuda(), None, reduction,
+                                             -100, total_weight.cuda())
+    two = _ops().softmax_backward(dense, logp.cuda(), -1, True)
+    if dtype == torch.float16:
+        # (fp16 only: the compiler may fold the last multiply-add into the conversion, one rounding
+        # instead of two, in one kernel and not in the other: a unit in the last place, rarely)
+        differ = got != two
+        assert int(differ.sum()) <= max(1, got.numel() // 1000)
+        assert ((got.double() - two.double()).abs() <= 2.0 ** -10 * two.double().abs() + 1e-12).all()
+    else:
+        assert torch.equal(got, two)
+    # rows of whole 16-byte vectors with zeros behind the last class
+    unit = 16 // logp.element_size()
+    if cols % unit:
+        assert got.stride(0) == (cols + 63) // 64 * 64 and got.stride(0) % unit == 0
+        whole = got.as_strided((rows, got.stride(0)), (got.stride(0), 1), got.storage_offset())
+        assert float(whole[:, cols:].abs().max()) == 0.0
+    else:
+        assert got.is_contiguous()
+
+
+def test_nll_log_softmax_backward_reads_strided_rows_and_feeds_the_products():
+    """Log-probabilities that are a column slice of something wider (pitch > classes), and the
+    products that take the result as an operand: the padded buffer is found instead of copied."""
+    rows, cols, hidden = 2048, 50257, 64
+    wide = torch.log_softmax(seeded((rows, cols + 3), seed=21) * 2, -1).bfloat16().cuda()
+    logp = wide[:, 1:cols + 1]
+    target = torch.randint(0, cols, (rows,), generator=torch.Generator().manual_seed(3)).cuda()
+    one, tw = torch.tensor(1.0).bfloat16().cuda(), torch.tensor(float(rows)).bfloat16().cuda()
+    ops = _ops()
+    copies = []
+    plain_copy = ops._pad_last_copy
+
+    def counting(t, size):
+        copies.append((tuple(t.shape), size))
+        return plain_copy(t, size)
+
+    w = (seeded((cols, hidden), seed=22) * 0.05).bfloat16().cuda()
+    x = seeded((rows, hidden), seed=23).bfloat16().cuda()
+    before = ops.pad_reuse_begin()
+    ops._pad_last_copy = counting
+    try:
+        dl = ops.nll_log_softmax_backward(one, logp, target, tw, 1, -100)
+        dx = ops.gemm(dl, w)            # contracts over the classes
+        dw = ops.gemm(dl.t(), x)        # has them as its transposed dimension
+        torch.cuda.synchronize()
+    finally:
+        ops._pad_last_copy = plain_copy
+        ops.pad_reuse_end(before)
+    assert not [c for c in copies if c[0] == (rows, cols)], copies
+    ref = oracle.nll_log_softmax_backward(one.cpu(), logp.cpu().contiguous(), target.cpu(), tw.cpu(), 1, -100)
+    assert torch.equal(dl.cpu(), ref) or (dl.cpu().double() - ref.double()).abs().max() <= 2.0 ** -8 / rows
+    for got, want in ((dx, ref.double() @ w.cpu().double()), (dw, ref.double().t() @ x.cpu().double())):
+        err = (got.cpu().double() - want).norm() / want.norm()
+        assert err < 4e-3, err
+
+
 # ---- layer norm ---------------------------------------------------------------------------------
 LN_SHAPES = [(1, 8), (5, 65), (33, 768), (64, 1000), (9, 4096), (300, 768), (7, 12288), (3, 50257)]
 

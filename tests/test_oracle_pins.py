@@ -529,6 +529,36 @@ def test_gelu_backward_oracle_vs_autograd_and_limits(dtype, approximate):
     assert torch.allclose(lim, torch.tensor([1.0, 2.0, 0.0]), atol=1e-6)
 
 
+@pytest.mark.parametrize("reduction", ["none", "mean", "sum"])
+def test_nll_log_softmax_backward_oracle_vs_autograd(reduction):
+    """The oracle's loss backward against float64 autograd of `nll_loss(log_softmax(x))`, with
+    ignored rows, for every reduction; and by brute force on a tiny case."""
+    torch.manual_seed(5)
+    x = torch.randn(9, 37, dtype=torch.float64, requires_grad=True)
+    t = torch.randint(0, 37, (9,))
+    t[3], t[7] = -100, -100
+    logp = torch.log_softmax(x, 1)
+    loss = torch.nn.functional.nll_loss(logp, t, reduction=reduction)
+    up = torch.rand(9, dtype=torch.float64) + 0.5 if reduction == "none" else torch.tensor(1.25, dtype=torch.float64)
+    loss.backward(up)
+    code = {"none": 0, "mean": 1, "sum": 2}[reduction]
+    got = oracle.nll_log_softmax_backward(up.float(), logp.detach().float(), t, torch.tensor(7.0), code, -100)
+    torch.testing.assert_close(got.double(), x.grad, rtol=1e-5, atol=1e-6)
+    assert float(got[3].abs().max()) == 0.0 and float(got[7].abs().max()) == 0.0
+    # brute force: w * (exp(logp) - [c == t])
+    lp = logp.detach().float()
+    for r in (0, 4):
+        w = float(up[r]) if reduction == "none" else float(up) / (7.0 if reduction == "mean" else 1.0)
+        for c in (0, int(t[r]), 36):
+            want = w * (float(torch.exp(lp[r, c])) - (1.0 if c == int(t[r]) else 0.0))
+            assert abs(float(got[r, c]) - want) <= 1e-6
+    # a target that is no class behaves like an ignored one (the reference kernel's rule)
+    t2 = t.clone()
+    t2[0] = 37
+    got2 = oracle.nll_log_softmax_backward(up.float(), lp, t2, torch.tensor(7.0), code, -100)
+    assert float(got2[0].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("log", [False, True])
 def test_softmax_backward_oracle_vs_autograd_and_invariants(log):
     x = seeded((7, 130), seed=3)

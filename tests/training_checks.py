@@ -287,6 +287,59 @@ def vocabulary_projection_backward_pads_its_gradient_once():
         assert err < 4e-3, err
 
 
+def cross_entropy_in_the_graph_sends_one_pass_back_to_the_logits():
+    """A cross-entropy loss computed inside the compiled function, over a 50257-wide vocabulary:
+    the backward graph's nll_loss_backward + _log_softmax_backward_data pair runs as one pass that
+    writes rows of whole vectors, so neither product of the projection's backward pads the
+    gradient again; ignored targets, mean and sum reductions, gradients against float64."""
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    torch.manual_seed(0)
+    rows, hidden, vocab = 1024, 128, 50257
+    w = (torch.randn(vocab, hidden) * 0.05).bfloat16()
+    x = torch.randn(rows, hidden).bfloat16()
+    t = torch.randint(0, vocab, (rows,))
+    t[::7] = -100
+
+    for reduction in ("mean", "sum"):
+        def fn(inp, weight, target):
+            return F.cross_entropy(inp @ weight.t(), target, reduction=reduction)
+
+        fused, copies = [], []
+        plain, plain_copy = hip_ops.nll_log_softmax_backward, hip_ops._pad_last_copy
+
+        def counting(*args):
+            fused.append(tuple(args[1].shape))
+            return plain(*args)
+
+        def counting_copy(tensor, size):
+            if tensor.numel() * tensor.element_size() >= hip_ops._PAD_REUSE_MIN_BYTES:
+                copies.append((tuple(tensor.shape), size))
+            return plain_copy(tensor, size)
+
+        hip_ops.nll_log_softmax_backward, hip_ops._pad_last_copy = counting, counting_copy
+        try:
+            xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+            torch._dynamo.reset()
+            loss = torch.compile(fn, backend=mojo_backend)(xd, wd, t.cuda())
+            loss.backward()
+            torch.cuda.synchronize()
+        finally:
+            hip_ops.nll_log_softmax_backward, hip_ops._pad_last_copy = plain, plain_copy
+        assert fused == [(rows, vocab)], fused
+        assert copies == [], copies
+        assert hip_ops.pad_reuse_active() is None
+        x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+        want = F.cross_entropy(x64 @ w64.t(), t, reduction=reduction)
+        want.backward()
+        assert abs(float(loss) - float(want)) <= 2e-2 * abs(float(want))
+        for got, ref in ((xd.grad, x64.grad), (wd.grad, w64.grad)):
+            assert got.shape == ref.shape and got.is_contiguous()
+            err = (got.cpu().double() - ref).norm() / ref.norm()
+            assert err < 2e-2, (reduction, err)
+
+
 if __name__ == "__main__":
     import os
 

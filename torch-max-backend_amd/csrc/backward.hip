@@ -944,6 +944,110 @@ extern "C" int tmb_gelu_backward(void* grad_in, const void* grad_out, const void
   }
 }
 
+namespace tmb {
+
+// What a cross-entropy loss sends back to the logits, from the saved log-probabilities in one
+// pass: dx[r, c] = g[c] - exp(logp[r, c]) * s with g the dense NLL gradient of row r (-w at the
+// row's target, 0 elsewhere) and s its row sum (-w), i.e. the arithmetic of
+// softmax_backward_long_rows_kernel on that gradient without the gradient ever being stored. w is
+// grad_out / total_weight (mean), grad_out (sum) or grad_out[r] (no reduction), rounded to the
+// tensor type as the separate kernel would have stored it; rows whose target is ignore_index or
+// no class get zeros. The rows of dx have a pitch of their own (ldo >= cols, whole 16-byte
+// vectors, zero beyond cols), so the products that consume the result need no padded copy of it.
+// A workgroup takes 256 * U vectors of one row: aligned stores, loads wherever the input row lies.
+template <typename T, int U>
+__global__ __launch_bounds__(256) void nll_log_softmax_backward_kernel(
+    T* __restrict__ dx, const T* __restrict__ logp, const int64_t* __restrict__ target,
+    const T* __restrict__ grad_out, const T* __restrict__ total_weight, int64_t cols, int64_t ldi,
+    int64_t ldo, int chunks, int reduction, int64_t ignore_index) {
+  constexpr int EPV = Vec16<T>::N;
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = static_cast<int>(blockIdx.x - row * chunks);
+  const int64_t t = target[row];
+  const bool valid = t != ignore_index && t >= 0 && t < cols;
+  float w = 0.0f;
+  if (valid) {
+    if (reduction == 1) w = to_f32(grad_out[0]) / to_f32(total_weight[0]);
+    else if (reduction == 2) w = to_f32(grad_out[0]);
+    else w = to_f32(grad_out[row]);
+  }
+  const float g_t = to_f32(from_f32<T>(-w));  // the gradient at the target, as it would be stored
+  const float s = g_t;                         // the row sum of that gradient
+  const T* src = logp + row * ldi;
+  T* dst = dx + row * ldo;
+  const bool stream = static_cast<int64_t>(gridDim.x) * 256 * U * 32 >= kStreamStoreBytes;
+  const int64_t nvec_out = ldo / EPV;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t vi = (static_cast<int64_t>(chunk) * U + u) * 256 + threadIdx.x;
+    if (vi >= nvec_out) continue;
+    const int64_t c0 = vi * EPV;
+    float r[EPV];
+    if (c0 + EPV <= cols) {
+      const Vec16<T> y = load_vec16_unaligned(src + c0);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float g = (c0 + e == t) ? g_t : 0.0f;
+        r[e] = valid ? g - exp_for<T>(to_f32(y.v[e])) * s : 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const int64_t c = c0 + e;
+        const float g = (c == t) ? g_t : 0.0f;
+        r[e] = (valid && c < cols) ? g - exp_for<T>(to_f32(src[c < cols ? c : 0])) * s : 0.0f;
+      }
+    }
+    store_converted_hinted<T, EPV>(dst + c0, r, stream);
+  }
+}
+
+template <typename T>
+static int nll_log_softmax_backward_dispatch(void* dx, const void* logp, const int64_t* target,
+                                             const void* grad_out, const void* total_weight,
+                                             int64_t rows, int64_t cols, int64_t ldi, int64_t ldo,
+                                             int reduction, int64_t ignore_index, hipStream_t stream) {
+  constexpr int EPV = Vec16<T>::N;
+  constexpr int U = 4;
+  if (ldo % EPV != 0 || ldo < cols || ldi < cols || !aligned16(dx)) return TMB_ERR_INVALID_ARGUMENT;
+  const int64_t nvec_out = ldo / EPV;
+  const int64_t chunks = (nvec_out + 256 * U - 1) / (256 * U);
+  if (rows * chunks >= (int64_t{1} << 31)) return TMB_ERR_UNSUPPORTED;
+  nll_log_softmax_backward_kernel<T, U><<<dim3(static_cast<unsigned>(rows * chunks)), dim3(256), 0, stream>>>(
+      static_cast<T*>(dx), static_cast<const T*>(logp), target, static_cast<const T*>(grad_out),
+      static_cast<const T*>(total_weight), cols, ldi, ldo, static_cast<int>(chunks), reduction,
+      ignore_index);
+  return check_launch();
+}
+
+}  // namespace tmb
+
+extern "C" int tmb_nll_log_softmax_backward_rows(void* dx, const void* logp, const int64_t* target,
+                                                 const void* grad_out, const void* total_weight,
+                                                 int64_t rows, int64_t cols, int64_t ldi, int64_t ldo,
+                                                 int reduction, int64_t ignore_index, int dtype,
+                                                 void* stream) {
+  if (rows < 0 || cols < 0 || reduction < 0 || reduction > 2) return TMB_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || cols == 0) return TMB_OK;
+  if (dx == nullptr || logp == nullptr || target == nullptr || grad_out == nullptr ||
+      (reduction == 1 && total_weight == nullptr))
+    return TMB_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  using namespace tmb;
+  switch (dtype) {
+    case TMB_F32:
+      return nll_log_softmax_backward_dispatch<float>(dx, logp, target, grad_out, total_weight, rows, cols,
+                                                      ldi, ldo, reduction, ignore_index, s);
+    case TMB_F16:
+      return nll_log_softmax_backward_dispatch<f16_t>(dx, logp, target, grad_out, total_weight, rows, cols,
+                                                      ldi, ldo, reduction, ignore_index, s);
+    case TMB_BF16:
+      return nll_log_softmax_backward_dispatch<bf16_t>(dx, logp, target, grad_out, total_weight, rows, cols,
+                                                       ldi, ldo, reduction, ignore_index, s);
+    default: return TMB_ERR_UNSUPPORTED;
+  }
+}
+
 extern "C" int tmb_softmax_backward_rows(void* grad_in, const void* grad_out, const void* out,
                                          int64_t rows, int64_t cols, int dtype, int log_mode,
                                          void* stream) {

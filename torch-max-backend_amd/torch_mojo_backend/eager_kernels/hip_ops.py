@@ -925,6 +925,46 @@ def softmax_backward(grad: torch.Tensor, out: torch.Tensor, dim: int, log: bool)
     return res if dim == last else res.transpose(dim, last).contiguous()
 
 
+def nll_log_softmax_backward(grad_output: torch.Tensor, logp: torch.Tensor, target: torch.Tensor,
+                             total_weight: Optional[torch.Tensor], reduction: int,
+                             ignore_index: int) -> torch.Tensor:
+    """``_log_softmax_backward_data(nll_loss_backward(grad_output, logp, target, None, reduction,
+    ignore_index, total_weight), logp, 1, logp.dtype)`` in one pass over the saved
+    log-probabilities ``logp`` [rows, classes], without the dense NLL gradient in between
+    (reference: eager_kernels/aten_fast.py:3450-3497 + aten_functions.py:788-833). The result is a
+    [rows, classes] view of rows of whole 16-byte vectors with zeros behind each row; while a
+    compiled graph keeps padded copies (`pad_reuse_begin`), the products that take it as an
+    operand find that buffer instead of padding the view again."""
+    require_hip(grad_output, logp, target, total_weight)
+    if logp.dim() != 2 or logp.dtype not in FLOAT_DTYPES or target.dtype != torch.int64 or \
+            tuple(target.shape) != (logp.shape[0],) or reduction not in (0, 1, 2):
+        raise TypeError(f"nll_log_softmax_backward: logp {tuple(logp.shape)} {logp.dtype}, target "
+                        f"{tuple(target.shape)} {target.dtype}, reduction {reduction}")
+    rows, cols = logp.shape
+    if grad_output.numel() != (rows if reduction == 0 else 1) or \
+            (reduction == 1 and (total_weight is None or total_weight.numel() != 1)):
+        raise ValueError("nll_log_softmax_backward: grad_output / total_weight do not fit the reduction")
+    lp = logp if logp.stride(1) == 1 and (rows <= 1 or logp.stride(0) >= cols) else logp.contiguous()
+    go = grad_output.to(logp.dtype).contiguous()
+    tw = None if total_weight is None else total_weight.to(logp.dtype).contiguous()
+    unit = 16 // logp.element_size()
+    ldo = cols if cols % unit == 0 else (cols + 63) // 64 * 64   # the width `_relayout_for_mfma` pads to
+    buf = torch.empty((rows, ldo), dtype=logp.dtype, device=logp.device)
+    if buf.numel():
+        _check("tmb_nll_log_softmax_backward_rows", _ek.lib().tmb_nll_log_softmax_backward_rows(
+            buf.data_ptr(), lp.data_ptr(), target.contiguous().data_ptr(), go.data_ptr(),
+            None if tw is None else tw.data_ptr(), rows, cols, lp.stride(0) if rows > 1 else cols, ldo,
+            int(reduction), int(ignore_index), code_of(logp.dtype), _stream()))
+    if ldo == cols:
+        return buf
+    out = buf[:, :cols]
+    reuse = getattr(_PAD_STATE, "reuse", None)
+    if reuse is not None and out.numel() * out.element_size() >= _PAD_REUSE_MIN_BYTES:
+        reuse.clear()
+        reuse[(out.data_ptr(), tuple(out.shape), out.stride(), out.dtype, ldo)] = (out, buf)
+    return out
+
+
 def layer_norm_backward(grad: torch.Tensor, x: torch.Tensor, normalized_shape: Sequence[int],
                         mean: torch.Tensor, rstd: torch.Tensor, weight: Optional[torch.Tensor],
                         output_mask: Sequence[bool]):

@@ -462,6 +462,44 @@ class _GraphFactory:
         return out
 
     @staticmethod
+    def _fuse_loss_backward(graph: torch.fx.Graph) -> dict:
+        """nll_loss_backward (no class weights, single user) -> _log_softmax_backward_data over
+        dimension 1 of the same 2-D log-probabilities: what a cross-entropy loss sends back to
+        the logits. The second node becomes one pass over the log-probabilities; the dense NLL
+        gradient is never written. Returns {node: None (skip) | ("loss_bwd", grad_output, logp,
+        target, total_weight, reduction, ignore_index)}."""
+        out: dict = {}
+        lsm = MAPPING_TORCH_ATEN_TO_MOJO.get(aten._log_softmax_backward_data)
+        if lsm is None or lsm is not _BUILTIN_LOG_SOFTMAX_BACKWARD or \
+                MAPPING_TORCH_ATEN_TO_MOJO.get(aten.nll_loss_backward) is not _BUILTIN_NLL_LOSS_BACKWARD:
+            return out  # (somebody replaced one of the two mappings: their nodes stay as they are)
+        for node in graph.nodes:
+            if node.op != "call_function" or node.target is not aten._log_softmax_backward_data.default:
+                continue
+            if len(node.args) < 4:
+                continue
+            grad, logp, dim, in_dtype = node.args[:4]
+            if not (isinstance(grad, torch.fx.Node) and grad.op == "call_function"
+                    and grad.target is aten.nll_loss_backward.default and len(grad.users) == 1):
+                continue
+            if len(grad.args) != 7 or grad.kwargs:
+                continue
+            g_out, self_, target, weight, reduction, ignore_index, total_weight = grad.args
+            lv = logp.meta.get("val") if isinstance(logp, torch.fx.Node) else None
+            sv = self_.meta.get("val") if isinstance(self_, torch.fx.Node) else None
+            # (nll_loss_backward takes nothing but the shape and type from its `self`, which in a
+            # backward graph is another saved alias of the same log-probabilities)
+            if sv is None or lv is None or tuple(sv.shape) != tuple(lv.shape) or sv.dtype != lv.dtype or \
+                    weight is not None or lv.dim() != 2 or \
+                    dim not in (1, -1) or in_dtype != lv.dtype or reduction not in (0, 1, 2) or \
+                    lv.dtype not in (torch.float32, torch.float16, torch.bfloat16) or \
+                    not isinstance(ignore_index, int):
+                continue
+            out[node] = ("loss_bwd", g_out, logp, target, total_weight, reduction, ignore_index)
+            out[grad] = None
+        return out
+
+    @staticmethod
     def _widen_residual_stream(plans: dict) -> None:
         """A fused residual step of a 16-bit graph whose result only feeds other fused residual
         steps (as their residual operand) and native_layer_norm nodes (as their input) hands that
@@ -564,6 +602,7 @@ class _GraphFactory:
             softmax_rewrites.update(self._fuse_residual_add(graph, {**rewrites, **softmax_rewrites}))
             if not twice:
                 self._widen_residual_stream(softmax_rewrites)
+            softmax_rewrites.update(self._fuse_loss_backward(graph))
         nodes = list(graph.nodes)
         # what each node reads after the rewrites (liveness must follow the rewritten program)
         reads: dict = {}
@@ -578,6 +617,8 @@ class _GraphFactory:
                     reads[node] = [plan[1], plan[2], plan[3], plan[4]]
                 elif plan[0] == "wide_ln":
                     reads[node] = list(node.all_input_nodes)
+                elif plan[0] == "loss_bwd":
+                    reads[node] = [x for x in plan[1:5] if isinstance(x, torch.fx.Node)]
                 else:
                     reads[node] = [plan[1], plan[2], plan[3], plan[5]]
             else:
@@ -614,6 +655,9 @@ class _GraphFactory:
                         args = plan[1:]
                     elif plan[0] == "wide_ln":
                         fn, kwargs = _WIDE_LAYER_NORM, {"out_dtype": plan[1]}
+                    elif plan[0] == "loss_bwd":
+                        fn, kwargs = _FUSED_LOSS_BACKWARD, {}
+                        args = plan[1:]
                     else:
                         fn, kwargs = _FUSED_ATTENTION, {}
                         args = plan[1:]
@@ -823,6 +867,21 @@ def _fused_addmm_residual(bias, mat1, mat2, residual, out_shape, out_dtype, *,
     return total.float() if out_dtype is torch.float32 else total
 
 
+def _fused_loss_backward(grad_output, logp, target, total_weight, reduction, ignore_index):
+    """The gradient of a cross-entropy loss with respect to its logits from the saved
+    log-probabilities (`hip_ops.nll_log_softmax_backward`); anything the kernel does not take
+    runs as the two nodes it stands for."""
+    if isinstance(logp, torch.Tensor) and logp.is_cuda and logp.dim() == 2 and target.is_cuda and \
+            target.dtype == torch.int64 and grad_output.is_cuda and \
+            (total_weight is None or total_weight.is_cuda):
+        from ..eager_kernels import hip_ops
+        return hip_ops.nll_log_softmax_backward(grad_output, logp, target, total_weight, reduction,
+                                                ignore_index)
+    dense = torch.ops.aten.nll_loss_backward.default(grad_output, logp, target, None, reduction,
+                                                     ignore_index, total_weight)
+    return MAPPING_TORCH_ATEN_TO_MOJO[aten._log_softmax_backward_data](dense, logp, 1, logp.dtype)
+
+
 def _wide_layer_norm(input, normalized_shape, weight, bias, eps, *, out_dtype):
     """native_layer_norm whose input is a float32 residual stream of a 16-bit graph: statistics
     and normalisation from the float32 row, one cast to the graph's dtype."""
@@ -969,11 +1028,14 @@ _BUILTIN_MUL = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.mul)
 _BUILTIN_EQ = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.eq)
 _BUILTIN_SLICE = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.slice)
 _BUILTIN_ALIAS = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.alias)
+_BUILTIN_LOG_SOFTMAX_BACKWARD = MAPPING_TORCH_ATEN_TO_MOJO.get(aten._log_softmax_backward_data)
+_BUILTIN_NLL_LOSS_BACKWARD = MAPPING_TORCH_ATEN_TO_MOJO.get(aten.nll_loss_backward)
 _FUSED_ADDMM_GELU = _fused_addmm_gelu
 _FUSED_MASKED_SOFTMAX = _fused_masked_softmax
 _FUSED_ATTENTION = _fused_attention
 _FUSED_ADDMM_RESIDUAL = _fused_addmm_residual
 _WIDE_LAYER_NORM = _wide_layer_norm
+_FUSED_LOSS_BACKWARD = _fused_loss_backward
 
 
 def _graph_home(gm: torch.fx.GraphModule, example_inputs: list) -> str:
