@@ -598,7 +598,18 @@ def main() -> int:
                     lambda i: lib.tmb_softmax_backward_rows(outs[0].data_ptr(), gs[0].data_ptr(),
                                                             ys[0].data_ptr(), rows, cols, code, 1, stream),
                     3 * nb, steps=20)
-            del ys, gs, outs
+            # the same gradient when it comes from a cross-entropy loss: one pass over the saved
+            # log-probabilities, rows of whole vectors out (pitch 50304)
+            ldo = (cols + 63) // 64 * 64
+            tgt = torch.randint(0, cols, (rows,), device=dev, generator=torch.Generator(device=dev).manual_seed(7))
+            one, tw = torch.ones((), dtype=dtype, device=dev), torch.full((), float(rows), dtype=dtype, device=dev)
+            padded = torch.empty((rows, ldo), dtype=dtype, device=dev)
+            hbm_row(f"cross_entropy_backward_{dn}_{rows}x{cols}", 1,
+                    lambda i: lib.tmb_nll_log_softmax_backward_rows(
+                        padded.data_ptr(), ys[0].data_ptr(), tgt.data_ptr(), one.data_ptr(), tw.data_ptr(),
+                        rows, cols, cols, ldo, 1, -100, code, stream),
+                    2 * nb, steps=20)
+            del ys, gs, outs, padded
             # layer norm backward (all three outputs)
             for (rows, cols) in ((32768, 768), (16384, 4096)):
                 nb = rows * cols * es
