@@ -400,9 +400,11 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
 }
 
 // grad_input and the parameter-gradient partials in one pass: a group of WPR waves walks `walk`
-// consecutive rows; every lane keeps the column sums of dy*xhat and dy for the columns it owns
-// in registers and writes them once, as one fp32 partial row per group, at the end. dy and x are
-// read exactly once.
+// rows, one from each sweep of all the launch's groups over the matrix (group g takes rows g,
+// g + groups, g + 2 groups, ...: at any moment the launch reads one contiguous span; a run of
+// consecutive rows per group, whose starts lie a power of two apart, measured 3-12 % slower);
+// every lane keeps the column sums of dy*xhat and dy for the columns it owns in registers and
+// writes them once, as one fp32 partial row per group, at the end. dy and x are read exactly once.
 template <typename T, int WPR, int VPL, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
     T* __restrict__ dx, float* __restrict__ partial, const T* __restrict__ dy,
@@ -418,7 +420,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
   const int nvec = cols / EPV;
   const float n = static_cast<float>(cols);
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * GROUPS + group;
-  const int64_t first = gid * walk;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * GROUPS;  // groups of the launch
 
   Vec16<T> gv[VPL];
   if (gamma != nullptr) {
@@ -437,7 +439,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
   // every group of the workgroup runs `walk` iterations (the reductions contain barriers); rows
   // past the end re-read the last row and contribute nothing
   for (int64_t i = 0; i < walk; ++i) {
-    int64_t row = first + i;
+    int64_t row = gid + i * step;
     const bool live = row < rows;
     if (!live) row = rows - 1;
     const T* dsrc = dy + row * static_cast<int64_t>(cols);
@@ -493,11 +495,12 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
   }
 }
 
-// Rows of up to 1024 columns: one wave per row and no barrier inside the walk. A workgroup of
-// four waves takes 4 * walk consecutive rows (wave w the w-th run of `walk` rows), two rows per
-// iteration so that four row reads are in flight per wave; every lane keeps the column sums of
-// dy * xhat and dy for its own columns in registers. At the end the four waves add their sums
-// through LDS in wave order and the workgroup writes one fp32 partial row.
+// Rows of up to 1024 columns: one wave per row and no barrier inside the walk. A wave takes
+// `walk` rows, one from each sweep of all the launch's waves over the matrix (wave w takes rows
+// w, w + waves, w + 2 waves, ...), two rows per iteration so that four row reads are in flight
+// per wave; every lane keeps the column sums of dy * xhat and dy for its own columns in
+// registers. At the end the four waves of a workgroup add their sums through LDS in wave order
+// and the workgroup writes one fp32 partial row.
 template <typename T, int VPL>
 __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
     T* __restrict__ dx, float* __restrict__ partial, const T* __restrict__ dy,
@@ -510,7 +513,8 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int nvec = cols / EPV;
   const float n = static_cast<float>(cols);
-  const int64_t first = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * walk;
+  const int64_t wid = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * 4;  // waves of the launch
 
   Vec16<T> gv[VPL];
   if (gamma != nullptr) {
@@ -532,7 +536,7 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
     bool live[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
-      row[r] = first + i + r;
+      row[r] = wid + (i + r) * step;
       live[r] = row[r] < rows && i + r < walk;
       if (!live[r]) row[r] = rows - 1;  // any valid row: its values are masked out below
 #pragma unroll
@@ -609,8 +613,9 @@ static int64_t narrow_groups(int64_t rows) {
 
 // Geometry of the fused kernel (a pure function of the shape: the workspace size and the order
 // of the final summation follow from it): waves per row as in the forward kernels, about 2048
-// waves in flight (measured best of 1024 .. 16384), 8 to 64 rows per group, partial rows for
-// whole workgroups.
+// waves in flight for rows of up to four waves and 4096 for wider ones (measured best of
+// 1024 .. 16384 in both classes: more groups cost more partial rows, fewer leave the memory
+// system short of requests), 8 to 64 rows per group, partial rows for whole workgroups.
 struct FusedPlan {
   int wpr, groups_per_block;
   int64_t walk, groups, padded_groups;
@@ -620,7 +625,7 @@ static FusedPlan fused_plan(int64_t rows, int64_t nvec) {
   p.wpr = nvec <= 64 ? 1 : nvec <= 256 ? 2 : nvec <= 512 ? 4 : nvec <= 1024 ? 8 : 16;
   const int block = nvec <= 512 ? 256 : nvec <= 1024 ? 512 : 1024;
   p.groups_per_block = block / kWave / p.wpr;
-  const int64_t target = 2048 / p.wpr;
+  const int64_t target = (p.wpr >= 8 ? 4096 : 2048) / p.wpr;
   p.walk = (rows + target - 1) / target;
   if (p.walk < 8) p.walk = 8;
   if (p.walk > 64) p.walk = 64;
