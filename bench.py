@@ -627,6 +627,19 @@ def main() -> int:
                             xs[i].data_ptr(), stats[i][0].data_ptr(), stats[i][1].data_ptr(),
                             gamma.data_ptr(), rows, cols, code, wsp.data_ptr(), ws_b, stream),
                         3 * nb + 3 * cols * es + 2 * rows * 4)
+                # the same pass where its grad_input re-joins a residual stream: the by-passing
+                # gradient added on the way out, the column sums of the result handed out as well
+                # (the add and the bias-gradient sum that would follow as passes of their own)
+                ws_a = lib.tmb_layer_norm_backward_add_workspace_bytes(rows, cols, code)
+                wsa = torch.empty(max(ws_a, 16), dtype=torch.uint8, device=dev)
+                dsm = torch.empty_like(gamma)
+                hbm_row(f"layer_norm_backward_add_{dn}_{rows}x{cols}", len(xs),
+                        lambda i: lib.tmb_layer_norm_backward_add_rows(
+                            dxs[i].data_ptr(), dgm.data_ptr(), dbt.data_ptr(), dsm.data_ptr(),
+                            gs[i].data_ptr(), xs[i].data_ptr(), stats[i][0].data_ptr(),
+                            stats[i][1].data_ptr(), gamma.data_ptr(), gs[(i + 1) % len(xs)].data_ptr(),
+                            rows, cols, code, wsa.data_ptr(), ws_a, stream),
+                        4 * nb + 4 * cols * es + 2 * rows * 4)
                 del xs, gs, dxs, stats
         # the two GEMMs of linear_backward for the MLP up-projection: dgrad (NN) and wgrad (TN)
         rows_, in_f, out_f = 32768, 768, 3072

@@ -325,6 +325,25 @@ int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_bet
                                  const float* rstd, const void* gamma, int64_t rows, int64_t cols,
                                  int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* tmb_layer_norm_backward_rows where the gradient re-joins the residual stream of a decoder
+ * block (x <- x + f(norm(x))): what is stored is grad_in = round(dx) + addend, rounded again
+ * (addend: the gradient that by-passed the block, same shape and type, may be NULL), and
+ * grad_sum [cols] receives the column sums of the stored grad_in (may be NULL): the bias gradient
+ * of the projection in front of the norm. At least one of the two is given; grad_in, grad_gamma
+ * and grad_beta are all wanted. The result equals the three separate steps it replaces, each
+ * storing its result in the tensor type: this layer-norm backward, `aten.add`
+ * (aten_functions.py:939, fast_aten_add aten_fast.py:1010-1024) and `aten.sum` over the leading
+ * dimension (aten_functions.py:3310-3312); the column sums are added in an order of their own
+ * that depends on the shape only. Shapes outside the one-pass kernels (cols not a whole number of
+ * 16-byte vectors, more than 8192 columns) report TMB_ERR_UNSUPPORTED and a workspace size of 0:
+ * the caller then runs the three steps. */
+size_t tmb_layer_norm_backward_add_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+int tmb_layer_norm_backward_add_rows(void* grad_in, void* grad_gamma, void* grad_beta,
+                                     void* grad_sum, const void* grad_out, const void* in,
+                                     const float* mean, const float* rstd, const void* gamma,
+                                     const void* addend, int64_t rows, int64_t cols, int dtype,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
 /* Concatenation of two contiguous row blocks: out[r] = a[r] ++ b[r] for `rows` rows of
  * `a_row_bytes` and `b_row_bytes` bytes (any element type; the widest of 16/4/2/1-byte pieces that
  * the lengths and the three addresses allow is moved). With rows = the product of the dims in

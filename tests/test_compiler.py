@@ -652,3 +652,92 @@ def test_training_partition_leaves_graphs_without_attention_alone():
         torch.testing.assert_close(g, w)
     for ga, gb in zip(a_graphs, b_graphs):
         assert [n.target for n in ga.graph.nodes] == [n.target for n in gb.graph.nodes]
+
+
+def test_layer_norm_backward_takes_the_residual_gradient_and_the_bias_sums_along(monkeypatch):
+    """A two-block decoder's backward graph: every native_layer_norm_backward whose grad_input
+    re-joins the residual stream becomes one step that takes the by-passing gradient along and
+    hands the bias gradient of the projection in front of it to the sum node; run with host
+    stand-ins for the three ops, the rewritten program returns what the graph itself returns."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch._functorch.partitioners import default_partition
+
+    idx, targets = seeded_tokens(2, 8, seed=0), seeded_tokens(2, 8, seed=1)
+    graphs, _ = _partitioned_training_graphs(build_gpt2_small(seed=0, n_layer=2), idx, targets,
+                                             default_partition)
+    bw = graphs[1]
+    plans = compiler._GraphFactory._fuse_norm_backward_add(bw.graph)
+    kinds = [p[0] for p in plans.values()]
+    # the final norm (bias sums only), two norms per block (an addend each; all but the first
+    # block's first norm also feed a projection's bias gradient)
+    assert kinds.count("ln_bwd_add") == 5 and kinds.count("take") == 4 and kinds.count("colsum") == 4
+    with_addend = [p for p in plans.values() if p[0] == "ln_bwd_add" and p[1] is not None]
+    assert len(with_addend) == 4 and sum(1 for p in plans.values() if p[0] == "ln_bwd_add" and p[2]) == 4
+    order = {n: i for i, n in enumerate(bw.graph.nodes)}
+    for node, plan in plans.items():
+        if plan[0] == "ln_bwd_add" and plan[1] is not None:
+            assert order[plan[1]] < order[node]       # the addend exists when the step runs
+        if plan[0] == "colsum":
+            assert tuple(node.meta["val"].shape) == plan[2]
+    # somebody else's layer-norm backward: nothing is rewritten
+    with monkeypatch.context() as mp:
+        mp.setitem(MAPPING_TORCH_ATEN_TO_MOJO, aten.native_layer_norm_backward, lambda *a: None)
+        assert compiler._GraphFactory._fuse_norm_backward_add(bw.graph) == {}
+
+    # execute: PyTorch's kernels behind every entry the backward graph uses
+    calls = []
+
+    def ln_bwd(*a):
+        calls.append("ln_bwd")
+        return aten.native_layer_norm_backward.default(*a)
+
+    def add(a, b, alpha=1):
+        calls.append("add")
+        return torch.add(a, b, alpha=alpha)
+
+    def total(x, dim=None, keepdim=False, dtype=None):
+        calls.append("sum")
+        return torch.sum(x, dim, keepdim, dtype=dtype) if dim is not None else torch.sum(x, dtype=dtype)
+
+    for op, name, fn in ((aten.native_layer_norm_backward, "_BUILTIN_LAYER_NORM_BACKWARD", ln_bwd),
+                         (aten.add, "_BUILTIN_ADD", add), (aten.sum, "_BUILTIN_SUM", total)):
+        monkeypatch.setitem(MAPPING_TORCH_ATEN_TO_MOJO, op, fn)
+        monkeypatch.setattr(compiler, name, fn)
+    for op in {n.target for n in bw.graph.nodes if n.op == "call_function"}:
+        key = op if op in MAPPING_TORCH_ATEN_TO_MOJO else getattr(op, "overloadpacket", op)
+        if key not in (aten.native_layer_norm_backward, aten.add, aten.sum, operator.getitem):
+            monkeypatch.setitem(MAPPING_TORCH_ATEN_TO_MOJO, key, op if key is op else getattr(torch.ops.aten, key.__name__))
+    program = compiler._GraphFactory().create_graph(bw.graph)
+    fused = [s for s in program.steps if s.fn is compiler._FUSED_NORM_BACKWARD_ADD]
+    assert len(fused) == 5
+    assert sum(1 for s in program.steps if s.fn is compiler._TAKE_COLUMN_SUMS) == 4
+    placeholders = [n for n in bw.graph.nodes if n.op == "placeholder"]
+    torch.manual_seed(3)
+    inputs = []
+    for p in placeholders:
+        v = p.meta["val"]
+        if v.dtype.is_floating_point:
+            inputs.append(torch.randn(v.shape, dtype=v.dtype))
+        else:
+            inputs.append(torch.randint(0, 2 if v.dtype == torch.bool else 50, tuple(v.shape)).to(v.dtype))
+    want = bw(*inputs)
+    env = [None] * len(program.slots)
+    for slot, value in zip(program.input_slots, inputs):
+        env[slot] = value
+    for slot, value in program.constants:
+        env[slot] = value
+    for step in program.steps:
+        a = compiler._materialize(step.args, env) if step.dynamic_args else step.args
+        k = compiler._materialize(step.kwargs, env) if step.dynamic_kwargs else step.kwargs
+        env[step.out] = step.fn(*a, **k)
+        for slot in step.release:
+            env[slot] = None
+    got = compiler._materialize(program.output_template, env)
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+        else:
+            torch.testing.assert_close(g, w, rtol=1e-5, atol=1e-6)
+    # the four joins ran inside the fused steps' host route, the four bias sums as well
+    assert calls.count("ln_bwd") == 5

@@ -274,6 +274,74 @@ def test_layer_norm_backward_invariants_and_masks():
     assert torch.equal(only_params[1], again[1]) and torch.equal(only_params[2], again[2])
 
 
+LN_ADD_SHAPES = [(5, 64), (33, 768), (300, 768), (1030, 1024), (64, 1000), (9, 4096), (70, 2048),
+                 (40, 8192), (7, 12288)]
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", LN_ADD_SHAPES)
+@pytest.mark.parametrize("form", ["add+sum", "add", "sum"])
+def test_layer_norm_backward_add(shape, dtype, form):
+    """grad_input + addend and its column sums in the layer-norm backward's own pass: the same
+    values as the three separate steps (bit for bit in bfloat16 and float32; float16 may round an
+    element the other way where the compiler folds the conversion into the multiply)."""
+    rows, cols = shape
+    ops = _ops()
+    x = seeded(shape, seed=31, dtype=dtype).cuda()
+    g = seeded(shape, seed=32, dtype=dtype).cuda()
+    a = seeded(shape, seed=33, dtype=dtype).cuda() if "add" in form else None
+    w = (1 + 0.1 * seeded((cols,), seed=34)).to(dtype).cuda()
+    _, mean, rstd = ops.layer_norm(x, [cols], w, None, 1e-5)
+    got = ops.layer_norm_backward_add(g, x, [cols], mean, rstd, w, a, "sum" in form)
+    epv = 16 // x.element_size()
+    covered = cols % epv == 0 and cols // epv <= (2048 if dtype == torch.float32 else 1024)
+    if not covered:
+        assert got is None
+        return
+    dx, dw, db, ds = got
+    rdx, rdw, rdb = ops.layer_norm_backward(g, x, [cols], mean, rstd, w, [True, True, True])
+    want = rdx if a is None else rdx + a
+    if dtype == torch.float16:
+        off = (dx != want)
+        assert off.float().mean().item() <= 1e-3
+        assert (dx.double() - want.double()).abs().max().item() <= \
+            2.0 ** -10 * (want.double().abs().max().item() + 1.0)
+    else:
+        assert torch.equal(dx, want)
+    for mine, theirs in ((dw, rdw), (db, rdb)):
+        scale = theirs.double().abs().max().item() + 1.0
+        assert (mine.double() - theirs.double()).abs().max().item() <= TOL[dtype] * scale
+    if "sum" in form:
+        ref = dx.double().sum(0)
+        bound = TOL[dtype] * (ref.abs().max().item() + 1.0) + rows * 2.0 ** -22 * dx.double().abs().max().item()
+        assert ds.shape == (cols,) and ds.dtype == dtype
+        assert (ds.double() - ref).abs().max().item() <= 4 * bound
+    else:
+        assert ds is None
+    # against the CPU restatement of the layer-norm backward, with the add and its two roundings
+    odx, _, _ = oracle.layer_norm_backward_rows(g.cpu(), x.cpu(), mean.cpu(), rstd.cpu(), w.cpu())
+    owant = odx if a is None else (odx + a.cpu())
+    scale = owant.double().abs().max().item() + 1.0
+    assert (dx.cpu().double() - owant.double()).abs().max().item() <= TOL[dtype] * scale * 4
+
+
+def test_layer_norm_backward_add_rejects_what_it_cannot_mean():
+    ops = _ops()
+    x = seeded((8, 64), seed=35).cuda()
+    _, mean, rstd = ops.layer_norm(x, [64], None, None, 1e-5)
+    with pytest.raises(ValueError):
+        ops.layer_norm_backward_add(x, x, [64], mean, rstd, None, None, False)
+    with pytest.raises(ValueError):
+        ops.layer_norm_backward_add(x, x, [64], mean, rstd, None, x[:4], True)
+    from torch_mojo_backend import eager_kernels
+    lib = eager_kernels.lib()
+    assert lib.tmb_layer_norm_backward_add_workspace_bytes(8, 63, 0) == 0
+    rc = lib.tmb_layer_norm_backward_add_rows(x.data_ptr(), x.data_ptr(), x.data_ptr(), None, x.data_ptr(),
+                                              x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), None, None,
+                                              8, 64, 0, None, 0, None)
+    assert rc == -1  # neither an addend nor the column sums
+
+
 # ---- linear -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [((4, 33, 64), 48), ((512, 768), 2304), ((8, 128, 768), 768)])

@@ -340,6 +340,50 @@ def cross_entropy_in_the_graph_sends_one_pass_back_to_the_logits():
             assert err < 2e-2, (reduction, err)
 
 
+def residual_gradient_joins_inside_the_layer_norm_backward():
+    """Two decoder blocks: each native_layer_norm_backward of the backward graph also adds the
+    gradient that by-passed its block and hands out the bias gradient of the projection in front
+    of it (one pass instead of three). Every matrix gradient equals, bit for bit, that of the same
+    graph run with the three ops apart; the vectors (bias and norm gradients, whose sums are
+    added in another order) agree to rounding."""
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.eager_kernels import hip_ops
+
+    idx, targets = seeded_tokens(4, 64, seed=0).cuda(), seeded_tokens(4, 64, seed=1).cuda()
+    plain = hip_ops.layer_norm_backward_add
+    for dtype in (torch.bfloat16, torch.float32):
+        grads = {}
+        for route in ("one pass", "apart"):
+            taken = []
+
+            def counting(*args):
+                taken.append((args[6] is not None, args[7]))
+                return plain(*args) if route == "one pass" else None
+
+            hip_ops.layer_norm_backward_add = counting
+            try:
+                torch._dynamo.reset()
+                model = build_gpt2_small(seed=0, n_layer=2).to(dtype).cuda()
+                loss = _loss(torch.compile(model, backend=mojo_backend), idx, targets)
+                loss.backward()
+                torch.cuda.synchronize()
+            finally:
+                hip_ops.layer_norm_backward_add = plain
+            # the final norm (sums only), then four norms with the by-passing gradient, the last
+            # of which feeds no projection
+            assert taken == [(False, True), (True, True), (True, True), (True, True), (True, False)], taken
+            grads[route] = {n: p.grad.clone() for n, p in model.named_parameters()}
+        for name, got in grads["one pass"].items():
+            want = grads["apart"][name]
+            if got.dim() >= 2:
+                assert torch.equal(got, want), (dtype, name)
+            else:
+                scale = want.double().abs().max().item() + 1e-6
+                tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+                assert (got.double() - want.double()).abs().max().item() <= tol * scale, (dtype, name)
+
+
 if __name__ == "__main__":
     import os
 

@@ -341,6 +341,20 @@ static int softmax_backward_dispatch(void* gin_, const void* gout_, const void* 
 // ---------------------------------------------------------------------------
 // layer norm backward: grad_input
 // ---------------------------------------------------------------------------
+// rstd * (g dy - mean(g dy) - xhat * mean(g dy xhat)) with b1 = -rstd * mean(g dy) and
+// b2 = -rstd * mean(g dy xhat): two multiply-adds per element.
+__device__ __forceinline__ float grad_input_of(float gd, float xh, float rs, float b1, float b2) {
+  return __builtin_fmaf(gd, rs, __builtin_fmaf(xh, b2, b1));
+}
+
+// The vector, or zeros: four selects for the 16 bytes instead of one per element.
+template <typename T>
+__device__ __forceinline__ Vec16<T> keep_if(const Vec16<T>& v, bool keep) {
+  const raw16_t zero = {0u, 0u, 0u, 0u};
+  const raw16_t r = keep ? __builtin_bit_cast(raw16_t, v) : zero;
+  return __builtin_bit_cast(Vec16<T>, r);
+}
+
 template <typename T, int WPR, int VPL, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
     T* __restrict__ dx, const T* __restrict__ dy, const T* __restrict__ x,
@@ -354,7 +368,7 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int group = wave / WPR, wave_in_row = wave - group * WPR;
   const int nvec = cols / EPV;
-  const float n = static_cast<float>(cols);
+  const float inv_n = 1.0f / static_cast<float>(cols);
   int64_t row = static_cast<int64_t>(blockIdx.x) * GROUPS + group;
   const bool live = row < rows;
   if (!live) row = rows - 1;
@@ -387,14 +401,14 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
   s2 = wave_sum(s2);
   s2 = group_reduce(s2, slot, wave, group * WPR, WPR, SumOp{});
   if (!live) return;
-  const float m1 = s1 / n, m2 = s2 / n;
+  const float b1 = -rs * (s1 * inv_n), b2 = -rs * (s2 * inv_n);
   T* dst = dx + row * static_cast<int64_t>(cols);
 #pragma unroll
   for (int v = 0; v < VPL; ++v) {
     const int vi = (v * WPR + wave_in_row) * kWave + lane;
     float r[EPV];
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) r[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
+    for (int e = 0; e < EPV; ++e) r[e] = grad_input_of(gd[v][e], xh[v][e], rs, b1, b2);
     if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r, stream);
   }
 }
@@ -405,12 +419,17 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_dx_kernel(
 // consecutive rows per group, whose starts lie a power of two apart, measured 3-12 % slower);
 // every lane keeps the column sums of dy*xhat and dy for the columns it owns in registers and
 // writes them once, as one fp32 partial row per group, at the end. dy and x are read exactly once.
-template <typename T, int WPR, int VPL, int BLOCK>
+// EXTRA: as in the narrow kernel below (round(dx) + addend is stored, its column sums are a third
+// partial row per group).
+template <typename T, int WPR, int VPL, int BLOCK, bool EXTRA = false>
 __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
     T* __restrict__ dx, float* __restrict__ partial, const T* __restrict__ dy,
     const T* __restrict__ x, const float* __restrict__ mean, const float* __restrict__ rstd,
-    const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk) {
+    const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk,
+    const T* __restrict__ addend = nullptr) {
   constexpr int EPV = Vec16<T>::N;
+  constexpr int NR = EXTRA ? 3 : 2;
+  constexpr int XV = EXTRA ? VPL : 1;
   const bool stream = rows * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WAVES = BLOCK / kWave;
   constexpr int GROUPS = WAVES / WPR;
@@ -418,23 +437,28 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int group = wave / WPR, wave_in_row = wave - group * WPR;
   const int nvec = cols / EPV;
-  const float n = static_cast<float>(cols);
+  const float inv_n = 1.0f / static_cast<float>(cols);
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * GROUPS + group;
   const int64_t step = static_cast<int64_t>(gridDim.x) * GROUPS;  // groups of the launch
 
-  Vec16<T> gv[VPL];
-  if (gamma != nullptr) {
+  float gf[VPL][EPV];  // gamma, unpacked once
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-      const int vi = (v * WPR + wave_in_row) * kWave + lane;
-      gv[v] = load_vec16(gamma + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV);
-    }
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = (v * WPR + wave_in_row) * kWave + lane;
+    Vec16<T> gv;
+    if (gamma != nullptr) gv = load_vec16(gamma + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) gf[v][e] = gamma != nullptr ? to_f32(gv.v[e]) : 1.0f;
   }
-  float dg[VPL][EPV], db[VPL][EPV];
+  float dg[VPL][EPV], db[VPL][EPV], ds[XV][EPV];
 #pragma unroll
   for (int v = 0; v < VPL; ++v)
 #pragma unroll
     for (int e = 0; e < EPV; ++e) dg[v][e] = db[v][e] = 0.0f;
+#pragma unroll
+  for (int v = 0; v < XV; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) ds[v][e] = 0.0f;
 
   // every group of the workgroup runs `walk` iterations (the reductions contain barriers); rows
   // past the end re-read the last row and contribute nothing
@@ -446,19 +470,23 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
     const T* xsrc = x + row * static_cast<int64_t>(cols);
     const float mu = mean[row], rs = rstd[row];
     float gd[VPL][EPV], xh[VPL][EPV];
+    Vec16<T> av[XV];
     float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
       const int vi = (v * WPR + wave_in_row) * kWave + lane;
       const bool ok = vi < nvec && live;
       const int64_t at = static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
-      const Vec16<T> dv = load_vec16_stream(dsrc + at);
+      // (lanes past the row and rows past the end take part with dy = 0: see the narrow kernel)
+      const Vec16<T> dv = keep_if(load_vec16_stream(dsrc + at), ok);
       const Vec16<T> xv = load_vec16_stream(xsrc + at);
+      if constexpr (EXTRA)
+        av[v] = load_vec16_stream((addend != nullptr ? addend : dy) + row * static_cast<int64_t>(cols) + at);
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
-        const float d = ok ? to_f32(dv.v[e]) : 0.0f;
-        const float h = ok ? (to_f32(xv.v[e]) - mu) * rs : 0.0f;
-        gd[v][e] = d * (gamma != nullptr ? to_f32(gv[v].v[e]) : 1.0f);
+        const float d = to_f32(dv.v[e]);
+        const float h = (to_f32(xv.v[e]) - mu) * rs;
+        gd[v][e] = d * gf[v][e];
         xh[v][e] = h;
         s1 += gd[v][e];
         s2 += gd[v][e] * h;
@@ -471,26 +499,39 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
     s2 = wave_sum(s2);
     s2 = group_reduce(s2, slot, wave, group * WPR, WPR, SumOp{});
     if (live) {
-      const float m1 = s1 / n, m2 = s2 / n;
+      const float b1 = -rs * (s1 * inv_n), b2 = -rs * (s2 * inv_n);
       T* dst = dx + row * static_cast<int64_t>(cols);
 #pragma unroll
       for (int v = 0; v < VPL; ++v) {
         const int vi = (v * WPR + wave_in_row) * kWave + lane;
         float r[EPV];
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) r[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
+        for (int e = 0; e < EPV; ++e) r[e] = grad_input_of(gd[v][e], xh[v][e], rs, b1, b2);
+        if constexpr (EXTRA) {
+          // the two roundings of separate kernels: dx to T, then the sum to T
+          const Vec16<T> az = keep_if(av[v], addend != nullptr);
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) {
+            r[e] = to_f32(from_f32<T>(pin_f32(r[e]))) + to_f32(az.v[e]);
+            r[e] = to_f32(from_f32<T>(pin_f32(r[e])));
+            ds[v][e] += vi < nvec ? r[e] : 0.0f;
+          }
+        }
         if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, r, stream);
       }
     }
   }
-  float* pg = partial + (gid * 2 + 0) * static_cast<int64_t>(cols);
-  float* pb = partial + (gid * 2 + 1) * static_cast<int64_t>(cols);
+  float* pg = partial + (gid * NR + 0) * static_cast<int64_t>(cols);
+  float* pb = partial + (gid * NR + 1) * static_cast<int64_t>(cols);
 #pragma unroll
   for (int v = 0; v < VPL; ++v) {
     const int vi = (v * WPR + wave_in_row) * kWave + lane;
     if (vi < nvec) {
       store_converted<float, EPV>(pg + static_cast<int64_t>(vi) * EPV, dg[v]);
       store_converted<float, EPV>(pb + static_cast<int64_t>(vi) * EPV, db[v]);
+      if constexpr (EXTRA)
+        store_converted<float, EPV>(partial + (gid * NR + 2) * static_cast<int64_t>(cols) +
+                                        static_cast<int64_t>(vi) * EPV, ds[v]);
     }
   }
 }
@@ -501,37 +542,47 @@ __global__ __launch_bounds__(BLOCK) void layer_norm_backward_fused_kernel(
 // per wave; every lane keeps the column sums of dy * xhat and dy for its own columns in
 // registers. At the end the four waves of a workgroup add their sums through LDS in wave order
 // and the workgroup writes one fp32 partial row.
-template <typename T, int VPL>
+// EXTRA: the residual stream's form. grad_input is stored as round(dx) + addend (addend may be
+// null) and the column sums of what was stored leave as a third partial row per workgroup.
+template <typename T, int VPL, bool EXTRA = false>
 __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
     T* __restrict__ dx, float* __restrict__ partial, const T* __restrict__ dy,
     const T* __restrict__ x, const float* __restrict__ mean, const float* __restrict__ rstd,
-    const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk) {
+    const T* __restrict__ gamma, int64_t rows, int cols, int64_t walk,
+    const T* __restrict__ addend = nullptr) {
   constexpr int EPV = Vec16<T>::N;
+  constexpr int NR = EXTRA ? 3 : 2;    // partial rows per workgroup
+  constexpr int XV = EXTRA ? VPL : 1;  // (arrays of the extra outputs shrink to one vector without them)
   const bool stream = rows * cols * static_cast<int64_t>(3 * sizeof(T)) >= kStreamStoreBytes;
   constexpr int WIDTH = VPL * kWave * EPV;  // columns a wave covers
-  __shared__ float sums[4][2][WIDTH];
+  __shared__ float sums[4][NR][WIDTH];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int nvec = cols / EPV;
-  const float n = static_cast<float>(cols);
+  const float inv_n = 1.0f / static_cast<float>(cols);
   const int64_t wid = static_cast<int64_t>(blockIdx.x) * 4 + wave;
   const int64_t step = static_cast<int64_t>(gridDim.x) * 4;  // waves of the launch
 
-  Vec16<T> gv[VPL];
-  if (gamma != nullptr) {
+  float gf[VPL][EPV];  // gamma, unpacked once
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-      const int vi = v * kWave + lane;
-      gv[v] = load_vec16(gamma + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV);
-    }
+  for (int v = 0; v < VPL; ++v) {
+    const int vi = v * kWave + lane;
+    Vec16<T> gv;
+    if (gamma != nullptr) gv = load_vec16(gamma + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) gf[v][e] = gamma != nullptr ? to_f32(gv.v[e]) : 1.0f;
   }
-  float dg[VPL][EPV], db[VPL][EPV];
+  float dg[VPL][EPV], db[VPL][EPV], ds[XV][EPV];
 #pragma unroll
   for (int v = 0; v < VPL; ++v)
 #pragma unroll
     for (int e = 0; e < EPV; ++e) dg[v][e] = db[v][e] = 0.0f;
+#pragma unroll
+  for (int v = 0; v < XV; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) ds[v][e] = 0.0f;
 
   for (int64_t i = 0; i < walk; i += 2) {
-    Vec16<T> dv[2][VPL], xv[2][VPL];
+    Vec16<T> dv[2][VPL], xv[2][VPL], av[2][XV];
     int64_t row[2];
     bool live[2];
 #pragma unroll
@@ -545,6 +596,9 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
         const int64_t at = row[r] * static_cast<int64_t>(cols) + static_cast<int64_t>(vi < nvec ? vi : 0) * EPV;
         dv[r][v] = load_vec16_stream(dy + at);
         xv[r][v] = load_vec16_stream(x + at);
+        // (without an addend the load re-reads dy and is cleared below: a load under a
+        // condition would make every later wait a wait for all loads)
+        if constexpr (EXTRA) av[r][v] = load_vec16_stream((addend != nullptr ? addend : dy) + at);
       }
     }
 #pragma unroll
@@ -554,12 +608,14 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
       float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
       for (int v = 0; v < VPL; ++v) {
-        const bool ok = v * kWave + lane < nvec && live[r];
+        // lanes past the row and rows past the end take part with dy = 0 (whole vectors are
+        // cleared, not elements): every sum they feed then gets 0, whatever x they re-read
+        const Vec16<T> dz = keep_if(dv[r][v], v * kWave + lane < nvec && live[r]);
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
-          const float d = ok ? to_f32(dv[r][v].v[e]) : 0.0f;
-          const float h = ok ? (to_f32(xv[r][v].v[e]) - mu) * rs : 0.0f;
-          gd[v][e] = d * (gamma != nullptr ? to_f32(gv[v].v[e]) : 1.0f);
+          const float d = to_f32(dz.v[e]);
+          const float h = (to_f32(xv[r][v].v[e]) - mu) * rs;
+          gd[v][e] = d * gf[v][e];
           xh[v][e] = h;
           s1 += gd[v][e];
           s2 += gd[v][e] * h;
@@ -570,14 +626,24 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
       s1 = wave_sum(s1);
       s2 = wave_sum(s2);
       if (live[r]) {
-        const float m1 = s1 / n, m2 = s2 / n;
+        const float b1 = -rs * (s1 * inv_n), b2 = -rs * (s2 * inv_n);
         T* dst = dx + row[r] * static_cast<int64_t>(cols);
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
           const int vi = v * kWave + lane;
           float out[EPV];
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) out[e] = rs * (gd[v][e] - m1 - xh[v][e] * m2);
+          for (int e = 0; e < EPV; ++e) out[e] = grad_input_of(gd[v][e], xh[v][e], rs, b1, b2);
+          if constexpr (EXTRA) {
+            // the two roundings of separate kernels: dx to T, then the sum to T
+            const Vec16<T> az = keep_if(av[r][v], addend != nullptr);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+              out[e] = to_f32(from_f32<T>(pin_f32(out[e]))) + to_f32(az.v[e]);
+              out[e] = to_f32(from_f32<T>(pin_f32(out[e])));
+              ds[v][e] += vi < nvec ? out[e] : 0.0f;
+            }
+          }
           if (vi < nvec) store_converted_hinted<T, EPV>(dst + static_cast<int64_t>(vi) * EPV, out, stream);
         }
       }
@@ -590,11 +656,12 @@ __global__ __launch_bounds__(256) void layer_norm_backward_narrow_kernel(
       const int c = (v * kWave + lane) * EPV + e;
       sums[wave][0][c] = dg[v][e];
       sums[wave][1][c] = db[v][e];
+      if constexpr (EXTRA) sums[wave][2][c] = ds[v][e];
     }
   __syncthreads();
-  float* out = partial + static_cast<int64_t>(blockIdx.x) * 2 * cols;
-  for (int c = threadIdx.x; c < 2 * cols; c += 256) {
-    const int which = c >= cols ? 1 : 0, col = c - which * cols;
+  float* out = partial + static_cast<int64_t>(blockIdx.x) * NR * cols;
+  for (int c = threadIdx.x; c < NR * cols; c += 256) {
+    const int which = c / cols, col = c - which * cols;
     out[c] = ((sums[0][which][col] + sums[1][which][col]) + sums[2][which][col]) + sums[3][which][col];
   }
 }
@@ -641,7 +708,7 @@ __global__ __launch_bounds__(256) void layer_norm_backward_dx_generic_kernel(
     int64_t rows, int64_t cols) {
   __shared__ float slot[4];
   const int wave = threadIdx.x >> 6;
-  const float n = static_cast<float>(cols);
+  const float inv_n = 1.0f / static_cast<float>(cols);
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const T* dsrc = dy + row * cols;
     const T* xsrc = x + row * cols;
@@ -656,11 +723,11 @@ __global__ __launch_bounds__(256) void layer_norm_backward_dx_generic_kernel(
     s1 = group_reduce(s1, slot, wave, 0, 4, SumOp{});
     s2 = wave_sum(s2);
     s2 = group_reduce(s2, slot, wave, 0, 4, SumOp{});
-    const float m1 = s1 / n, m2 = s2 / n;
+    const float b1 = -rs * (s1 * inv_n), b2 = -rs * (s2 * inv_n);
     for (int64_t j = threadIdx.x; j < cols; j += 256) {
       const float d = to_f32(dsrc[j]) * (gamma != nullptr ? to_f32(gamma[j]) : 1.0f);
       const float xh = (to_f32(xsrc[j]) - mu) * rs;
-      dx[row * cols + j] = from_f32<T>(rs * (d - m1 - xh * m2));
+      dx[row * cols + j] = from_f32<T>(grad_input_of(d, xh, rs, b1, b2));
     }
   }
 }
@@ -754,46 +821,49 @@ __global__ __launch_bounds__(kParamWaves* kWave) void layer_norm_param_partial_k
 }
 
 // 32 columns per workgroup; the 32 threads that share a column take every 32nd slab and their
-// sums are added in thread order (fixed), so the result depends on the shape only.
-template <typename T>
+// sums are added in thread order (fixed), so the result depends on the shape only. A slab holds NR
+// partial rows (grad_gamma, grad_beta and, with NR = 3, the column sums of grad_input).
+template <typename T, int NR = 2>
 __global__ __launch_bounds__(1024) void layer_norm_param_final_kernel(
     T* __restrict__ dgamma, T* __restrict__ dbeta, const float* __restrict__ partial, int64_t cols,
-    int64_t slabs) {
-  __shared__ float lds[2][32][33];
+    int64_t slabs, T* __restrict__ dsum = nullptr) {
+  __shared__ float lds[NR][32][33];
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
   const int64_t col = static_cast<int64_t>(blockIdx.x) * 32 + tx;
-  float sg = 0.0f, sb = 0.0f;
+  float acc[NR];
+#pragma unroll
+  for (int k = 0; k < NR; ++k) acc[k] = 0.0f;
   if (col < cols) {
     int64_t s = ty;
-    for (; s + 96 < slabs; s += 128) {  // eight loads in flight, added in slab order
-      float vg[4], vb[4];
+    for (; s + 96 < slabs; s += 128) {  // 4 * NR loads in flight, added in slab order
+      float v[NR][4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        vg[u] = partial[((s + 32 * u) * 2 + 0) * cols + col];
-        vb[u] = partial[((s + 32 * u) * 2 + 1) * cols + col];
-      }
+      for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        sg += vg[u];
-        sb += vb[u];
-      }
+        for (int k = 0; k < NR; ++k) v[k][u] = partial[((s + 32 * u) * NR + k) * cols + col];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < NR; ++k) acc[k] += v[k][u];
     }
-    for (; s < slabs; s += 32) {
-      sg += partial[(s * 2 + 0) * cols + col];
-      sb += partial[(s * 2 + 1) * cols + col];
-    }
+    for (; s < slabs; s += 32)
+#pragma unroll
+      for (int k = 0; k < NR; ++k) acc[k] += partial[(s * NR + k) * cols + col];
   }
-  lds[0][ty][tx] = sg;
-  lds[1][ty][tx] = sb;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) lds[k][ty][tx] = acc[k];
   __syncthreads();
   if (ty == 0 && col < cols) {
-    float tg = lds[0][0][tx], tb = lds[1][0][tx];
-    for (int i = 1; i < 32; ++i) {
-      tg += lds[0][i][tx];
-      tb += lds[1][i][tx];
-    }
-    if (dgamma != nullptr) dgamma[col] = from_f32<T>(tg);
-    if (dbeta != nullptr) dbeta[col] = from_f32<T>(tb);
+    float t[NR];
+#pragma unroll
+    for (int k = 0; k < NR; ++k) t[k] = lds[k][0][tx];
+    for (int i = 1; i < 32; ++i)
+#pragma unroll
+      for (int k = 0; k < NR; ++k) t[k] += lds[k][i][tx];
+    if (dgamma != nullptr) dgamma[col] = from_f32<T>(t[0]);
+    if (dbeta != nullptr) dbeta[col] = from_f32<T>(t[1]);
+    if constexpr (NR == 3)
+      if (dsum != nullptr) dsum[col] = from_f32<T>(t[2]);
   }
 }
 
@@ -819,63 +889,95 @@ static int layer_norm_backward_dispatch(void* dx_, void* dgamma_, void* dbeta_, 
                                         const void* x_, const float* mean, const float* rstd,
                                         const void* gamma_, int64_t rows, int64_t cols,
                                         void* workspace, size_t workspace_bytes,
-                                        hipStream_t stream) {
+                                        hipStream_t stream, const void* addend_ = nullptr,
+                                        void* dsum_ = nullptr) {
   T* dx = static_cast<T*>(dx_);
   const T* dy = static_cast<const T*>(dy_);
   const T* x = static_cast<const T*>(x_);
   const T* gamma = static_cast<const T*>(gamma_);
+  const T* addend = static_cast<const T*>(addend_);
+  // the residual stream's form (an addend, column sums of grad_input, or both) exists in the two
+  // one-pass kernels only
+  const bool extra = addend_ != nullptr || dsum_ != nullptr;
   constexpr int EPV = Vec16<T>::N;
+  // (rows of up to 1024 columns are at most two 16-bit or four fp32 vectors per lane)
+  constexpr int kNarrowVpl = 1024 / (kWave * EPV);
   int rc = 0;
   if (dx != nullptr && (dgamma_ != nullptr || dbeta_ != nullptr) && cols % EPV == 0 && cols <= 1024 &&
       aligned16(dx) && aligned16(dy) && aligned16(x) && (gamma == nullptr || aligned16(gamma)) &&
-      rows < (int64_t{1} << 31)) {
+      (addend == nullptr || aligned16(addend)) && rows < (int64_t{1} << 31)) {
     const int64_t nvec = cols / EPV;
     const int64_t walk = narrow_walk(rows), groups = narrow_groups(rows);
-    if (workspace == nullptr || workspace_bytes < static_cast<size_t>(groups) * 2 * cols * 4)
+    const int nr = extra ? 3 : 2;
+    if (workspace == nullptr || workspace_bytes < static_cast<size_t>(groups) * nr * cols * 4)
       return TMB_ERR_WORKSPACE;
     float* partial = static_cast<float*>(workspace);
     const dim3 grid(static_cast<unsigned>(groups));
-#define TMB_LN(VPL)                                                                    \
-  layer_norm_backward_narrow_kernel<T, VPL><<<grid, dim3(256), 0, stream>>>(           \
-      dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), walk);
-    if (nvec <= 64) TMB_LN(1)
-    else if (nvec <= 128) TMB_LN(2)
-    else if (nvec <= 192) TMB_LN(3)
-    else TMB_LN(4)
+#define TMB_LN(VPL)                                                                              \
+  if constexpr (VPL <= kNarrowVpl) {                                                             \
+    if (extra)                                                                                   \
+      layer_norm_backward_narrow_kernel<T, VPL, true><<<grid, dim3(256), 0, stream>>>(           \
+          dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), walk, addend);    \
+    else                                                                                         \
+      layer_norm_backward_narrow_kernel<T, VPL, false><<<grid, dim3(256), 0, stream>>>(          \
+          dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), walk);            \
+  }
+    if (nvec <= 64) { TMB_LN(1) }
+    else if (nvec <= 128) { TMB_LN(2) }
+    else if (nvec <= 192) { TMB_LN(3) }
+    else { TMB_LN(4) }
 #undef TMB_LN
     rc = check_launch();
     if (rc != 0) return rc;
-    layer_norm_param_final_kernel<T><<<dim3(static_cast<unsigned>((cols + 31) / 32)), dim3(1024), 0, stream>>>(
-        static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, groups);
+    const dim3 fgrid(static_cast<unsigned>((cols + 31) / 32));
+    if (extra)
+      layer_norm_param_final_kernel<T, 3><<<fgrid, dim3(1024), 0, stream>>>(
+          static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, groups, static_cast<T*>(dsum_));
+    else
+      layer_norm_param_final_kernel<T, 2><<<fgrid, dim3(1024), 0, stream>>>(
+          static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, groups);
     return check_launch();
   }
   if (dx != nullptr && (dgamma_ != nullptr || dbeta_ != nullptr) && cols % EPV == 0 &&
       cols / EPV > 128 && cols / EPV <= 16 * 64 * 2 && aligned16(dx) && aligned16(dy) && aligned16(x) &&
-      (gamma == nullptr || aligned16(gamma)) && rows < (int64_t{1} << 31)) {
+      (gamma == nullptr || aligned16(gamma)) && (addend == nullptr || aligned16(addend)) &&
+      rows < (int64_t{1} << 31)) {
     const int64_t nvec = cols / EPV;
     const FusedPlan plan = fused_plan(rows, nvec);
+    const int nr = extra ? 3 : 2;
     if (workspace == nullptr ||
-        workspace_bytes < static_cast<size_t>(plan.padded_groups) * 2 * cols * 4)
+        workspace_bytes < static_cast<size_t>(plan.padded_groups) * nr * cols * 4)
       return TMB_ERR_WORKSPACE;
     float* partial = static_cast<float*>(workspace);
     const dim3 grid(static_cast<unsigned>(plan.padded_groups / plan.groups_per_block));
-#define TMB_LF(WPR, VPL, BLOCK)                                                               \
-  layer_norm_backward_fused_kernel<T, WPR, VPL, BLOCK><<<grid, dim3(BLOCK), 0, stream>>>(     \
-      dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), plan.walk);
+#define TMB_LF(WPR, VPL, BLOCK)                                                                      \
+  if (extra)                                                                                         \
+    layer_norm_backward_fused_kernel<T, WPR, VPL, BLOCK, true><<<grid, dim3(BLOCK), 0, stream>>>(    \
+        dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), plan.walk, addend);     \
+  else                                                                                               \
+    layer_norm_backward_fused_kernel<T, WPR, VPL, BLOCK, false><<<grid, dim3(BLOCK), 0, stream>>>(   \
+        dx, partial, dy, x, mean, rstd, gamma, rows, static_cast<int>(cols), plan.walk);
     // (groups past the last row write partial rows of zeros, which the final stage adds)
-    if (nvec <= 64) TMB_LF(1, 1, 256)
-    else if (nvec <= 128) TMB_LF(2, 1, 256)
-    else if (nvec <= 256) TMB_LF(2, 2, 256)
-    else if (nvec <= 512) TMB_LF(4, 2, 256)
-    else if (nvec <= 1024) TMB_LF(8, 2, 512)
-    else TMB_LF(16, 2, 1024)
+    if (nvec <= 64) { TMB_LF(1, 1, 256) }
+    else if (nvec <= 128) { TMB_LF(2, 1, 256) }
+    else if (nvec <= 256) { TMB_LF(2, 2, 256) }
+    else if (nvec <= 512) { TMB_LF(4, 2, 256) }
+    else if (nvec <= 1024) { TMB_LF(8, 2, 512) }
+    else { TMB_LF(16, 2, 1024) }
 #undef TMB_LF
     rc = check_launch();
     if (rc != 0) return rc;
-    layer_norm_param_final_kernel<T><<<dim3(static_cast<unsigned>((cols + 31) / 32)), dim3(1024), 0, stream>>>(
-        static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, plan.padded_groups);
+    const dim3 fgrid(static_cast<unsigned>((cols + 31) / 32));
+    if (extra)
+      layer_norm_param_final_kernel<T, 3><<<fgrid, dim3(1024), 0, stream>>>(
+          static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, plan.padded_groups,
+          static_cast<T*>(dsum_));
+    else
+      layer_norm_param_final_kernel<T, 2><<<fgrid, dim3(1024), 0, stream>>>(
+          static_cast<T*>(dgamma_), static_cast<T*>(dbeta_), partial, cols, plan.padded_groups);
     return check_launch();
   }
+  if (extra) return TMB_ERR_UNSUPPORTED;
   if (dx != nullptr) {
     const bool vec_ok = cols % EPV == 0 && aligned16(dx) && aligned16(dy) && aligned16(x) &&
                         (gamma == nullptr || aligned16(gamma)) && rows < (int64_t{1} << 31);
@@ -1089,6 +1191,40 @@ extern "C" size_t tmb_layer_norm_backward_workspace_bytes(int64_t rows, int64_t 
     if (cols <= 1024 && narrow > most) most = narrow;
   }
   return static_cast<size_t>(most) * 2 * static_cast<size_t>(cols) * 4;
+}
+
+extern "C" size_t tmb_layer_norm_backward_add_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
+  if (rows <= 0 || cols <= 0) return 0;
+  const int epv = dtype == TMB_F32 ? 4 : 8;
+  // (16-bit rows of more than 8192 columns run 1024-thread workgroups, whose 128 registers per
+  // lane the third set of column sums does not fit)
+  if (cols % epv != 0 || cols / epv > (dtype == TMB_F32 ? 16 * 64 * 2 : 16 * 64)) return 0;
+  const int64_t groups = cols <= 1024 ? tmb::narrow_groups(rows) : tmb::fused_plan(rows, cols / epv).padded_groups;
+  return static_cast<size_t>(groups) * 3 * static_cast<size_t>(cols) * 4;
+}
+
+extern "C" int tmb_layer_norm_backward_add_rows(void* grad_in, void* grad_gamma, void* grad_beta,
+                                                void* grad_sum, const void* grad_out, const void* in,
+                                                const float* mean, const float* rstd,
+                                                const void* gamma, const void* addend, int64_t rows,
+                                                int64_t cols, int dtype, void* workspace,
+                                                size_t workspace_bytes, void* stream) {
+  if (rows <= 0 || cols <= 0) return TMB_ERR_INVALID_ARGUMENT;
+  if (grad_in == nullptr || grad_gamma == nullptr || grad_beta == nullptr || grad_out == nullptr ||
+      in == nullptr || mean == nullptr || rstd == nullptr || (addend == nullptr && grad_sum == nullptr))
+    return TMB_ERR_INVALID_ARGUMENT;
+  if (tmb_layer_norm_backward_add_workspace_bytes(rows, cols, dtype) == 0) return TMB_ERR_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  using namespace tmb;
+  switch (dtype) {
+    case TMB_F32:
+      return layer_norm_backward_dispatch<float>(grad_in, grad_gamma, grad_beta, grad_out, in, mean, rstd, gamma, rows, cols, workspace, workspace_bytes, s, addend, grad_sum);
+    case TMB_F16:
+      return layer_norm_backward_dispatch<f16_t>(grad_in, grad_gamma, grad_beta, grad_out, in, mean, rstd, gamma, rows, cols, workspace, workspace_bytes, s, addend, grad_sum);
+    case TMB_BF16:
+      return layer_norm_backward_dispatch<bf16_t>(grad_in, grad_gamma, grad_beta, grad_out, in, mean, rstd, gamma, rows, cols, workspace, workspace_bytes, s, addend, grad_sum);
+    default: return TMB_ERR_UNSUPPORTED;
+  }
 }
 
 extern "C" int tmb_layer_norm_backward_rows(void* grad_in, void* grad_gamma, void* grad_beta,

@@ -54,6 +54,8 @@ SIGNATURES = {
     "tmb_nll_log_softmax_backward_rows": (_ci, [_vp] * 5 + [_i64] * 4 + [_ci, _i64, _ci, _vp]),
     "tmb_layer_norm_backward_workspace_bytes": (_sz, [_i64, _i64, _ci]),
     "tmb_layer_norm_backward_rows": (_ci, [_vp] * 8 + [_i64, _i64, _ci, _vp, _sz, _vp]),
+    "tmb_layer_norm_backward_add_workspace_bytes": (_sz, [_i64, _i64, _ci]),
+    "tmb_layer_norm_backward_add_rows": (_ci, [_vp] * 10 + [_i64, _i64, _ci, _vp, _sz, _vp]),
     "tmb_copy_bytes": (_ci, [_vp, _vp, _sz, _vp]),
     "tmb_read_bytes": (_ci, [_vp, _sz, _vp, _vp]),
     "tmb_cat2_rows": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),

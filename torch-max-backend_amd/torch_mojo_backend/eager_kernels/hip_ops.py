@@ -1010,6 +1010,59 @@ def layer_norm_backward(grad: torch.Tensor, x: torch.Tensor, normalized_shape: S
     return dx, dw, db
 
 
+def layer_norm_backward_add(grad: torch.Tensor, x: torch.Tensor, normalized_shape: Sequence[int],
+                            mean: torch.Tensor, rstd: torch.Tensor, weight: Optional[torch.Tensor],
+                            addend: Optional[torch.Tensor], want_sum: bool):
+    """``layer_norm_backward`` with all three outputs where its grad_input re-joins a residual
+    stream: returns (grad_input + addend, grad_weight, grad_bias, column sums of the first over
+    all leading dimensions or None), each stored in the tensor type step by step as the separate
+    ops would (this one, ``aten.add``, ``aten.sum``). Returns None when the shape is outside the
+    one-pass kernels: the caller then runs the separate ops."""
+    require_hip(grad, x, mean, rstd, weight, addend)
+    normalized_shape = tuple(normalized_shape)
+    k = len(normalized_shape)
+    if addend is None and not want_sum:
+        raise ValueError("layer_norm_backward_add: neither an addend nor the column sums are asked for")
+    if x.dtype not in FLOAT_DTYPES or grad.dtype != x.dtype or grad.shape != x.shape or k < 1 \
+            or tuple(x.shape[x.dim() - k:]) != normalized_shape:
+        raise ValueError(f"layer_norm_backward_add: grad {tuple(grad.shape)} {grad.dtype}, input "
+                         f"{tuple(x.shape)} {x.dtype}, normalized_shape {normalized_shape}")
+    if addend is not None and (addend.dtype != x.dtype or addend.shape != x.shape):
+        raise ValueError(f"layer_norm_backward_add: addend {tuple(addend.shape)} {addend.dtype} for "
+                         f"input {tuple(x.shape)} {x.dtype}")
+    cols = math.prod(normalized_shape)
+    rows = x.numel() // cols if cols else 0
+    if mean.dtype != torch.float32 or rstd.dtype != torch.float32 or mean.numel() != rows \
+            or rstd.numel() != rows:
+        raise ValueError("layer_norm_backward_add: mean / rstd must be float32 with one value per row")
+    if weight is not None and (weight.dtype != x.dtype or tuple(weight.shape) != normalized_shape):
+        raise ValueError(f"layer_norm_backward_add: weight must be {normalized_shape} {x.dtype}")
+    if rows == 0 or cols == 0:
+        return None
+    code = code_of(x.dtype)
+    lib = _ek.lib()
+    ws_bytes = int(lib.tmb_layer_norm_backward_add_workspace_bytes(rows, cols, code))
+    if ws_bytes == 0:
+        return None
+    gc, xc = grad.contiguous(), x.contiguous()
+    ac = None if addend is None else addend.contiguous()
+    wc = None if weight is None else weight.contiguous()
+    dx = torch.empty_like(xc)
+    dw = torch.empty(normalized_shape, dtype=x.dtype, device=x.device)
+    db = torch.empty(normalized_shape, dtype=x.dtype, device=x.device)
+    ds = torch.empty(normalized_shape, dtype=x.dtype, device=x.device) if want_sum else None
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    rc = lib.tmb_layer_norm_backward_add_rows(
+        dx.data_ptr(), dw.data_ptr(), db.data_ptr(), None if ds is None else ds.data_ptr(),
+        gc.data_ptr(), xc.data_ptr(), mean.contiguous().data_ptr(), rstd.contiguous().data_ptr(),
+        None if wc is None else wc.data_ptr(), None if ac is None else ac.data_ptr(), rows, cols,
+        code, ws.data_ptr(), ws_bytes, _stream())
+    if rc == _ek.ERR_UNSUPPORTED:
+        return None
+    _check("tmb_layer_norm_backward_add_rows", rc)
+    return dx, dw, db, ds
+
+
 def linear_backward(x: torch.Tensor, grad: torch.Tensor, weight: torch.Tensor,
                     output_mask: Sequence[bool]):
     """(grad_input, grad_weight, grad_bias) of ``x @ weight.T + bias`` (reference:
