@@ -697,7 +697,42 @@ def main() -> int:
             row["cpu_note"] = (f"PyTorch CPU eager fp32 of the same module at B={cb}, T={ct} "
                                f"(the workload's CPU configuration), {cpu_threads} threads")
         sweep[f"gpt2_small_fwd_bf16_B{B}_T{T}"] = row
-        del model, compiled
+        # the workload's small configuration (B=1, T=128) is bound by the host's step per node:
+        # the same forward step by step and as replays of one recorded HIP graph
+        # (TORCH_MOJO_BACKEND_HIP_GRAPH=1), beside PyTorch-ROCm eager
+        torch._dynamo.reset()
+        sb, st = 1, 128
+        sidx = seeded_tokens(sb, st, seed=0).to(dev)
+        small = torch.compile(model, backend=mojo_backend, fullgraph=True)
+        small_row = {"batch": sb, "seq": st, "dtype": "bf16"}
+        saved_flag = os.environ.get("TORCH_MOJO_BACKEND_HIP_GRAPH")
+        try:
+            with torch.no_grad():
+                for flag, key in (("0", "ms_step_by_step"), ("1", "ms_hip_graph_replay")):
+                    os.environ["TORCH_MOJO_BACKEND_HIP_GRAPH"] = flag
+                    for _ in range(3):
+                        small(sidx)
+                    sync()
+                    t0 = time.perf_counter()
+                    for _ in range(30):
+                        small(sidx)
+                    sync()
+                    small_row[key] = round((time.perf_counter() - t0) / 30 * 1e3, 3)
+                for _ in range(3):
+                    model(sidx)
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(30):
+                    model(sidx)
+                sync()
+                small_row["pytorch_rocm_eager_ms"] = round((time.perf_counter() - t0) / 30 * 1e3, 3)
+        finally:
+            if saved_flag is None:
+                os.environ.pop("TORCH_MOJO_BACKEND_HIP_GRAPH", None)
+            else:
+                os.environ["TORCH_MOJO_BACKEND_HIP_GRAPH"] = saved_flag
+        sweep[f"gpt2_small_fwd_bf16_B{sb}_T{st}"] = small_row
+        del model, compiled, small
 
     # ------------------------------------------------------------------ GPT-2 training step
     # Forward + backward of the same module through mojo_backend (bf16, B=16, T=1024, mean

@@ -44,3 +44,16 @@ def cache_host_parameters() -> bool:
     moment, as the reference's aliasing buffer import sees them
     (torch_compile_backend/compiler.py:535-566)."""
     return _flag("CACHE_HOST_PARAMETERS")
+
+
+def hip_graph() -> bool:
+    """Inference graphs over HIP tensors: after one ordinary run per set of input shapes the step
+    program is captured into a HIP graph and later calls replay it (one graph launch instead of a
+    Python step per node; a launch-bound forward such as GPT-2 small at batch 1 runs several times
+    faster). Inputs whose address changes from call to call are copied into buffers the graph
+    owns, results are handed out as copies. Off by default: the graph keeps the memory of one
+    whole run, and what the steps decide on the host while it is recorded (a mask buffer found to
+    be causal) stays decided until an input's address, shape or version counter changes. The
+    reference has no counterpart (MAX compiles the whole graph; its executor is one call,
+    torch_compile_backend/compiler.py:455-532)."""
+    return _flag("HIP_GRAPH")

@@ -34,6 +34,7 @@ import operator
 import os
 import time
 import traceback
+import weakref
 from typing import Any, Callable, List, Optional
 
 import torch
@@ -46,7 +47,7 @@ from torch_mojo_backend.aten_functions import (
     DECOMPOSITION_TABLE,
     MAPPING_TORCH_ATEN_TO_MOJO,
 )
-from torch_mojo_backend.flags import (cache_host_parameters, debug_graph, profiling_enabled,
+from torch_mojo_backend.flags import (cache_host_parameters, debug_graph, hip_graph, profiling_enabled,
                                       round_like_unfused, verbose_enabled)
 from torch_mojo_backend.torch_compile_backend.utils import get_accelerators, get_error_message
 
@@ -1283,8 +1284,12 @@ class BaseMaxCompiler:
     on a HIP device, on the eager `mojo` device (wrappers over HIP memory: consumed and returned
     zero-copy) or on the host (copied in, results copied back: there is no CPU kernel path)."""
 
-    def __init__(self, gm: torch.fx.GraphModule, example_inputs: list, mode=None):
+    def __init__(self, gm: torch.fx.GraphModule, example_inputs: list, mode=None, inference: bool = False):
         self.gm = gm
+        # HIP-graph replays (flags.hip_graph): only graphs that hand nothing to a backward pass
+        self.inference = inference
+        self.replays: dict = {}
+        self.last_replay = None
         start = time.time_ns() if profiling_enabled() else 0
         if verbose_enabled():
             print(f"Graph has {len(gm.graph.nodes)} nodes.")
@@ -1325,6 +1330,59 @@ class BaseMaxCompiler:
         ) from exc
 
     def __call__(self, *args) -> list:
+        if self.inference and self.run_device is None and self.home == "cuda" and hip_graph() \
+                and not COLLECT_OP_TIMINGS and not debug_graph():
+            replayed = self._replay(args)
+            if replayed is not None:
+                return replayed
+        return self._run(args)
+
+    # ---- HIP-graph replays ------------------------------------------------------------------
+    _MAX_REPLAY_KEYS = 8
+
+    def _replay(self, args):
+        """The results of this call from a captured HIP graph, or None when the call has to run
+        step by step: the first call per key (shapes, strides, types and non-tensor values of the
+        inputs) runs ordinarily and notes the input addresses, the second records the graph."""
+        last = self.last_replay
+        if last is not None:      # the graph of the call before, checked without building a key
+            out = last.run(args)
+            if out is not None:
+                return out
+        key = tuple((tuple(a.shape), tuple(a.stride()), a.dtype, a.device.index)
+                    if isinstance(a, torch.Tensor) else ("value", a) for a in args)
+        state = self.replays.get(key)
+        if state is False:
+            return None
+        tensors_ok = all(a.is_cuda for a in args if isinstance(a, torch.Tensor))
+        if state is None:
+            if len(self.replays) >= self._MAX_REPLAY_KEYS or not tensors_ok:
+                self.replays[key] = False
+                return None
+            self.replays[key] = ("seen", [weakref.ref(a) if isinstance(a, torch.Tensor) else None for a in args])
+            return None
+        if not tensors_ok:
+            self.replays[key] = False
+            return None
+        if isinstance(state, tuple):   # ("seen", the tensors of the call before)
+            try:
+                state = _CapturedRun(self, args, state[1])
+            except Exception as exc:  # noqa: BLE001 - a step that cannot be recorded: run step by step
+                if verbose_enabled():
+                    print(f"[mojo_backend] graph not recorded, running step by step: {exc!r}")
+                self.replays[key] = False
+                return None
+            self.replays[key] = state
+        out = state.run(args)
+        if out is None:   # an input the graph reads in place has moved or was written to
+            del self.replays[key]
+            if self.last_replay is state:
+                self.last_replay = None
+        else:
+            self.last_replay = state
+        return out
+
+    def _run(self, args) -> list:
         start = time.time_ns() if profiling_enabled() else 0
         program = self.program
         env: List[Any] = [None] * self.num_slots
@@ -1402,6 +1460,65 @@ class BaseMaxCompiler:
         return value.cpu()
 
 
+GRAPH_REPLAYS = {"recorded": 0, "replayed": 0}   # counters, for tests and diagnostics
+
+
+class _CapturedRun:
+    """One HIP graph of a step program for one input key. Inputs that are parameters, or the very
+    tensor objects the call before was given, are read where they are (their address, and for
+    anything but a parameter the version counter, must still stand at every replay: the steps may
+    have decided something from their contents while the graph was recorded); all others are
+    copied into a buffer of the graph's before each replay. Results are handed out as copies, the
+    graph's own result tensors are overwritten by the next replay."""
+
+    def __init__(self, owner: "BaseMaxCompiler", args, seen):
+        self.inputs = []
+        self.copied = []      # positions whose value is copied in
+        self.values = []      # positions of non-tensor inputs
+        self.in_place = []    # (position, address, version or None)
+        for i, a in enumerate(args):
+            if not isinstance(a, torch.Tensor):
+                self.inputs.append(a)
+                self.values.append(i)
+            elif isinstance(a, torch.nn.Parameter):
+                self.inputs.append(a)
+                self.in_place.append((i, a.data_ptr(), None))
+            elif seen[i]() is a:   # the very tensor of the call before: a module's buffer
+                self.inputs.append(a)
+                self.in_place.append((i, a.data_ptr(), a._version))
+            else:
+                self.inputs.append(a.clone())
+                self.copied.append(i)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.results = owner._run(self.inputs)
+        GRAPH_REPLAYS["recorded"] += 1
+
+    def run(self, args):
+        """The results of a replay with these inputs, or None if they are not the ones this graph
+        was recorded for."""
+        inputs = self.inputs
+        if len(args) != len(inputs):
+            return None
+        for i, ptr, version in self.in_place:
+            a = args[i]
+            if a is not inputs[i] or a.data_ptr() != ptr or (version is not None and a._version != version):
+                return None
+        for i in self.copied:
+            a, mine = args[i], inputs[i]
+            if not isinstance(a, torch.Tensor) or a.shape != mine.shape or a.dtype != mine.dtype \
+                    or a.device != mine.device or a.stride() != mine.stride():
+                return None
+        for i in self.values:
+            if type(args[i]) is not type(inputs[i]) or args[i] != inputs[i]:
+                return None
+        for i in self.copied:
+            inputs[i].copy_(args[i])
+        self.graph.replay()
+        GRAPH_REPLAYS["replayed"] += 1
+        return [r.clone() if isinstance(r, torch.Tensor) else r for r in self.results]
+
+
 def _compare_with_torch(step: _Step, args, kwargs, out) -> None:
     """TORCH_MOJO_BACKEND_DEBUG_GRAPH=1: run the node's own aten op with PyTorch-ROCm and report
     the largest deviation (the reference compares MAX against torch per node, debug.py:27-128)."""
@@ -1431,6 +1548,11 @@ def _compare_with_torch(step: _Step, args, kwargs, out) -> None:
 
 def boxed_func(*args, **kwargs):
     return make_boxed_func(BaseMaxCompiler(*args, **kwargs).__call__)
+
+
+def boxed_inference_func(*args, **kwargs):
+    """The compiler of graphs no backward pass follows (aot_autograd's `inference_compiler`)."""
+    return make_boxed_func(BaseMaxCompiler(*args, inference=True, **kwargs).__call__)
 
 
 def _match_forward_attention(joint_module: torch.fx.GraphModule, num_fwd_outputs: int):
@@ -1672,8 +1794,8 @@ class mojo_backend:
         _REAL_EXAMPLE_INPUTS.append(list(example_inputs))
         try:
             self.func_to_execute = aot_autograd(
-                fw_compiler=boxed_func, partition_fn=attention_recompute_partition,
-                decompositions=DECOMPOSITION_TABLE
+                fw_compiler=boxed_func, inference_compiler=boxed_inference_func,
+                partition_fn=attention_recompute_partition, decompositions=DECOMPOSITION_TABLE
             )(gm, example_inputs)
         finally:
             _REAL_EXAMPLE_INPUTS.pop()
