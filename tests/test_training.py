@@ -17,7 +17,8 @@ CHECKS = ["gpt2_training_step_gradients_match_cpu", "training_graph_runs_the_fus
           "log_softmax_and_linear_backward_in_a_compiled_graph",
           "vocabulary_projection_backward_pads_its_gradient_once",
           "cross_entropy_in_the_graph_sends_one_pass_back_to_the_logits",
-          "residual_gradient_joins_inside_the_layer_norm_backward"]
+          "residual_gradient_joins_inside_the_layer_norm_backward",
+          "training_graphs_are_never_replayed"]
 
 
 @pytest.mark.parametrize("check", CHECKS)

@@ -384,6 +384,34 @@ def residual_gradient_joins_inside_the_layer_norm_backward():
                 assert (got.double() - want.double()).abs().max().item() <= tol * scale, (dtype, name)
 
 
+def training_graphs_are_never_replayed():
+    """TORCH_MOJO_BACKEND_HIP_GRAPH=1 records inference graphs only: the forward graph of a
+    training step hands tensors to the backward pass, and neither of the two is ever replayed."""
+    import os
+
+    from demo_scripts.gpt2 import build_gpt2_small, seeded_tokens
+    from torch_mojo_backend import mojo_backend
+    from torch_mojo_backend.torch_compile_backend import compiler
+
+    os.environ["TORCH_MOJO_BACKEND_HIP_GRAPH"] = "1"
+    model = build_gpt2_small(seed=0, n_layer=1).bfloat16().cuda().train()
+    compiled = torch.compile(model, backend=mojo_backend)
+    before = dict(compiler.GRAPH_REPLAYS)
+    for seed in range(3):
+        logits, _ = compiled(seeded_tokens(2, 32, seed=seed).cuda())
+        logits.float().sum().backward()
+    torch.cuda.synchronize()
+    assert compiler.GRAPH_REPLAYS == before, compiler.GRAPH_REPLAYS
+    assert all(p.grad is not None for p in model.parameters())
+    # the same module under no_grad is an inference graph: recorded at its second call
+    with torch.no_grad():
+        idx = seeded_tokens(2, 32, seed=5).cuda()
+        outs = [compiled(idx)[0] for _ in range(4)]
+    torch.cuda.synchronize()
+    assert compiler.GRAPH_REPLAYS["recorded"] == before["recorded"] + 1
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
+
+
 if __name__ == "__main__":
     import os
 
