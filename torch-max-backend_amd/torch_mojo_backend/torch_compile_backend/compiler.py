@@ -180,9 +180,24 @@ def _materialize(value, env):
     return value
 
 
+def _flat_plan(args):
+    """(template list, ((position, slot index), ...)) for an argument tuple whose slots all sit at
+    its top level (what most nodes have: tensors and a few constants), else None. The executor
+    then fills a copy of the template instead of walking the arguments recursively."""
+    if not isinstance(args, tuple):
+        return None
+    fills = []
+    for pos, value in enumerate(args):
+        if isinstance(value, _Slot):
+            fills.append((pos, value.index))
+        elif _has_slot(value) or isinstance(value, slice):
+            return None
+    return [None if isinstance(v, _Slot) else v for v in args], tuple(fills)
+
+
 class _Step:
     __slots__ = ("fn", "args", "kwargs", "dynamic_args", "dynamic_kwargs", "out", "node",
-                 "node_idx", "release", "key")
+                 "node_idx", "release", "key", "flat")
 
 
 class _GraphFactory:
@@ -771,6 +786,7 @@ class _GraphFactory:
                 step.kwargs = self._convert(kwargs)
                 step.dynamic_args = _has_slot(step.args)
                 step.dynamic_kwargs = _has_slot(step.kwargs)
+                step.flat = _flat_plan(step.args) if step.dynamic_args else None
                 self.slots[node.name] = len(self.slots)
                 step.out = self.slots[node.name]
                 step.node = node
@@ -1426,7 +1442,13 @@ class BaseMaxCompiler:
 
     def _run_steps(self, program, env, check) -> None:
         for step in program.steps:
-            a = _materialize(step.args, env) if step.dynamic_args else step.args
+            flat = step.flat
+            if flat is not None:
+                a = flat[0].copy()
+                for pos, index in flat[1]:
+                    a[pos] = env[index]
+            else:
+                a = _materialize(step.args, env) if step.dynamic_args else step.args
             kw = _materialize(step.kwargs, env) if step.dynamic_kwargs else step.kwargs
             token = CURRENT_FX_NODE.set(step.node)
             if COLLECT_OP_TIMINGS:
